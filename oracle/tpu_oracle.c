@@ -1,0 +1,443 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- see tpu_oracle.h.  CPU restatement of the
+ * tpuc-interpreter INT8 arithmetic; the checker for the HIP kernels.
+ *
+ * Build: make -C oracle   (gcc, -ffp-contract=off so no fused multiply-add
+ * can change a float result).
+ */
+#include "tpu_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------- */
+/* scalar arithmetic                                                          */
+/* ------------------------------------------------------------------------- */
+
+/* QuantizationArithmetic.cpp:501-509.  C '/' truncates toward zero; with the
+ * sign-dependent nudge this rounds a*b/2^31 to nearest, ties toward +inf.  The
+ * final static_cast keeps the low 32 bits. */
+int32_t orc_srdhm(int32_t a, int32_t b) {
+  int64_t ab = (int64_t)a * (int64_t)b;
+  int32_t nudge = ab >= 0 ? (1 << 30) : (1 - (1 << 30));
+  int64_t q = (ab + nudge) / (1ll << 31);
+  return (int32_t)(uint32_t)(uint64_t)q;
+}
+
+/* QuantizationArithmetic.cpp:487-499 */
+int32_t orc_rdbp(int32_t x, int exponent) {
+  if (x == 0) return 0;
+  if (exponent == 0) return x;
+  if (exponent < 0 || exponent > 31) return x; /* outside the reference's assert */
+  const int32_t mask = (int32_t)((1ll << exponent) - 1);
+  const int32_t remainder = x & mask;
+  const int32_t threshold = (mask >> 1) + ((x < 0) ? 1 : 0);
+  return (x >> exponent) + ((remainder > threshold) ? 1 : 0);
+}
+
+/* QuantizationArithmetic.cpp:301-334: "int q = floor(f + 0.5)" -- the sum is
+ * formed in double (0.5 is a double literal), so it is exact. */
+int8_t orc_saturate_int8(float f) {
+  double s = floor((double)f + 0.5);
+  int q;
+  /* the reference converts the double to int; outside int range that is
+   * undefined, x86 yields INT_MIN.  Clamp first: same result wherever the
+   * reference's is defined, and saturation for the rest. */
+  if (s > 127.0)
+    q = 127;
+  else if (s < -128.0)
+    q = -128;
+  else
+    q = (int)s;
+  return (int8_t)q;
+}
+
+/* QuantizationArithmetic.cpp:481-483: v / (1 << rshift) in float */
+int8_t orc_apply_rshift_sat8(float v, uint32_t rshift) {
+  return orc_saturate_int8(v / (float)(1 << rshift));
+}
+
+/* QuantizationArithmetic.cpp:518-528 */
+int8_t orc_apply_mult_rshift_sat8_f(float v, uint32_t rshift, uint32_t multiplier, int qdm) {
+  if (qdm) {
+    int32_t q = orc_rdbp(orc_srdhm((int32_t)v, (int32_t)multiplier), (int)rshift);
+    return orc_saturate_int8((float)q);
+  }
+  /* float * uint32 -> float product, then float / int -> float quotient */
+  float prod = v * (float)multiplier;
+  return orc_saturate_int8(prod / (float)(1 << rshift));
+}
+
+/* QuantizationArithmetic.cpp:530-539.  Without qdm "v * multiplier" is int32 *
+ * uint32, i.e. unsigned arithmetic, and so is the division. */
+int8_t orc_apply_mult_rshift_sat8_i(int32_t v, uint32_t rshift, uint32_t multiplier, int qdm) {
+  if (qdm) {
+    int32_t q = orc_rdbp(orc_srdhm(v, (int32_t)multiplier), (int)rshift);
+    return orc_saturate_int8((float)q);
+  }
+  uint32_t prod = (uint32_t)v * multiplier;
+  uint32_t quo = prod / (uint32_t)(1 << rshift);
+  return orc_saturate_int8((float)quo);
+}
+
+uint32_t orc_f2u32(float f) { return (uint32_t)(uint64_t)(int64_t)f; }
+
+/* ------------------------------------------------------------------------- */
+/* convolution                                                                */
+/* ------------------------------------------------------------------------- */
+
+static inline int div_floor(int a, int b) { /* b > 0 */
+  int q = a / b, r = a % b;
+  return (r != 0 && r < 0) ? q - 1 : q;
+}
+static inline int div_ceil(int a, int b) { return -div_floor(-a, b); }
+
+/* valid output range [lo, hi) along one axis for a tap at offset 'koff'
+ * (= k*dilation - pad) over an input extent 'in' with stride s */
+static inline void tap_range(int koff, int s, int in, int out, int *lo, int *hi) {
+  int l = div_ceil(-koff, s);
+  int h = div_floor(in - 1 - koff, s) + 1;
+  if (l < 0) l = 0;
+  if (h > out) h = out;
+  *lo = l;
+  *hi = h;
+}
+
+#define CONV_BODY(ACC_T, X_T, W_T, MUL)                                                     \
+  const int icg = d->ic / d->g, ocg = d->oc / d->g;                                         \
+  const int ihd = (d->ih - 1) * (d->ins_h + 1) + 1;                                         \
+  const int iwd = (d->iw - 1) * (d->ins_w + 1) + 1;                                         \
+  const int64_t osz = (int64_t)d->oh * d->ow;                                               \
+  _Pragma("omp parallel for collapse(2) schedule(dynamic, 1)")                              \
+  for (int n = 0; n < d->n; ++n) {                                                          \
+    for (int oc = 0; oc < d->oc; ++oc) {                                                    \
+      ACC_T *a = acc + ((int64_t)n * d->oc + oc) * osz;                                     \
+      for (int64_t i = 0; i < osz; ++i) a[i] = 0;                                           \
+      const int gi = oc / ocg;                                                              \
+      for (int c = 0; c < icg; ++c) {                                                       \
+        const X_T *xp = x + ((int64_t)n * d->ic + (int64_t)gi * icg + c) * d->ih * d->iw;   \
+        for (int kh = 0; kh < d->kh; ++kh) {                                                \
+          for (int kw = 0; kw < d->kw; ++kw) {                                              \
+            const W_T wv = w[(((int64_t)oc * icg + c) * d->kh + kh) * d->kw + kw];          \
+            if (wv == 0) continue;                                                          \
+            const int hoff = kh * d->dh - d->pt, woff = kw * d->dw - d->pl;                 \
+            int oh0, oh1, ow0, ow1;                                                         \
+            tap_range(hoff, d->sh, ihd, d->oh, &oh0, &oh1);                                 \
+            tap_range(woff, d->sw, iwd, d->ow, &ow0, &ow1);                                 \
+            for (int oh = oh0; oh < oh1; ++oh) {                                            \
+              const int hp = oh * d->sh + hoff;                                             \
+              if (d->ins_h && (hp % (d->ins_h + 1))) continue;                              \
+              const X_T *xr = xp + (int64_t)(hp / (d->ins_h + 1)) * d->iw;                  \
+              ACC_T *ar = a + (int64_t)oh * d->ow;                                          \
+              if (d->ins_w == 0 && d->sw == 1) {                                            \
+                const X_T *xs = xr + woff;                                                  \
+                for (int ow = ow0; ow < ow1; ++ow) ar[ow] += MUL(wv, xs[ow]);               \
+              } else if (d->ins_w == 0) {                                                   \
+                for (int ow = ow0; ow < ow1; ++ow) ar[ow] += MUL(wv, xr[ow * d->sw + woff]); \
+              } else {                                                                      \
+                for (int ow = ow0; ow < ow1; ++ow) {                                        \
+                  const int wp = ow * d->sw + woff;                                         \
+                  if (wp % (d->ins_w + 1)) continue;                                        \
+                  ar[ow] += MUL(wv, xr[wp / (d->ins_w + 1)]);                               \
+                }                                                                           \
+              }                                                                             \
+            }                                                                               \
+          }                                                                                 \
+        }                                                                                   \
+      }                                                                                     \
+    }                                                                                       \
+  }
+
+#define MUL_I32(a, b) ((int32_t)(a) * (int32_t)(b))
+#define MUL_ABS(a, b) (abs((int32_t)(a)) * abs((int32_t)(b)))
+#define MUL_F32(a, b) ((a) * (b))
+
+/* include/tpuc/NativeCpuImplementation.h:11-102 (MKL-DNN convolution_direct,
+ * zero padding, dilation passed as d-1, groups) restated as the integer
+ * cross-correlation it computes inside the exact domain. */
+void orc_conv2d_acc(const int8_t *x, const int8_t *w, int32_t *acc, const orc_conv_desc *d) {
+  CONV_BODY(int32_t, int8_t, int8_t, MUL_I32)
+}
+
+static void conv2d_abs(const int8_t *x, const int8_t *w, int32_t *acc, const orc_conv_desc *d) {
+  CONV_BODY(int32_t, int8_t, int8_t, MUL_ABS)
+}
+
+void orc_conv2d_acc_f32(const float *x, const float *w, float *acc, const orc_conv_desc *d) {
+  CONV_BODY(float, float, float, MUL_F32)
+}
+
+int64_t orc_conv2d_guard(const int8_t *x, const int8_t *w, const orc_conv_desc *d) {
+  const int64_t total = (int64_t)d->n * d->oc * d->oh * d->ow;
+  int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)total);
+  conv2d_abs(x, w, acc, d);
+  int64_t m = 0;
+  for (int64_t i = 0; i < total; ++i)
+    if (acc[i] > m) m = acc[i];
+  free(acc);
+  return m;
+}
+
+/* QuantizationArithmetic.cpp:849-871 */
+void orc_requant_per_channel(const int32_t *acc, int8_t *y, const float *bias, int do_relu,
+                             int64_t on, int64_t oc, int64_t isz, const float *rshift,
+                             const float *multiplier) {
+#pragma omp parallel for collapse(2)
+  for (int64_t n = 0; n < on; ++n) {
+    for (int64_t i = 0; i < oc; ++i) {
+      /* the float -> uint32_t conversions happen at the call (:863-865) */
+      const uint32_t rs = orc_f2u32(rshift[i]);
+      const uint32_t mu = orc_f2u32(multiplier[i]);
+      const int32_t b = bias ? (int32_t)bias[i] : 0;
+      for (int64_t j = 0; j < isz; ++j) {
+        int32_t v = acc[n * oc * isz + i * isz + j];
+        v = (int32_t)((uint32_t)v + (uint32_t)b);
+        v = orc_apply_mult_rshift_sat8_i(v, rs, mu, 1);
+        if (do_relu && v < 0) v = 0;
+        y[n * oc * isz + i * isz + j] = (int8_t)v;
+      }
+    }
+  }
+}
+
+/* conv.cpp:80-104, INT8 branch.  The MKL-DNN conv runs with a zero bias
+ * (:57-65); the int32 bias is added in the epilogue.  Without with_bias the
+ * epilogue adds a zero tensor (:59-61). */
+void orc_conv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                   const float *multiplier, int8_t *y, const orc_conv_desc *d) {
+  const int64_t total = (int64_t)d->n * d->oc * d->oh * d->ow;
+  int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)total);
+  orc_conv2d_acc(x, w, acc, d);
+  orc_requant_per_channel(acc, y, d->with_bias ? bias : NULL, d->do_relu, d->n, d->oc,
+                          (int64_t)d->oh * d->ow, rshift, multiplier);
+  free(acc);
+}
+
+/* ------------------------------------------------------------------------- */
+/* fully connected                                                            */
+/* ------------------------------------------------------------------------- */
+
+/* fullyconnected.cpp:44-91: inner product (weights n x k, NativeCpuImplementation.cpp:185-288)
+ * with the bias added inside the fp32 primitive, ReLU on the float sums, then
+ * one qdm requant per batch matmul (rshift_data->at(i), multiplier_data->at(i)).
+ * Inside the exact domain the fp32 sum equals the integer sum, which is what
+ * is computed here. */
+void orc_fc_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+               const float *multiplier, int8_t *y, int batch, int m, int k, int n, int do_relu) {
+  for (int b = 0; b < batch; ++b) {
+    const uint32_t rs = orc_f2u32(rshift[b]);
+    const uint32_t mu = orc_f2u32(multiplier[b]);
+#pragma omp parallel for collapse(2)
+    for (int i = 0; i < m; ++i) {
+      for (int j = 0; j < n; ++j) {
+        const int8_t *xr = x + ((int64_t)b * m + i) * k;
+        const int8_t *wr = w + ((int64_t)b * n + j) * k;
+        int32_t s = 0;
+        for (int t = 0; t < k; ++t) s += (int32_t)xr[t] * (int32_t)wr[t];
+        float f = (float)s;
+        if (bias) f = (float)(s + (int32_t)bias[(int64_t)b * n + j]);
+        if (do_relu && !(f > 0)) f = 0;
+        y[((int64_t)b * m + i) * n + j] = orc_apply_mult_rshift_sat8_f(f, rs, mu, 1);
+      }
+    }
+  }
+}
+
+int64_t orc_fc_guard(const int8_t *x, const int8_t *w, const float *bias, int batch, int m, int k,
+                     int n) {
+  int64_t worst = 0;
+  for (int b = 0; b < batch; ++b)
+    for (int i = 0; i < m; ++i)
+      for (int j = 0; j < n; ++j) {
+        const int8_t *xr = x + ((int64_t)b * m + i) * k;
+        const int8_t *wr = w + ((int64_t)b * n + j) * k;
+        int64_t s = 0;
+        for (int t = 0; t < k; ++t) s += llabs((int64_t)xr[t] * wr[t]);
+        if (bias) s += llabs((int64_t)bias[(int64_t)b * n + j]);
+        if (s > worst) worst = s;
+      }
+  return worst;
+}
+
+/* ------------------------------------------------------------------------- */
+/* eltwise add                                                                */
+/* ------------------------------------------------------------------------- */
+
+/* eltwise.cpp:52-85: each input times (int8_t)multiplier[i] in float, summed
+ * in float, ReLU, then v / 2^rshift[0] in float and floor(.+0.5), saturate. */
+void orc_eltwise_add_i8(const int8_t *const *xs, int nin, const float *multiplier,
+                        const float *rshift, int do_relu, int8_t *y, size_t count) {
+  const uint32_t rs = orc_f2u32(rshift[0]);
+#pragma omp parallel for
+  for (size_t i = 0; i < count; ++i) {
+    float s = 0;
+    for (int k = 0; k < nin; ++k) {
+      float t = (float)xs[k][i];
+      t *= (int8_t)(int)multiplier[k];
+      s += t;
+    }
+    if (do_relu) s = s > 0 ? s : 0;
+    y[i] = orc_apply_rshift_sat8(s, rs);
+  }
+}
+
+/* ------------------------------------------------------------------------- */
+/* pooling                                                                    */
+/* ------------------------------------------------------------------------- */
+
+/* pooling.cpp:155-157 -> MKLPooling (NativeCpuImplementation.h:104-174):
+ * pooling_max ignores padded positions. */
+void orc_pool_max_i8(const int8_t *x, int8_t *y, const orc_pool_desc *d) {
+#pragma omp parallel for
+  for (int64_t nc = 0; nc < (int64_t)d->n * d->c; ++nc) {
+    const int8_t *xp = x + nc * d->ih * d->iw;
+    int8_t *yp = y + nc * d->oh * d->ow;
+    for (int oh = 0; oh < d->oh; ++oh)
+      for (int ow = 0; ow < d->ow; ++ow) {
+        int best = -128; /* an all-padding window cannot occur for valid shapes */
+        for (int kh = 0; kh < d->kh; ++kh) {
+          int ih = oh * d->sh - d->pt + kh;
+          if (ih < 0 || ih >= d->ih) continue;
+          for (int kw = 0; kw < d->kw; ++kw) {
+            int iw = ow * d->sw - d->pl + kw;
+            if (iw < 0 || iw >= d->iw) continue;
+            int v = xp[ih * d->iw + iw];
+            if (v > best) best = v;
+          }
+        }
+        yp[oh * d->ow + ow] = (int8_t)best;
+      }
+  }
+}
+
+/* pooling.cpp:72-82,147-154: depthwise fp32 conv with an all-ones filter and
+ * zero padding (MKLInt8AvgPooling, NativeCpuImplementation.h:176-192) = window
+ * sum that counts padding as zeros; then the non-qdm float overload with the
+ * scalar (uint32_t)rshift / (uint32_t)multiplier. */
+void orc_pool_avg_i8(const int8_t *x, int8_t *y, const orc_pool_desc *d, float rshift,
+                     float multiplier) {
+  const uint32_t rs = orc_f2u32(rshift);
+  const uint32_t mu = orc_f2u32(multiplier);
+#pragma omp parallel for
+  for (int64_t nc = 0; nc < (int64_t)d->n * d->c; ++nc) {
+    const int8_t *xp = x + nc * d->ih * d->iw;
+    int8_t *yp = y + nc * d->oh * d->ow;
+    for (int oh = 0; oh < d->oh; ++oh)
+      for (int ow = 0; ow < d->ow; ++ow) {
+        int32_t s = 0;
+        for (int kh = 0; kh < d->kh; ++kh) {
+          int ih = oh * d->sh - d->pt + kh;
+          if (ih < 0 || ih >= d->ih) continue;
+          for (int kw = 0; kw < d->kw; ++kw) {
+            int iw = ow * d->sw - d->pl + kw;
+            if (iw < 0 || iw >= d->iw) continue;
+            s += xp[ih * d->iw + iw];
+          }
+        }
+        yp[oh * d->ow + ow] = orc_apply_mult_rshift_sat8_f((float)s, rs, mu, 0);
+      }
+  }
+}
+
+/* ------------------------------------------------------------------------- */
+/* activations                                                                */
+/* ------------------------------------------------------------------------- */
+
+/* activation.cpp:126-153.  rshift is cast explicitly to uint32_t; the
+ * multiplier float is converted implicitly at the call. */
+void orc_leaky_relu_i8(const int8_t *x, int8_t *y, size_t count, float rshift_pos,
+                       float multiplier_pos, float rshift_neg, float multiplier_neg) {
+  const int do_pos_scale = (multiplier_pos != 0.0);
+#pragma omp parallel for
+  for (size_t i = 0; i < count; ++i) {
+    float v = (float)x[i];
+    if (v > 0) {
+      if (do_pos_scale)
+        y[i] = orc_apply_mult_rshift_sat8_f(v, orc_f2u32(rshift_pos), orc_f2u32(multiplier_pos), 0);
+      else
+        y[i] = x[i];
+    } else {
+      y[i] = orc_apply_mult_rshift_sat8_f(v, orc_f2u32(rshift_neg), orc_f2u32(multiplier_neg), 0);
+    }
+  }
+}
+
+/* activation.cpp:47-53: y0_table_op->at((unsigned char)input).  float ->
+ * unsigned char of a negative value keeps the low byte on x86-64 gcc, i.e. the
+ * index is the two's-complement byte of the int8 input. */
+void orc_lut_i8(const int8_t *x, int8_t *y, size_t count, const float *table256) {
+#pragma omp parallel for
+  for (size_t i = 0; i < count; ++i) {
+    unsigned char idx = (unsigned char)(int)(float)x[i];
+    y[i] = (int8_t)table256[idx];
+  }
+}
+
+/* core/internal.cpp:13-18 */
+void orc_relu_i8(const int8_t *x, int8_t *y, size_t count) {
+#pragma omp parallel for
+  for (size_t i = 0; i < count; ++i) y[i] = x[i] > 0 ? x[i] : 0;
+}
+
+/* clip.cpp:29-40 */
+void orc_clip_i8(const int8_t *x, int8_t *y, size_t count, float min, float max, float rshift,
+                 float multiplier) {
+  const uint32_t rs = orc_f2u32(rshift);
+  const uint32_t mu = orc_f2u32(multiplier);
+#pragma omp parallel for
+  for (size_t i = 0; i < count; ++i) {
+    float v = (float)x[i];
+    float c = fmaxf(min, fminf(v, max)); /* std::max(min, std::min(v, max)) */
+    y[i] = orc_apply_mult_rshift_sat8_f(c, rs, mu, 0);
+  }
+}
+
+/* ------------------------------------------------------------------------- */
+/* data movement                                                              */
+/* ------------------------------------------------------------------------- */
+
+/* upsample.cpp:20-41 */
+void orc_upsample_i8(const int8_t *x, int8_t *y, int n, int c, int ih, int iw, int scale_h,
+                     int scale_w) {
+  const int h = ih * scale_h, w = iw * scale_w;
+#pragma omp parallel for
+  for (int64_t nc = 0; nc < (int64_t)n * c; ++nc)
+    for (int hi = 0; hi < h; ++hi)
+      for (int wi = 0; wi < w; ++wi)
+        y[(nc * h + hi) * w + wi] = x[(nc * ih + hi / scale_h) * iw + wi / scale_w];
+}
+
+/* concat.cpp:34-90 */
+void orc_concat_i8(const int8_t *const *xs, int nin, const int64_t *shapes, int ndim, int axis,
+                   const float *rshift, const float *multiplier, int do_relu, int8_t *y) {
+  int64_t num_concats = 1;
+  for (int i = 0; i < axis; ++i) num_concats *= shapes[i];
+  int64_t out_axis = 0;
+  for (int k = 0; k < nin; ++k) out_axis += shapes[(int64_t)k * ndim + axis];
+  int64_t inner = 1;
+  for (int i = axis + 1; i < ndim; ++i) inner *= shapes[i];
+  const int64_t concat_output_size = out_axis * inner;
+  const int need_quant = rshift != NULL && multiplier != NULL;
+  int64_t global_offset = 0;
+  for (int k = 0; k < nin; ++k) {
+    const int64_t concat_input_size = shapes[(int64_t)k * ndim + axis] * inner;
+    for (int64_t c = 0; c < num_concats; ++c) {
+      const int8_t *src = xs[k] + c * concat_input_size;
+      int8_t *dst = y + global_offset + concat_output_size * c;
+      for (int64_t i = 0; i < concat_input_size; ++i) {
+        int8_t v = src[i];
+        if (need_quant && !(multiplier[k] == 1 && rshift[k] == 0))
+          v = orc_apply_mult_rshift_sat8_f((float)v, orc_f2u32(rshift[k]),
+                                           orc_f2u32(multiplier[k]), 0);
+        dst[i] = v;
+      }
+    }
+    global_offset += concat_input_size;
+  }
+  if (do_relu) {
+    const int64_t total = concat_output_size * num_concats;
+    for (int64_t i = 0; i < total; ++i)
+      if (y[i] < 0) y[i] = 0;
+  }
+}

@@ -1,0 +1,126 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement (plain C) of the arithmetic the
+ * tpuc-interpreter performs on its INT8 path.  It is the checker the HIP
+ * kernels are compared against; nothing that ships may link or call it.
+ *
+ * Tensors are NCHW (W fastest) like the reference's.  Activations and
+ * weights are int8; every quantisation parameter is passed the way the
+ * reference stores it -- as a float holding an integer -- so that the
+ * float -> uint32 -> int32 conversions of the reference are reproduced here
+ * and not by the caller.
+ *
+ * Each function names the reference lines it follows (paths relative to the
+ * reference tree).
+ *
+ * Parity status: the reference has no stored expected outputs for this path
+ * and cannot be built offline (needs MLIR and MKL-DNN 1.0.2).  Every function
+ * below is pinned by closed forms / brute force / library cross-checks in
+ * tests/; the one behaviour that nothing pins is MKL-DNN's fp32 accumulation
+ * order when partial sums exceed 2^24 ("parity unpinned"); orc_conv2d_guard
+ * and orc_fc_guard report when an input leaves the exact domain.
+ */
+#ifndef TPU_ORACLE_H
+#define TPU_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar arithmetic: lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp ---- */
+
+/* :501-509 */
+int32_t orc_srdhm(int32_t a, int32_t b);
+/* :487-499.  exponent outside [0,31] is outside the reference's assert; returns x. */
+int32_t orc_rdbp(int32_t x, int exponent);
+/* :301-334 (the "#elif 1" branch: floor(f + 0.5), clamp) */
+int8_t orc_saturate_int8(float f);
+/* :481-483 */
+int8_t orc_apply_rshift_sat8(float v, uint32_t rshift);
+/* :518-528 (float overload) */
+int8_t orc_apply_mult_rshift_sat8_f(float v, uint32_t rshift, uint32_t multiplier, int qdm);
+/* :530-539 (int32 overload) */
+int8_t orc_apply_mult_rshift_sat8_i(int32_t v, uint32_t rshift, uint32_t multiplier, int qdm);
+/* the implicit float -> uint32_t conversion at :849-863 as x86-64 gcc emits it
+ * (cvttss2si to 64 bit, low 32 bits kept) */
+uint32_t orc_f2u32(float f);
+
+/* ---- convolution: lib/Dialect/TPU/Interpreter/core/conv.cpp:11-104 ---- */
+typedef struct {
+  int n, ic, ih, iw;
+  int oc, oh, ow;
+  int g;
+  int kh, kw;
+  int sh, sw;
+  int pt, pb, pl, pr;
+  int dh, dw;
+  int ins_h, ins_w; /* zeros inserted between input rows / columns (conv.cpp:66-77) */
+  int do_relu;
+  int with_bias;
+} orc_conv_desc;
+
+/* Integer cross-correlation, zero padding (include/tpuc/NativeCpuImplementation.h:11-102
+ * restated in int32).  x: n*ic*ih*iw, w: oc*(ic/g)*kh*kw, acc: n*oc*oh*ow. */
+void orc_conv2d_acc(const int8_t *x, const int8_t *w, int32_t *acc, const orc_conv_desc *d);
+/* max over outputs of sum_k |x_k * w_k|: fp32 accumulation is order-independent
+ * and equal to the int32 sum whenever this is < 2^24. */
+int64_t orc_conv2d_guard(const int8_t *x, const int8_t *w, const orc_conv_desc *d);
+/* The same contraction done the reference's way: float-stored operands, fp32
+ * accumulate (one fixed order).  Used to show fp32 == int32 under the guard. */
+void orc_conv2d_acc_f32(const float *x, const float *w, float *acc, const orc_conv_desc *d);
+/* QuantizationArithmetic.cpp:849-871, input = int32 accumulators.
+ * bias may be NULL. */
+void orc_requant_per_channel(const int32_t *acc, int8_t *y, const float *bias, int do_relu,
+                             int64_t on, int64_t oc, int64_t isz, const float *rshift,
+                             const float *multiplier);
+/* whole op: conv.cpp:80-104 (INT8 branch).  bias/rshift/multiplier hold oc floats. */
+void orc_conv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                   const float *multiplier, int8_t *y, const orc_conv_desc *d);
+
+/* ---- fully connected: core/fullyconnected.cpp:44-91 (no transposes), one
+ * rshift / multiplier per batch matmul.  x: batch*m*k, w: batch*n*k,
+ * bias: batch*n or NULL, y: batch*m*n ---- */
+void orc_fc_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+               const float *multiplier, int8_t *y, int batch, int m, int k, int n, int do_relu);
+int64_t orc_fc_guard(const int8_t *x, const int8_t *w, const float *bias, int batch, int m, int k,
+                     int n);
+
+/* ---- eltwise add: core/eltwise.cpp:52-85 ---- */
+void orc_eltwise_add_i8(const int8_t *const *xs, int nin, const float *multiplier,
+                        const float *rshift, int do_relu, int8_t *y, size_t count);
+
+/* ---- pooling: core/pooling.cpp:89-160 (normal path only) ---- */
+typedef struct {
+  int n, c, ih, iw, oh, ow, kh, kw, sh, sw, pt, pb, pl, pr;
+} orc_pool_desc;
+void orc_pool_max_i8(const int8_t *x, int8_t *y, const orc_pool_desc *d);
+void orc_pool_avg_i8(const int8_t *x, int8_t *y, const orc_pool_desc *d, float rshift,
+                     float multiplier);
+
+/* ---- activations: core/activation.cpp ---- */
+/* :126-153 */
+void orc_leaky_relu_i8(const int8_t *x, int8_t *y, size_t count, float rshift_pos,
+                       float multiplier_pos, float rshift_neg, float multiplier_neg);
+/* :47-53 and siblings: y = table[(unsigned char)x]; table holds 256 floats */
+void orc_lut_i8(const int8_t *x, int8_t *y, size_t count, const float *table256);
+/* :155-164 + core/internal.cpp:13-18 */
+void orc_relu_i8(const int8_t *x, int8_t *y, size_t count);
+/* core/clip.cpp:29-40 */
+void orc_clip_i8(const int8_t *x, int8_t *y, size_t count, float min, float max, float rshift,
+                 float multiplier);
+
+/* ---- data movement ---- */
+/* core/upsample.cpp:20-41 */
+void orc_upsample_i8(const int8_t *x, int8_t *y, int n, int c, int ih, int iw, int scale_h,
+                     int scale_w);
+/* core/concat.cpp:34-90.  shapes: nin*ndim int64 (row per input).  rshift /
+ * multiplier NULL when the op carries none. */
+void orc_concat_i8(const int8_t *const *xs, int nin, const int64_t *shapes, int ndim, int axis,
+                   const float *rshift, const float *multiplier, int do_relu, int8_t *y);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
