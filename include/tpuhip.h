@@ -1,0 +1,199 @@
+/*
+ * tpuhip -- C ABI of the MI355X (gfx950) INT8 kernels that stand in for the
+ * tpuc-interpreter's CPU op kernels.  Plain pointers and sizes only.
+ *
+ * Every entry point returns 0 on success or a tpuhip_status; the message of
+ * the last failure on the calling thread is available from
+ * tpuhip_last_error().  (The reference aborts through llvm_unreachable /
+ * assert instead: lib/Dialect/TPU/Interpreter/MlirModuleInterpreter.cpp:339-344.)
+ *
+ * Device tensors are int8, channels-last: element (n, h, w, c) of a tensor
+ * with channel stride cs lives at byte ((n*H + h)*W + w)*cs + c.  cs is a
+ * multiple of 16 (or exactly 4 for a graph input with <= 4 channels) and the
+ * bytes c..cs-1 of every pixel are zero; every kernel keeps that invariant.
+ * The reference's NCHW float tensors (include/tpuc/Interpreter/cpukernel.h:15-78)
+ * are converted at the edge by the tpuhip_*_nchw_* entry points.
+ *
+ * A context owns one HIP stream; all work of a context is issued to it in call
+ * order and is asynchronous until tpuhip_sync().  Calls on one context must be
+ * serialised by the caller (the reference is single-threaded as well).
+ */
+#ifndef TPUHIP_H
+#define TPUHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  TPUHIP_OK = 0,
+  TPUHIP_ERR_INVALID = 1,     /* bad argument / shape the kernels cannot take */
+  TPUHIP_ERR_HIP = 2,         /* a HIP runtime call failed */
+  TPUHIP_ERR_NOMEM = 3,
+  TPUHIP_ERR_UNSUPPORTED = 4
+} tpuhip_status;
+
+typedef struct tpuhip_ctx tpuhip_ctx;
+
+/* ---- context, memory -------------------------------------------------- */
+
+/* Replaces the construction of MlirModuleInterpreter (include/tpuc/MlirModuleInterpreter.h:34-37):
+ * one context per interpreter instance. */
+int tpuhip_ctx_create(int device, tpuhip_ctx **out);
+/* Same, but work is issued to an existing hipStream_t owned by the caller. */
+int tpuhip_ctx_create_on_stream(int device, void *hip_stream, tpuhip_ctx **out);
+int tpuhip_ctx_destroy(tpuhip_ctx *ctx);
+void *tpuhip_ctx_stream(tpuhip_ctx *ctx);
+const char *tpuhip_last_error(void);
+const char *tpuhip_version(void);
+
+/* Replaces TensorData's std::vector<float> storage (cpukernel.h:15-24). */
+int tpuhip_malloc(tpuhip_ctx *ctx, size_t bytes, void **dptr);
+int tpuhip_free(tpuhip_ctx *ctx, void *dptr);
+int tpuhip_memset(tpuhip_ctx *ctx, void *dptr, int value, size_t bytes);
+int tpuhip_upload(tpuhip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+int tpuhip_download(tpuhip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+int tpuhip_sync(tpuhip_ctx *ctx);
+
+/* HIP events on the context's stream, for timing what was issued between two
+ * records (the reference has no counterpart: its Timer is commented out,
+ * bindings/python/pytuner.cpp:55-73). */
+int tpuhip_event_create(tpuhip_ctx *ctx, void **event);
+int tpuhip_event_destroy(tpuhip_ctx *ctx, void *event);
+int tpuhip_event_record(tpuhip_ctx *ctx, void *event);
+/* waits for 'stop', then returns the milliseconds between the two records */
+int tpuhip_event_elapsed_ms(tpuhip_ctx *ctx, void *start, void *stop, float *ms);
+
+/* channel stride the library uses for a tensor with c channels */
+int tpuhip_channel_stride(int c);
+
+/* ---- layout / storage conversion at the API edge ----------------------- */
+
+/* int8 NCHW (dense, device) <-> int8 channels-last with stride cs (device) */
+int tpuhip_nchw_to_nhwc_i8(tpuhip_ctx *ctx, const void *src_nchw, void *dst_nhwc, int n, int c,
+                           int h, int w, int cs);
+int tpuhip_nhwc_to_nchw_i8(tpuhip_ctx *ctx, const void *src_nhwc, void *dst_nchw, int n, int c,
+                           int h, int w, int cs);
+/* float-stored NCHW (device) <-> int8 channels-last: the float <-> int8 edge of
+ * InputOpKernel::set_tensor (core/input.cpp:16-24) and CPUOpKernel::get_tensor
+ * (cpukernel.h:124-128).  Floats must hold integers in [-128,127]. */
+int tpuhip_nchw_f32_to_nhwc_i8(tpuhip_ctx *ctx, const void *src_f32, void *dst_nhwc, int n, int c,
+                               int h, int w, int cs);
+int tpuhip_nhwc_i8_to_nchw_f32(tpuhip_ctx *ctx, const void *src_nhwc, void *dst_f32, int n, int c,
+                               int h, int w, int cs);
+
+/* ---- Conv2D (dense, grouped, depthwise) -------------------------------- */
+
+/* Field meaning follows parseConvParam (lib/Dialect/TPU/IR/TPUOperationSupport.cpp:366-428). */
+typedef struct {
+  int n, ic, ih, iw;
+  int oc, oh, ow;
+  int g;
+  int kh, kw;
+  int sh, sw;
+  int pt, pb, pl, pr;
+  int dh, dw;
+  int ins_h, ins_w;
+  int do_relu;
+  int with_bias;
+  int x_cs, y_cs;    /* channel strides of input / output */
+  int relu_first;    /* 0: ReLU after saturation (conv); 1: ReLU on the sum before requant (FC) */
+  int algo;          /* 0 auto, 1 direct (one thread per output), 2 MFMA implicit GEMM, 3 depthwise */
+} tpuhip_conv_desc;
+
+typedef struct tpuhip_conv_weights tpuhip_conv_weights;
+
+/* Replaces Conv2DOpKernel's constructor + MKLConv::setup (core/conv.cpp:11-78,
+ * include/tpuc/NativeCpuImplementation.h:18-56): takes host OIHW int8 filter
+ * (G x OC/G x IC/G x KH x KW for groups), int32 bias (may be NULL), and the
+ * per-channel int32 multiplier / rshift the epilogue uses, and stores them on
+ * the device in the layout the chosen kernel reads.  rshift must be in [0,31]. */
+int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const int8_t *filter_oihw,
+                          const int32_t *bias, const int32_t *multiplier, const int32_t *rshift,
+                          tpuhip_conv_weights **out);
+int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w);
+/* Replaces Conv2DOpKernel::invoke, INT8 branch: MKLConv::run +
+ * quantizeActivationInt8PerChannelMultiplierAndRShift (core/conv.cpp:80-104,
+ * lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp:849-871). */
+int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
+/* name of the kernel variant a prepacked conv dispatches to (for profiling) */
+const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
+
+/* ---- FullyConnected ----------------------------------------------------- */
+
+/* Replaces FullyConnectedOpKernel::invoke, INT8 branch (core/fullyconnected.cpp:44-91)
+ * for batch == 1, no transposes: y[m][n] = qdm(relu?(sum_k x[m][k]*w[n][k] + bias[n])),
+ * one multiplier / rshift for the whole tensor.  Built on the conv path: prepack
+ * with tpuhip_fc_prepack, run with tpuhip_conv2d_i8.  x rows have stride x_cs,
+ * y rows stride y_cs. */
+int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,
+                      const int8_t *filter_nk, const int32_t *bias, int32_t multiplier,
+                      int32_t rshift, tpuhip_conv_weights **out);
+
+/* ---- EltwiseAdd ---------------------------------------------------------- */
+
+/* Replaces EltwiseAddOpKernel::i8_invoke (core/eltwise.cpp:52-85):
+ * y = sat8(floor(relu?(sum_i x_i * multiplier_i) / 2^rshift + 0.5)).
+ * All tensors share pixels x cs bytes. nin <= 8. */
+int tpuhip_eltwise_add_i8(tpuhip_ctx *ctx, const void *const *xs, int nin,
+                          const int8_t *multiplier, int rshift, int do_relu, void *y,
+                          size_t bytes);
+
+/* ---- Pooling -------------------------------------------------------------- */
+
+/* Field meaning follows parsePoolParam (TPUOperationSupport.cpp:479-522). */
+typedef struct {
+  int n, c, ih, iw, oh, ow, kh, kw, sh, sw, pt, pb, pl, pr;
+  int x_cs, y_cs;
+} tpuhip_pool_desc;
+
+/* Replaces PoolingOpKernel::invoke, INT8 max (core/pooling.cpp:155-157). */
+int tpuhip_pool_max_i8(tpuhip_ctx *ctx, const tpuhip_pool_desc *d, const void *x, void *y);
+/* Replaces PoolingOpKernel::invoke, INT8 average, normal path (core/pooling.cpp:147-154):
+ * window sum with zero padding, then sat8(floor(sum * multiplier / 2^rshift + 0.5))
+ * evaluated in float32 like the reference. */
+int tpuhip_pool_avg_i8(tpuhip_ctx *ctx, const tpuhip_pool_desc *d, const void *x, void *y,
+                       uint32_t multiplier, uint32_t rshift);
+
+/* ---- 256-entry table ops ---------------------------------------------------- */
+
+/* Replaces the INT8 branch of the LUT activations: y = table[(unsigned char)x]
+ * (core/activation.cpp:47-53 and siblings).  table256: 256 int8 on the host.
+ * Pad channels (c..cs-1) stay zero. */
+int tpuhip_lut_i8(tpuhip_ctx *ctx, const void *x, void *y, const int8_t *table256, size_t pixels,
+                  int c, int cs);
+/* Replaces LeakyReluOpKernel::invoke, INT8 branch (core/activation.cpp:126-153):
+ * builds the 256-entry table from the four scalars and runs tpuhip_lut_i8. */
+int tpuhip_leaky_relu_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t pixels, int c, int cs,
+                         uint32_t rshift_pos, uint32_t multiplier_pos, uint32_t rshift_neg,
+                         uint32_t multiplier_neg);
+/* host helper: the table tpuhip_leaky_relu_i8 uses */
+int tpuhip_leaky_relu_table(uint32_t rshift_pos, uint32_t multiplier_pos, uint32_t rshift_neg,
+                            uint32_t multiplier_neg, int8_t *table256);
+/* Replaces ClipOpKernel::invoke, INT8 (core/clip.cpp:29-40); min/max as float. */
+int tpuhip_clip_table(float min, float max, uint32_t rshift, uint32_t multiplier,
+                      int8_t *table256);
+/* Replaces ReluOpKernel::invoke (core/activation.cpp:155-164). */
+int tpuhip_relu_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t bytes);
+
+/* ---- Upsample, Concat ----------------------------------------------------- */
+
+/* Replaces UpsampleOpKernel::invoke (core/upsample.cpp:20-41), nearest. */
+int tpuhip_upsample_nearest_i8(tpuhip_ctx *ctx, const void *x, void *y, int n, int c, int ih,
+                               int iw, int scale_h, int scale_w, int x_cs, int y_cs);
+
+/* Replaces ConcatOpKernel::invoke (core/concat.cpp:34-90).  axis is the NCHW
+ * axis (0..3).  in_dims: nin x 4 ints (n, c, h, w per input); in_cs: channel
+ * stride per input.  rshift / multiplier may be NULL (no requant); an input
+ * with multiplier 1 and rshift 0 is copied unchanged. */
+int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int *in_dims,
+                     const int *in_cs, int axis, const uint32_t *rshift,
+                     const uint32_t *multiplier, int do_relu, void *y, int y_cs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TPUHIP_H */

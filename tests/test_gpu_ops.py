@@ -1,0 +1,330 @@
+"""GPU parity tests, op by op, through the C ABI: every result must equal the
+oracle's byte for byte (int8 outputs, so the bar is exact equality)."""
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from gpu_helpers import conv_desc, f2i32, pool_desc, run_conv
+from tpu_compiler_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def rnd_i8(rng, shape, lo=-128, hi=127):
+    return rng.integers(lo, hi + 1, size=shape, dtype=np.int64).astype(np.int8)
+
+
+def rnd_w(rng, shape, sigma=32):
+    return np.clip(np.rint(rng.normal(0, sigma, shape)), -127, 127).astype(np.int8)
+
+
+def rnd_params(rng, oc, rs_lo=8, rs_hi=20, bias_mag=4096):
+    bias = rng.integers(-bias_mag, bias_mag + 1, oc).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, oc) * 128).astype(np.float32)
+    rsh = rng.integers(rs_lo, rs_hi + 1, oc).astype(np.float32)
+    return bias, rsh, mult
+
+
+def oracle_conv(x, w, bias, rsh, mult, g=1, stride=(1, 1), pads=(0, 0, 0, 0), dil=(1, 1),
+                ins=(0, 0), do_relu=False, with_bias=True, out_hw=None):
+    d = O.make_conv_desc(x.shape, w.shape, g, stride, pads, dil, ins, do_relu, with_bias, out_hw)
+    return O.conv2d_i8(x, w, bias, rsh, mult, d)
+
+
+# n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu  (dense convolutions, g = 1)
+DENSE = [
+    (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),      # config 1
+    (2, 64, 14, 14, 256, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),    # 1x1, tile 128x128
+    (2, 256, 14, 14, 64, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), True),     # tile 64x256
+    (1, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3, 3, 3), (1, 1), True),       # stem: 3 channels, 7x7 s2
+    (3, 24, 9, 11, 144, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),     # ic, oc not multiples of 16/64
+    (1, 144, 9, 11, 24, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),     # oc 24 -> tile 32x256
+    (2, 32, 13, 13, 16, 3, 3, (2, 2), (0, 1, 0, 1), (1, 1), True),      # asymmetric pads, s2
+    (1, 48, 10, 10, 80, 3, 3, (1, 1), (2, 2, 2, 2), (2, 2), True),      # dilation 2
+    (2, 128, 7, 7, 255, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),     # 255 output channels
+    (1, 512, 5, 5, 128, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),      # K = 4608
+    (2, 64, 8, 8, 64, 1, 1, (2, 2), (0, 0, 0, 0), (1, 1), False),       # 1x1 stride 2 (downsample)
+    (1, 16, 6, 5, 32, 5, 3, (1, 2), (2, 2, 1, 1), (1, 1), False),       # non-square kernel
+]
+
+
+@pytest.mark.parametrize("case", DENSE)
+@pytest.mark.parametrize("algo", [capi.ALGO_MFMA, capi.ALGO_DIRECT])
+def test_conv_dense(ctx, case, algo):
+    n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
+    rng = np.random.default_rng(ic * 1000 + oc + kh)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=algo, stride=stride, pads=pads, dil=dil,
+                         do_relu=relu)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want), "%s: %d mismatches" % (name, (got != want).sum())
+    # outputs must not be degenerate, or equality proves little
+    assert len(np.unique(want)) > 8
+
+
+def test_conv_auto_picks_mfma_for_dense_and_depthwise_for_dw(ctx):
+    rng = np.random.default_rng(1)
+    x = rnd_i8(rng, (1, 32, 8, 8))
+    w = rnd_w(rng, (32, 32, 3, 3))
+    bias, rsh, mult = rnd_params(rng, 32)
+    _, name = run_conv(ctx, x, w, bias, rsh, mult, pads=(1, 1, 1, 1))
+    assert name.startswith("mfma")
+    wd = rnd_w(rng, (32, 1, 3, 3))
+    _, name = run_conv(ctx, x, wd, bias, rsh, mult, g=32, pads=(1, 1, 1, 1))
+    assert name == "depthwise"
+    wg = rnd_w(rng, (32, 8, 3, 3))
+    _, name = run_conv(ctx, x, wg, bias, rsh, mult, g=4, pads=(1, 1, 1, 1))
+    assert name == "direct"
+
+
+# n, c, ih, iw, k, stride, pads, relu
+DEPTHWISE = [
+    (2, 256, 56, 56, 3, (1, 1), (1, 1, 1, 1), True),     # config 2 (smaller batch)
+    (2, 96, 15, 15, 3, (2, 2), (0, 1, 0, 1), True),
+    (1, 24, 9, 9, 3, (1, 1), (1, 1, 1, 1), False),       # 24 channels: padded group
+    (1, 32, 12, 12, 5, (1, 1), (2, 2, 2, 2), False),
+    (1, 16, 7, 7, 7, (1, 1), (0, 0, 0, 0), False),       # global depthwise
+]
+
+
+@pytest.mark.parametrize("case", DEPTHWISE)
+@pytest.mark.parametrize("algo", [capi.ALGO_DEPTHWISE, capi.ALGO_DIRECT])
+def test_conv_depthwise(ctx, case, algo):
+    n, c, ih, iw, k, stride, pads, relu = case
+    rng = np.random.default_rng(c + k)
+    x = rnd_i8(rng, (n, c, ih, iw))
+    w = rnd_w(rng, (c, 1, k, k), 24)
+    bias, rsh, mult = rnd_params(rng, c, 5, 12, 2048)
+    want = oracle_conv(x, w, bias, rsh, mult, c, stride, pads, (1, 1), (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=algo, g=c, stride=stride, pads=pads,
+                         do_relu=relu)
+    assert np.array_equal(got, want), name
+    assert len(np.unique(want)) > 8
+
+
+def test_conv_grouped_and_inserted_zeros_direct(ctx):
+    rng = np.random.default_rng(3)
+    x = rnd_i8(rng, (2, 12, 7, 6))
+    w = rnd_w(rng, (8, 3, 3, 3))
+    bias, rsh, mult = rnd_params(rng, 8, 4, 9)
+    want = oracle_conv(x, w, bias, rsh, mult, 4, (1, 1), (1, 1, 1, 1))
+    got, _ = run_conv(ctx, x, w, bias, rsh, mult, g=4, pads=(1, 1, 1, 1))
+    assert np.array_equal(got, want)
+    w2 = rnd_w(rng, (5, 12, 3, 3))
+    bias, rsh, mult = rnd_params(rng, 5, 6, 10)
+    want = oracle_conv(x, w2, bias, rsh, mult, 1, (1, 1), (1, 1, 1, 1), (1, 1), (1, 2))
+    got, name = run_conv(ctx, x, w2, bias, rsh, mult, pads=(1, 1, 1, 1), ins=(1, 2))
+    assert name == "direct" and np.array_equal(got, want)
+
+
+def test_conv_without_bias_and_null_bias(ctx):
+    rng = np.random.default_rng(5)
+    x = rnd_i8(rng, (1, 16, 6, 6))
+    w = rnd_w(rng, (16, 16, 3, 3))
+    bias, rsh, mult = rnd_params(rng, 16)
+    want = oracle_conv(x, w, bias, rsh, mult, pads=(1, 1, 1, 1), with_bias=False)
+    got, _ = run_conv(ctx, x, w, bias, rsh, mult, pads=(1, 1, 1, 1), with_bias=False)
+    assert np.array_equal(got, want)
+    got, _ = run_conv(ctx, x, w, None, rsh, mult, pads=(1, 1, 1, 1), with_bias=True)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("algo", [capi.ALGO_MFMA, capi.ALGO_DIRECT])
+def test_conv_requant_edge_parameters(ctx, algo):
+    """rshift 0 and 31, multipliers that are not float32-exact, zero, 2^31 (which the
+    reference turns into INT_MIN) and large accumulators."""
+    rng = np.random.default_rng(7)
+    oc = 32
+    x = rnd_i8(rng, (1, 256, 4, 4), 100, 127)
+    w = rnd_i8(rng, (oc, 256, 3, 3), 100, 127)       # sums near 9*256*127*127 = 3.7e7
+    w[1::2] = -w[1::2]
+    bias = rng.integers(-(1 << 23), 1 << 23, oc).astype(np.float32)
+    mult = (rng.integers(1 << 30, (1 << 31) - 1, oc)).astype(np.float32)   # rounded by float32
+    mult[0] = 0
+    mult[1] = float(2 ** 31)       # -> uint32 2^31 -> int32 INT_MIN
+    mult[2] = 1.0
+    mult[3] = float((1 << 31) - 1)  # rounds up to 2^31 as a float
+    rsh = rng.integers(0, 32, oc).astype(np.float32)
+    rsh[4], rsh[5], rsh[6], rsh[7] = 0, 31, 1, 30
+    want = oracle_conv(x, w, bias, rsh, mult, pads=(1, 1, 1, 1))
+    got, _ = run_conv(ctx, x, w, bias, rsh, mult, algo=algo, pads=(1, 1, 1, 1))
+    assert np.array_equal(got, want)
+
+
+def test_conv_rejects_bad_arguments(ctx):
+    d = conv_desc((1, 16, 4, 4), (16, 16, 3, 3), pads=(1, 1, 1, 1))
+    w = np.zeros((16, 16, 3, 3), np.int8)
+    ok = np.zeros(16, np.int32)
+    bad = ok.copy()
+    bad[3] = 32
+    with pytest.raises(capi.TpuHipError, match="rshift"):
+        ctx.conv_prepack(d, w, None, ok, bad)
+    d2 = conv_desc((1, 16, 4, 4), (16, 16, 3, 3), pads=(1, 1, 1, 1), out_hw=(9, 9))
+    with pytest.raises(capi.TpuHipError, match="window"):
+        ctx.conv_prepack(d2, w, None, ok, ok)
+    d3 = conv_desc((1, 16, 4, 4), (16, 4, 3, 3), g=4, pads=(1, 1, 1, 1), algo=capi.ALGO_MFMA)
+    with pytest.raises(capi.TpuHipError, match="MFMA"):
+        ctx.conv_prepack(d3, np.zeros((16, 4, 3, 3), np.int8), None, ok, ok)
+
+
+@pytest.mark.parametrize("m,k,n,relu", [(32, 2048, 1000, False), (5, 100, 37, True),
+                                        (64, 1280, 1000, True)])
+def test_fully_connected(ctx, m, k, n, relu):
+    rng = np.random.default_rng(m + k + n)
+    x = rnd_i8(rng, (m, k))
+    w = rnd_w(rng, (n, k), 20)
+    bias = rng.integers(-3000, 3000, n).astype(np.float32)
+    mult, rsh = np.float32((1 << 30) + 128 * 12345), np.float32(9)
+    want = O.fc_i8(x, w, bias, [rsh], [mult], 1, m, k, n, relu)[0]
+    xt = ctx.from_nchw(x.reshape(m, k, 1, 1))
+    yt = ctx.tensor((m, n, 1, 1))
+    wh = ctx.fc_prepack(m, k, n, xt.cs, yt.cs, relu, w, f2i32(bias), f2i32([mult])[0],
+                        f2i32([rsh])[0])
+    ctx.conv(wh, xt, yt)
+    got = ctx.to_nchw(yt).reshape(m, n)
+    assert np.array_equal(got, want)
+    assert O.fc_guard(x, w, bias, 1, m, k, n) < (1 << 24)
+    ctx.conv_weights_destroy(wh)
+
+
+@pytest.mark.parametrize("nin,relu,rs", [(2, True, 5), (2, False, 0), (3, False, 7), (1, True, 2),
+                                         (8, True, 9)])
+def test_eltwise_add(ctx, nin, relu, rs):
+    rng = np.random.default_rng(nin * 10 + rs)
+    shape = (2, 24, 7, 9)
+    xs = [rnd_i8(rng, shape) for _ in range(nin)]
+    mult = rng.integers(-128, 128, nin).astype(np.float32)
+    want = O.eltwise_add_i8(xs, mult, [rs], relu)
+    ts = [ctx.from_nchw(a) for a in xs]
+    yt = ctx.tensor(shape)
+    ctx.eltwise_add(ts, mult.astype(np.int8), rs, relu, yt)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., 24:].any()
+
+
+@pytest.mark.parametrize("k,s,pads,shape,out_hw", [
+    ((3, 3), (2, 2), (0, 1, 0, 1), (2, 64, 28, 28), None),   # ResNet-50 pool1 (Caffe ceil mode)
+    ((3, 3), (2, 2), (1, 1, 1, 1), (1, 24, 9, 11), None),
+    ((2, 2), (2, 2), (0, 0, 0, 0), (1, 5, 8, 8), None),
+    ((3, 2), (1, 2), (1, 0, 0, 1), (1, 40, 7, 9), None),
+])
+def test_pool_max(ctx, k, s, pads, shape, out_hw):
+    rng = np.random.default_rng(sum(shape))
+    x = rnd_i8(rng, shape)
+    want = O.pool_max_i8(x, O.make_pool_desc(shape, k, s, pads, out_hw))
+    d = pool_desc(shape, k, s, pads, out_hw)
+    xt = ctx.from_nchw(x)
+    yt = ctx.tensor((d.n, d.c, d.oh, d.ow))
+    ctx.pool_max(d, xt, yt)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., shape[1]:].any()
+
+
+@pytest.mark.parametrize("k,s,pads,shape,mult,rs", [
+    ((7, 7), (1, 1), (0, 0, 0, 0), (4, 2048, 7, 7), 167, 13),   # ResNet-50 global average
+    ((7, 7), (1, 1), (0, 0, 0, 0), (2, 1280, 7, 7), 84, 12),
+    ((3, 3), (2, 2), (1, 1, 1, 1), (1, 20, 9, 9), 57, 9),
+    ((2, 2), (2, 2), (0, 0, 0, 0), (1, 3, 6, 6), 1, 0),
+    ((3, 3), (1, 1), (1, 1, 1, 1), (1, 16, 5, 5), 255, 3),      # saturates
+])
+def test_pool_avg(ctx, k, s, pads, shape, mult, rs):
+    rng = np.random.default_rng(sum(shape) + mult)
+    x = rnd_i8(rng, shape)
+    want = O.pool_avg_i8(x, O.make_pool_desc(shape, k, s, pads), rs, mult)
+    d = pool_desc(shape, k, s, pads)
+    xt = ctx.from_nchw(x)
+    yt = ctx.tensor((d.n, d.c, d.oh, d.ow))
+    ctx.pool_avg(d, xt, yt, mult, rs)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+
+
+def test_leaky_relu_lut_relu(ctx):
+    rng = np.random.default_rng(41)
+    shape = (2, 40, 6, 5)
+    x = rnd_i8(rng, shape)
+    x.reshape(-1)[:256] = np.arange(-128, 128)      # every input value occurs
+    xt = ctx.from_nchw(x)
+    yt = ctx.tensor(shape)
+    for rp, mp, rn, mn in ((0, 1, 7, 13), (5, 33, 10, 102), (0, 0, 6, 6)):
+        ctx.leaky_relu(xt, yt, rp, mp, rn, mn)
+        assert np.array_equal(ctx.to_nchw(yt), O.leaky_relu_i8(x, rp, mp, rn, mn))
+        assert not ctx.raw(yt)[..., 40:].any()
+    table = rng.integers(-128, 128, 256).astype(np.int8)
+    ctx.lut(xt, yt, table)
+    assert np.array_equal(ctx.to_nchw(yt), O.lut_i8(x, table.astype(np.float32)))
+    assert not ctx.raw(yt)[..., 40:].any()       # table[0] != 0 must not leak into the pads
+    ctx.relu(xt, yt)
+    assert np.array_equal(ctx.to_nchw(yt), O.relu_i8(x))
+    ctx.lut(xt, yt, ctx.clip_table(0, 77, 0, 1))
+    assert np.array_equal(ctx.to_nchw(yt), O.clip_i8(x, 0, 77, 0, 1))
+
+
+def test_upsample(ctx):
+    rng = np.random.default_rng(43)
+    for shape, sh, sw in (((2, 256, 19, 19), 2, 2), ((1, 24, 5, 4), 3, 1), ((1, 8, 3, 3), 1, 2)):
+        x = rnd_i8(rng, shape)
+        xt = ctx.from_nchw(x)
+        yt = ctx.tensor((shape[0], shape[1], shape[2] * sh, shape[3] * sw))
+        ctx.upsample(xt, yt, sh, sw)
+        assert np.array_equal(ctx.to_nchw(yt), O.upsample_i8(x, sh, sw))
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, 3])
+def test_concat_axes(ctx, axis):
+    rng = np.random.default_rng(47 + axis)
+    base = [2, 32, 5, 6]
+    shapes = []
+    for extent in (3, 1, 4) if axis != 1 else (32, 16, 48):
+        s = list(base)
+        s[axis] = extent
+        shapes.append(tuple(s))
+    xs = [rnd_i8(rng, s) for s in shapes]
+    want = O.concat_i8(xs, axis)
+    ts = [ctx.from_nchw(a) for a in xs]
+    yt = ctx.tensor(want.shape)
+    ctx.concat(ts, axis, yt)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+
+
+def test_concat_channels_unaligned_requant_relu(ctx):
+    rng = np.random.default_rng(53)
+    xs = [rnd_i8(rng, (2, c, 4, 5)) for c in (24, 7, 40)]
+    rsh, mult = [0, 3, 6], [1, 5, 77]
+    want = O.concat_i8(xs, 1, rsh, mult, True)
+    ts = [ctx.from_nchw(a) for a in xs]
+    yt = ctx.tensor(want.shape)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.concat(ts, 1, yt, rsh, mult, True)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., 71:].any()
+
+
+def test_layout_round_trip_and_float_edge(ctx):
+    rng = np.random.default_rng(59)
+    x = rnd_i8(rng, (3, 37, 11, 13))
+    t = ctx.from_nchw(x)
+    raw = ctx.raw(t)
+    assert np.array_equal(raw[..., :37], x.transpose(0, 2, 3, 1))
+    assert not raw[..., 37:].any()
+    assert np.array_equal(ctx.to_nchw(t), x)
+    # float-stored edge
+    xf = x.astype(np.float32)
+    src = ctx.malloc(xf.nbytes)
+    ctx.upload(src, xf)
+    t2 = ctx.tensor(x.shape)
+    n, c, h, w = x.shape
+    ctx._ck(ctx.lib.tpuhip_nchw_f32_to_nhwc_i8(ctx.h, src, t2.ptr, n, c, h, w, t2.cs))
+    assert np.array_equal(ctx.raw(t2), raw)
+    dst = ctx.malloc(xf.nbytes)
+    ctx._ck(ctx.lib.tpuhip_nhwc_i8_to_nchw_f32(ctx.h, t2.ptr, dst, n, c, h, w, t2.cs))
+    assert np.array_equal(ctx.download(dst, x.shape, np.float32), xf)

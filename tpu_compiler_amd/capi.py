@@ -1,0 +1,291 @@
+"""ctypes binding of the tpuhip C ABI (include/tpuhip.h) plus small numpy
+conveniences.  Every call goes to the HIP library; nothing here computes."""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+c_void_pp = C.POINTER(C.c_void_p)
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in (
+        "n", "ic", "ih", "iw", "oc", "oh", "ow", "g", "kh", "kw", "sh", "sw",
+        "pt", "pb", "pl", "pr", "dh", "dw", "ins_h", "ins_w", "do_relu", "with_bias",
+        "x_cs", "y_cs", "relu_first", "algo")]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in (
+        "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
+        "x_cs", "y_cs")]
+
+
+ALGO_AUTO, ALGO_DIRECT, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
+
+# name -> (restype, argtypes); every symbol include/tpuhip.h declares
+PROTOTYPES = {
+    "tpuhip_ctx_create": (C.c_int, [C.c_int, c_void_pp]),
+    "tpuhip_ctx_create_on_stream": (C.c_int, [C.c_int, C.c_void_p, c_void_pp]),
+    "tpuhip_ctx_destroy": (C.c_int, [C.c_void_p]),
+    "tpuhip_ctx_stream": (C.c_void_p, [C.c_void_p]),
+    "tpuhip_last_error": (C.c_char_p, []),
+    "tpuhip_version": (C.c_char_p, []),
+    "tpuhip_malloc": (C.c_int, [C.c_void_p, C.c_size_t, c_void_pp]),
+    "tpuhip_free": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_memset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t]),
+    "tpuhip_upload": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "tpuhip_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "tpuhip_sync": (C.c_int, [C.c_void_p]),
+    "tpuhip_event_create": (C.c_int, [C.c_void_p, c_void_pp]),
+    "tpuhip_event_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p,
+                                          C.POINTER(C.c_float)]),
+    "tpuhip_channel_stride": (C.c_int, [C.c_int]),
+    "tpuhip_nchw_to_nhwc_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
+    "tpuhip_nhwc_to_nchw_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
+    "tpuhip_nchw_f32_to_nhwc_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
+    "tpuhip_nhwc_i8_to_nchw_f32": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
+    "tpuhip_conv2d_prepack": (C.c_int, [C.c_void_p, C.POINTER(ConvDesc), C.c_void_p, C.c_void_p,
+                                        C.c_void_p, C.c_void_p, c_void_pp]),
+    "tpuhip_conv2d_weights_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_conv2d_i8": (C.c_int, [C.c_void_p] * 4),
+    "tpuhip_conv2d_algo_name": (C.c_char_p, [C.c_void_p]),
+    "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
+                                                                   C.c_int32, C.c_int32,
+                                                                   c_void_pp]),
+    "tpuhip_eltwise_add_i8": (C.c_int, [C.c_void_p, c_void_pp, C.c_int, C.c_void_p, C.c_int,
+                                        C.c_int, C.c_void_p, C.c_size_t]),
+    "tpuhip_pool_max_i8": (C.c_int, [C.c_void_p, C.POINTER(PoolDesc), C.c_void_p, C.c_void_p]),
+    "tpuhip_pool_avg_i8": (C.c_int, [C.c_void_p, C.POINTER(PoolDesc), C.c_void_p, C.c_void_p,
+                                     C.c_uint32, C.c_uint32]),
+    "tpuhip_lut_i8": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t, C.c_int, C.c_int]),
+    "tpuhip_leaky_relu_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int, C.c_int] +
+                             [C.c_uint32] * 4),
+    "tpuhip_leaky_relu_table": (C.c_int, [C.c_uint32] * 4 + [C.c_void_p]),
+    "tpuhip_clip_table": (C.c_int, [C.c_float, C.c_float, C.c_uint32, C.c_uint32, C.c_void_p]),
+    "tpuhip_relu_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t]),
+    "tpuhip_upsample_nearest_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 8),
+    "tpuhip_concat_i8": (C.c_int, [C.c_void_p, c_void_pp, C.c_int, C.c_void_p, C.c_void_p,
+                                   C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int]),
+}
+
+
+class TpuHipError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("tpuhip status %d: %s" % (status, message))
+        self.status = status
+
+
+def bind(lib=None, prototypes=None):
+    lib = lib or _lib.load()
+    for name, (res, args) in (prototypes or PROTOTYPES).items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def check(lib, status):
+    if status != 0:
+        raise TpuHipError(status, lib.tpuhip_last_error().decode())
+
+
+def channel_stride(c):
+    return (c + 15) // 16 * 16
+
+
+class DeviceTensor:
+    """An int8 channels-last tensor in HBM: logical NCHW shape, channel stride cs."""
+
+    def __init__(self, ctx, shape, cs=None, ptr=None, owner=True):
+        self.ctx = ctx
+        self.shape = tuple(int(v) for v in shape)
+        n, c, h, w = self.shape
+        self.cs = cs or channel_stride(c)
+        self.nbytes = n * h * w * self.cs
+        self._owner = owner and ptr is None
+        self.ptr = ptr if ptr is not None else ctx.malloc(self.nbytes)
+
+    @property
+    def pixels(self):
+        n, _, h, w = self.shape
+        return n * h * w
+
+    def free(self):
+        if self._owner and self.ptr:
+            self.ctx.free(self.ptr)
+            self.ptr = None
+
+
+class Context:
+    """One tpuhip context (one HIP stream) with numpy conveniences."""
+
+    def __init__(self, device=0):
+        self.lib = bind()
+        h = C.c_void_p()
+        check(self.lib, self.lib.tpuhip_ctx_create(device, C.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            self.lib.tpuhip_ctx_destroy(self.h)
+            self.h = None
+
+    def _ck(self, status):
+        check(self.lib, status)
+
+    # -- memory -----------------------------------------------------------
+    def malloc(self, nbytes):
+        p = C.c_void_p()
+        self._ck(self.lib.tpuhip_malloc(self.h, max(int(nbytes), 1), C.byref(p)))
+        return p.value
+
+    def free(self, ptr):
+        self._ck(self.lib.tpuhip_free(self.h, ptr))
+
+    def upload(self, ptr, arr):
+        arr = np.ascontiguousarray(arr)
+        self._ck(self.lib.tpuhip_upload(self.h, ptr, arr.ctypes.data, arr.nbytes))
+
+    def download(self, ptr, shape, dtype):
+        out = np.empty(shape, dtype)
+        self._ck(self.lib.tpuhip_download(self.h, out.ctypes.data, ptr, out.nbytes))
+        return out
+
+    def sync(self):
+        self._ck(self.lib.tpuhip_sync(self.h))
+
+    # -- events ------------------------------------------------------------
+    def event(self):
+        e = C.c_void_p()
+        self._ck(self.lib.tpuhip_event_create(self.h, C.byref(e)))
+        return e.value
+
+    def record(self, ev):
+        self._ck(self.lib.tpuhip_event_record(self.h, ev))
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        self._ck(self.lib.tpuhip_event_elapsed_ms(self.h, start, stop, C.byref(ms)))
+        return ms.value
+
+    # -- tensors -------------------------------------------------------------
+    def tensor(self, shape, cs=None):
+        return DeviceTensor(self, shape, cs)
+
+    def from_nchw(self, arr, cs=None):
+        """int8 NCHW numpy array -> channels-last device tensor (conversion on the GPU)."""
+        arr = np.ascontiguousarray(arr)
+        assert arr.dtype == np.int8 and arr.ndim == 4
+        t = DeviceTensor(self, arr.shape, cs)
+        tmp = self.malloc(arr.nbytes)
+        try:
+            self.upload(tmp, arr)
+            n, c, h, w = arr.shape
+            self._ck(self.lib.tpuhip_nchw_to_nhwc_i8(self.h, tmp, t.ptr, n, c, h, w, t.cs))
+            self.sync()
+        finally:
+            self.free(tmp)
+        return t
+
+    def to_nchw(self, t):
+        n, c, h, w = t.shape
+        tmp = self.malloc(n * c * h * w)
+        try:
+            self._ck(self.lib.tpuhip_nhwc_to_nchw_i8(self.h, t.ptr, tmp, n, c, h, w, t.cs))
+            return self.download(tmp, t.shape, np.int8)
+        finally:
+            self.free(tmp)
+
+    def raw(self, t):
+        """the channels-last bytes, pad channels included"""
+        n, c, h, w = t.shape
+        return self.download(t.ptr, (n, h, w, t.cs), np.int8)
+
+    # -- ops -------------------------------------------------------------------
+    def conv_prepack(self, desc, filt, bias, mult, rshift):
+        filt = np.ascontiguousarray(filt, dtype=np.int8)
+        mult = np.ascontiguousarray(mult, dtype=np.int32)
+        rshift = np.ascontiguousarray(rshift, dtype=np.int32)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_conv2d_prepack(
+            self.h, C.byref(desc), filt.ctypes.data, None if b is None else b.ctypes.data,
+            mult.ctypes.data, rshift.ctypes.data, C.byref(w)))
+        return w.value
+
+    def fc_prepack(self, m, k, n, x_cs, y_cs, do_relu, filt, bias, mult, rshift):
+        filt = np.ascontiguousarray(filt, dtype=np.int8)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_fc_prepack(
+            self.h, m, k, n, x_cs, y_cs, int(do_relu), filt.ctypes.data,
+            None if b is None else b.ctypes.data, int(mult), int(rshift), C.byref(w)))
+        return w.value
+
+    def conv_weights_destroy(self, w):
+        self._ck(self.lib.tpuhip_conv2d_weights_destroy(self.h, w))
+
+    def conv(self, w, x, y):
+        self._ck(self.lib.tpuhip_conv2d_i8(self.h, w, x.ptr if hasattr(x, "ptr") else x,
+                                           y.ptr if hasattr(y, "ptr") else y))
+
+    def conv_algo_name(self, w):
+        return self.lib.tpuhip_conv2d_algo_name(w).decode()
+
+    def eltwise_add(self, xs, mult, rshift, do_relu, y):
+        ptrs = (C.c_void_p * len(xs))(*[t.ptr for t in xs])
+        m = np.ascontiguousarray(mult, dtype=np.int8)
+        self._ck(self.lib.tpuhip_eltwise_add_i8(self.h, ptrs, len(xs), m.ctypes.data, int(rshift),
+                                                int(do_relu), y.ptr, y.nbytes))
+
+    def pool_max(self, d, x, y):
+        self._ck(self.lib.tpuhip_pool_max_i8(self.h, C.byref(d), x.ptr, y.ptr))
+
+    def pool_avg(self, d, x, y, mult, rshift):
+        self._ck(self.lib.tpuhip_pool_avg_i8(self.h, C.byref(d), x.ptr, y.ptr, int(mult),
+                                             int(rshift)))
+
+    def lut(self, x, y, table):
+        t = np.ascontiguousarray(table, dtype=np.int8)
+        assert t.size == 256
+        self._ck(self.lib.tpuhip_lut_i8(self.h, x.ptr, y.ptr, t.ctypes.data, x.pixels,
+                                        x.shape[1], x.cs))
+
+    def leaky_relu(self, x, y, rp, mp, rn, mn):
+        self._ck(self.lib.tpuhip_leaky_relu_i8(self.h, x.ptr, y.ptr, x.pixels, x.shape[1], x.cs,
+                                               int(rp), int(mp), int(rn), int(mn)))
+
+    def leaky_relu_table(self, rp, mp, rn, mn):
+        t = np.empty(256, np.int8)
+        self._ck(self.lib.tpuhip_leaky_relu_table(int(rp), int(mp), int(rn), int(mn),
+                                                  t.ctypes.data))
+        return t
+
+    def clip_table(self, lo, hi, rshift, mult):
+        t = np.empty(256, np.int8)
+        self._ck(self.lib.tpuhip_clip_table(float(lo), float(hi), int(rshift), int(mult),
+                                            t.ctypes.data))
+        return t
+
+    def relu(self, x, y):
+        self._ck(self.lib.tpuhip_relu_i8(self.h, x.ptr, y.ptr, x.nbytes))
+
+    def upsample(self, x, y, sh, sw):
+        n, c, h, w = x.shape
+        self._ck(self.lib.tpuhip_upsample_nearest_i8(self.h, x.ptr, y.ptr, n, c, h, w, sh, sw,
+                                                     x.cs, y.cs))
+
+    def concat(self, xs, axis, y, rshift=None, mult=None, do_relu=False):
+        ptrs = (C.c_void_p * len(xs))(*[t.ptr for t in xs])
+        dims = np.ascontiguousarray(np.array([t.shape for t in xs], dtype=np.int32))
+        cs = np.ascontiguousarray(np.array([t.cs for t in xs], dtype=np.int32))
+        r = None if rshift is None else np.ascontiguousarray(rshift, dtype=np.uint32)
+        m = None if mult is None else np.ascontiguousarray(mult, dtype=np.uint32)
+        self._ck(self.lib.tpuhip_concat_i8(
+            self.h, ptrs, len(xs), dims.ctypes.data, cs.ctypes.data, axis,
+            None if r is None else r.ctypes.data, None if m is None else m.ctypes.data,
+            int(do_relu), y.ptr, y.cs))
