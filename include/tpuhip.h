@@ -193,6 +193,73 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
                      const int *in_cs, int axis, const uint32_t *rshift,
                      const uint32_t *multiplier, int do_relu, void *y, int y_cs);
 
+/* ---- module interpreter ------------------------------------------------------ */
+
+/* Flat view of the C++ ModuleInterpreter (include/tpuhip/interpreter.hpp), which
+ * mirrors MlirModuleInterpreter (include/tpuc/MlirModuleInterpreter.h:32-83) and
+ * what pymlir.module exposes on top of it (bindings/python/pymlir.cpp:289-311).
+ * Tensors cross this boundary the way the reference passes them: float32 NCHW
+ * arrays holding integers. */
+typedef struct tpuhip_module tpuhip_module;
+
+/* One TPU-dialect op: what the reference reads from an mlir::Operation. */
+typedef struct {
+  const char *type;          /* "tpu.conv_2d", "tpu.eltwise_add", ... */
+  const char *name;
+  const char *quant;         /* "INT8" | "UINT8" | "BF16" | "NONE" */
+  const char *param_type;    /* "RSHIFT_AND_M_I32", "RSHIFT_AND_M_I8", "NONE", ... */
+  int ndim;
+  const int64_t *shape;      /* result shape */
+  int n_operands;
+  const char *const *operands; /* value / weight names in operand order, "" for none */
+  int n_attrs;
+  const char *const *attr_keys;
+  const double *attr_values;
+} tpuhip_op_desc;
+
+/* MlirModuleInterpreter(batch) */
+int tpuhip_module_create(int device, int max_batch, tpuhip_module **out);
+int tpuhip_module_destroy(tpuhip_module *m);
+/* updateWeightMap: one call per tpu.load_weight (MlirModuleInterpreter.cpp:352-369) */
+int tpuhip_module_set_weight(tpuhip_module *m, const char *name, const float *data, size_t count);
+/* describe the function body: ops in program order, then the returned values */
+int tpuhip_module_clear_ops(tpuhip_module *m);
+int tpuhip_module_add_op(tpuhip_module *m, const tpuhip_op_desc *op);
+int tpuhip_module_set_returns(tpuhip_module *m, const char *const *names, int n);
+/* loadModule(module, target_op): builds / refreshes the kernel list; unchanged
+ * kernels are kept (MlirModuleInterpreter.cpp:73-83, 118-350).  target_op may be NULL. */
+int tpuhip_module_load(tpuhip_module *m, const char *target_op);
+/* setTensor / getTensor (:407-430) */
+int tpuhip_module_set_tensor(tpuhip_module *m, const char *name, const float *data, size_t count,
+                             int bidx);
+int tpuhip_module_get_tensor(tpuhip_module *m, const char *name, float *dst, size_t count,
+                             int bidx);
+/* same tensor as int8 NCHW, without the float detour */
+int tpuhip_module_get_tensor_i8(tpuhip_module *m, const char *name, int8_t *dst, size_t count,
+                                int bidx);
+/* invoke / invokeTo / fastInvokeAllBatch (:371-405).  Work is queued on the
+ * module's stream; tpuhip_module_sync (or any get_tensor) waits for it. */
+int tpuhip_module_invoke(tpuhip_module *m, int bidx);
+int tpuhip_module_invoke_to(tpuhip_module *m, const char *name, int bidx);
+int tpuhip_module_fast_invoke_all_batch(tpuhip_module *m, const char *name, int batch);
+int tpuhip_module_sync(tpuhip_module *m);
+/* getTensorShape / getDataType / getAllTensorName / outputDetails / input_details */
+int tpuhip_module_tensor_shape(tpuhip_module *m, const char *name, int64_t *dims8, int *ndim);
+const char *tpuhip_module_tensor_dtype(tpuhip_module *m, const char *name);
+int tpuhip_module_num_tensors(tpuhip_module *m);
+const char *tpuhip_module_tensor_name(tpuhip_module *m, int i);
+int tpuhip_module_num_inputs(tpuhip_module *m);
+const char *tpuhip_module_input_name(tpuhip_module *m, int i);
+int tpuhip_module_num_outputs(tpuhip_module *m);
+const char *tpuhip_module_output_name(tpuhip_module *m, int i);
+/* kernels in execution order; algo is the conv variant or "" */
+int tpuhip_module_num_kernels(tpuhip_module *m);
+const char *tpuhip_module_kernel_name(tpuhip_module *m, int i);
+const char *tpuhip_module_kernel_algo(tpuhip_module *m, int i);
+/* HIP-event time of every kernel in execution order: ms[i] = mean over iters runs */
+int tpuhip_module_time_kernels(tpuhip_module *m, int bidx, int iters, float *ms, int capacity);
+tpuhip_ctx *tpuhip_module_ctx(tpuhip_module *m);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,351 @@
+// C++ op-level API of tpuhip: the classes a caller of the reference's
+// interpreter works with -- TensorData, CPUOpKernel and its per-op subclasses,
+// and the module interpreter -- with the same names, members, operand order and
+// invoke() contract, running on the MI355X through the C ABI in tpuhip.h.
+//
+// Differences forced by the environment, and only these:
+//   * mlir::Operation& is replaced by OpDesc, a plain description of one TPU
+//     dialect op (MLIR is not available to build against); everything the
+//     reference reads from the operation -- result shape, name, quant mode and
+//     param type, operands, attributes -- is a field of OpDesc;
+//   * an activation TensorData lives in HBM as int8 channels-last; the float
+//     NCHW view the reference exposes is produced on set/get;
+//   * failures throw std::runtime_error where the reference aborts.
+//
+// Reference: include/tpuc/Interpreter/cpukernel.h:15-159,
+// include/tpuc/MlirModuleInterpreter.h:32-83.
+#pragma once
+
+#include <cstdint>
+#include <list>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "tpuhip.h"
+
+namespace tpuhip {
+
+using SyncedDataShape = std::vector<int64_t>;
+
+// One TPU-dialect operation as the interpreter sees it.
+struct OpDesc {
+  std::string type;                    // "tpu.conv_2d", "tpu.eltwise_add", ...
+  std::string name;                    // getOpName(op)
+  SyncedDataShape shape;               // result tensor shape
+  std::string quant = "INT8";          // getOpQuant(op): "INT8" | "UINT8" | "BF16" | "NONE"
+  std::string param_type = "NONE";     // getOpQuantParamType(op)
+  std::vector<std::string> operands;   // value names in operand order; "" is a NoneOp
+  std::map<std::string, double> attrs; // numeric attributes (param struct fields, do_relu, axis...)
+
+  double attr(const std::string &key, double dflt) const;
+  double attr(const std::string &key) const;  // throws if absent
+  std::string signature() const;              // text of everything but the name (dirty check)
+};
+
+// A weight tensor as tpu.load_weight yields it: float-stored values
+// (MlirModuleInterpreter.cpp:353-369).
+struct WeightData {
+  std::vector<float> data;
+  size_t size() const { return data.size(); }
+  float at(size_t i) const { return data.at(i); }
+};
+
+// An activation tensor: `batch` slots of one int8 channels-last image set in HBM.
+// Mirrors mlir::TensorData (cpukernel.h:15-78): size(), set_batch_idx(),
+// assign(), tensor(bidx).
+class TensorData {
+public:
+  TensorData(tpuhip_ctx *ctx, int32_t batch, const SyncedDataShape &shape);
+  ~TensorData();
+  TensorData(const TensorData &) = delete;
+  TensorData &operator=(const TensorData &) = delete;
+
+  size_t size() const { return size_; }          // logical elements of one slot
+  void *data() const { return ptr_; }            // device address of the current slot
+  void set_batch_idx(int32_t bidx);
+  int32_t batch_idx() const { return cur_; }
+  // float-stored NCHW host data -> slot bidx (values must be integers in [-128,127])
+  void assign(const float *first, size_t num, int32_t bidx);
+  // slot bidx as float-stored NCHW host data
+  std::shared_ptr<std::vector<float>> tensor(int32_t bidx) const;
+  // slot bidx as int8 NCHW host data (no float detour)
+  void read_i8(int8_t *dst, size_t num, int32_t bidx) const;
+
+  int32_t batch;
+  int n = 1, c = 1, h = 1, w = 1;  // 4-d view of the shape (missing dims are 1)
+  int cs = 16;                     // channel stride in bytes
+  size_t slot_bytes() const { return (size_t)n * h * w * cs; }
+  tpuhip_ctx *ctx() const { return ctx_; }
+
+private:
+  tpuhip_ctx *ctx_;
+  size_t size_;
+  void *base_ = nullptr;
+  void *ptr_ = nullptr;
+  int32_t cur_ = 0;
+};
+
+enum class DataType { INT8, BF16, FP32 };
+
+using SyncedData = std::shared_ptr<TensorData>;
+using SyncedWeight = std::shared_ptr<WeightData>;
+
+struct value_map_t : std::map<std::string, SyncedData> {
+  tpuhip_ctx *ctx = nullptr;
+  std::map<std::string, SyncedDataShape> shapes;  // result shape of every value
+};
+using weight_map_t = std::map<std::string, SyncedWeight>;
+
+// One operand: an activation, a weight, or none (cpukernel.cpp:50-73).
+struct Operand {
+  SyncedData act;
+  SyncedWeight weight;
+  explicit operator bool() const { return act || weight; }
+};
+
+class CPUOpKernel {
+public:
+  CPUOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+              bool hasOpds = true);
+  CPUOpKernel() = delete;
+  virtual ~CPUOpKernel() {}
+
+  virtual void set_tensor(const std::vector<float> &data);
+  virtual void invoke() = 0;
+
+  std::string get_name() { return name; }
+  SyncedDataShape get_shape() { return shape; }
+  std::string get_data_type();
+  void set_name(std::string n) { name = std::move(n); }
+  void set_shape(SyncedDataShape &s) { shape = s; }
+  void set_datatype(std::string type);
+  std::string get_op_type() { return op_type; }
+  virtual void dump();
+  std::vector<float> get_tensor();
+  static std::string generateSignature(OpDesc &op);
+
+  SyncedDataShape shape;
+  std::string name;
+  std::string op_type;
+  size_t size = 0;
+  DataType datatype = DataType::FP32;
+  OpDesc *op = nullptr;
+  std::string signature;
+  bool dirty = true;
+  static int32_t max_batch_size;
+
+protected:
+  void assignOperandTensors(OpDesc &op, const value_map_t &valueMapping,
+                            const weight_map_t &weightMapping);
+  void assignResultTensor(OpDesc &op, value_map_t &valueMapping);
+  void require_int8(const char *what) const;
+  tpuhip_ctx *ctx = nullptr;
+  std::vector<Operand> opdTensors;
+  SyncedData resTensor;
+};
+
+// ---- per-op kernels (same class names as the reference's) -----------------
+
+class InputOpKernel : public CPUOpKernel {  // core/input.cpp
+public:
+  static constexpr const char *OpName = "CPUInputOp";
+  InputOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+                std::vector<std::pair<std::string, size_t>> &input_details);
+  void invoke() override {}
+  void set_tensor(const std::vector<float> &data) override;
+};
+
+class Conv2DOpKernel : public CPUOpKernel {  // core/conv.cpp
+public:
+  static constexpr const char *OpName = "CPUConv2DOp";
+  Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~Conv2DOpKernel() override;
+  void invoke() override;
+  const char *algo_name() const;
+  tpuhip_conv_desc desc{};
+
+private:
+  tpuhip_conv_weights *packed = nullptr;
+  SyncedData input_data, output_data;
+};
+
+class FullyConnectedOpKernel : public CPUOpKernel {  // core/fullyconnected.cpp
+public:
+  static constexpr const char *OpName = "CPUFullyConnectedOp";
+  FullyConnectedOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~FullyConnectedOpKernel() override;
+  void invoke() override;
+  int m = 0, k = 0, n = 0;
+
+private:
+  tpuhip_conv_weights *packed = nullptr;
+  SyncedData input_data, output_data;
+};
+
+class EltwiseAddOpKernel : public CPUOpKernel {  // core/eltwise.cpp:7-100
+public:
+  static constexpr const char *OpName = "CPUEltwiseAddOp";
+  EltwiseAddOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  std::vector<SyncedData> inputs_data;
+  SyncedData output_data;
+  std::vector<int8_t> multiplier;
+  int rshift = 0;
+  bool do_relu = false;
+};
+
+class PoolingOpKernel : public CPUOpKernel {  // core/pooling.cpp
+public:
+  static constexpr const char *OpName = "CPUPoolingOp";
+  PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  tpuhip_pool_desc desc{};
+  bool is_avg = false;
+  uint32_t rshift = 0, multiplier = 0;
+  SyncedData input_data, output_data;
+};
+
+// 256-entry table ops.  LeakyRelu (core/activation.cpp:104-153), Clip
+// (core/clip.cpp) and the y0_table activations -- Sigmoid, Exp, Mish, Swish,
+// Elu, SoftPlus, Pow, TanH, Log -- (core/activation.cpp:47-53 and siblings) all
+// reduce to one lookup per int8 element.
+class LutOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPULutOp";
+  LutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+  int8_t table[256];
+
+protected:
+  SyncedData input_data, output_data;
+};
+
+class LeakyReluOpKernel : public LutOpKernel {
+public:
+  static constexpr const char *OpName = "CPULeakyReluOp";
+  LeakyReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+};
+
+class ClipOpKernel : public LutOpKernel {
+public:
+  static constexpr const char *OpName = "CPUClipOp";
+  ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+};
+
+class ReluOpKernel : public CPUOpKernel {  // core/activation.cpp:155-164
+public:
+  static constexpr const char *OpName = "CPUReluOp";
+  ReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+};
+
+class UpsampleOpKernel : public CPUOpKernel {  // core/upsample.cpp
+public:
+  static constexpr const char *OpName = "CPUUpsampleOp";
+  UpsampleOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  int scale_h = 1, scale_w = 1;
+  SyncedData input_data, output_data;
+};
+
+class ConcatOpKernel : public CPUOpKernel {  // core/concat.cpp
+public:
+  static constexpr const char *OpName = "CPUConcatOp";
+  ConcatOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  int axis = 1;
+  size_t input_number = 0;
+  bool do_relu = false, need_quant = false;
+  std::vector<uint32_t> rshift, multiplier;
+  std::vector<SyncedData> inputs_data;
+  SyncedData output_data;
+};
+
+// tpu.reshape whose source and result are not the same bytes in channels-last
+// order (the reference aliases the NCHW buffer: MlirModuleInterpreter.cpp:331-338).
+class ReshapeOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPUReshapeOp";
+  ReshapeOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~ReshapeOpKernel() override;
+  void invoke() override;
+  static bool is_alias(const SyncedDataShape &from, const SyncedDataShape &to);
+
+private:
+  SyncedData input_data, output_data;
+  void *scratch = nullptr;
+};
+
+// ---- module interpreter -------------------------------------------------------
+
+using activations_map_t = std::map<std::string, SyncedData>;
+using kernel_map_t = std::map<std::string, std::shared_ptr<CPUOpKernel>>;
+using kernel_list_t = std::list<std::shared_ptr<CPUOpKernel>>;
+
+// Mirrors mlir::MlirModuleInterpreter (include/tpuc/MlirModuleInterpreter.h:32-83,
+// lib/Dialect/TPU/Interpreter/MlirModuleInterpreter.cpp:73-457).  A "module" is
+// the list of OpDesc in program order plus the names the function returns.
+struct ModuleDesc {
+  std::vector<OpDesc> ops;
+  std::vector<std::string> returns;
+};
+
+class ModuleInterpreter {
+public:
+  explicit ModuleInterpreter(int32_t batch = 1, int device = 0);
+  ~ModuleInterpreter();
+
+  void loadModule(ModuleDesc &module, std::string target_op);
+  void loadModule(ModuleDesc &module) { loadModule(module, ""); }
+  void fastInvokeAllBatch(std::string name, int32_t batch);
+  void invokeTo(std::string name, int32_t bidx);
+  void invoke(int32_t bidx) { invokeTo("", bidx); }
+  void setTensor(std::string &name, const std::vector<float> &data, int32_t bidx);
+  std::shared_ptr<std::vector<float>> getTensor(std::string &name, int32_t bidx);
+  void getTensorI8(const std::string &name, int8_t *dst, size_t num, int32_t bidx);
+  std::vector<int64_t> getTensorShape(std::string &name);
+  std::string getDataType(std::string &name);
+  // the reference's updateWeightMap reads every tpu.load_weight from the npz
+  // (MlirModuleInterpreter.cpp:352-369); here the caller hands the arrays over
+  void updateWeightMap(const std::string &name, const float *data, size_t count);
+  std::vector<std::string> &outputDetails() { return output_details; }
+  void dump(std::string &name);
+  std::vector<std::string> getAllTensorName();
+  void sync();
+
+  // per-kernel HIP-event timing of one invoke (ms per kernel, in kernel_list_ order)
+  std::vector<std::pair<std::string, float>> timeKernels(int32_t bidx, int iters);
+  // kernels in execution order
+  const kernel_list_t &kernels() const { return kernel_list_; }
+  tpuhip_ctx *context() const { return ctx_; }
+
+  std::vector<std::pair<std::string, size_t>> input_details;
+  std::vector<std::string> output_details;
+  weight_map_t weightMapping;
+  activations_map_t activationMapping;
+  value_map_t valueMapping;
+
+private:
+  void updateKernelList(ModuleDesc &module, std::string &target_op);
+  bool isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op);
+  tpuhip_ctx *ctx_ = nullptr;
+  kernel_map_t kernel_map_;
+  kernel_list_t kernel_list_;
+};
+
+}  // namespace tpuhip

@@ -87,67 +87,76 @@ uint32_t orc_f2u32(float f) { return (uint32_t)(uint64_t)(int64_t)f; }
 /* convolution                                                                */
 /* ------------------------------------------------------------------------- */
 
-static inline int div_floor(int a, int b) { /* b > 0 */
-  int q = a / b, r = a % b;
-  return (r != 0 && r < 0) ? q - 1 : q;
-}
-static inline int div_ceil(int a, int b) { return -div_floor(-a, b); }
-
-/* valid output range [lo, hi) along one axis for a tap at offset 'koff'
- * (= k*dilation - pad) over an input extent 'in' with stride s */
-static inline void tap_range(int koff, int s, int in, int out, int *lo, int *hi) {
-  int l = div_ceil(-koff, s);
-  int h = div_floor(in - 1 - koff, s) + 1;
-  if (l < 0) l = 0;
-  if (h > out) h = out;
-  *lo = l;
-  *hi = h;
-}
-
+/* The reference pads with zeros (MKL-DNN convolution, conv.cpp ignores
+ * pad_value) and inserts ins_h / ins_w zeros between input samples
+ * (my_dilateActivation, NativeCpuImplementation.cpp:480-503).  Both are done
+ * here by materialising the dilated, padded planes once; the contraction then
+ * runs over plain in-bounds windows.  For stride 1 a tap contributes to the
+ * whole output plane (kept at the padded row pitch) as one long vector
+ * operation, which is what makes full-size graphs checkable in seconds. */
 #define CONV_BODY(ACC_T, X_T, W_T, MUL)                                                     \
   const int icg = d->ic / d->g, ocg = d->oc / d->g;                                         \
   const int ihd = (d->ih - 1) * (d->ins_h + 1) + 1;                                         \
   const int iwd = (d->iw - 1) * (d->ins_w + 1) + 1;                                         \
+  const int ihp = ihd + d->pt + d->pb, iwp = iwd + d->pl + d->pr;                           \
+  const int64_t plane = (int64_t)ihp * iwp;                                                 \
+  /* rows the windows may touch beyond ihp when oh was rounded up by the importer */       \
+  const int need_h = (d->oh - 1) * d->sh + (d->kh - 1) * d->dh + 1;                         \
+  const int need_w = (d->ow - 1) * d->sw + (d->kw - 1) * d->dw + 1;                         \
+  if (need_h > ihp || need_w > iwp) abort(); /* caller passed an impossible output size */ \
+  X_T *xp = (X_T *)calloc((size_t)d->n * d->ic * plane + 64, sizeof(X_T));                  \
+  _Pragma("omp parallel for")                                                               \
+  for (int64_t nc = 0; nc < (int64_t)d->n * d->ic; ++nc)                                    \
+    for (int h = 0; h < d->ih; ++h)                                                         \
+      for (int w_ = 0; w_ < d->iw; ++w_)                                                    \
+        xp[nc * plane + (int64_t)(d->pt + h * (d->ins_h + 1)) * iwp + d->pl +               \
+           w_ * (d->ins_w + 1)] = x[(nc * d->ih + h) * d->iw + w_];                         \
   const int64_t osz = (int64_t)d->oh * d->ow;                                               \
-  _Pragma("omp parallel for collapse(2) schedule(dynamic, 1)")                              \
-  for (int n = 0; n < d->n; ++n) {                                                          \
-    for (int oc = 0; oc < d->oc; ++oc) {                                                    \
-      ACC_T *a = acc + ((int64_t)n * d->oc + oc) * osz;                                     \
-      for (int64_t i = 0; i < osz; ++i) a[i] = 0;                                           \
-      const int gi = oc / ocg;                                                              \
-      for (int c = 0; c < icg; ++c) {                                                       \
-        const X_T *xp = x + ((int64_t)n * d->ic + (int64_t)gi * icg + c) * d->ih * d->iw;   \
-        for (int kh = 0; kh < d->kh; ++kh) {                                                \
-          for (int kw = 0; kw < d->kw; ++kw) {                                              \
-            const W_T wv = w[(((int64_t)oc * icg + c) * d->kh + kh) * d->kw + kw];          \
-            if (wv == 0) continue;                                                          \
-            const int hoff = kh * d->dh - d->pt, woff = kw * d->dw - d->pl;                 \
-            int oh0, oh1, ow0, ow1;                                                         \
-            tap_range(hoff, d->sh, ihd, d->oh, &oh0, &oh1);                                 \
-            tap_range(woff, d->sw, iwd, d->ow, &ow0, &ow1);                                 \
-            for (int oh = oh0; oh < oh1; ++oh) {                                            \
-              const int hp = oh * d->sh + hoff;                                             \
-              if (d->ins_h && (hp % (d->ins_h + 1))) continue;                              \
-              const X_T *xr = xp + (int64_t)(hp / (d->ins_h + 1)) * d->iw;                  \
-              ACC_T *ar = a + (int64_t)oh * d->ow;                                          \
-              if (d->ins_w == 0 && d->sw == 1) {                                            \
-                const X_T *xs = xr + woff;                                                  \
-                for (int ow = ow0; ow < ow1; ++ow) ar[ow] += MUL(wv, xs[ow]);               \
-              } else if (d->ins_w == 0) {                                                   \
-                for (int ow = ow0; ow < ow1; ++ow) ar[ow] += MUL(wv, xr[ow * d->sw + woff]); \
+  const int64_t span = (int64_t)(d->oh - 1) * iwp + d->ow; /* stride-1 plane at pitch iwp */ \
+  _Pragma("omp parallel")                                                                   \
+  {                                                                                         \
+    ACC_T *ap = (ACC_T *)malloc(sizeof(ACC_T) * (size_t)(d->oh * (int64_t)iwp + 64));       \
+    _Pragma("omp for collapse(2) schedule(dynamic, 1)")                                     \
+    for (int n = 0; n < d->n; ++n) {                                                        \
+      for (int oc = 0; oc < d->oc; ++oc) {                                                  \
+        const int gi = oc / ocg;                                                            \
+        const int unit = (d->sh == 1 && d->sw == 1);                                        \
+        if (unit) {                                                                         \
+          for (int64_t i = 0; i < span; ++i) ap[i] = 0;                                     \
+        } else {                                                                            \
+          for (int64_t i = 0; i < osz; ++i) ap[i] = 0;                                      \
+        }                                                                                   \
+        for (int c = 0; c < icg; ++c) {                                                     \
+          const X_T *xc = xp + ((int64_t)n * d->ic + (int64_t)gi * icg + c) * plane;        \
+          for (int kh = 0; kh < d->kh; ++kh) {                                              \
+            for (int kw = 0; kw < d->kw; ++kw) {                                            \
+              const W_T wv = w[(((int64_t)oc * icg + c) * d->kh + kh) * d->kw + kw];        \
+              if (wv == 0) continue;                                                        \
+              const X_T *xt = xc + (int64_t)kh * d->dh * iwp + kw * d->dw;                  \
+              if (unit) {                                                                   \
+                for (int64_t i = 0; i < span; ++i) ap[i] += MUL(wv, xt[i]);                 \
               } else {                                                                      \
-                for (int ow = ow0; ow < ow1; ++ow) {                                        \
-                  const int wp = ow * d->sw + woff;                                         \
-                  if (wp % (d->ins_w + 1)) continue;                                        \
-                  ar[ow] += MUL(wv, xr[wp / (d->ins_w + 1)]);                               \
+                for (int oh = 0; oh < d->oh; ++oh) {                                        \
+                  const X_T *xr = xt + (int64_t)oh * d->sh * iwp;                           \
+                  ACC_T *ar = ap + (int64_t)oh * d->ow;                                     \
+                  for (int ow = 0; ow < d->ow; ++ow) ar[ow] += MUL(wv, xr[ow * d->sw]);     \
                 }                                                                           \
               }                                                                             \
             }                                                                               \
           }                                                                                 \
         }                                                                                   \
+        ACC_T *a = acc + ((int64_t)n * d->oc + oc) * osz;                                   \
+        if (unit) {                                                                         \
+          for (int oh = 0; oh < d->oh; ++oh)                                                \
+            for (int ow = 0; ow < d->ow; ++ow) a[oh * d->ow + ow] = ap[(int64_t)oh * iwp + ow]; \
+        } else {                                                                            \
+          for (int64_t i = 0; i < osz; ++i) a[i] = ap[i];                                   \
+        }                                                                                   \
       }                                                                                     \
     }                                                                                       \
-  }
+    free(ap);                                                                               \
+  }                                                                                         \
+  free(xp);
 
 #define MUL_I32(a, b) ((int32_t)(a) * (int32_t)(b))
 #define MUL_ABS(a, b) (abs((int32_t)(a)) * abs((int32_t)(b)))

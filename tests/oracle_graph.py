@@ -1,0 +1,88 @@
+"""Runs a graphs.Graph through the CPU oracle (test infrastructure): NCHW int8
+tensors, every op's result kept, so the GPU run can be compared layer by layer."""
+import numpy as np
+
+import oracle_lib as O
+
+
+def _conv(op, x):
+    a = op.attrs
+    w = op.weights["filter"].astype(np.int8)
+    g = int(a["group"])
+    oc = op.shape[1]
+    w = w.reshape(oc, -1, int(a["kernel_h"]), int(a["kernel_w"]))
+    d = O.make_conv_desc(
+        x.shape, w.shape, g, (int(a["stride_h"]), int(a["stride_w"])),
+        (int(a["padding_t"]), int(a["padding_b"]), int(a["padding_l"]), int(a["padding_r"])),
+        (int(a["dilation_h"]), int(a["dilation_w"])), (int(a.get("ins_h", 0)), int(a.get("ins_w", 0))),
+        bool(a["do_relu"]), bool(a["with_bias"]), (op.shape[2], op.shape[3]))
+    return O.conv2d_i8(x, w, op.weights.get("bias"), op.weights["rshift"],
+                       op.weights["multiplier"], d), d, w
+
+
+def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=None):
+    """Returns {name: int8 NCHW array}.  batch_slice selects images (ops are
+    independent across the batch, which is also how the reference runs a batch:
+    one N=1 pass per slot).  guards: dict filled with the fp32-exactness guard of
+    every conv / fc when given."""
+    vals = {}
+    for op in graph.ops:
+        ins = [vals[n] for n in op.inputs]
+        t = op.type
+        if t == "tpu.input":
+            y = op.data if input_data is None else input_data
+            if batch_slice is not None:
+                y = np.ascontiguousarray(y[batch_slice])
+        elif t == "tpu.conv_2d":
+            y, d, w = _conv(op, ins[0])
+            if guards is not None:
+                guards[op.name] = O.conv2d_guard(ins[0], w, d) + int(
+                    np.abs(op.weights["bias"]).max())
+        elif t == "tpu.fully_connected":
+            x = ins[0].reshape(ins[0].shape[0], -1)
+            w = op.weights["filter"].astype(np.int8)
+            y = O.fc_i8(x, w, op.weights.get("bias"), op.weights["rshift"],
+                        op.weights["multiplier"], 1, x.shape[0], x.shape[1], w.shape[0],
+                        bool(op.attrs.get("do_relu", 0)))[0]
+            if guards is not None:
+                guards[op.name] = O.fc_guard(x, w, op.weights.get("bias"), 1, x.shape[0],
+                                             x.shape[1], w.shape[0])
+        elif t == "tpu.eltwise_add":
+            y = O.eltwise_add_i8(ins, op.weights["multiplier"], op.weights["rshift"],
+                                 bool(op.attrs["do_relu"]))
+        elif t in ("tpu.pool_max_2d", "tpu.pool_avg_2d"):
+            a = op.attrs
+            d = O.make_pool_desc(ins[0].shape, (int(a["kernel_h"]), int(a["kernel_w"])),
+                                 (int(a["stride_h"]), int(a["stride_w"])),
+                                 (int(a["padding_t"]), int(a["padding_b"]), int(a["padding_l"]),
+                                  int(a["padding_r"])), (op.shape[2], op.shape[3]))
+            if t == "tpu.pool_max_2d":
+                y = O.pool_max_i8(ins[0], d)
+            else:
+                y = O.pool_avg_i8(ins[0], d, op.weights["rshift"][0], op.weights["multiplier"][0])
+        elif t == "tpu.leaky_relu":
+            w = op.weights
+            y = O.leaky_relu_i8(ins[0], w["rshift_pos"][0], w["multiplier_pos"][0],
+                                w["rshift_neg"][0], w["multiplier_neg"][0])
+        elif t == "tpu.clip":
+            y = O.clip_i8(ins[0], op.attrs["min"], op.attrs["max"], op.weights["rshift"][0],
+                          op.weights["multiplier"][0])
+        elif t == "tpu.lut":
+            y = O.lut_i8(ins[0], op.weights["table"])
+        elif t == "tpu.relu":
+            y = O.relu_i8(ins[0])
+        elif t == "tpu.upsample":
+            y = O.upsample_i8(ins[0], int(op.attrs["scale_h"]), int(op.attrs["scale_w"]))
+        elif t == "tpu.concat":
+            y = O.concat_i8(ins, int(op.attrs["axis"]), op.weights.get("rshift"),
+                            op.weights.get("multiplier"), bool(op.attrs.get("do_relu", 0)))
+        elif t == "tpu.reshape":
+            y = ins[0].reshape((ins[0].shape[0],) + tuple(op.shape[1:]))
+        else:
+            raise NotImplementedError(t)
+        vals[op.name] = y
+        if upto is not None and op.name == upto:
+            break
+    if keep is not None:
+        return {k: vals[k] for k in keep}
+    return vals

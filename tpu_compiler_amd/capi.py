@@ -73,6 +73,50 @@ PROTOTYPES = {
 }
 
 
+class OpDescC(C.Structure):
+    _fields_ = [("type", C.c_char_p), ("name", C.c_char_p), ("quant", C.c_char_p),
+                ("param_type", C.c_char_p), ("ndim", C.c_int), ("shape", C.POINTER(C.c_int64)),
+                ("n_operands", C.c_int), ("operands", C.POINTER(C.c_char_p)),
+                ("n_attrs", C.c_int), ("attr_keys", C.POINTER(C.c_char_p)),
+                ("attr_values", C.POINTER(C.c_double))]
+
+
+PROTOTYPES.update({
+    "tpuhip_module_create": (C.c_int, [C.c_int, C.c_int, c_void_pp]),
+    "tpuhip_module_destroy": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_set_weight": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]),
+    "tpuhip_module_clear_ops": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_add_op": (C.c_int, [C.c_void_p, C.POINTER(OpDescC)]),
+    "tpuhip_module_set_returns": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), C.c_int]),
+    "tpuhip_module_load": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "tpuhip_module_set_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,
+                                           C.c_int]),
+    "tpuhip_module_get_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,
+                                           C.c_int]),
+    "tpuhip_module_get_tensor_i8": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,
+                                              C.c_int]),
+    "tpuhip_module_invoke": (C.c_int, [C.c_void_p, C.c_int]),
+    "tpuhip_module_invoke_to": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
+    "tpuhip_module_fast_invoke_all_batch": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
+    "tpuhip_module_sync": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_tensor_shape": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64),
+                                             C.POINTER(C.c_int)]),
+    "tpuhip_module_tensor_dtype": (C.c_char_p, [C.c_void_p, C.c_char_p]),
+    "tpuhip_module_num_tensors": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_tensor_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_module_num_inputs": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_input_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_module_num_outputs": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_output_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_module_num_kernels": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_kernel_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_module_kernel_algo": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_module_time_kernels": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float),
+                                             C.c_int]),
+    "tpuhip_module_ctx": (C.c_void_p, [C.c_void_p]),
+})
+
+
 class TpuHipError(RuntimeError):
     def __init__(self, status, message):
         super().__init__("tpuhip status %d: %s" % (status, message))

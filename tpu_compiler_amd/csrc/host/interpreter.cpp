@@ -1,0 +1,238 @@
+// ModuleInterpreter: builds the kernel list from a module description and runs
+// it in program order on the context's stream.  Mirrors
+// lib/Dialect/TPU/Interpreter/MlirModuleInterpreter.cpp:73-457.
+#include "tpuhip/interpreter.hpp"
+
+#include <cstdio>
+
+namespace tpuhip {
+
+namespace {
+[[noreturn]] void fail(const std::string &msg) { throw std::runtime_error(msg); }
+void ck(int status, const char *what) {
+  if (status != 0) fail(std::string(what) + ": " + tpuhip_last_error());
+}
+
+bool is_lut_op(const std::string &t) {
+  static const char *names[] = {"tpu.sigmoid", "tpu.exp", "tpu.mish", "tpu.swish", "tpu.elu",
+                                "tpu.softplus", "tpu.pow", "tpu.tanh", "tpu.log", "tpu.sqrt",
+                                "tpu.lut"};
+  for (auto n : names)
+    if (t == n) return true;
+  return false;
+}
+}  // namespace
+
+ModuleInterpreter::ModuleInterpreter(int32_t batch, int device) {
+  if (batch < 1) fail("ModuleInterpreter: batch < 1");
+  CPUOpKernel::max_batch_size = batch;
+  ck(tpuhip_ctx_create(device, &ctx_), "ModuleInterpreter");
+  valueMapping.ctx = ctx_;
+}
+
+ModuleInterpreter::~ModuleInterpreter() {
+  if (ctx_) tpuhip_sync(ctx_);
+  kernel_list_.clear();
+  kernel_map_.clear();
+  activationMapping.clear();
+  valueMapping.clear();
+  if (ctx_) tpuhip_ctx_destroy(ctx_);
+}
+
+void ModuleInterpreter::updateWeightMap(const std::string &name, const float *data, size_t count) {
+  auto w = std::make_shared<WeightData>();
+  w->data.assign(data, data + count);
+  weightMapping[name] = w;
+}
+
+void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
+  updateKernelList(module, target_op);
+}
+
+// MlirModuleInterpreter.cpp:85-116
+bool ModuleInterpreter::isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op) {
+  if (op->type == "tpu.input") return false;
+  if (krnl->dirty) return true;
+  auto new_signature = CPUOpKernel::generateSignature(*op);
+  bool dirty = krnl->signature != new_signature;
+  if (!dirty) {
+    for (auto &opd : op->operands) {
+      if (opd.empty()) continue;
+      auto it = kernel_map_.find(opd);
+      if (it == kernel_map_.end()) continue;
+      if (it->second && it->second->dirty) {
+        dirty = true;
+        break;
+      }
+    }
+  }
+  return dirty;
+}
+
+// MlirModuleInterpreter.cpp:118-350
+void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target_op) {
+  kernel_list_.clear();
+  static_cast<std::map<std::string, SyncedData> &>(valueMapping).clear();
+  output_details = module.returns;
+  bool completed = false;
+  for (auto &opd : module.ops) {
+    if (completed) break;
+    OpDesc *op = &opd;
+    const std::string &name = op->name;
+    if (!target_op.empty() && target_op == name) completed = true;
+
+    auto it = kernel_map_.find(name);
+    if (it != kernel_map_.end() && it->second && op->type != "tpu.reshape") {
+      auto &krnl = it->second;
+      bool dirty = isKernelDirty(krnl, op);
+      if (!dirty) {
+        krnl->dirty = false;
+        krnl->op = op;
+        valueMapping[name] = activationMapping[name];
+        valueMapping.shapes[name] = op->shape;
+        kernel_list_.emplace_back(krnl);
+        continue;
+      }
+      activationMapping.erase(name);
+    }
+
+    std::shared_ptr<CPUOpKernel> krnl;
+    const std::string &t = op->type;
+    if (t == "tpu.input") {
+      // a reloaded module keeps its input kernel (and the data set on it)
+      krnl = std::make_shared<InputOpKernel>(*op, valueMapping, weightMapping, input_details);
+    } else if (t == "tpu.conv_2d") {
+      krnl = std::make_shared<Conv2DOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.fully_connected") {
+      krnl = std::make_shared<FullyConnectedOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.eltwise_add") {
+      krnl = std::make_shared<EltwiseAddOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.pool_avg_2d" || t == "tpu.pool_max_2d") {
+      krnl = std::make_shared<PoolingOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.leaky_relu") {
+      krnl = std::make_shared<LeakyReluOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.clip") {
+      krnl = std::make_shared<ClipOpKernel>(*op, valueMapping, weightMapping);
+    } else if (is_lut_op(t)) {
+      krnl = std::make_shared<LutOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.relu") {
+      krnl = std::make_shared<ReluOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.upsample") {
+      krnl = std::make_shared<UpsampleOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.concat") {
+      krnl = std::make_shared<ConcatOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.reshape") {
+      if (op->operands.empty()) fail("reshape '" + name + "': no operand");
+      const std::string &src = op->operands[0];
+      auto vit = valueMapping.find(src);
+      if (vit == valueMapping.end()) fail("reshape '" + name + "': operand '" + src + "' not found");
+      if (ReshapeOpKernel::is_alias(valueMapping.shapes[src], op->shape)) {
+        // zero-copy alias (MlirModuleInterpreter.cpp:331-338)
+        auto resTensor = vit->second;
+        activationMapping[name] = resTensor;
+        valueMapping[name] = resTensor;
+        valueMapping.shapes[name] = op->shape;
+        kernel_map_[name] = kernel_map_[src];
+        continue;
+      }
+      krnl = std::make_shared<ReshapeOpKernel>(*op, valueMapping, weightMapping);
+    } else {
+      fail("no support " + t + " op in interpreter_v2");
+    }
+    activationMapping[name] = valueMapping[name];
+    kernel_map_[name] = krnl;
+    kernel_list_.emplace_back(krnl);
+  }
+}
+
+// MlirModuleInterpreter.cpp:371-381
+void ModuleInterpreter::invokeTo(std::string name, int32_t bidx) {
+  for (auto &kv : valueMapping) kv.second->set_batch_idx(bidx);
+  for (auto &krnl : kernel_list_) {
+    krnl->invoke();
+    if (!name.empty() && name == krnl->name) break;
+  }
+}
+
+// MlirModuleInterpreter.cpp:383-405
+void ModuleInterpreter::fastInvokeAllBatch(std::string name, int32_t batch) {
+  bool last_batch = false;
+  for (int i = 0; i < batch; i++) {
+    if (i == batch - 1) last_batch = true;
+    for (auto &kv : valueMapping) kv.second->set_batch_idx(i);
+    for (auto &krnl : kernel_list_) {
+      if (krnl->dirty) {
+        krnl->invoke();
+        if (last_batch) krnl->dirty = false;
+      }
+      if (!name.empty() && name == krnl->name) break;
+    }
+  }
+}
+
+void ModuleInterpreter::setTensor(std::string &name, const std::vector<float> &data, int32_t bidx) {
+  auto it = activationMapping.find(name);
+  if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");
+  it->second->assign(data.data(), data.size(), bidx);
+}
+
+std::shared_ptr<std::vector<float>> ModuleInterpreter::getTensor(std::string &name, int32_t bidx) {
+  auto it = activationMapping.find(name);
+  if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");
+  return it->second->tensor(bidx);
+}
+
+void ModuleInterpreter::getTensorI8(const std::string &name, int8_t *dst, size_t num, int32_t bidx) {
+  auto it = activationMapping.find(name);
+  if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");
+  it->second->read_i8(dst, num, bidx);
+}
+
+std::vector<int64_t> ModuleInterpreter::getTensorShape(std::string &name) {
+  auto it = valueMapping.shapes.find(name);
+  if (it == valueMapping.shapes.end()) fail(" Not Find Op name: " + name + " tensor");
+  return it->second;
+}
+
+std::string ModuleInterpreter::getDataType(std::string &name) {
+  auto it = kernel_map_.find(name);
+  if (it == kernel_map_.end() || !it->second) fail(" Not Find Op name: " + name + " tensor");
+  return it->second->get_data_type();
+}
+
+void ModuleInterpreter::dump(std::string &name) {
+  for (auto &krnl : kernel_list_)
+    if (krnl->get_name() == name) return krnl->dump();
+  fprintf(stderr, " Not Find Op name: %s tensor \n", name.c_str());
+}
+
+std::vector<std::string> ModuleInterpreter::getAllTensorName() {
+  std::vector<std::string> ret;
+  for (auto &kv : activationMapping) ret.push_back(kv.first);
+  return ret;
+}
+
+void ModuleInterpreter::sync() { ck(tpuhip_sync(ctx_), "sync"); }
+
+std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_t bidx, int iters) {
+  if (iters < 1) iters = 1;
+  for (auto &kv : valueMapping) kv.second->set_batch_idx(bidx);
+  std::vector<std::pair<std::string, float>> out;
+  void *e0 = nullptr, *e1 = nullptr;
+  ck(tpuhip_event_create(ctx_, &e0), "timeKernels");
+  ck(tpuhip_event_create(ctx_, &e1), "timeKernels");
+  for (auto &krnl : kernel_list_) {
+    krnl->invoke();  // warm
+    ck(tpuhip_event_record(ctx_, e0), "timeKernels");
+    for (int i = 0; i < iters; ++i) krnl->invoke();
+    ck(tpuhip_event_record(ctx_, e1), "timeKernels");
+    float ms = 0;
+    ck(tpuhip_event_elapsed_ms(ctx_, e0, e1, &ms), "timeKernels");
+    out.emplace_back(krnl->name, ms / (float)iters);
+  }
+  tpuhip_event_destroy(ctx_, e0);
+  tpuhip_event_destroy(ctx_, e1);
+  return out;
+}
+
+}  // namespace tpuhip

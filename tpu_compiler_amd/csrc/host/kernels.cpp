@@ -1,0 +1,629 @@
+// Host side of the op-level C++ API: TensorData, CPUOpKernel and the per-op
+// kernel classes.  Each class parses its OpDesc the way the reference's
+// constructor parses the mlir::Operation, converts the float-stored parameters
+// with the reference's own conversions, and invoke() issues the HIP work
+// through the C ABI.
+#include "tpuhip/interpreter.hpp"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <sstream>
+
+namespace tpuhip {
+
+namespace {
+
+[[noreturn]] void fail(const std::string &msg) { throw std::runtime_error(msg); }
+
+void ck(int status, const char *what) {
+  if (status != 0) fail(std::string(what) + ": " + tpuhip_last_error());
+}
+
+// (uint32_t)float as x86-64 gcc compiles the reference's implicit and explicit
+// conversions: truncate to a 64-bit integer, keep the low 32 bits.
+uint32_t f2u32(float f) { return (uint32_t)(uint64_t)(int64_t)f; }
+
+// (int8_t)float the same way (eltwise.cpp:66)
+int8_t f2i8(float f) { return (int8_t)(int32_t)f; }
+
+int32_t f2i32(float f) {
+  if (!(f > -2147483904.0f)) return INT32_MIN;
+  if (!(f < 2147483648.0f)) return INT32_MIN;  // x86 cvttss2si "integer indefinite"
+  return (int32_t)f;
+}
+
+int8_t weight_to_i8(float v, const std::string &op, const char *role) {
+  if (!(v >= -128.0f && v <= 127.0f) || v != std::nearbyint(v))
+    fail(op + ": " + role + " value " + std::to_string(v) +
+         " is not an int8; only INT8-quantized weights are supported");
+  return (int8_t)v;
+}
+
+void view4(const SyncedDataShape &s, int *n, int *c, int *h, int *w) {
+  if (s.empty() || s.size() > 4) fail("tensor rank " + std::to_string(s.size()) + " not supported");
+  int64_t d[4] = {1, 1, 1, 1};
+  if (s.size() == 1) {
+    d[1] = s[0];
+  } else {
+    for (size_t i = 0; i < s.size(); ++i) d[i] = s[i];
+  }
+  for (int i = 0; i < 4; ++i)
+    if (d[i] <= 0 || d[i] > INT32_MAX) fail("bad tensor dimension");
+  *n = (int)d[0]; *c = (int)d[1]; *h = (int)d[2]; *w = (int)d[3];
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// OpDesc
+// ---------------------------------------------------------------------------
+double OpDesc::attr(const std::string &key, double dflt) const {
+  auto it = attrs.find(key);
+  return it == attrs.end() ? dflt : it->second;
+}
+
+double OpDesc::attr(const std::string &key) const {
+  auto it = attrs.find(key);
+  if (it == attrs.end()) fail(type + " '" + name + "': missing attribute " + key);
+  return it->second;
+}
+
+std::string OpDesc::signature() const {
+  std::ostringstream os;
+  os << type << "|" << quant << "|" << param_type << "|";
+  for (auto d : shape) os << d << "x";
+  os << "|";
+  for (auto &o : operands) os << o << ",";
+  os << "|";
+  for (auto &kv : attrs) os << kv.first << "=" << kv.second << ";";
+  return os.str();
+}
+
+// ---------------------------------------------------------------------------
+// TensorData
+// ---------------------------------------------------------------------------
+TensorData::TensorData(tpuhip_ctx *ctx, int32_t batch_, const SyncedDataShape &shape)
+    : batch(batch_), ctx_(ctx) {
+  if (batch < 1) fail("TensorData: batch < 1");
+  view4(shape, &n, &c, &h, &w);
+  cs = tpuhip_channel_stride(c);
+  size_ = (size_t)n * c * h * w;
+  ck(tpuhip_malloc(ctx_, slot_bytes() * (size_t)batch, &base_), "TensorData");
+  ptr_ = base_;
+}
+
+TensorData::~TensorData() {
+  if (base_) tpuhip_free(ctx_, base_);
+}
+
+void TensorData::set_batch_idx(int32_t bidx) {
+  if (bidx < 0 || bidx >= batch) fail("TensorData::set_batch_idx: slot out of range");
+  ptr_ = (char *)base_ + slot_bytes() * (size_t)bidx;
+  cur_ = bidx;
+}
+
+void TensorData::assign(const float *first, size_t num, int32_t bidx) {
+  if (num != size_) fail("TensorData::assign: size mismatch");
+  if (bidx < 0 || bidx >= batch) fail("TensorData::assign: slot out of range");
+  for (size_t i = 0; i < num; ++i)
+    if (!(first[i] >= -128.0f && first[i] <= 127.0f) || first[i] != std::nearbyint(first[i]))
+      fail("TensorData::assign: element " + std::to_string(i) + " = " + std::to_string(first[i]) +
+           " is not an int8 value");
+  void *tmp = nullptr;
+  ck(tpuhip_malloc(ctx_, num * sizeof(float), &tmp), "TensorData::assign");
+  int rc = tpuhip_upload(ctx_, tmp, first, num * sizeof(float));
+  if (!rc)
+    rc = tpuhip_nchw_f32_to_nhwc_i8(ctx_, tmp, (char *)base_ + slot_bytes() * (size_t)bidx, n, c, h,
+                                    w, cs);
+  tpuhip_free(ctx_, tmp);  // synchronises the stream first
+  ck(rc, "TensorData::assign");
+}
+
+std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
+  if (bidx < 0 || bidx >= batch) fail("TensorData::tensor: slot out of range");
+  auto out = std::make_shared<std::vector<float>>(size_);
+  void *tmp = nullptr;
+  ck(tpuhip_malloc(ctx_, size_ * sizeof(float), &tmp), "TensorData::tensor");
+  int rc = tpuhip_nhwc_i8_to_nchw_f32(ctx_, (char *)base_ + slot_bytes() * (size_t)bidx, tmp, n, c,
+                                      h, w, cs);
+  if (!rc) rc = tpuhip_download(ctx_, out->data(), tmp, size_ * sizeof(float));
+  tpuhip_free(ctx_, tmp);
+  ck(rc, "TensorData::tensor");
+  return out;
+}
+
+void TensorData::read_i8(int8_t *dst, size_t num, int32_t bidx) const {
+  if (num != size_) fail("TensorData::read_i8: size mismatch");
+  if (bidx < 0 || bidx >= batch) fail("TensorData::read_i8: slot out of range");
+  void *tmp = nullptr;
+  ck(tpuhip_malloc(ctx_, size_, &tmp), "TensorData::read_i8");
+  int rc = tpuhip_nhwc_to_nchw_i8(ctx_, (char *)base_ + slot_bytes() * (size_t)bidx, tmp, n, c, h, w,
+                                  cs);
+  if (!rc) rc = tpuhip_download(ctx_, dst, tmp, size_);
+  tpuhip_free(ctx_, tmp);
+  ck(rc, "TensorData::read_i8");
+}
+
+// ---------------------------------------------------------------------------
+// CPUOpKernel (core/cpukernel.cpp:6-80)
+// ---------------------------------------------------------------------------
+int32_t CPUOpKernel::max_batch_size = 1;
+
+CPUOpKernel::CPUOpKernel(OpDesc &op_, value_map_t &valueMapping, weight_map_t &weightMapping,
+                         bool hasOpds) {
+  ctx = valueMapping.ctx;
+  if (!ctx) fail("CPUOpKernel: the value map carries no context");
+  shape = op_.shape;
+  name = op_.name;
+  op_type = op_.type;
+  set_datatype(op_.quant);
+  size = 1;
+  for (auto d : shape) size *= (size_t)d;
+  if (hasOpds) assignOperandTensors(op_, valueMapping, weightMapping);
+  assignResultTensor(op_, valueMapping);
+  signature = generateSignature(op_);
+  op = &op_;
+}
+
+void CPUOpKernel::set_tensor(const std::vector<float> &) { fail("NOT support set_tensor"); }
+
+std::string CPUOpKernel::get_data_type() {
+  if (datatype == DataType::BF16) return "BF16";
+  if (datatype == DataType::INT8) return "INT8";
+  return "FP32";
+}
+
+void CPUOpKernel::set_datatype(std::string type) {
+  if (type == "NONE")
+    datatype = DataType::FP32;
+  else if (type == "BF16")
+    datatype = DataType::BF16;
+  else if (type == "INT8" || type == "UINT8")
+    datatype = DataType::INT8;
+  else
+    fail("Not support type " + type);
+}
+
+void CPUOpKernel::dump() {
+  if (shape.empty()) fail("No shape");
+  std::string shape_str;
+  for (auto &i : shape) shape_str += std::to_string(i) + " ";
+  printf("%s\n\tName: %s\n\tShape: %s\n\tDataType: %s\n", op_type.c_str(), name.c_str(),
+         shape_str.c_str(), get_data_type().c_str());
+}
+
+std::vector<float> CPUOpKernel::get_tensor() {
+  // deep copy of the current slot, like the reference
+  auto t = resTensor->tensor(resTensor->batch_idx());
+  return *t;
+}
+
+std::string CPUOpKernel::generateSignature(OpDesc &op) { return op.signature(); }
+
+void CPUOpKernel::assignOperandTensors(OpDesc &op_, const value_map_t &valueMapping,
+                                       const weight_map_t &weightMapping) {
+  for (auto &opd : op_.operands) {
+    Operand o;
+    if (opd.empty()) {
+      opdTensors.push_back(o);
+      continue;
+    }
+    auto wit = weightMapping.find(opd);
+    if (wit != weightMapping.end()) {
+      o.weight = wit->second;
+    } else {
+      auto it = valueMapping.find(opd);
+      if (it == valueMapping.end()) fail(op_.name + ": operand '" + opd + "' not found (value mapping false)");
+      o.act = it->second;
+    }
+    opdTensors.push_back(o);
+  }
+}
+
+void CPUOpKernel::assignResultTensor(OpDesc &op_, value_map_t &valueMapping) {
+  resTensor = std::make_shared<TensorData>(ctx, max_batch_size, op_.shape);
+  valueMapping[op_.name] = resTensor;
+  valueMapping.shapes[op_.name] = op_.shape;
+}
+
+void CPUOpKernel::require_int8(const char *what) const {
+  if (datatype != DataType::INT8)
+    fail(std::string(what) + " '" + name + "': only the INT8 path is implemented on the GPU");
+}
+
+// ---------------------------------------------------------------------------
+// Input (core/input.cpp:7-24)
+// ---------------------------------------------------------------------------
+InputOpKernel::InputOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+                             std::vector<std::pair<std::string, size_t>> &input_details)
+    : CPUOpKernel(op, valueMapping, weightMapping, false) {
+  input_details.push_back(std::make_pair(name, resTensor->size()));
+}
+
+void InputOpKernel::set_tensor(const std::vector<float> &data) {
+  if (data.size() != resTensor->size())
+    fail(" Input op: [" + name + "] required memsize :" + std::to_string(resTensor->size()) +
+         ", input data size: " + std::to_string(data.size()) + ": size not same!");
+  resTensor->assign(data.data(), data.size(), resTensor->batch_idx());
+}
+
+// ---------------------------------------------------------------------------
+// Conv2D (core/conv.cpp:11-104)
+// ---------------------------------------------------------------------------
+Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Conv2D");
+  if (opdTensors.size() != 7) fail("Conv2D '" + name + "': expected 7 operands");
+  input_data = opdTensors[0].act;
+  output_data = resTensor;
+  auto filter = opdTensors[1].weight;
+  auto bias = opdTensors[2].weight;
+  auto quant_rshift = opdTensors[5].weight;
+  auto quant_multiplier = opdTensors[6].weight;
+  if (!input_data || !filter) fail("Conv2D '" + name + "': input / filter operand missing");
+  if (!quant_rshift || !quant_multiplier)
+    fail("Conv2D '" + name + "': INT8 conv needs per-channel rshift and multiplier operands");
+
+  // parseConvParam (TPUOperationSupport.cpp:366-428)
+  tpuhip_conv_desc &d = desc;
+  d.kh = (int)op.attr("kernel_h");
+  d.kw = (int)op.attr("kernel_w");
+  d.dh = (int)op.attr("dilation_h", 1);
+  d.dw = (int)op.attr("dilation_w", 1);
+  d.sh = (int)op.attr("stride_h", 1);
+  d.sw = (int)op.attr("stride_w", 1);
+  d.pt = (int)op.attr("padding_t", 0);
+  d.pb = (int)op.attr("padding_b", 0);
+  d.pl = (int)op.attr("padding_l", 0);
+  d.pr = (int)op.attr("padding_r", 0);
+  d.g = (int)op.attr("group", 1);
+  d.with_bias = (int)op.attr("with_bias", bias ? 1 : 0);
+  d.do_relu = (int)op.attr("do_relu", 0);
+  d.ins_h = (int)op.attr("ins_h", 0);
+  d.ins_w = (int)op.attr("ins_w", 0);
+  if (d.kw == 0) d.kw = 1;
+  if (input_data->n != output_data->n) fail("input N not equal to output N");
+  d.n = input_data->n; d.ic = input_data->c; d.ih = input_data->h; d.iw = input_data->w;
+  d.oc = output_data->c; d.oh = output_data->h; d.ow = output_data->w;
+  d.x_cs = input_data->cs;
+  d.y_cs = output_data->cs;
+  d.relu_first = 0;
+  d.algo = (int)op.attr("algo", 0);
+  if (d.g <= 0 || d.ic % d.g || d.oc % d.g) fail("Conv2D '" + name + "': bad group");
+
+  const size_t fsz = (size_t)d.oc * (d.ic / d.g) * d.kh * d.kw;
+  if (filter->size() != fsz) fail("Conv2D '" + name + "': filter size mismatch");
+  if (quant_rshift->size() < (size_t)d.oc || quant_multiplier->size() < (size_t)d.oc)
+    fail("Conv2D '" + name + "': rshift / multiplier need one entry per output channel");
+  std::vector<int8_t> w8(fsz);
+  for (size_t i = 0; i < fsz; ++i) w8[i] = weight_to_i8(filter->at(i), name, "filter");
+  std::vector<int32_t> b32, m32((size_t)d.oc), r32((size_t)d.oc);
+  // without with_bias the epilogue adds a zero tensor (conv.cpp:59-61)
+  if (d.with_bias) {
+    if (!bias || bias->size() < (size_t)d.oc) fail("Conv2D '" + name + "': bias operand missing");
+    b32.resize((size_t)d.oc);
+    for (int i = 0; i < d.oc; ++i) b32[i] = f2i32(bias->at(i));   // (int32_t)bias[i], :859-861
+  }
+  for (int i = 0; i < d.oc; ++i) {
+    // float -> uint32_t at the call, uint32_t -> int32_t inside (:863-865, :534)
+    m32[i] = (int32_t)f2u32(quant_multiplier->at(i));
+    r32[i] = (int32_t)f2u32(quant_rshift->at(i));
+  }
+  ck(tpuhip_conv2d_prepack(ctx, &d, w8.data(), d.with_bias ? b32.data() : nullptr, m32.data(),
+                           r32.data(), &packed),
+     ("Conv2D '" + name + "'").c_str());
+}
+
+Conv2DOpKernel::~Conv2DOpKernel() {
+  if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
+}
+
+void Conv2DOpKernel::invoke() {
+  ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+}
+
+const char *Conv2DOpKernel::algo_name() const { return tpuhip_conv2d_algo_name(packed); }
+
+// ---------------------------------------------------------------------------
+// FullyConnected (core/fullyconnected.cpp:7-91)
+// ---------------------------------------------------------------------------
+FullyConnectedOpKernel::FullyConnectedOpKernel(OpDesc &op, value_map_t &valueMapping,
+                                               weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("FullyConnected");
+  if (opdTensors.size() != 7) fail("FullyConnected '" + name + "': expected 7 operands");
+  if (op.attr("input_transpose", 0) != 0 || op.attr("output_transpose", 0) != 0)
+    fail("FullyConnected '" + name + "': transposed variants are not implemented");
+  input_data = opdTensors[0].act;
+  output_data = resTensor;
+  auto filter = opdTensors[1].weight;
+  auto bias = opdTensors[2].weight;
+  auto rshift_data = opdTensors[5].weight;
+  auto multiplier_data = opdTensors[6].weight;
+  if (!input_data || !filter || !rshift_data || !multiplier_data)
+    fail("FullyConnected '" + name + "': operand missing");
+  // parseFullyConnectedParam (TPUOperationSupport.cpp:568-605), batch_low == batch_high == 1:
+  // m = product of the leading input dims, n = rows of the filter, k = its columns
+  n = output_data->c * output_data->h * output_data->w;
+  if (op.shape.size() != 2) fail("FullyConnected '" + name + "': result must be [m, n]");
+  m = (int)op.shape[0];
+  n = (int)op.shape[1];
+  if (filter->size() % (size_t)n) fail("FullyConnected '" + name + "': filter size mismatch");
+  k = (int)(filter->size() / (size_t)n);
+  if (input_data->size() != (size_t)m * k) fail("FullyConnected '" + name + "': input size mismatch");
+  if (input_data->h * input_data->w != 1)
+    fail("FullyConnected '" + name + "': input must be [m, k] (reshape first)");
+  std::vector<int8_t> w8(filter->size());
+  for (size_t i = 0; i < w8.size(); ++i) w8[i] = weight_to_i8(filter->at(i), name, "filter");
+  std::vector<int32_t> b32;
+  if (bias) {
+    if (bias->size() < (size_t)n) fail("FullyConnected '" + name + "': bias size mismatch");
+    b32.resize((size_t)n);
+    for (int i = 0; i < n; ++i) b32[i] = f2i32(bias->at(i));
+  }
+  // (uint32_t)rshift_data->at(i), (uint32_t)multiplier_data->at(i) with i the batch index
+  // (:78-87); batch == 1 here
+  const int32_t rs = (int32_t)f2u32(rshift_data->at(0));
+  const int32_t mu = (int32_t)f2u32(multiplier_data->at(0));
+  ck(tpuhip_fc_prepack(ctx, m, k, n, input_data->cs, output_data->cs, (int)op.attr("do_relu", 0),
+                       w8.data(), bias ? b32.data() : nullptr, mu, rs, &packed),
+     ("FullyConnected '" + name + "'").c_str());
+}
+
+FullyConnectedOpKernel::~FullyConnectedOpKernel() {
+  if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
+}
+
+void FullyConnectedOpKernel::invoke() {
+  ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// EltwiseAdd (core/eltwise.cpp:7-100)
+// ---------------------------------------------------------------------------
+EltwiseAddOpKernel::EltwiseAddOpKernel(OpDesc &op, value_map_t &valueMapping,
+                                       weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("EltwiseAdd");
+  if (opdTensors.size() < 5) fail("EltwiseAdd '" + name + "': expected inputs + 4 operands");
+  const size_t nInputs = opdTensors.size() - 4;
+  if (op.param_type == "NONE")
+    fail("EltwiseAdd '" + name + "': the unquantized (fp32) fallback is not implemented");
+  do_relu = op.attr("do_relu", 0) != 0;
+  auto quant_rshift = opdTensors[nInputs + 2].weight;
+  auto quant_multiplier = opdTensors[nInputs + 3].weight;
+  if (!quant_rshift || !quant_multiplier) fail("EltwiseAdd '" + name + "': rshift / multiplier missing");
+  if (quant_multiplier->size() < nInputs || quant_rshift->size() < 1)
+    fail("EltwiseAdd '" + name + "': one multiplier per input and one rshift needed");
+  rshift = (int)f2u32(quant_rshift->at(0));                                    // :81-83
+  for (size_t i = 0; i < nInputs; ++i) multiplier.push_back(f2i8(quant_multiplier->at(i)));  // :66
+  for (size_t i = 0; i < nInputs; ++i) {
+    auto t = opdTensors[i].act;
+    if (!t) fail("EltwiseAdd '" + name + "': input " + std::to_string(i) + " is not an activation");
+    if (t->slot_bytes() != resTensor->slot_bytes() || t->size() != resTensor->size())
+      fail("EltwiseAdd '" + name + "': input shapes differ");
+    inputs_data.push_back(t);
+  }
+  output_data = resTensor;
+}
+
+void EltwiseAddOpKernel::invoke() {
+  std::vector<const void *> ptrs;
+  for (auto &t : inputs_data) ptrs.push_back(t->data());
+  ck(tpuhip_eltwise_add_i8(ctx, ptrs.data(), (int)ptrs.size(), multiplier.data(), rshift,
+                           do_relu ? 1 : 0, output_data->data(), output_data->slot_bytes()),
+     name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// Pooling (core/pooling.cpp:33-160)
+// ---------------------------------------------------------------------------
+PoolingOpKernel::PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Pooling");
+  is_avg = op.type == "tpu.pool_avg_2d";
+  if (op.attr("do_relu", 0) != 0) fail("Pooling '" + name + "': do_relu is not allowed");  // :59
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail("Pooling '" + name + "': input missing");
+  // parsePoolParam (TPUOperationSupport.cpp:479-522)
+  tpuhip_pool_desc &d = desc;
+  d.kh = (int)op.attr("kernel_h");
+  d.kw = (int)op.attr("kernel_w");
+  if (d.kw == 0) d.kw = 1;
+  d.sh = (int)op.attr("stride_h", 1);
+  d.sw = (int)op.attr("stride_w", 1);
+  d.pt = (int)op.attr("padding_t", 0);
+  d.pb = (int)op.attr("padding_b", 0);
+  d.pl = (int)op.attr("padding_l", 0);
+  d.pr = (int)op.attr("padding_r", 0);
+  d.n = input_data->n; d.c = input_data->c; d.ih = input_data->h; d.iw = input_data->w;
+  d.oh = output_data->h; d.ow = output_data->w;
+  d.x_cs = input_data->cs;
+  d.y_cs = output_data->cs;
+  if (output_data->n != d.n || output_data->c != d.c) fail("Pooling '" + name + "': N/C mismatch");
+  if (is_avg) {
+    if (opdTensors.size() < 5 || !opdTensors[3].weight || !opdTensors[4].weight)
+      fail("Pooling '" + name + "': quant_rshift / quant_multiplier is null!");   // :74-79
+    rshift = f2u32(opdTensors[3].weight->at(0));
+    multiplier = f2u32(opdTensors[4].weight->at(0));
+  }
+}
+
+void PoolingOpKernel::invoke() {
+  if (is_avg)
+    ck(tpuhip_pool_avg_i8(ctx, &desc, input_data->data(), output_data->data(), multiplier, rshift),
+       name.c_str());
+  else
+    ck(tpuhip_pool_max_i8(ctx, &desc, input_data->data(), output_data->data()), name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// table ops
+// ---------------------------------------------------------------------------
+LutOpKernel::LutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8(op.type.c_str());
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail(op.type + " '" + name + "': input missing");
+  if (input_data->size() != output_data->size()) fail(op.type + " '" + name + "': shape mismatch");
+  memset(table, 0, sizeof(table));
+  if (op.type != "tpu.leaky_relu" && op.type != "tpu.clip") {
+    // y0_table_op = opdTensors[1] (core/activation.cpp:34-37): 256 float-stored int8 entries,
+    // indexed by the two's-complement byte of the input
+    auto y0 = opdTensors.size() > 1 ? opdTensors[1].weight : nullptr;
+    if (!y0 || y0->size() < 256) fail(op.type + " '" + name + "': y0 table operand missing");
+    for (int i = 0; i < 256; ++i) table[i] = weight_to_i8(y0->at(i), name, "table");
+  }
+}
+
+void LutOpKernel::invoke() {
+  ck(tpuhip_lut_i8(ctx, input_data->data(), output_data->data(), table,
+                   (size_t)input_data->n * input_data->h * input_data->w, input_data->c,
+                   input_data->cs),
+     name.c_str());
+}
+
+LeakyReluOpKernel::LeakyReluOpKernel(OpDesc &op, value_map_t &valueMapping,
+                                     weight_map_t &weightMapping)
+    : LutOpKernel(op, valueMapping, weightMapping) {
+  if (opdTensors.size() < 9) fail("LeakyRelu '" + name + "': expected 9 operands");
+  for (int i = 5; i <= 8; ++i)
+    if (!opdTensors[i].weight) fail("LeakyRelu '" + name + "': rshift / multiplier operand missing");
+  // rshift cast explicitly, multiplier converted implicitly (activation.cpp:137-146)
+  ck(tpuhip_leaky_relu_table(f2u32(opdTensors[5].weight->at(0)), f2u32(opdTensors[6].weight->at(0)),
+                             f2u32(opdTensors[7].weight->at(0)), f2u32(opdTensors[8].weight->at(0)),
+                             table),
+     name.c_str());
+}
+
+ClipOpKernel::ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : LutOpKernel(op, valueMapping, weightMapping) {
+  if (opdTensors.size() < 5 || !opdTensors[3].weight || !opdTensors[4].weight)
+    fail("Clip '" + name + "': rshift / multiplier operand missing");
+  ck(tpuhip_clip_table((float)op.attr("min"), (float)op.attr("max"),
+                       f2u32(opdTensors[3].weight->at(0)), f2u32(opdTensors[4].weight->at(0)),
+                       table),
+     name.c_str());
+}
+
+ReluOpKernel::ReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Relu");
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data || input_data->slot_bytes() != output_data->slot_bytes())
+    fail("Relu '" + name + "': shape mismatch");
+}
+
+void ReluOpKernel::invoke() {
+  ck(tpuhip_relu_i8(ctx, input_data->data(), output_data->data(), output_data->slot_bytes()),
+     name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// Upsample (core/upsample.cpp:7-41)
+// ---------------------------------------------------------------------------
+UpsampleOpKernel::UpsampleOpKernel(OpDesc &op, value_map_t &valueMapping,
+                                   weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Upsample");
+  scale_h = (int)op.attr("scale_h");
+  scale_w = (int)op.attr("scale_w");
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail("Upsample '" + name + "': input missing");
+  if (output_data->h != input_data->h * scale_h || output_data->w != input_data->w * scale_w ||
+      output_data->c != input_data->c || output_data->n != input_data->n)
+    fail("Upsample '" + name + "': result shape does not match the scales");
+}
+
+void UpsampleOpKernel::invoke() {
+  ck(tpuhip_upsample_nearest_i8(ctx, input_data->data(), output_data->data(), input_data->n,
+                                input_data->c, input_data->h, input_data->w, scale_h, scale_w,
+                                input_data->cs, output_data->cs),
+     name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// Concat (core/concat.cpp:8-90)
+// ---------------------------------------------------------------------------
+ConcatOpKernel::ConcatOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Concat");
+  axis = (int)op.attr("axis");
+  if (opdTensors.size() < 5) fail("Concat '" + name + "': expected inputs + 4 operands");
+  input_number = opdTensors.size() - 4;
+  do_relu = op.attr("do_relu", 0) != 0;
+  auto quant_rshift = opdTensors[input_number + 2].weight;
+  auto quant_multiplier = opdTensors[input_number + 3].weight;
+  if (quant_rshift && quant_multiplier) {
+    need_quant = true;
+    if (quant_rshift->size() < input_number || quant_multiplier->size() < input_number)
+      fail("Concat '" + name + "': one rshift / multiplier per input needed");
+    for (size_t i = 0; i < input_number; ++i) {
+      rshift.push_back(f2u32(quant_rshift->at(i)));
+      multiplier.push_back(f2u32(quant_multiplier->at(i)));
+    }
+  }
+  for (size_t i = 0; i < input_number; ++i) {
+    if (!opdTensors[i].act) fail("Concat '" + name + "': input " + std::to_string(i) + " missing");
+    inputs_data.push_back(opdTensors[i].act);
+  }
+  output_data = resTensor;
+  if (op.shape.size() != 4 && axis != 1) fail("Concat '" + name + "': only 4-d tensors off axis 1");
+}
+
+void ConcatOpKernel::invoke() {
+  std::vector<const void *> ptrs;
+  std::vector<int> dims, css;
+  for (auto &t : inputs_data) {
+    ptrs.push_back(t->data());
+    dims.insert(dims.end(), {t->n, t->c, t->h, t->w});
+    css.push_back(t->cs);
+  }
+  ck(tpuhip_concat_i8(ctx, ptrs.data(), (int)ptrs.size(), dims.data(), css.data(), axis,
+                      need_quant ? rshift.data() : nullptr, need_quant ? multiplier.data() : nullptr,
+                      do_relu ? 1 : 0, output_data->data(), output_data->cs),
+     name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// Reshape that cannot alias
+// ---------------------------------------------------------------------------
+bool ReshapeOpKernel::is_alias(const SyncedDataShape &from, const SyncedDataShape &to) {
+  int n0, c0, h0, w0, n1, c1, h1, w1;
+  view4(from, &n0, &c0, &h0, &w0);
+  view4(to, &n1, &c1, &h1, &w1);
+  if (n0 == n1 && c0 == c1 && h0 == h1 && w0 == w1) return true;
+  // [n, c, 1, 1] <-> [n, c]: same bytes in channels-last order
+  return h0 * w0 == 1 && h1 * w1 == 1 && n0 == n1 && c0 == c1;
+}
+
+ReshapeOpKernel::ReshapeOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Reshape");
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data || input_data->size() != output_data->size())
+    fail("Reshape '" + name + "': element count changes");
+  ck(tpuhip_malloc(ctx, input_data->size(), &scratch), name.c_str());
+}
+
+ReshapeOpKernel::~ReshapeOpKernel() {
+  if (scratch) tpuhip_free(ctx, scratch);
+}
+
+void ReshapeOpKernel::invoke() {
+  // channels-last -> NCHW bytes (which the reshape leaves untouched) -> channels-last
+  ck(tpuhip_nhwc_to_nchw_i8(ctx, input_data->data(), scratch, input_data->n, input_data->c,
+                            input_data->h, input_data->w, input_data->cs),
+     name.c_str());
+  ck(tpuhip_nchw_to_nhwc_i8(ctx, scratch, output_data->data(), output_data->n, output_data->c,
+                            output_data->h, output_data->w, output_data->cs),
+     name.c_str());
+}
+
+}  // namespace tpuhip

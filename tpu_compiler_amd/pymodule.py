@@ -1,0 +1,193 @@
+"""`module`: the Python face of the interpreter, shaped like the reference's
+pymlir.module (bindings/python/pymlir.cpp:87-311): load / run / set_tensor /
+get_tensor / invoke / invoke_to / get_all_tensor / op_info / get_input_details /
+get_output_details.  Where pymlir.load parses an .mlir file, `load` takes a
+`graphs.Graph` (ops in program order with their float-stored weights).
+
+Tensors cross this API as float32 NCHW arrays holding integers, like the
+reference's; `get_tensor_i8` is the cheaper int8 view of the same data.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+
+# operand layout of each op: names of weight roles in operand order after the
+# activation inputs; None marks an operand the INT8 path leaves empty
+_WEIGHT_OPERANDS = {
+    "tpu.conv_2d": ["filter", "bias", None, None, "rshift", "multiplier"],
+    "tpu.fully_connected": ["filter", "bias", None, None, "rshift", "multiplier"],
+    "tpu.eltwise_add": [None, None, "rshift", "multiplier"],
+    "tpu.pool_avg_2d": [None, None, "rshift", "multiplier"],
+    "tpu.pool_max_2d": [],
+    "tpu.leaky_relu": [None, None, None, None, "rshift_pos", "multiplier_pos", "rshift_neg",
+                       "multiplier_neg"],
+    "tpu.clip": [None, None, "rshift", "multiplier"],
+    "tpu.lut": ["table", None],
+    "tpu.relu": [],
+    "tpu.upsample": [],
+    "tpu.concat": [None, None, "rshift", "multiplier"],
+    "tpu.reshape": [],
+    "tpu.input": [],
+}
+
+
+class module:
+    version = "tpuhip"
+
+    def __init__(self, device=0, max_batch=1):
+        self.lib = capi.bind()
+        h = C.c_void_p()
+        capi.check(self.lib, self.lib.tpuhip_module_create(device, max_batch, C.byref(h)))
+        self.h = h
+        self.op_info = []
+        self.graph = None
+
+    def close(self):
+        if self.h:
+            self.lib.tpuhip_module_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _ck(self, status):
+        capi.check(self.lib, status)
+
+    # -- loading ----------------------------------------------------------
+    def load(self, graph, target_op=""):
+        """updateWeightMap + loadModule for `graph` (pymlir.cpp:99-122)."""
+        self.graph = graph
+        self._ck(self.lib.tpuhip_module_clear_ops(self.h))
+        self.op_info = []
+        for op in graph.ops:
+            roles = _WEIGHT_OPERANDS.get(op.type)
+            if roles is None:
+                roles = _WEIGHT_OPERANDS["tpu.lut"] if "table" in op.weights else []
+            operands = [s.encode() for s in op.inputs]
+            for role in roles:
+                if role is None or role not in op.weights:
+                    operands.append(b"")
+                    continue
+                wname = ("%s_%s" % (op.name, role)).encode()
+                arr = np.ascontiguousarray(op.weights[role], dtype=np.float32)
+                self._ck(self.lib.tpuhip_module_set_weight(self.h, wname, arr.ctypes.data,
+                                                           arr.size))
+                operands.append(wname)
+            shape = (C.c_int64 * len(op.shape))(*op.shape)
+            opd = (C.c_char_p * max(len(operands), 1))(*operands)
+            keys = [k.encode() for k in op.attrs]
+            vals = [float(v) for v in op.attrs.values()]
+            ak = (C.c_char_p * max(len(keys), 1))(*keys)
+            av = (C.c_double * max(len(vals), 1))(*vals)
+            d = capi.OpDescC(op.type.encode(), op.name.encode(), op.quant.encode(),
+                             op.param_type.encode(), len(op.shape), shape, len(operands), opd,
+                             len(keys), ak, av)
+            self._ck(self.lib.tpuhip_module_add_op(self.h, C.byref(d)))
+            self.op_info.append({"name": op.name, "type": op.type, "quant": op.quant})
+        rets = [s.encode() for s in graph.outputs]
+        ra = (C.c_char_p * max(len(rets), 1))(*rets)
+        self._ck(self.lib.tpuhip_module_set_returns(self.h, ra, len(rets)))
+        self._ck(self.lib.tpuhip_module_load(self.h, target_op.encode() if target_op else None))
+
+    # -- details ------------------------------------------------------------
+    def get_input_details(self):
+        out = {}
+        for i in range(self.lib.tpuhip_module_num_inputs(self.h)):
+            name = self.lib.tpuhip_module_input_name(self.h, i).decode()
+            out[name] = int(np.prod(self.tensor_shape(name)))
+        return out
+
+    def get_output_details(self):
+        return [self.lib.tpuhip_module_output_name(self.h, i).decode()
+                for i in range(self.lib.tpuhip_module_num_outputs(self.h))]
+
+    def tensor_names(self):
+        return [self.lib.tpuhip_module_tensor_name(self.h, i).decode()
+                for i in range(self.lib.tpuhip_module_num_tensors(self.h))]
+
+    def tensor_shape(self, name):
+        dims = (C.c_int64 * 8)()
+        nd = C.c_int()
+        self._ck(self.lib.tpuhip_module_tensor_shape(self.h, name.encode(), dims, C.byref(nd)))
+        return tuple(dims[i] for i in range(nd.value))
+
+    def tensor_dtype(self, name):
+        r = self.lib.tpuhip_module_tensor_dtype(self.h, name.encode())
+        if r is None:
+            raise capi.TpuHipError(1, self.lib.tpuhip_last_error().decode())
+        return r.decode()
+
+    def kernels(self):
+        """(name, algo) of every kernel in execution order"""
+        return [(self.lib.tpuhip_module_kernel_name(self.h, i).decode(),
+                 self.lib.tpuhip_module_kernel_algo(self.h, i).decode())
+                for i in range(self.lib.tpuhip_module_num_kernels(self.h))]
+
+    # -- data ---------------------------------------------------------------
+    def set_tensor(self, name, data, bidx=0):
+        arr = np.ascontiguousarray(data, dtype=np.float32)
+        self._ck(self.lib.tpuhip_module_set_tensor(self.h, name.encode(), arr.ctypes.data,
+                                                   arr.size, bidx))
+
+    def get_tensor(self, name, bidx=0):
+        shape = self.tensor_shape(name)
+        out = np.empty(shape, np.float32)
+        self._ck(self.lib.tpuhip_module_get_tensor(self.h, name.encode(), out.ctypes.data,
+                                                   out.size, bidx))
+        return out
+
+    def get_tensor_i8(self, name, bidx=0):
+        shape = self.tensor_shape(name)
+        out = np.empty(shape, np.int8)
+        self._ck(self.lib.tpuhip_module_get_tensor_i8(self.h, name.encode(), out.ctypes.data,
+                                                      out.size, bidx))
+        return out
+
+    def get_all_tensor(self):
+        return {n: self.get_tensor(n) for n in self.tensor_names()}
+
+    # -- execution ------------------------------------------------------------
+    def invoke(self, bidx=0):
+        self._ck(self.lib.tpuhip_module_invoke(self.h, bidx))
+
+    def invoke_to(self, name, bidx=0):
+        self._ck(self.lib.tpuhip_module_invoke_to(self.h, name.encode(), bidx))
+
+    def fast_invoke_all_batch(self, name, batch):
+        self._ck(self.lib.tpuhip_module_fast_invoke_all_batch(self.h, name.encode(), batch))
+
+    def sync(self):
+        self._ck(self.lib.tpuhip_module_sync(self.h))
+
+    def run(self, array, target_op=""):
+        """pymlir.module.run (pymlir.cpp:215-269): slice one flat float array over the
+        inputs, invoke, return {name: array} for the outputs (or for target_op)."""
+        flat = np.ascontiguousarray(array, dtype=np.float32).reshape(-1)
+        details = self.get_input_details()
+        need = sum(details.values())
+        if flat.size != need:
+            raise ValueError("input data size %d not same with all input needed size %d" %
+                             (flat.size, need))
+        off = 0
+        for name, size in details.items():
+            self.set_tensor(name, flat[off:off + size])
+            off += size
+        if target_op:
+            self.invoke_to(target_op)
+            return {target_op: self.get_tensor(target_op)}
+        self.invoke()
+        return {n: self.get_tensor(n) for n in self.get_output_details()}
+
+    def time_kernels(self, iters=5, bidx=0):
+        n = self.lib.tpuhip_module_num_kernels(self.h)
+        ms = (C.c_float * max(n, 1))()
+        self._ck(self.lib.tpuhip_module_time_kernels(self.h, bidx, iters, ms, n))
+        return [(k[0], k[1], ms[i]) for i, k in enumerate(self.kernels())]
+
+    def context_handle(self):
+        return self.lib.tpuhip_module_ctx(self.h)
