@@ -1,0 +1,184 @@
+"""GPU parity on whole graphs through the module API (C++ op classes +
+ModuleInterpreter behind the C ABI): every tensor of every layer must equal the
+oracle's, for the five benchmark configurations at their full sizes."""
+import numpy as np
+import pytest
+
+import oracle_graph
+from tpu_compiler_amd import capi, graphs, module
+
+pytestmark = pytest.mark.gpu
+
+
+def run_and_compare(g, check_stats=True):
+    m = module()
+    try:
+        m.load(g)
+        inp = g.input_op()
+        m.set_tensor(inp.name, inp.data.astype(np.float32))
+        m.invoke()
+        guards = {}
+        want = oracle_graph.run(g, guards=guards if g.input_op().shape[0] <= 8 else None)
+        bad = []
+        for op in g.ops:
+            got = m.get_tensor_i8(op.name)
+            ref = want[op.name].reshape(got.shape)
+            if not np.array_equal(got, ref):
+                bad.append((op.name, op.type, int((got != ref).sum()), got.size))
+        assert not bad, "mismatching layers (name, type, wrong, total): %s" % bad[:8]
+        for name, gv in guards.items():
+            assert gv < (1 << 24), "fp32-exactness guard broken at %s: %d" % (name, gv)
+        if check_stats:
+            # the comparison must not be trivially true: activations are alive everywhere
+            for op in g.ops:
+                if op.type in ("tpu.conv_2d", "tpu.fully_connected", "tpu.eltwise_add"):
+                    y = want[op.name]
+                    assert len(np.unique(y)) > 16, op.name
+                    assert np.mean(y == 0) < 0.9, op.name
+        return m, want
+    except Exception:
+        m.close()
+        raise
+
+
+def test_cfg1_single_conv():
+    g = graphs.cfg1_single_conv()
+    m, want = run_and_compare(g)
+    # float view of the same tensor, as the reference hands it out
+    f = m.get_tensor("conv")
+    assert f.dtype == np.float32 and np.array_equal(f, want["conv"].astype(np.float32))
+    assert dict(m.kernels())["conv"].startswith("mfma")
+    m.close()
+
+
+def test_cfg2_mobilenet_block():
+    g = graphs.cfg2_mobilenet_block()
+    m, _ = run_and_compare(g)
+    k = dict(m.kernels())
+    assert k["dw"] == "depthwise" and k["pw"].startswith("mfma")
+    m.close()
+
+
+def test_cfg3_resnet50_batch32():
+    g = graphs.cfg3_resnet50()
+    assert len(g.conv_ops()) == 54 and g.input_op().shape == (32, 3, 224, 224)
+    m, want = run_and_compare(g)
+    assert want["fc1000"].shape == (32, 1000)
+    m.close()
+
+
+def test_cfg4_mobilenet_v2_batch64():
+    g = graphs.cfg4_mobilenet_v2()
+    assert g.input_op().shape == (64, 3, 224, 224)
+    m, _ = run_and_compare(g)
+    m.close()
+
+
+def test_cfg5_yolo_v3_batch8():
+    g = graphs.cfg5_yolo_v3()
+    assert g.input_op().shape == (8, 3, 608, 608) and len(g.outputs) == 3
+    m, want = run_and_compare(g)
+    assert [want[o].shape for o in g.outputs] == [(8, 255, 19, 19), (8, 255, 38, 38),
+                                                  (8, 255, 76, 76)]
+    m.close()
+
+
+def test_module_api_semantics():
+    """batch slots, invoke_to, run(), get_all_tensor, reload keeps clean kernels."""
+    g = graphs.cfg3_resnet50(batch=1, hw=64)
+    m = module(max_batch=2)
+    m.load(g)
+    assert list(m.get_input_details()) == ["input"]
+    assert m.get_input_details()["input"] == 3 * 64 * 64
+    assert m.get_output_details() == ["fc1000"]
+    assert m.tensor_dtype("conv1") == "INT8"
+    assert m.tensor_shape("pool5_flat") == (1, 2048)
+    x0 = g.input_op().data
+    x1 = np.ascontiguousarray(x0[:, :, ::-1, :])
+    want0 = oracle_graph.run(g)
+    want1 = oracle_graph.run(g, input_data=x1)
+    # slot 1 and slot 0 are independent runs of the N=1 graph
+    m.set_tensor("input", x1.astype(np.float32), 1)
+    m.set_tensor("input", x0.astype(np.float32), 0)
+    m.invoke(1)
+    m.invoke(0)
+    assert np.array_equal(m.get_tensor_i8("fc1000", 1), want1["fc1000"])
+    assert np.array_equal(m.get_tensor_i8("fc1000", 0), want0["fc1000"])
+    # fastInvokeAllBatch runs every dirty kernel for each slot
+    m2 = module(max_batch=2)
+    m2.load(g)
+    m2.set_tensor("input", x0.astype(np.float32), 0)
+    m2.set_tensor("input", x1.astype(np.float32), 1)
+    m2.fast_invoke_all_batch("", 2)
+    assert np.array_equal(m2.get_tensor_i8("res3a", 1), want1["res3a"])
+    assert np.array_equal(m2.get_tensor_i8("res3a", 0), want0["res3a"])
+    m2.close()
+    # run(): flat float array in, dict of outputs out; target_op stops early
+    out = m.run(x0.astype(np.float32))
+    assert list(out) == ["fc1000"] and np.array_equal(out["fc1000"], want0["fc1000"])
+    out = m.run(x0.astype(np.float32), "res2a")
+    assert np.array_equal(out["res2a"], want0["res2a"].astype(np.float32))
+    allt = m.get_all_tensor()
+    assert set(allt) == {op.name for op in g.ops}
+    # reload with one op changed: only it and its consumers are rebuilt (dirty check)
+    g.by_name["res5c_branch2c"].attrs["do_relu"] = 1
+    m.load(g)
+    m.invoke(0)
+    want2 = oracle_graph.run(g)
+    assert np.array_equal(m.get_tensor_i8("fc1000", 0), want2["fc1000"])
+    assert not np.array_equal(want2["res5c_branch2c"], want0["res5c_branch2c"])
+    m.close()
+
+
+def test_module_errors_are_reported():
+    g = graphs.cfg1_single_conv()
+    m = module()
+    m.load(g)
+    with pytest.raises(capi.TpuHipError, match="size"):
+        m.set_tensor("input", np.zeros(10, np.float32))
+    with pytest.raises(capi.TpuHipError, match="Not Find"):
+        m.get_tensor_i8("nope")
+    bad = np.zeros(g.input_op().shape, np.float32)
+    bad[0, 0, 0, 0] = 0.5
+    with pytest.raises(capi.TpuHipError, match="int8"):
+        m.set_tensor("input", bad)
+    g2 = graphs.cfg1_single_conv()
+    g2.ops[1].type = "tpu.softmax"
+    with pytest.raises(capi.TpuHipError, match="no support"):
+        module().load(g2)
+    g3 = graphs.cfg1_single_conv()
+    del g3.ops[1].weights["multiplier"]
+    with pytest.raises(capi.TpuHipError, match="multiplier"):
+        module().load(g3)
+    g4 = graphs.cfg1_single_conv()
+    g4.ops[1].quant = "BF16"
+    with pytest.raises(capi.TpuHipError, match="INT8"):
+        module().load(g4)
+    m.close()
+
+
+def test_lut_activation_and_general_reshape():
+    """a y0-table activation (sigmoid-style op) and a reshape that is not an alias in
+    channels-last order."""
+    b = graphs.Builder("lut_reshape", 77, 2, (4, 18))
+    x = b.input("input", 24, 5, 6)
+    y = b.conv("conv", x, 40, 3, relu=False)
+    g = b.finish([y])
+    table = np.clip(np.rint(127 / (1 + np.exp(-np.arange(-128, 128) / 16.0))), -128, 127)
+    table = np.roll(table, 128).astype(np.float32)   # entry i <-> two's-complement byte i
+    g.add(graphs.Op("tpu.sigmoid", "sig", ["conv"], g.by_name["conv"].shape, {},
+                    {"table": table}, "LUT_INT8"))
+    g.add(graphs.Op("tpu.reshape", "flat", ["sig"], (2, 40 * 5 * 6)))
+    g.add(graphs.Op("tpu.reshape", "back", ["flat"], (2, 8, 25, 6)))
+    g.outputs = ["back"]
+    m = module()
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    conv = oracle_graph.run(g, upto="conv")["conv"]
+    import oracle_lib as O
+    sig = O.lut_i8(conv, table)
+    assert np.array_equal(m.get_tensor_i8("sig"), sig)
+    assert np.array_equal(m.get_tensor_i8("flat"), sig.reshape(2, -1))
+    assert np.array_equal(m.get_tensor_i8("back"), sig.reshape(2, 8, 25, 6))
+    m.close()
