@@ -1,0 +1,153 @@
+#!/usr/bin/env python3
+"""Benchmark of the INT8 interpreter path on one MI355X.
+
+A step is one pass of the whole quantized graph over one batch of synthetic
+input already resident in HBM.  Default workload: the ResNet-50-shaped INT8
+graph at batch 32.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+
+def conv_bytes(op, graph):
+    """algorithmic bytes of a conv / fc: int8 input + output + filter, 12 B of int32
+    parameters per output channel"""
+    import numpy as np
+    x = graph.by_name[op.inputs[0]].shape
+    oc = op.shape[1]
+    return int(np.prod(x)) + int(np.prod(op.shape)) + int(op.weights["filter"].size) + 12 * oc
+
+
+def cpu_baseline(graph_fn, images):
+    """The oracle (CPU restatement of the reference's arithmetic) on a bounded sample of
+    the same workload, on this host's cores."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_graph
+    g = graph_fn(batch=images)
+    oracle_graph.run(g, keep=g.outputs)      # page in
+    t0 = time.perf_counter()
+    oracle_graph.run(g, keep=g.outputs)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": round(images / dt, 2), "unit": "images/s", "cores": cores, "kind": "port",
+            "sample": "%s, %d images, one pass through the integer-exact C/OpenMP oracle"
+                      % (g.name, images)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--per-layer", action="store_true", help="print the per-layer table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (--gpus %d refused); the path shards "
+                 "by batch with no exchange step, see DESIGN.md" % args.gpus)
+
+    import numpy as np
+    from tpu_compiler_amd import graphs, module
+
+    graph_fn = graphs.CONFIGS[args.config]
+    g = graph_fn()
+    batch = g.input_op().shape[0]
+    m = module(device=0)
+    m.load(g)
+    m.set_tensor(g.input_op().name, g.input_op().data.astype(np.float32))
+    lib, ctxh = m.lib, m.context_handle()
+
+    for _ in range(max(args.warmup, 1)):
+        m.invoke()
+    m.sync()
+
+    import ctypes as C
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.tpuhip_event_create(ctxh, C.byref(e0))
+    lib.tpuhip_event_create(ctxh, C.byref(e1))
+    m.sync()
+    t0 = time.perf_counter()
+    lib.tpuhip_event_record(ctxh, e0)
+    for _ in range(args.steps):
+        m.invoke()
+    lib.tpuhip_event_record(ctxh, e1)
+    m.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ev_ms = C.c_float()
+    lib.tpuhip_event_elapsed_ms(ctxh, e0, e1, C.byref(ev_ms))
+    ms_per_step = wall_ms / args.steps
+    images_per_s = batch / (ms_per_step / 1e3)
+    total_ops = 2.0 * g.macs
+    tops = total_ops / (ms_per_step / 1e3) / 1e12
+
+    # per-kernel times, HIP events on the stream the kernels run on
+    rows = m.time_kernels(iters=max(5, min(args.steps, 20)))
+    by_algo = {}
+    for name, algo, ms in rows:
+        op = g.by_name[name]
+        if op.type in ("tpu.conv_2d", "tpu.fully_connected"):
+            key = algo if algo != "fc" else "fc"
+            d = by_algo.setdefault(key, {"ms": 0.0, "ops": 0.0, "bytes": 0.0, "launches": 0})
+            d["ms"] += ms
+            d["ops"] += 2.0 * op.macs
+            d["bytes"] += conv_bytes(op, g)
+            d["launches"] += 1
+    mfma = {k: v for k, v in by_algo.items() if k.startswith("mfma")}
+    conv_ms = sum(v["ms"] for v in mfma.values())
+    conv_ops = sum(v["ops"] for v in mfma.values())
+    dom_name, dom = max(mfma.items(), key=lambda kv: kv[1]["ms"]) if mfma else (None, None)
+    roofline = None
+    if dom:
+        achieved = dom["ops"] / (dom["ms"] / 1e3) / 1e12
+        roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<%s>" % dom_name.replace("mfma_", ""),
+                    "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                    "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None,
+                    "launches": dom["launches"],
+                    "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 2),
+                    "all_mfma_conv_layers": {
+                        "achieved": round(conv_ops / (conv_ms / 1e3) / 1e12, 2),
+                        "frac": round(conv_ops / (conv_ms / 1e3) / 1e12 / PEAK_INT8_TOPS, 4),
+                        "ms": round(conv_ms, 4)}}
+    if args.per_layer:
+        for name, algo, ms in rows:
+            op = g.by_name[name]
+            macs = getattr(op, "macs", 0)
+            print("%-22s %-18s %-14s %9.2f us %8.1f TOP/s" %
+                  (name, op.type, algo, ms * 1e3, 2 * macs / (ms / 1e3) / 1e12 if ms > 0 else 0),
+                  file=sys.stderr)
+
+    out = {
+        "metric": "images_per_sec", "value": round(images_per_s, 1), "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "%s: %s INT8 graph, batch %d, %s input, random-init seeded weights"
+                               % (args.config, g.name, batch,
+                                  "x".join(str(v) for v in g.input_op().shape[1:])),
+                   "global_batch": batch},
+        "tops": round(tops, 2),
+        "ops_per_step": total_ops,
+        "event_ms_per_step": round(ev_ms.value / args.steps, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        sample = {"cfg1": 8, "cfg2": 8, "cfg3": 8, "cfg4": 16, "cfg5": 1}[args.config]
+        out["cpu_baseline"] = cpu_baseline(graph_fn, sample)
+    m.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

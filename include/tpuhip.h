@@ -47,6 +47,11 @@ int tpuhip_ctx_create(int device, tpuhip_ctx **out);
 int tpuhip_ctx_create_on_stream(int device, void *hip_stream, tpuhip_ctx **out);
 int tpuhip_ctx_destroy(tpuhip_ctx *ctx);
 void *tpuhip_ctx_stream(tpuhip_ctx *ctx);
+/* When enabled (the default; TPUHIP_AUTOTUNE=0 in the environment disables it) a
+ * dense conv times its tile variants on first use and keeps the fastest.  Every
+ * variant produces the same bytes.  The first use of a layer is then not
+ * capturable into a HIP graph. */
+int tpuhip_ctx_set_autotune(tpuhip_ctx *ctx, int enable);
 const char *tpuhip_last_error(void);
 const char *tpuhip_version(void);
 

@@ -72,6 +72,36 @@ def test_conv_dense(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
+TILE_CASES = [
+    (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),
+    (2, 96, 17, 13, 200, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),   # ragged pixel / channel tails
+    (1, 40, 9, 9, 72, 3, 3, (2, 2), (1, 1, 1, 1), (1, 1), True),
+    (3, 16, 5, 5, 16, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),      # one K step, tiny
+    (1, 256, 6, 6, 300, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),     # 36 K steps
+]
+
+
+@pytest.mark.parametrize("case", TILE_CASES)
+@pytest.mark.parametrize("tile", range(7))
+def test_conv_every_mfma_tile_variant(ctx, case, tile):
+    n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
+    rng = np.random.default_rng(ic * 7 + oc + tile)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=16 + tile, stride=stride, pads=pads,
+                         dil=dil, do_relu=relu)
+    assert np.array_equal(got, want), "%s: %d mismatches" % (name, (got != want).sum())
+    # the general (non-fast) requant form of the same tile: an rshift of 0 forces it
+    rsh2 = rsh.copy()
+    rsh2[::3] = 0
+    want = oracle_conv(x, w, bias, rsh2, mult, 1, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh2, mult, algo=16 + tile, stride=stride, pads=pads,
+                         dil=dil, do_relu=relu)
+    assert np.array_equal(got, want), "%s general: %d mismatches" % (name, (got != want).sum())
+
+
 def test_conv_auto_picks_mfma_for_dense_and_depthwise_for_dw(ctx):
     rng = np.random.default_rng(1)
     x = rnd_i8(rng, (1, 32, 8, 8))

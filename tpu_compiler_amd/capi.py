@@ -30,6 +30,7 @@ PROTOTYPES = {
     "tpuhip_ctx_create_on_stream": (C.c_int, [C.c_int, C.c_void_p, c_void_pp]),
     "tpuhip_ctx_destroy": (C.c_int, [C.c_void_p]),
     "tpuhip_ctx_stream": (C.c_void_p, [C.c_void_p]),
+    "tpuhip_ctx_set_autotune": (C.c_int, [C.c_void_p, C.c_int]),
     "tpuhip_last_error": (C.c_char_p, []),
     "tpuhip_version": (C.c_char_p, []),
     "tpuhip_malloc": (C.c_int, [C.c_void_p, C.c_size_t, c_void_pp]),

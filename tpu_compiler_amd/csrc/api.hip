@@ -1,6 +1,7 @@
 // Context, memory and error plumbing of the tpuhip C ABI.
 #include "common.hpp"
 
+#include <cstdlib>
 #include <cstring>
 
 namespace tpuhip {
@@ -41,6 +42,7 @@ static int ctx_create(int device, void *stream, bool own, tpuhip_ctx **out) {
   tpuhip_ctx *c = new tpuhip_ctx();
   c->device = device;
   c->num_cu = prop.multiProcessorCount;
+  if (const char *e = getenv("TPUHIP_AUTOTUNE")) c->autotune = atoi(e) != 0;
   if (own) {
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
@@ -69,6 +71,12 @@ int tpuhip_ctx_destroy(tpuhip_ctx *ctx) {
     (void)hipStreamDestroy(ctx->stream);
   }
   delete ctx;
+  return TPUHIP_OK;
+}
+
+int tpuhip_ctx_set_autotune(tpuhip_ctx *ctx, int enable) {
+  TPUHIP_REQUIRE(ctx, "tpuhip_ctx_set_autotune: NULL context");
+  ctx->autotune = enable != 0;
   return TPUHIP_OK;
 }
 

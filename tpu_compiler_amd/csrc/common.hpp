@@ -16,6 +16,7 @@ struct tpuhip_ctx {
   hipStream_t stream = nullptr;
   bool owns_stream = false;
   int num_cu = 0;
+  bool autotune = true;  // time the conv tile variants on a layer's first use
 };
 
 namespace tpuhip {

@@ -12,6 +12,9 @@
 // (lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp:849-871).
 #include "common.hpp"
 
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
 #include <vector>
 
 using namespace tpuhip;
@@ -21,24 +24,25 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3 };
 
-// Per-output-channel epilogue parameters, one 32-byte record per channel so a
-// lane fetches a channel's record with two 16-byte loads.
-struct __attribute__((aligned(32))) ChanParams {
-  int32_t bias;
+// per-channel requantisation record
+struct __attribute__((aligned(16))) QParam {
   int32_t mult;
   int32_t rshift;
   int32_t mask;   // 2^rshift - 1
-  int32_t half;   // mask >> 1
-  int32_t pad[3];
+  int32_t hpot;   // 2^(rshift-1), 0 for rshift 0
 };
 
 struct tpuhip_conv_weights {
   tpuhip_conv_desc d;
   int algo = ALGO_DIRECT;
   int tile = 0;          // MFMA tile variant
+  int fast = 0;          // the overflow-free requant form is provably exact for this layer
+  bool tuned = true;     // false: the tile is chosen by timing the candidates on first use
+  std::vector<int8_t> host_filter;  // OIHW copy, kept while the layer can still be repacked
   int8_t *w = nullptr;   // packed filter
-  ChanParams *cp = nullptr;
-  int ocp = 0;           // padded output channels (rows of w / entries of cp)
+  int32_t *bias = nullptr;
+  QParam *qp = nullptr;
+  int ocp = 0;           // padded output channels (rows of w / entries of bias, qp)
   int kp = 0;            // padded K in bytes (row stride of w) for the MFMA path
   int c16 = 0;           // input 16-channel groups per tap
   int k16 = 0;           // 16-byte K groups in total
@@ -47,23 +51,28 @@ struct tpuhip_conv_weights {
 struct ConvArgs {
   const int8_t *x;
   const int8_t *w;
-  const ChanParams *cp;
+  const int32_t *bias;
+  const QParam *qp;
   int8_t *y;
   int n, ih, iw, x_cs;
   int oh, ow, y_cs;
   int oc, ocw, icg, ocg, g;  // ocw = oc rounded up to 16: channels written per pixel
   int kh, kw, sh, sw, pt, pl, dh, dw, ins_h, ins_w;
   int c16, k16, kp;
+  uint32_t magic_c16, magic_kw;   // floor(2^20 / d) + 1: x / d == (x * magic) >> 20 for x < 4095
+  uint32_t x_bytes, w_bytes;      // sizes behind x and w (buffer descriptors)
+  uint32_t magic_ow, magic_oh;    // ceil(2^32 / d): x / d == umulhi(x, magic) for x, d < 2^16
+  int n_oc_tiles, n_tiles, tiles_per_xcd;
   int npix;
   int lo;          // lower clamp bound: 0 with ReLU after saturation, else -128
   int relu_first;  // ReLU on the sum before requantisation (FC)
 };
 
-__device__ __forceinline__ int32_t epilogue(int32_t acc, const ChanParams &p, int lo,
+__device__ __forceinline__ int32_t epilogue(int32_t acc, int32_t bias, const QParam &p, int lo,
                                             int relu_first) {
-  int32_t v = (int32_t)((uint32_t)acc + (uint32_t)p.bias);
+  int32_t v = (int32_t)((uint32_t)acc + (uint32_t)bias);
   if (relu_first) v = max(v, 0);
-  return requant_qdm(v, p.mult, p.rshift, p.mask, p.half, lo);
+  return requant_qdm(v, p.mult, p.rshift, p.mask, p.mask >> 1, lo);
 }
 
 // ---------------------------------------------------------------------------
@@ -101,7 +110,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(ConvArgs a) {
         for (int c = 0; c < a.icg; ++c) acc += (int32_t)xp[c] * (int32_t)wp_[c];
       }
     }
-    *yp = (int8_t)epilogue(acc, a.cp[oc], a.lo, a.relu_first);
+    *yp = (int8_t)epilogue(acc, a.bias[oc], a.qp[oc], a.lo, a.relu_first);
   }
 }
 
@@ -150,7 +159,7 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(ConvArgs a) {
       for (int b = 0; b < 4; ++b) {
         const int c = cg * 16 + q * 4 + b;
         int32_t v = 0;
-        if (c < a.oc) v = epilogue(acc[q * 4 + b], a.cp[c], a.lo, a.relu_first);
+        if (c < a.oc) v = epilogue(acc[q * 4 + b], a.bias[c], a.qp[c], a.lo, a.relu_first);
         word |= ((uint32_t)v & 0xffu) << (8 * b);
       }
       out[q] = (int)word;
@@ -162,22 +171,81 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(ConvArgs a) {
 // ---------------------------------------------------------------------------
 // MFMA implicit-GEMM kernel.
 //
-//   D[oc][pix] = sum_k W[oc][k] * X[pix][k],   k = (kh*KW + kw)*cs_in + c
+//   D[oc][pix] = sum_k W[oc][k] * X[pix][k],   k = (kh*KW + kw)*icp + c
 //
-// Workgroup = 4 waves, tile BM output channels x BN pixels, K consumed 64 bytes
-// per step.  LDS rows are 64 bytes (4 chunks of 16); chunk index is XOR-swizzled
-// with (row >> 2) & 3 so that both the 16-byte stores of the loader and the
-// 16-byte fragment reads of the MFMA loop spread over all banks.
+// (icp = input channels rounded up to 16).  A workgroup of WM x WN waves owns a
+// tile of BM output channels x BN pixels; every wave owns (BM/WM) x (BN/WN) of it
+// as TM x TN blocks of 32x32 (v_mfma_i32_32x32x32_i8).  K is consumed 64 bytes per
+// step.  Global loads run DEPTH steps ahead of the MFMAs in a ring of registers,
+// LDS is double-buffered, one barrier per step.
+//
+// LDS rows are 64 bytes (4 chunks of 16); the chunk index is XOR-swizzled with
+// (row >> 2) & 3 so that both the 16-byte stores of the loader and the 16-byte
+// fragment reads spread over all banks.
+//
+// The rows of a weight tile are stored permuted (see mfma_row_to_oc) so that in
+// the 32x32 result layout -- lane l holds column l & 31 and rows
+// 8*(r/4) + 4*(l/32) + r%4 for register r -- the 16 registers of a lane are 16
+// consecutive output channels of one pixel: one 16-byte store per block.
 // ---------------------------------------------------------------------------
-template <int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void conv_mfma_kernel(ConvArgs a) {
-  static_assert(WM * WN == 4, "four waves per workgroup");
+
+// tile-local weight row (as the MFMA sees it) -> tile-local output channel
+__host__ __device__ inline int mfma_row_to_oc(int row, int tm) {
+  const int wave_rows = tm * 32;
+  const int wrow = row % wave_rows, wbase = row - wrow;
+  const int i = wrow / 32, ri = wrow % 32;
+  const int fk = (ri >> 2) & 1;
+  const int r = (ri >> 3) * 4 + (ri & 3);
+  return wbase + fk * 16 * tm + i * 16 + r;
+}
+
+typedef short v2s __attribute__((ext_vector_type(2)));
+
+// four int32 -> four saturated int8 in one dword; lo is -128 or 0 (fused ReLU)
+__device__ __forceinline__ uint32_t pack_sat4(int32_t a, int32_t b, int32_t c, int32_t d, int lo) {
+  v2s p0 = __builtin_amdgcn_cvt_pk_i16(a, b);
+  v2s p1 = __builtin_amdgcn_cvt_pk_i16(c, d);
+  const v2s vlo = {(short)lo, (short)lo}, vhi = {127, 127};
+  p0 = __builtin_elementwise_min(__builtin_elementwise_max(p0, vlo), vhi);
+  p1 = __builtin_elementwise_min(__builtin_elementwise_max(p1, vlo), vhi);
+  return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, p1), __builtin_bit_cast(uint32_t, p0),
+                               0x06040200u);
+}
+
+// FAST: every channel has 1 <= rshift <= 31 and |acc + bias| + 1 + 2^(rshift-1) < 2^31
+// (proved on the host from the weights), so RoundingDivideByPOT is
+// (x + 2^(e-1) - (x < 0)) >> e without overflow.
+template <bool FAST>
+__device__ __forceinline__ int32_t requant_core(int32_t v, const QParam &q) {
+  const int32_t x = srdhm(v, q.mult);
+  if (FAST) return (x + q.hpot + (x >> 31)) >> q.rshift;
+  return rdbp(x, q.rshift, q.mask, q.mask >> 1);
+}
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+// 16-byte load through a buffer descriptor: an offset at or beyond the
+// descriptor's size yields zeros, which is how padding taps, pixels past the end
+// of the tensor and K steps past the end of the filter are fed to the MFMAs
+// without a branch.
+__device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t offset) {
+  return (v4i)__builtin_amdgcn_raw_buffer_load_b128(rsrc, offset, 0, 0);
+}
+constexpr uint32_t kOobOffset = 0x7fffffffu;
+
+// UNI: the input channel count is a multiple of 64, so the four 16-byte K groups of
+// a step lie in one filter tap and all tap arithmetic is wave-uniform (scalar).
+template <int BM, int BN, int WM, int WN, int DEPTH, bool FAST, bool UNI>
+__global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
+  constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32;  // 32x32 blocks per wave along oc
   constexpr int TN = BN / WN / 32;  // 32x32 blocks per wave along pixels
-  static_assert(TM >= 1 && TN >= 1, "tile too small");
-  constexpr int NW = BM * 4 / 256;  // 16-byte weight chunks per thread per step
-  constexpr int NX = BN * 4 / 256;  // 16-byte activation chunks per thread per step
-  static_assert(NX >= 1, "pixel tile too small");
+  static_assert(TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
+  constexpr int RP = NT / 4;                 // tile rows fetched per pass of the workgroup
+  constexpr int NW = (BM + RP - 1) / RP;     // 16-byte weight chunks per thread per step
+  constexpr int NX = BN / RP;                // 16-byte activation chunks per thread per step
+  static_assert(BN % RP == 0, "pixel tile must be a multiple of the loader pass");
+  static_assert(DEPTH == 2 || DEPTH == 4, "register ring depth");
 
   __shared__ v4i lds[2][(BM + BN) * 4];
 
@@ -185,161 +253,209 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(ConvArgs a) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  const int oc0 = blockIdx.y * BM;
-  const int pix0 = blockIdx.x * BN;
+  // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run
+  // of tiles, output-channel tiles of one pixel tile next to each other, so that the
+  // workgroups sharing activations (and writing the same output rows) share an L2.
+  const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  if (logical >= a.n_tiles) return;
+  const int pix_tile = logical / a.n_oc_tiles;
+  const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;
+  const int pix0 = pix_tile * BN;
 
-  // ---- loader state: this thread always fetches K-chunk kc of rows (tid>>2)+64*s
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  // ---- loader state: this thread fetches K-chunk kc of rows lrow + RP*s
   const int kc = tid & 3;
   const int lrow = tid >> 2;
-  int64_t xbase[NX];  // byte offset of image n in x
+  int poff[NX];     // byte offset of (n, oh*sh - pt, ow*sw - pl, kc*16) in x (may lie before the image)
   int ih0[NX], iw0[NX];
-  bool pvalid[NX];
+  // (n, oh, ow) of the tile's first pixel: one generic division per workgroup ...
+  const int ow_first = pix0 % a.ow;
+  const int t_first = pix0 / a.ow;
+  const int oh_first = t_first % a.oh;
+  const int n_first = t_first / a.oh;
 #pragma unroll
   for (int s = 0; s < NX; ++s) {
-    const int pix = pix0 + lrow + 64 * s;
-    pvalid[s] = pix < a.npix;
-    const int p = pvalid[s] ? pix : 0;
-    const int ow = p % a.ow;
-    const int t = p / a.ow;
-    const int oh = t % a.oh;
-    const int n = t / a.oh;
-    xbase[s] = (int64_t)n * a.ih * a.iw * a.x_cs;
-    ih0[s] = oh * a.sh - a.pt;
+    // ... and exact multiply-high divisions of small numbers per row
+    const int delta = lrow + RP * s;
+    const bool pv = pix0 + delta < a.npix;
+    const uint32_t t1 = (uint32_t)(ow_first + delta);
+    const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
+    const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
+    const uint32_t t2 = (uint32_t)oh_first + q1;
+    const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
+    const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
+    const int n = n_first + (int)q2;
+    ih0[s] = pv ? oh * a.sh - a.pt : -(1 << 28);   // an invalid pixel never passes the bounds test
     iw0[s] = ow * a.sw - a.pl;
+    poff[s] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[s]) * a.x_cs + (UNI ? kc * 16 : 0);
+    // keep the three values in registers instead of recomputing them every K step
+    asm volatile("" : "+v"(poff[s]), "+v"(ih0[s]), "+v"(iw0[s]));
   }
-  // position of this thread's K group inside the filter window
-  int kg = kc;                 // 16-byte group index along K
-  int cgrp = kc % a.c16;       // 16-channel group inside the tap
-  int tap = kc / a.c16;
-  int tkh = tap / a.kw, tkw = tap % a.kw;
+  uint32_t woff[NW];
+#pragma unroll
+  for (int s = 0; s < NW; ++s) {
+    const int r = lrow + RP * s;
+    woff[s] = r < BM ? (uint32_t)((oc0 + r) * a.kp + kc * 16) : kOobOffset;
+    asm volatile("" : "+v"(woff[s]));
+  }
 
-  const int8_t *wrow[NW > 0 ? NW : 1];
-#pragma unroll
-  for (int s = 0; s < NW; ++s)
-    wrow[s] = a.w + (int64_t)(oc0 + lrow + 64 * s) * a.kp + kc * 16;
-  // BM == 32: only threads with lrow < 32 carry a weight chunk
-  const bool wsmall = (BM * 4 < 256);
-  const int8_t *wrow_small = a.w + (int64_t)(oc0 + (lrow & (BM - 1))) * a.kp + kc * 16;
-
-  v4i wreg[NW > 0 ? NW : 1], xreg[NX];
-
-  auto load_tile = [&](int step) {
-    if (wsmall) {
-      if (lrow < BM) wreg[0] = *reinterpret_cast<const v4i *>(wrow_small + (int64_t)step * 64);
-    } else {
-#pragma unroll
-      for (int s = 0; s < NW; ++s)
-        wreg[s] = *reinterpret_cast<const v4i *>(wrow[s] + (int64_t)step * 64);
-    }
-    const bool kvalid = kg < a.k16;
-    const int dh_off = tkh * a.dh, dw_off = tkw * a.dw;
-#pragma unroll
-    for (int s = 0; s < NX; ++s) {
-      const int ih = ih0[s] + dh_off, iw = iw0[s] + dw_off;
-      const bool ok = kvalid && pvalid[s] && (unsigned)ih < (unsigned)a.ih &&
-                      (unsigned)iw < (unsigned)a.iw;
-      v4i v = {0, 0, 0, 0};
-      if (ok)
-        v = *reinterpret_cast<const v4i *>(a.x + xbase[s] +
-                                           ((int64_t)ih * a.iw + iw) * a.x_cs + cgrp * 16);
-      xreg[s] = v;
-    }
-    // advance to the next step's K group
-    kg += 4;
-    cgrp += 4;
-    while (cgrp >= a.c16) {
-      cgrp -= a.c16;
-      if (++tkw == a.kw) {
-        tkw = 0;
-        ++tkh;
-      }
-    }
-  };
-
-  auto store_tile = [&](int buf) {
-    v4i *base = lds[buf];
-    if (wsmall) {
-      if (lrow < BM) base[lrow * 4 + (kc ^ ((lrow >> 2) & 3))] = wreg[0];
-    } else {
-#pragma unroll
-      for (int s = 0; s < NW; ++s) {
-        const int r = lrow + 64 * s;
-        base[r * 4 + (kc ^ ((r >> 2) & 3))] = wreg[s];
-      }
-    }
-#pragma unroll
-    for (int s = 0; s < NX; ++s) {
-      const int r = lrow + 64 * s;
-      base[(BM + r) * 4 + (kc ^ ((r >> 2) & 3))] = xreg[s];
-    }
-  };
-
-  v16i acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
+  v4i wreg[DEPTH][NW], xreg[DEPTH][NX];
   const int nsteps = a.kp / 64;
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
+
+  // fetch the tile of K step `step` into ring slot `slot`; no branches, no state.
+  // A 16-byte K group kg = tap * c16 + cgrp with tap = tkh * kw + tkw; the divisions
+  // are exact multiply-shifts.
+  auto load_tile = [&](int slot, int step) {
+    const bool in_k = step < nsteps;
+#pragma unroll
+    for (int s = 0; s < NW; ++s)
+      wreg[slot][s] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+          wrsrc, in_k ? woff[s] : kOobOffset, step * 64, 0);
+    if (UNI) {
+      const uint32_t kg0 = (uint32_t)(step * 4);
+      const uint32_t tap = (kg0 * a.magic_c16) >> 20;
+      const int cgrp0 = (int)(kg0 - tap * (uint32_t)a.c16);
+      const int tkh = (int)((tap * a.magic_kw) >> 20);
+      const int tkw = (int)tap - tkh * a.kw;
+      // past the end of K the row offset is pushed out of every image
+      const int dh_off = (int)kg0 < a.k16 ? tkh * a.dh : (1 << 28);
+      const int dw_off = tkw * a.dw;
+      const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp0 * 16;
+#pragma unroll
+      for (int s = 0; s < NX; ++s) {
+        const int ih = ih0[s] + dh_off, iw = iw0[s] + dw_off;
+        const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+        xreg[slot][s] = buffer_load16(xrsrc, ok ? (uint32_t)(poff[s] + tap_off) : kOobOffset);
+      }
+    } else {
+      const uint32_t kg = (uint32_t)(step * 4 + kc);
+      const uint32_t tap = (kg * a.magic_c16) >> 20;
+      const int cgrp = (int)(kg - tap * (uint32_t)a.c16);
+      const int tkh = (int)((tap * a.magic_kw) >> 20);
+      const int tkw = (int)tap - tkh * a.kw;
+      const int dh_off = (int)kg < a.k16 ? tkh * a.dh : (1 << 28);
+      const int dw_off = tkw * a.dw;
+      const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp * 16;
+#pragma unroll
+      for (int s = 0; s < NX; ++s) {
+        const int ih = ih0[s] + dh_off, iw = iw0[s] + dw_off;
+        const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+        xreg[slot][s] = buffer_load16(xrsrc, ok ? (uint32_t)(poff[s] + tap_off) : kOobOffset);
+      }
+    }
+  };
+
+  auto store_tile = [&](int slot, int buf) {
+    v4i *base = lds[buf];
+#pragma unroll
+    for (int s = 0; s < NW; ++s) {
+      const int r = lrow + RP * s;
+      if (BM % RP == 0 || r < BM) base[r * 4 + (kc ^ ((r >> 2) & 3))] = wreg[slot][s];
+    }
+#pragma unroll
+    for (int s = 0; s < NX; ++s) {
+      const int r = lrow + RP * s;
+      base[(BM + r) * 4 + (kc ^ ((r >> 2) & 3))] = xreg[slot][s];
+    }
+  };
 
   const int frow = lane & 31;   // row inside a 32-row block
   const int fk = lane >> 5;     // which 16-byte half of a 32-byte MFMA K slice
 
-  for (int step = 0; step < nsteps; ++step) {
-    const int buf = step & 1;
-    if (step + 1 < nsteps) load_tile(step + 1);
-    const v4i *wl = lds[buf];
-    const v4i *xl = lds[buf] + BM * 4;
+  // accumulators start from the bias (the int32 add of the epilogue commutes with the sum)
+  v16i acc[TM][TN];
+  const int ocw0 = oc0 + wm * TM * 32 + fk * 16 * TM;   // first of this lane's 16*TM channels
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const int chunk = kk * 2 + fk;
-      v4i af[TM], bf[TN];
+  for (int i = 0; i < TM; ++i) {
+    const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int r = (wm * TM + i) * 32 + frow;
-        af[i] = wl[r * 4 + (chunk ^ ((r >> 2) & 3))];
-      }
+    for (int q = 0; q < 4; ++q) {
+      const v4i b = bp[q];
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int r = (wn * TN + j) * 32 + frow;
-        bf[j] = xl[r * 4 + (chunk ^ ((r >> 2) & 3))];
+        acc[i][j][q * 4 + 0] = b[0];
+        acc[i][j][q * 4 + 1] = b[1];
+        acc[i][j][q * 4 + 2] = b[2];
+        acc[i][j][q * 4 + 3] = b[3];
       }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
-    if (step + 1 < nsteps) store_tile(buf ^ 1);
-    __syncthreads();
   }
 
-  // ---- epilogue.  In a 32x32 result block lane l holds column (pixel) l & 31
-  // and rows (channels) 8*(r/4) + 4*(l/32) + r%4 for register r = 0..15, i.e.
-  // four runs of 4 consecutive channels: each run becomes one 32-bit store.
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int pix = pix0 + (wn * TN + j) * 32 + frow;
-    if (pix >= a.npix) continue;
-    int8_t *yrow = a.y + (int64_t)pix * a.y_cs;
+  for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
+  store_tile(0, 0);
+  __syncthreads();
+
+  // Steps are processed DEPTH at a time so that ring slots and LDS buffers are
+  // compile-time indices; steps past the end of K multiply zeros.
+  for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int d = 0; d < DEPTH; ++d) {
+      const int step = s0 + d;
+      const int buf = d & 1;   // == step & 1 because DEPTH is even
+      // slot d went to LDS one step ago: refill it with the tile DEPTH steps ahead
+      load_tile(d, step + DEPTH);
+      if (step >= nsteps) break;   // uniform: only the last group can be short
+      const v4i *wl = lds[buf];
+      const v4i *xl = lds[buf] + BM * 4;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int oc = oc0 + (wm * TM + i) * 32 + q * 8 + fk * 4;
-        if (oc >= a.ocw) continue;
-        uint32_t word = 0;
+      for (int kk = 0; kk < 2; ++kk) {
+        const int chunk = kk * 2 + fk;
+        v4i af[TM], bf[TN];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const int32_t v = epilogue(acc[i][j][q * 4 + b], a.cp[oc + b], a.lo, a.relu_first);
-          word |= ((uint32_t)v & 0xffu) << (8 * b);
+        for (int i = 0; i < TM; ++i) {
+          const int r = (wm * TM + i) * 32 + frow;
+          af[i] = wl[r * 4 + (chunk ^ ((r >> 2) & 3))];
         }
-        *reinterpret_cast<uint32_t *>(yrow + oc) = word;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int r = (wn * TN + j) * 32 + frow;
+          bf[j] = xl[r * 4 + (chunk ^ ((r >> 2) & 3))];
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+      store_tile((d + 1) % DEPTH, buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: requantise, saturate (+ReLU), one 16-byte store per block
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int oc = ocw0 + i * 16;
+    if (oc >= a.ocw) continue;
+    const QParam *qp = a.qp + oc;
+    uint32_t outw[TN][4];
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const QParam q0 = qp[qd * 4 + 0], q1 = qp[qd * 4 + 1], q2 = qp[qd * 4 + 2],
+                   q3 = qp[qd * 4 + 3];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        int32_t v0 = acc[i][j][qd * 4 + 0], v1 = acc[i][j][qd * 4 + 1],
+                v2 = acc[i][j][qd * 4 + 2], v3 = acc[i][j][qd * 4 + 3];
+        if (a.relu_first) {
+          v0 = max(v0, 0); v1 = max(v1, 0); v2 = max(v2, 0); v3 = max(v3, 0);
+        }
+        outw[j][qd] = pack_sat4(requant_core<FAST>(v0, q0), requant_core<FAST>(v1, q1),
+                                       requant_core<FAST>(v2, q2), requant_core<FAST>(v3, q3),
+                                       a.lo);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int pix = pix0 + (wn * TN + j) * 32 + frow;
+      if (pix < a.npix) {
+        v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+        *reinterpret_cast<v4i *>(a.y + (int64_t)pix * a.y_cs + oc) = o;
       }
     }
   }
@@ -351,14 +467,60 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(ConvArgs a) {
 namespace {
 
 struct TileCfg {
-  int bm, bn;
+  int bm, bn, wm, wn;
+  const char *name;
 };
-const TileCfg kTiles[] = {{128, 128}, {64, 256}, {32, 256}};
+// wave tile = (bm/wm) x (bn/wn)
+const TileCfg kTiles[] = {
+    {128, 256, 2, 2, "mfma_128x256"},   // 0: waves of 64x128
+    {64, 256, 1, 4, "mfma_64x256"},     // 1: waves of 64x64
+    {64, 512, 1, 4, "mfma_64x512"},     // 2: waves of 64x128
+    {32, 256, 1, 4, "mfma_32x256"},     // 3: waves of 32x64
+    {128, 128, 2, 2, "mfma_128x128"},   // 4: waves of 64x64
+    {64, 128, 2, 2, "mfma_64x128"},     // 5: waves of 32x64
+    {64, 64, 2, 2, "mfma_64x64"},       // 6: waves of 32x32
+};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-int pick_tile(int ocp16) {
-  if (ocp16 > 64) return 0;
-  if (ocp16 > 32) return 1;
-  return 2;
+template <bool FAST, bool UNI>
+void launch_mfma(int tile, dim3 grid, hipStream_t st, const ConvArgs &a) {
+  switch (tile) {
+    case 0: hipLaunchKernelGGL((conv_mfma_kernel<128, 256, 2, 2, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((conv_mfma_kernel<64, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((conv_mfma_kernel<64, 512, 1, 4, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 3: hipLaunchKernelGGL((conv_mfma_kernel<32, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((conv_mfma_kernel<128, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 5: hipLaunchKernelGGL((conv_mfma_kernel<64, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    default: hipLaunchKernelGGL((conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+  }
+}
+
+// Rough cost model (cycles) used to pick a tile: workgroup rounds over the CUs
+// times the per-workgroup time (K steps bounded by MFMA issue or LDS reads, plus
+// the VALU epilogue), with two workgroups assumed to overlap on one CU.
+int pick_tile(const tpuhip_conv_desc &d, int k16, int num_cu) {
+  const int64_t npix = (int64_t)d.n * d.oh * d.ow;
+  const int nsteps = (k16 * 16 + 63) / 64;
+  double best = 1e30;
+  int best_tile = 1;
+  for (int t = 0; t < kNumTiles; ++t) {
+    const TileCfg &c = kTiles[t];
+    if (c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32)) continue;   // more than half the rows idle
+    const int tm = c.bm / c.wm / 32, tn = c.bn / c.wn / 32;
+    const int64_t wgs = ceil_div64(npix, c.bn) * ceil_div64(d.oc, c.bm);
+    const double mfma = tm * tn * 2 * 32.0;
+    const double ldsr = (tm + tn) * 2 * 8.0 * 4;          // four waves share the LDS port
+    const double step = std::max(std::max(mfma, ldsr), 160.0);
+    const double epi = tm * tn * 16 * 44.0;
+    const double per_wg = nsteps * step + epi + 1500.0;
+    const double rounds = std::ceil((double)wgs / (2.0 * num_cu));
+    const double cost = rounds * per_wg * (wgs < num_cu ? 1.0 : 1.0);
+    if (cost < best) {
+      best = cost;
+      best_tile = t;
+    }
+  }
+  return best_tile;
 }
 
 int check_desc(const tpuhip_conv_desc &d) {
@@ -379,10 +541,133 @@ int check_desc(const tpuhip_conv_desc &d) {
   // that matters for memory safety is that every output maps to a legal window
   TPUHIP_REQUIRE(d.oh <= oh && d.ow <= ow, "conv: output %dx%d larger than the window grid %dx%d",
                  d.oh, d.ow, oh, ow);
-  TPUHIP_REQUIRE((int64_t)d.n * d.oh * d.ow < (1ll << 31) &&
-                     (int64_t)d.n * d.ih * d.iw * d.x_cs < (1ll << 40),
+  // the kernels index pixels and input bytes with 32-bit integers
+  TPUHIP_REQUIRE(d.oh < 65536 && d.ow < 65536 && (int64_t)d.n * d.oh * d.ow < (1ll << 30) &&
+                     (int64_t)d.n * (d.ih + d.pt + d.pb + 2) * (d.iw + d.pl + d.pr + 2) * d.x_cs <
+                         (1ll << 31) &&
+                     (int64_t)d.n * d.oh * d.ow * d.y_cs < (1ll << 40),
                  "conv: tensor too large");
   return TPUHIP_OK;
+}
+
+// (re)builds the device filter of an MFMA conv for tile variant `tile`
+int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
+  const tpuhip_conv_desc &d = cw->d;
+  const TileCfg &t = kTiles[tile];
+  const int tm = t.bm / t.wm / 32;
+  const int icp = round_up(d.ic, 16);
+  const int ocp = round_up(d.oc, t.bm);
+  std::vector<int8_t> packed((size_t)ocp * cw->kp, 0);
+  const int8_t *filter = cw->host_filter.data();
+  for (int row = 0; row < ocp; ++row) {
+    const int tile0 = row / t.bm * t.bm;
+    const int oc = tile0 + mfma_row_to_oc(row - tile0, tm);
+    if (oc >= d.oc) continue;
+    int8_t *dst = packed.data() + (size_t)row * cw->kp;
+    const int8_t *src = filter + (size_t)oc * d.ic * d.kh * d.kw;
+    for (int c = 0; c < d.ic; ++c)
+      for (int k = 0; k < d.kh * d.kw; ++k) dst[(size_t)k * icp + c] = src[(size_t)c * d.kh * d.kw + k];
+  }
+  if (cw->w) {
+    if (int rc = tpuhip_free(ctx, cw->w)) return rc;
+    cw->w = nullptr;
+  }
+  if (int rc = tpuhip_malloc(ctx, packed.size(), (void **)&cw->w)) return rc;
+  if (int rc = tpuhip_upload(ctx, cw->w, packed.data(), packed.size())) return rc;
+  cw->tile = tile;
+  cw->ocp = ocp;
+  return TPUHIP_OK;
+}
+
+bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
+  const TileCfg &c = kTiles[t];
+  return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
+}
+
+void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *out) {
+  const tpuhip_conv_desc &d = w->d;
+  ConvArgs a{};
+  a.x = (const int8_t *)x;
+  a.w = w->w;
+  a.bias = w->bias;
+  a.qp = w->qp;
+  a.y = (int8_t *)y;
+  a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.x_cs = d.x_cs;
+  a.oh = d.oh; a.ow = d.ow; a.y_cs = d.y_cs;
+  a.oc = d.oc; a.ocw = round_up(d.oc, 16); a.icg = d.ic / d.g; a.ocg = d.oc / d.g; a.g = d.g;
+  a.kh = d.kh; a.kw = d.kw; a.sh = d.sh; a.sw = d.sw; a.pt = d.pt; a.pl = d.pl;
+  a.dh = d.dh; a.dw = d.dw; a.ins_h = d.ins_h; a.ins_w = d.ins_w;
+  a.c16 = w->c16; a.k16 = w->k16; a.kp = w->kp;
+  a.npix = d.n * d.oh * d.ow;
+  a.lo = (d.do_relu && !d.relu_first) ? 0 : -128;
+  a.relu_first = (d.do_relu && d.relu_first) ? 1 : 0;
+  if (w->algo == ALGO_MFMA) {
+    const TileCfg &t = kTiles[w->tile];
+    a.magic_c16 = (1u << 20) / (uint32_t)w->c16 + 1;
+    a.magic_kw = (1u << 20) / (uint32_t)d.kw + 1;
+    a.x_bytes = (uint32_t)((int64_t)d.n * d.ih * d.iw * d.x_cs);
+    a.w_bytes = (uint32_t)((int64_t)w->ocp * w->kp);
+    a.magic_ow = d.ow > 1 ? (uint32_t)(((1ull << 32) + d.ow - 1) / (uint64_t)d.ow) : 0;
+    a.magic_oh = d.oh > 1 ? (uint32_t)(((1ull << 32) + d.oh - 1) / (uint64_t)d.oh) : 0;
+    a.n_oc_tiles = w->ocp / t.bm;
+    a.n_tiles = (int)(ceil_div64(a.npix, t.bn) * a.n_oc_tiles);
+    a.tiles_per_xcd = (a.n_tiles + 7) / 8;
+  }
+  *out = a;
+}
+
+void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvArgs &a) {
+  dim3 grid((unsigned)(a.tiles_per_xcd * 8));
+  const bool uni = (w->c16 % 4) == 0;
+  if (w->fast && uni)
+    launch_mfma<true, true>(w->tile, grid, ctx->stream, a);
+  else if (w->fast)
+    launch_mfma<true, false>(w->tile, grid, ctx->stream, a);
+  else if (uni)
+    launch_mfma<false, true>(w->tile, grid, ctx->stream, a);
+  else
+    launch_mfma<false, false>(w->tile, grid, ctx->stream, a);
+}
+
+// Times every candidate tile on the layer's real buffers (the kernels are
+// idempotent and bit-identical across tiles) and keeps the fastest.
+int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *y) {
+  hipEvent_t e0, e1;
+  TPUHIP_CHECK_HIP(hipEventCreate(&e0));
+  TPUHIP_CHECK_HIP(hipEventCreate(&e1));
+  float best_ms = 1e30f;
+  int best = -1;
+  int rc = TPUHIP_OK;
+  for (int t = 0; t < kNumTiles && !rc; ++t) {
+    if (!tile_is_candidate(w->d, t)) continue;
+    rc = pack_mfma_weights(ctx, w, t);
+    if (rc) break;
+    ConvArgs a;
+    fill_args(w, x, y, &a);
+    for (int i = 0; i < 2; ++i) launch_conv_mfma(ctx, w, a);
+    hipEventRecord(e0, ctx->stream);
+    for (int i = 0; i < 5; ++i) launch_conv_mfma(ctx, w, a);
+    hipEventRecord(e1, ctx->stream);
+    if (hipEventSynchronize(e1) != hipSuccess || hipGetLastError() != hipSuccess) {
+      rc = set_error(TPUHIP_ERR_HIP, "conv autotune: kernel launch failed");
+      break;
+    }
+    float ms = 0;
+    hipEventElapsedTime(&ms, e0, e1);
+    if (ms < best_ms) {
+      best_ms = ms;
+      best = t;
+    }
+  }
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
+  if (rc) return rc;
+  if (best < 0) return set_error(TPUHIP_ERR_INVALID, "conv autotune: no candidate tile");
+  if (best != w->tile) rc = pack_mfma_weights(ctx, w, best);
+  w->tuned = true;
+  w->host_filter.clear();
+  w->host_filter.shrink_to_fit();
+  return rc;
 }
 
 }  // namespace
@@ -401,13 +686,26 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
                    rshift[i]);
   TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
 
-  const int icg = d.ic / d.g, ocg = d.oc / d.g;
+  const int icg = d.ic / d.g;
   const bool dense = d.g == 1 && d.ins_h == 0 && d.ins_w == 0;
   const bool depthwise = d.g == d.ic && d.g == d.oc && d.ins_h == 0 && d.ins_w == 0;
-  int algo = d.algo;
+  int algo = d.algo, forced_tile = -1;
+  if (algo >= 16) {   // MFMA with an explicit tile variant (tests, tuning)
+    forced_tile = algo - 16;
+    algo = ALGO_MFMA;
+    TPUHIP_REQUIRE(forced_tile < kNumTiles, "conv: unknown MFMA tile %d", forced_tile);
+  }
   if (algo == ALGO_AUTO) algo = dense ? ALGO_MFMA : depthwise ? ALGO_DEPTHWISE : ALGO_DIRECT;
   TPUHIP_REQUIRE(algo >= ALGO_DIRECT && algo <= ALGO_DEPTHWISE, "conv: unknown algo %d", d.algo);
-  TPUHIP_REQUIRE(algo != ALGO_MFMA || dense, "conv: MFMA path needs g == 1 and no inserted zeros");
+  // the MFMA kernel locates a K group with multiply-shift divisions that are exact
+  // for at most 4094 groups of at most 256 16-channel groups each
+  const bool mfma_ok = dense && round_up(d.ic, 16) / 16 <= 256 &&
+                       (int64_t)d.kh * d.kw * (round_up(d.ic, 16) / 16) + 16 < 4095 &&
+                       (int64_t)round_up(d.oc, 128) * (d.kh * d.kw * round_up(d.ic, 16) + 64) <
+                           (1ll << 31);
+  if (d.algo == ALGO_AUTO && algo == ALGO_MFMA && !mfma_ok) algo = ALGO_DIRECT;
+  TPUHIP_REQUIRE(algo != ALGO_MFMA || mfma_ok,
+                 "conv: MFMA path needs g == 1, no inserted zeros, ic <= 4096 and K < 65000");
   TPUHIP_REQUIRE(algo != ALGO_DEPTHWISE || depthwise,
                  "conv: depthwise path needs g == ic == oc and no inserted zeros");
 
@@ -415,21 +713,23 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   cw->d = d;
   cw->algo = algo;
   std::vector<int8_t> packed;
+  const size_t per_oc = (size_t)icg * d.kh * d.kw;
   if (algo == ALGO_MFMA) {
-    cw->tile = pick_tile(round_up(d.oc, 16));
-    const int bm = kTiles[cw->tile].bm;
-    cw->ocp = round_up(d.oc, bm);
     const int icp = round_up(d.ic, 16);
     cw->c16 = icp / 16;
     cw->k16 = d.kh * d.kw * cw->c16;
     cw->kp = round_up(cw->k16 * 16, 64);
-    packed.assign((size_t)cw->ocp * cw->kp, 0);
-    for (int oc = 0; oc < d.oc; ++oc)
-      for (int c = 0; c < d.ic; ++c)
-        for (int kh = 0; kh < d.kh; ++kh)
-          for (int kw = 0; kw < d.kw; ++kw)
-            packed[(size_t)oc * cw->kp + (size_t)(kh * d.kw + kw) * icp + c] =
-                filter[(((size_t)oc * d.ic + c) * d.kh + kh) * d.kw + kw];
+    cw->host_filter.assign(filter, filter + (size_t)d.oc * per_oc);
+    const int tile = forced_tile >= 0 ? forced_tile : pick_tile(d, cw->k16, ctx->num_cu);
+    if (int rc = pack_mfma_weights(ctx, cw, tile)) {
+      tpuhip_conv2d_weights_destroy(ctx, cw);
+      return rc;
+    }
+    cw->tuned = forced_tile >= 0 || !ctx->autotune;
+    if (cw->tuned) {
+      cw->host_filter.clear();
+      cw->host_filter.shrink_to_fit();
+    }
   } else if (algo == ALGO_DEPTHWISE) {
     cw->ocp = round_up(d.oc, 16);
     packed.assign((size_t)d.kh * d.kw * cw->ocp, 0);
@@ -448,23 +748,42 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
             packed[(((size_t)oc * d.kh + kh) * d.kw + kw) * icg + c] =
                 filter[(((size_t)oc * icg + c) * d.kh + kh) * d.kw + kw];
   }
-  (void)ocg;
-  std::vector<ChanParams> cp((size_t)cw->ocp);
-  for (int i = 0; i < cw->ocp; ++i) {
-    ChanParams p{};
+  // epilogue parameters, indexed by the true output channel.  `fast` holds when,
+  // for every channel, 1 <= rshift and |acc + bias| + 1 + 2^(rshift-1) cannot reach
+  // 2^31: |acc| <= 128 * sum|w|, and |x| <= |v| + 1 after the doubling high multiply.
+  const size_t nparam = (size_t)round_up(d.oc, 128) + 16;   // covers every tile's padding
+  std::vector<int32_t> b32(nparam, 0);
+  std::vector<QParam> qp(nparam);
+  bool fast = true;
+  for (int i = 0; i < (int)qp.size(); ++i) {
+    QParam q{};
     if (i < d.oc) {
-      p.bias = (d.with_bias && bias) ? bias[i] : 0;
-      p.mult = multiplier[i];
-      p.rshift = rshift[i];
-      p.mask = (int32_t)((1ll << rshift[i]) - 1);
-      p.half = p.mask >> 1;
+      b32[i] = (d.with_bias && bias) ? bias[i] : 0;
+      q.mult = multiplier[i];
+      q.rshift = rshift[i];
+      q.mask = (int32_t)((1ll << rshift[i]) - 1);
+      q.hpot = rshift[i] > 0 ? (int32_t)(1ll << (rshift[i] - 1)) : 0;
+      int64_t sumw = 0;
+      for (size_t k = 0; k < per_oc; ++k) sumw += std::abs((int)filter[(size_t)i * per_oc + k]);
+      const int64_t bound = 128 * sumw + std::llabs((long long)b32[i]) + 1 + q.hpot;
+      if (rshift[i] < 1 || bound >= (1ll << 31)) fast = false;
+    } else {
+      q.rshift = 1;   // pad channels: multiplier 0 gives 0 on either path
+      q.mask = 1;
+      q.hpot = 1;
     }
-    cp[i] = p;
+    qp[i] = q;
   }
-  int rc = tpuhip_malloc(ctx, packed.size(), (void **)&cw->w);
-  if (!rc) rc = tpuhip_malloc(ctx, cp.size() * sizeof(ChanParams), (void **)&cw->cp);
-  if (!rc) rc = tpuhip_upload(ctx, cw->w, packed.data(), packed.size());
-  if (!rc) rc = tpuhip_upload(ctx, cw->cp, cp.data(), cp.size() * sizeof(ChanParams));
+  cw->fast = fast ? 1 : 0;
+  int rc = TPUHIP_OK;
+  if (algo != ALGO_MFMA) {
+    rc = tpuhip_malloc(ctx, packed.size(), (void **)&cw->w);
+    if (!rc) rc = tpuhip_upload(ctx, cw->w, packed.data(), packed.size());
+  }
+  if (!rc) rc = tpuhip_malloc(ctx, b32.size() * sizeof(int32_t), (void **)&cw->bias);
+  if (!rc) rc = tpuhip_malloc(ctx, qp.size() * sizeof(QParam), (void **)&cw->qp);
+  if (!rc) rc = tpuhip_upload(ctx, cw->bias, b32.data(), b32.size() * sizeof(int32_t));
+  if (!rc) rc = tpuhip_upload(ctx, cw->qp, qp.data(), qp.size() * sizeof(QParam));
   if (rc) {
     tpuhip_conv2d_weights_destroy(ctx, cw);
     return rc;
@@ -477,9 +796,10 @@ int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w) {
   if (!w) return TPUHIP_OK;
   TPUHIP_REQUIRE(ctx, "tpuhip_conv2d_weights_destroy: NULL context");
   int rc = tpuhip_free(ctx, w->w);
-  int rc2 = tpuhip_free(ctx, w->cp);
+  int rc2 = tpuhip_free(ctx, w->bias);
+  int rc3 = tpuhip_free(ctx, w->qp);
   delete w;
-  return rc ? rc : rc2;
+  return rc ? rc : rc2 ? rc2 : rc3;
 }
 
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
@@ -487,44 +807,21 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
   switch (w->algo) {
     case ALGO_DIRECT: return "direct";
     case ALGO_DEPTHWISE: return "depthwise";
-    case ALGO_MFMA:
-      return w->tile == 0 ? "mfma_128x128" : w->tile == 1 ? "mfma_64x256" : "mfma_32x256";
+    case ALGO_MFMA: return kTiles[w->tile].name;
   }
   return "?";
 }
 
 int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_conv2d_i8: NULL argument");
-  const tpuhip_conv_desc &d = w->d;
-  ConvArgs a{};
-  a.x = (const int8_t *)x;
-  a.w = w->w;
-  a.cp = w->cp;
-  a.y = (int8_t *)y;
-  a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.x_cs = d.x_cs;
-  a.oh = d.oh; a.ow = d.ow; a.y_cs = d.y_cs;
-  a.oc = d.oc; a.ocw = round_up(d.oc, 16); a.icg = d.ic / d.g; a.ocg = d.oc / d.g; a.g = d.g;
-  a.kh = d.kh; a.kw = d.kw; a.sh = d.sh; a.sw = d.sw; a.pt = d.pt; a.pl = d.pl;
-  a.dh = d.dh; a.dw = d.dw; a.ins_h = d.ins_h; a.ins_w = d.ins_w;
-  a.c16 = w->c16; a.k16 = w->k16; a.kp = w->kp;
-  a.npix = d.n * d.oh * d.ow;
-  a.lo = (d.do_relu && !d.relu_first) ? 0 : -128;
-  a.relu_first = (d.do_relu && d.relu_first) ? 1 : 0;
-
+  if (w->algo == ALGO_MFMA && !w->tuned) {
+    // first use: pick the tile by measurement (not capturable into a HIP graph)
+    if (int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, y)) return rc;
+  }
+  ConvArgs a;
+  fill_args(w, x, y, &a);
   if (w->algo == ALGO_MFMA) {
-    const TileCfg t = kTiles[w->tile];
-    dim3 grid((unsigned)((a.npix + t.bn - 1) / t.bn), (unsigned)(w->ocp / t.bm));
-    switch (w->tile) {
-      case 0:
-        hipLaunchKernelGGL((conv_mfma_kernel<128, 128, 2, 2>), grid, dim3(256), 0, ctx->stream, a);
-        break;
-      case 1:
-        hipLaunchKernelGGL((conv_mfma_kernel<64, 256, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
-        break;
-      default:
-        hipLaunchKernelGGL((conv_mfma_kernel<32, 256, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
-        break;
-    }
+    launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
     const int64_t total = (int64_t)a.npix * (a.ocw / 16);
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(total, 256), 1 << 20);

@@ -215,23 +215,31 @@ std::vector<std::string> ModuleInterpreter::getAllTensorName() {
 void ModuleInterpreter::sync() { ck(tpuhip_sync(ctx_), "sync"); }
 
 std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_t bidx, int iters) {
+  // One HIP event between consecutive kernels of a normal invoke, on the stream
+  // the kernels run on: kernel i's time is event[i+1] - event[i], averaged.
   if (iters < 1) iters = 1;
   for (auto &kv : valueMapping) kv.second->set_batch_idx(bidx);
-  std::vector<std::pair<std::string, float>> out;
-  void *e0 = nullptr, *e1 = nullptr;
-  ck(tpuhip_event_create(ctx_, &e0), "timeKernels");
-  ck(tpuhip_event_create(ctx_, &e1), "timeKernels");
-  for (auto &krnl : kernel_list_) {
-    krnl->invoke();  // warm
-    ck(tpuhip_event_record(ctx_, e0), "timeKernels");
-    for (int i = 0; i < iters; ++i) krnl->invoke();
-    ck(tpuhip_event_record(ctx_, e1), "timeKernels");
-    float ms = 0;
-    ck(tpuhip_event_elapsed_ms(ctx_, e0, e1, &ms), "timeKernels");
-    out.emplace_back(krnl->name, ms / (float)iters);
+  const size_t nk = kernel_list_.size();
+  std::vector<void *> ev(nk + 1, nullptr);
+  for (auto &e : ev) ck(tpuhip_event_create(ctx_, &e), "timeKernels");
+  std::vector<double> acc(nk, 0.0);
+  for (int it = 0; it < iters; ++it) {
+    size_t i = 0;
+    ck(tpuhip_event_record(ctx_, ev[0]), "timeKernels");
+    for (auto &krnl : kernel_list_) {
+      krnl->invoke();
+      ck(tpuhip_event_record(ctx_, ev[++i]), "timeKernels");
+    }
+    for (i = 0; i < nk; ++i) {
+      float ms = 0;
+      ck(tpuhip_event_elapsed_ms(ctx_, ev[i], ev[i + 1], &ms), "timeKernels");
+      acc[i] += ms;
+    }
   }
-  tpuhip_event_destroy(ctx_, e0);
-  tpuhip_event_destroy(ctx_, e1);
+  std::vector<std::pair<std::string, float>> out;
+  size_t i = 0;
+  for (auto &krnl : kernel_list_) out.emplace_back(krnl->name, (float)(acc[i++] / iters));
+  for (auto &e : ev) tpuhip_event_destroy(ctx_, e);
   return out;
 }
 
