@@ -53,6 +53,12 @@ def main():
     ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-layer", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--save-tiles", default="", help="write the conv tile chosen for every layer")
+    ap.add_argument("--tiles", default="", help="use the conv tiles recorded in this file instead "
+                                                "of timing the variants (repeatable profiling)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB read + 256 MiB write kernel (relu) so HBM "
+                         "counters can be scaled against a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus %d refused); the path shards "
@@ -64,6 +70,12 @@ def main():
     graph_fn = graphs.CONFIGS[args.config]
     g = graph_fn()
     batch = g.input_op().shape[0]
+    tile_names = ["mfma_128x256", "mfma_64x256", "mfma_64x512", "mfma_32x256", "mfma_128x128",
+                  "mfma_64x128", "mfma_64x64"]
+    if args.tiles:
+        for name, algo in json.load(open(args.tiles)).items():
+            if algo in tile_names:
+                g.by_name[name].attrs["algo"] = 16 + tile_names.index(algo)
     m = module(device=0)
     m.load(g)
     m.set_tensor(g.input_op().name, g.input_op().data.astype(np.float32))
@@ -72,6 +84,22 @@ def main():
     for _ in range(max(args.warmup, 1)):
         m.invoke()
     m.sync()
+    if args.save_tiles:
+        json.dump({name: algo for name, algo in m.kernels() if algo.startswith("mfma")},
+                  open(args.save_tiles, "w"))
+
+    if args.copy_calibration:
+        from tpu_compiler_amd import capi
+        cal = capi.Context(0)
+        n = 256 << 20
+        src, dst = cal.malloc(n), cal.malloc(n)
+        cal._ck(cal.lib.tpuhip_memset(cal.h, src, 1, n))
+        for _ in range(3):
+            cal._ck(cal.lib.tpuhip_relu_i8(cal.h, src, dst, n))
+        cal.sync()
+        cal.free(src)
+        cal.free(dst)
+        cal.close()
 
     import ctypes as C
     e0, e1 = C.c_void_p(), C.c_void_p()

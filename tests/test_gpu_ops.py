@@ -82,7 +82,7 @@ TILE_CASES = [
 
 
 @pytest.mark.parametrize("case", TILE_CASES)
-@pytest.mark.parametrize("tile", range(7))
+@pytest.mark.parametrize("tile", range(12))
 def test_conv_every_mfma_tile_variant(ctx, case, tile):
     n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
     rng = np.random.default_rng(ic * 7 + oc + tile)

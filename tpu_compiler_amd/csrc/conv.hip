@@ -15,6 +15,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 
 using namespace tpuhip;
@@ -42,6 +43,8 @@ struct tpuhip_conv_weights {
   int8_t *w = nullptr;   // packed filter
   int32_t *bias = nullptr;
   QParam *qp = nullptr;
+  int32_t *qplanes = nullptr;   // mult | rshift | hpot planes of nparam entries each
+  int nparam = 0;
   int ocp = 0;           // padded output channels (rows of w / entries of bias, qp)
   int kp = 0;            // padded K in bytes (row stride of w) for the MFMA path
   int c16 = 0;           // input 16-channel groups per tap
@@ -53,6 +56,7 @@ struct ConvArgs {
   const int8_t *w;
   const int32_t *bias;
   const QParam *qp;
+  const int32_t *qmult, *qshift, *qhpot;   // the same per-channel data as planes (MFMA epilogue)
   int8_t *y;
   int n, ih, iw, x_cs;
   int oh, ow, y_cs;
@@ -216,10 +220,48 @@ __device__ __forceinline__ uint32_t pack_sat4(int32_t a, int32_t b, int32_t c, i
 // (proved on the host from the weights), so RoundingDivideByPOT is
 // (x + 2^(e-1) - (x < 0)) >> e without overflow.
 template <bool FAST>
-__device__ __forceinline__ int32_t requant_core(int32_t v, const QParam &q) {
-  const int32_t x = srdhm(v, q.mult);
-  if (FAST) return (x + q.hpot + (x >> 31)) >> q.rshift;
-  return rdbp(x, q.rshift, q.mask, q.mask >> 1);
+__device__ __forceinline__ int32_t requant_core(int32_t v, int32_t mult, int32_t rshift,
+                                                int32_t hpot) {
+  const int32_t x = srdhm(v, mult);
+  if (FAST) return (x + hpot + (x >> 31)) >> rshift;
+  const int32_t mask = (int32_t)((1u << rshift) - 1u);   // rshift <= 31
+  return rdbp(x, rshift, mask, mask >> 1);
+}
+
+// Epilogue of one wave tile row block: the lane's 16 consecutive channels
+// (starting at oc) of TN pixels.  Requantise, saturate (+ReLU) and store 16 bytes
+// per pixel.  Parameters are read four channels at a time to keep few registers live.
+template <int TN, bool FAST>
+__device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
+                                              int pix_first, int pix_stride) {
+  uint32_t outw[TN][4];
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    const v4i m4 = *reinterpret_cast<const v4i *>(a.qmult + oc + qd * 4);
+    const v4i r4 = *reinterpret_cast<const v4i *>(a.qshift + oc + qd * 4);
+    const v4i h4 = *reinterpret_cast<const v4i *>(a.qhpot + oc + qd * 4);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int32_t v0 = acc[j][qd * 4 + 0], v1 = acc[j][qd * 4 + 1], v2 = acc[j][qd * 4 + 2],
+              v3 = acc[j][qd * 4 + 3];
+      if (a.relu_first) {
+        v0 = max(v0, 0); v1 = max(v1, 0); v2 = max(v2, 0); v3 = max(v3, 0);
+      }
+      outw[j][qd] = pack_sat4(requant_core<FAST>(v0, m4[0], r4[0], h4[0]),
+                              requant_core<FAST>(v1, m4[1], r4[1], h4[1]),
+                              requant_core<FAST>(v2, m4[2], r4[2], h4[2]),
+                              requant_core<FAST>(v3, m4[3], r4[3], h4[3]), a.lo);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int pix = pix_first + j * pix_stride;
+    if (pix < a.npix) {
+      v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+      *reinterpret_cast<v4i *>(a.y + (int64_t)pix * a.y_cs + oc) = o;
+    }
+  }
 }
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
@@ -390,74 +432,222 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
   store_tile(0, 0);
   __syncthreads();
 
-  // Steps are processed DEPTH at a time so that ring slots and LDS buffers are
-  // compile-time indices; steps past the end of K multiply zeros.
-  for (int s0 = 0; s0 < nsteps; s0 += DEPTH) {
+  auto compute = [&](int buf) {
+    const v4i *wl = lds[buf];
+    const v4i *xl = lds[buf] + BM * 4;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const int chunk = kk * 2 + fk;
+      v4i af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int r = (wm * TM + i) * 32 + frow;
+        af[i] = wl[r * 4 + (chunk ^ ((r >> 2) & 3))];
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int r = (wn * TN + j) * 32 + frow;
+        bf[j] = xl[r * 4 + (chunk ^ ((r >> 2) & 3))];
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+  };
+  // Whole groups of DEPTH steps: ring slots and LDS buffers are compile-time indices
+  // (DEPTH is even, so buffer parity == slot parity) and the body has no branch.
+  const int full = nsteps / DEPTH;
+#pragma nounroll
+  for (int g = 0; g < full; ++g) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      const int step = s0 + d;
-      const int buf = d & 1;   // == step & 1 because DEPTH is even
       // slot d went to LDS one step ago: refill it with the tile DEPTH steps ahead
-      load_tile(d, step + DEPTH);
-      if (step >= nsteps) break;   // uniform: only the last group can be short
-      const v4i *wl = lds[buf];
-      const v4i *xl = lds[buf] + BM * 4;
+      load_tile(d, (g + 1) * DEPTH + d);
+      compute(d & 1);
+      store_tile((d + 1) % DEPTH, (d & 1) ^ 1);
+      __syncthreads();
+    }
+  }
+  // the last nsteps % DEPTH steps: their tiles are already in the ring / in LDS
+  const int rem = nsteps - full * DEPTH;
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        const int chunk = kk * 2 + fk;
-        v4i af[TM], bf[TN];
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int r = (wm * TM + i) * 32 + frow;
-          af[i] = wl[r * 4 + (chunk ^ ((r >> 2) & 3))];
-        }
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int r = (wn * TN + j) * 32 + frow;
-          bf[j] = xl[r * 4 + (chunk ^ ((r >> 2) & 3))];
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-      }
-      store_tile((d + 1) % DEPTH, buf ^ 1);
+  for (int d = 0; d < DEPTH - 1; ++d) {
+    if (d < rem) {
+      compute(d & 1);
+      store_tile((d + 1) % DEPTH, (d & 1) ^ 1);
       __syncthreads();
     }
   }
 
-  // ---- epilogue: requantise, saturate (+ReLU), one 16-byte store per block
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int oc = ocw0 + i * 16;
-    if (oc >= a.ocw) continue;
-    const QParam *qp = a.qp + oc;
-    uint32_t outw[TN][4];
+    if (oc < a.ocw) epilogue_rows<TN, FAST>(acc[i], a, oc, pix0 + wn * TN * 32 + frow, 32);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA kernel without LDS: every wave owns a tile of TM*32 output channels x
+// TN*32 pixels and loads its MFMA operands straight from global memory in the
+// fragment layout (lane l: row l & 31, bytes 16*(l >> 5) .. +15 of a 32-byte K
+// slice), DEPTH K steps ahead in registers.  Waves never synchronise.  Weights are
+// stored fragment by fragment so their loads are 1 KiB contiguous per wave;
+// an activation load touches 32 bytes of 32 pixel rows.  Feeds the MFMAs at up to
+// what the vector L1 delivers, which is all the small layers can use, at none of
+// the LDS / barrier cost.
+// ---------------------------------------------------------------------------
+template <int TM, int TN, int DEPTH, int OCC, bool FAST, bool UNI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+conv_mfma_reg_kernel(ConvArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int logical_wg = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  const int wt = logical_wg * 4 + wave;        // this wave's tile; oc tiles of a pixel tile adjacent
+  if (wt >= a.n_tiles) return;                 // no barriers anywhere below
+  const int pix_tile = wt / a.n_oc_tiles;
+  const int oc_tile = wt - pix_tile * a.n_oc_tiles;
+  const int oc0 = oc_tile * (TM * 32);
+  const int pix0 = pix_tile * (TN * 32);
+
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  const int nsteps = a.kp / 64;
+
+  int poff[TN], ih0[TN], iw0[TN];
+  const int ow_first = pix0 % a.ow;
+  const int t_first = pix0 / a.ow;
+  const int oh_first = t_first % a.oh;
+  const int n_first = t_first / a.oh;
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      const QParam q0 = qp[qd * 4 + 0], q1 = qp[qd * 4 + 1], q2 = qp[qd * 4 + 2],
-                   q3 = qp[qd * 4 + 3];
+  for (int j = 0; j < TN; ++j) {
+    const int delta = j * 32 + frow;
+    const bool pv = pix0 + delta < a.npix;
+    const uint32_t t1 = (uint32_t)(ow_first + delta);
+    const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
+    const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
+    const uint32_t t2 = (uint32_t)oh_first + q1;
+    const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
+    const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
+    const int n = n_first + (int)q2;
+    ih0[j] = pv ? oh * a.sh - a.pt : -(1 << 28);
+    iw0[j] = ow * a.sw - a.pl;
+    poff[j] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[j]) * a.x_cs + (UNI ? fk * 16 : 0);
+    asm volatile("" : "+v"(poff[j]), "+v"(ih0[j]), "+v"(iw0[j]));
+  }
+  // weight fragments: [oc block of 32][K step][kk][lane] x 16 bytes
+  uint32_t woff[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    woff[i] = (uint32_t)(((oc0 / 32 + i) * nsteps) * 2048 + lane * 16);
+    asm volatile("" : "+v"(woff[i]));
+  }
+
+  v4i af[DEPTH][2][TM], bf[DEPTH][2][TN];
+
+  auto load_step = [&](int slot, int step) {
+    const bool in_k = step < nsteps;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[slot][kk][i] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+            wrsrc, in_k ? woff[i] : kOobOffset, step * 2048 + kk * 1024, 0);
+    if (UNI) {
+      const uint32_t kg0 = (uint32_t)(step * 4);
+      const uint32_t tap = (kg0 * a.magic_c16) >> 20;
+      const int cgrp0 = (int)(kg0 - tap * (uint32_t)a.c16);
+      const int tkh = (int)((tap * a.magic_kw) >> 20);
+      const int tkw = (int)tap - tkh * a.kw;
+      const int dh_off = (int)kg0 < a.k16 ? tkh * a.dh : (1 << 28);
+      const int dw_off = tkw * a.dw;
+      const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp0 * 16;
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        int32_t v0 = acc[i][j][qd * 4 + 0], v1 = acc[i][j][qd * 4 + 1],
-                v2 = acc[i][j][qd * 4 + 2], v3 = acc[i][j][qd * 4 + 3];
-        if (a.relu_first) {
-          v0 = max(v0, 0); v1 = max(v1, 0); v2 = max(v2, 0); v3 = max(v3, 0);
-        }
-        outw[j][qd] = pack_sat4(requant_core<FAST>(v0, q0), requant_core<FAST>(v1, q1),
-                                       requant_core<FAST>(v2, q2), requant_core<FAST>(v3, q3),
-                                       a.lo);
+        const int ih = ih0[j] + dh_off, iw = iw0[j] + dw_off;
+        const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+        const uint32_t off = ok ? (uint32_t)(poff[j] + tap_off) : kOobOffset;
+        bf[slot][0][j] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 0, 0);
+        bf[slot][1][j] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 32, 0);
       }
-    }
+    } else {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int pix = pix0 + (wn * TN + j) * 32 + frow;
-      if (pix < a.npix) {
-        v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
-        *reinterpret_cast<v4i *>(a.y + (int64_t)pix * a.y_cs + oc) = o;
+      for (int kk = 0; kk < 2; ++kk) {
+        const uint32_t kg = (uint32_t)(step * 4 + kk * 2 + fk);
+        const uint32_t tap = (kg * a.magic_c16) >> 20;
+        const int cgrp = (int)(kg - tap * (uint32_t)a.c16);
+        const int tkh = (int)((tap * a.magic_kw) >> 20);
+        const int tkw = (int)tap - tkh * a.kw;
+        const int dh_off = (int)kg < a.k16 ? tkh * a.dh : (1 << 28);
+        const int dw_off = tkw * a.dw;
+        const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp * 16;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int ih = ih0[j] + dh_off, iw = iw0[j] + dw_off;
+          const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+          bf[slot][kk][j] = buffer_load16(xrsrc, ok ? (uint32_t)(poff[j] + tap_off) : kOobOffset);
+        }
       }
     }
+  };
+
+  v16i acc[TM][TN];
+  const int ocw0 = oc0 + fk * 16 * TM;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4i b = bp[q];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j][q * 4 + 0] = b[0];
+        acc[i][j][q * 4 + 1] = b[1];
+        acc[i][j][q * 4 + 2] = b[2];
+        acc[i][j][q * 4 + 3] = b[3];
+      }
+    }
+  }
+
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
+
+  auto mfma_step = [&](int slot) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[slot][kk][i], bf[slot][kk][j],
+                                                            acc[i][j], 0, 0, 0);
+  };
+  // whole groups of DEPTH steps: branch-free body, ring slots are compile-time indices
+  const int full = nsteps / DEPTH;
+#pragma nounroll
+  for (int g = 0; g < full; ++g) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      mfma_step(d);
+      load_step(d, (g + 1) * DEPTH + d);
+    }
+  }
+  // the last nsteps % DEPTH steps are already in the ring
+  const int rem = nsteps - full * DEPTH;
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < rem) mfma_step(d);
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int oc = ocw0 + i * 16;
+    if (oc < a.ocw) epilogue_rows<TN, FAST>(acc[i], a, oc, pix0 + frow, 32);
   }
 }
 
@@ -469,6 +659,7 @@ namespace {
 struct TileCfg {
   int bm, bn, wm, wn;
   const char *name;
+  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave
 };
 // wave tile = (bm/wm) x (bn/wn)
 const TileCfg kTiles[] = {
@@ -479,6 +670,11 @@ const TileCfg kTiles[] = {
     {128, 128, 2, 2, "mfma_128x128"},   // 4: waves of 64x64
     {64, 128, 2, 2, "mfma_64x128"},     // 5: waves of 32x64
     {64, 64, 2, 2, "mfma_64x64"},       // 6: waves of 32x32
+    {64, 64, 1, 1, "mfma_reg_64x64", 1},    // 7
+    {32, 64, 1, 1, "mfma_reg_32x64", 1},    // 8
+    {64, 128, 1, 1, "mfma_reg_64x128", 1},  // 9
+    {32, 32, 1, 1, "mfma_reg_32x32", 1},    // 10
+    {64, 32, 1, 1, "mfma_reg_64x32", 1},    // 11
 };
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
@@ -491,7 +687,12 @@ void launch_mfma(int tile, dim3 grid, hipStream_t st, const ConvArgs &a) {
     case 3: hipLaunchKernelGGL((conv_mfma_kernel<32, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
     case 4: hipLaunchKernelGGL((conv_mfma_kernel<128, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
     case 5: hipLaunchKernelGGL((conv_mfma_kernel<64, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    default: hipLaunchKernelGGL((conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 6: hipLaunchKernelGGL((conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 7: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 8: hipLaunchKernelGGL((conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 9: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 10: hipLaunchKernelGGL((conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    default: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), 0, st, a); break;
   }
 }
 
@@ -505,6 +706,7 @@ int pick_tile(const tpuhip_conv_desc &d, int k16, int num_cu) {
   int best_tile = 1;
   for (int t = 0; t < kNumTiles; ++t) {
     const TileCfg &c = kTiles[t];
+    if (c.reg) continue;
     if (c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32)) continue;   // more than half the rows idle
     const int tm = c.bm / c.wm / 32, tn = c.bn / c.wn / 32;
     const int64_t wgs = ceil_div64(npix, c.bn) * ceil_div64(d.oc, c.bm);
@@ -559,14 +761,29 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
   const int ocp = round_up(d.oc, t.bm);
   std::vector<int8_t> packed((size_t)ocp * cw->kp, 0);
   const int8_t *filter = cw->host_filter.data();
+  std::vector<int8_t> rowbuf((size_t)cw->kp);
+  const int nsteps = cw->kp / 64;
   for (int row = 0; row < ocp; ++row) {
     const int tile0 = row / t.bm * t.bm;
     const int oc = tile0 + mfma_row_to_oc(row - tile0, tm);
     if (oc >= d.oc) continue;
-    int8_t *dst = packed.data() + (size_t)row * cw->kp;
+    std::fill(rowbuf.begin(), rowbuf.end(), 0);
     const int8_t *src = filter + (size_t)oc * d.ic * d.kh * d.kw;
     for (int c = 0; c < d.ic; ++c)
-      for (int k = 0; k < d.kh * d.kw; ++k) dst[(size_t)k * icp + c] = src[(size_t)c * d.kh * d.kw + k];
+      for (int k = 0; k < d.kh * d.kw; ++k)
+        rowbuf[(size_t)k * icp + c] = src[(size_t)c * d.kh * d.kw + k];
+    if (!t.reg) {
+      memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
+    } else {
+      // fragment order: [row / 32][K step][kk][lane = (row & 31) + 32 * half][16 bytes]
+      const int blk = row / 32, r = row % 32;
+      for (int step = 0; step < nsteps; ++step)
+        for (int kk = 0; kk < 2; ++kk)
+          for (int half = 0; half < 2; ++half)
+            memcpy(packed.data() + ((size_t)(blk * nsteps + step) * 2 + kk) * 1024 +
+                       (size_t)(r + 32 * half) * 16,
+                   rowbuf.data() + (size_t)step * 64 + (kk * 2 + half) * 16, 16);
+    }
   }
   if (cw->w) {
     if (int rc = tpuhip_free(ctx, cw->w)) return rc;
@@ -591,6 +808,9 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
   a.w = w->w;
   a.bias = w->bias;
   a.qp = w->qp;
+  a.qmult = w->qplanes;
+  a.qshift = w->qplanes + w->nparam;
+  a.qhpot = w->qplanes + 2 * w->nparam;
   a.y = (int8_t *)y;
   a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.x_cs = d.x_cs;
   a.oh = d.oh; a.ow = d.ow; a.y_cs = d.y_cs;
@@ -611,7 +831,9 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
     a.magic_oh = d.oh > 1 ? (uint32_t)(((1ull << 32) + d.oh - 1) / (uint64_t)d.oh) : 0;
     a.n_oc_tiles = w->ocp / t.bm;
     a.n_tiles = (int)(ceil_div64(a.npix, t.bn) * a.n_oc_tiles);
-    a.tiles_per_xcd = (a.n_tiles + 7) / 8;
+    // workgroups per XCD (a workgroup of the LDS-free kernel holds four wave tiles)
+    const int n_wgs = t.reg ? (a.n_tiles + 3) / 4 : a.n_tiles;
+    a.tiles_per_xcd = (n_wgs + 7) / 8;
   }
   *out = a;
 }
@@ -784,6 +1006,17 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   if (!rc) rc = tpuhip_malloc(ctx, qp.size() * sizeof(QParam), (void **)&cw->qp);
   if (!rc) rc = tpuhip_upload(ctx, cw->bias, b32.data(), b32.size() * sizeof(int32_t));
   if (!rc) rc = tpuhip_upload(ctx, cw->qp, qp.data(), qp.size() * sizeof(QParam));
+  if (!rc && algo == ALGO_MFMA) {
+    std::vector<int32_t> planes(3 * nparam);
+    for (size_t i = 0; i < nparam; ++i) {
+      planes[i] = qp[i].mult;
+      planes[nparam + i] = qp[i].rshift;
+      planes[2 * nparam + i] = qp[i].hpot;
+    }
+    cw->nparam = (int)nparam;
+    rc = tpuhip_malloc(ctx, planes.size() * sizeof(int32_t), (void **)&cw->qplanes);
+    if (!rc) rc = tpuhip_upload(ctx, cw->qplanes, planes.data(), planes.size() * sizeof(int32_t));
+  }
   if (rc) {
     tpuhip_conv2d_weights_destroy(ctx, cw);
     return rc;
@@ -798,8 +1031,9 @@ int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w) {
   int rc = tpuhip_free(ctx, w->w);
   int rc2 = tpuhip_free(ctx, w->bias);
   int rc3 = tpuhip_free(ctx, w->qp);
+  int rc4 = tpuhip_free(ctx, w->qplanes);
   delete w;
-  return rc ? rc : rc2 ? rc2 : rc3;
+  return rc ? rc : rc2 ? rc2 : rc3 ? rc3 : rc4;
 }
 
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
