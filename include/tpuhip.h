@@ -72,6 +72,12 @@ int tpuhip_event_record(tpuhip_ctx *ctx, void *event);
 /* waits for 'stop', then returns the milliseconds between the two records */
 int tpuhip_event_elapsed_ms(tpuhip_ctx *ctx, void *start, void *stop, float *ms);
 
+/* While a pair of events is set, every kernel the context launches records its own
+ * begin and end of execution into them (the last launch wins), so
+ * tpuhip_event_elapsed_ms(start, stop) is that kernel's duration without the gaps
+ * around it.  Pass NULL, NULL to switch back. */
+int tpuhip_ctx_set_kernel_events(tpuhip_ctx *ctx, void *start, void *stop);
+
 /* channel stride the library uses for a tensor with c channels */
 int tpuhip_channel_stride(int c);
 
@@ -124,6 +130,20 @@ int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w);
  * quantizeActivationInt8PerChannelMultiplierAndRShift (core/conv.cpp:80-104,
  * lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp:849-871). */
 int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
+/* Conv2D with an EltwiseAdd folded into its epilogue (a dense conv on the MFMA path
+ * only): besides y (written unless y is NULL) the call writes
+ *   add_out = sat8(floor(relu?(add_src * m_src + y * m_conv) / 2^rshift + 0.5)),
+ * i.e. EltwiseAddOpKernel::i8_invoke (core/eltwise.cpp:52-85) applied to
+ * (add_src, y).  add_src / add_out have the shape and channel stride of y.
+ * The results equal running the two ops one after the other. */
+typedef struct {
+  int enable;
+  int m_src, m_conv;   /* int8 multipliers of add_src and of the conv result */
+  int rshift;          /* 0..30 */
+  int do_relu;
+} tpuhip_fused_add;
+int tpuhip_conv2d_add_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+                         const void *add_src, void *add_out, const tpuhip_fused_add *f);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 

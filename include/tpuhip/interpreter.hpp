@@ -167,10 +167,19 @@ public:
   void invoke() override;
   const char *algo_name() const;
   tpuhip_conv_desc desc{};
+  // Fold an EltwiseAdd of (src, this conv's result) into this kernel's epilogue:
+  // invoke() then also writes dst.  Results are unchanged; only the module
+  // interpreter arranges this (it also silences the eltwise kernel).
+  bool can_fuse_add() const;
+  void fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift, bool relu);
+  void clear_fusion();
+  SyncedData result() const { return output_data; }
 
 private:
   tpuhip_conv_weights *packed = nullptr;
   SyncedData input_data, output_data;
+  SyncedData add_src, add_dst;
+  tpuhip_fused_add fused{};
 };
 
 class FullyConnectedOpKernel : public CPUOpKernel {  // core/fullyconnected.cpp
@@ -191,6 +200,13 @@ public:
   static constexpr const char *OpName = "CPUEltwiseAddOp";
   EltwiseAddOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
   void invoke() override;
+  // set by the module interpreter when a producing conv computes this op's result
+  bool fused_into_producer = false;
+  const std::vector<SyncedData> &inputs() const { return inputs_data; }
+  SyncedData result() const { return output_data; }
+  const std::vector<int8_t> &multipliers() const { return multiplier; }
+  int rshift_value() const { return rshift; }
+  bool relu() const { return do_relu; }
 
 private:
   std::vector<SyncedData> inputs_data;
@@ -333,6 +349,8 @@ public:
   // kernels in execution order
   const kernel_list_t &kernels() const { return kernel_list_; }
   tpuhip_ctx *context() const { return ctx_; }
+  // conv + eltwise-add fusion (on by default; TPUHIP_FUSE=0 disables); applies at the next loadModule
+  bool fuse_eltwise = true;
 
   std::vector<std::pair<std::string, size_t>> input_details;
   std::vector<std::string> output_details;
@@ -343,6 +361,7 @@ public:
 private:
   void updateKernelList(ModuleDesc &module, std::string &target_op);
   bool isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op);
+  void fuseKernels();
   tpuhip_ctx *ctx_ = nullptr;
   kernel_map_t kernel_map_;
   kernel_list_t kernel_list_;

@@ -130,6 +130,21 @@ def test_module_api_semantics():
     m.close()
 
 
+def test_fusion_on_and_off_give_the_same_tensors(monkeypatch):
+    g = graphs.cfg3_resnet50(batch=2, hw=96)
+    want = oracle_graph.run(g)
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("TPUHIP_FUSE", fuse)
+        m = module()
+        m.load(g)
+        m.set_tensor("input", g.input_op().data.astype(np.float32))
+        m.invoke()
+        for op in g.ops:
+            assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), \
+                (fuse, op.name)
+        m.close()
+
+
 def test_module_errors_are_reported():
     g = graphs.cfg1_single_conv()
     m = module()

@@ -191,6 +191,33 @@ def test_conv_requant_edge_parameters(ctx, algo):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("tile", [1, 4, 5, 6, 7, 10])
+@pytest.mark.parametrize("relu,rs,keep_y", [(True, 6, True), (False, 0, True), (True, 9, False)])
+def test_conv_with_fused_eltwise_add(ctx, tile, relu, rs, keep_y):
+    """conv + EltwiseAdd in one kernel == the two ops run one after the other"""
+    rng = np.random.default_rng(tile * 31 + rs)
+    x = rnd_i8(rng, (2, 64, 13, 11))
+    w = rnd_w(rng, (72, 64, 3, 3))
+    bias, rsh, mult = rnd_params(rng, 72)
+    other = rnd_i8(rng, (2, 72, 13, 11))
+    m_src, m_conv = int(rng.integers(-100, 100)), int(rng.integers(20, 100))
+    y_ref = oracle_conv(x, w, bias, rsh, mult, 1, (1, 1), (1, 1, 1, 1))
+    z_ref = O.eltwise_add_i8([other, y_ref], [m_src, m_conv], [rs], relu)
+    d = conv_desc(x.shape, w.shape, pads=(1, 1, 1, 1), algo=16 + tile)
+    xt, ot = ctx.from_nchw(x), ctx.from_nchw(other)
+    yt, zt = ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    ctx.conv_add(wh, xt, yt if keep_y else None, ot, zt, m_src, m_conv, rs, relu)
+    assert np.array_equal(ctx.to_nchw(zt), z_ref)
+    assert not ctx.raw(zt)[..., 72:].any()
+    if keep_y:
+        assert np.array_equal(ctx.to_nchw(yt), y_ref)
+    else:
+        assert (ctx.raw(yt) == 0x55).all()      # the conv result was not written
+    ctx.conv_weights_destroy(wh)
+
+
 def test_conv_rejects_bad_arguments(ctx):
     d = conv_desc((1, 16, 4, 4), (16, 16, 3, 3), pads=(1, 1, 1, 1))
     w = np.zeros((16, 16, 3, 3), np.int8)

@@ -16,6 +16,10 @@ class ConvDesc(C.Structure):
         "x_cs", "y_cs", "relu_first", "algo")]
 
 
+class FusedAdd(C.Structure):
+    _fields_ = [(k, C.c_int) for k in ("enable", "m_src", "m_conv", "rshift", "do_relu")]
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
@@ -44,6 +48,7 @@ PROTOTYPES = {
     "tpuhip_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p,
                                           C.POINTER(C.c_float)]),
+    "tpuhip_ctx_set_kernel_events": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
     "tpuhip_channel_stride": (C.c_int, [C.c_int]),
     "tpuhip_nchw_to_nhwc_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
     "tpuhip_nhwc_to_nchw_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5),
@@ -54,6 +59,7 @@ PROTOTYPES = {
     "tpuhip_conv2d_weights_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_conv2d_i8": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_conv2d_algo_name": (C.c_char_p, [C.c_void_p]),
+    "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
                                                                    c_void_pp]),
@@ -277,6 +283,11 @@ class Context:
     def conv(self, w, x, y):
         self._ck(self.lib.tpuhip_conv2d_i8(self.h, w, x.ptr if hasattr(x, "ptr") else x,
                                            y.ptr if hasattr(y, "ptr") else y))
+
+    def conv_add(self, w, x, y, add_src, add_out, m_src, m_conv, rshift, do_relu):
+        f = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(do_relu))
+        self._ck(self.lib.tpuhip_conv2d_add_i8(self.h, w, x.ptr, None if y is None else y.ptr,
+                                               add_src.ptr, add_out.ptr, C.byref(f)))
 
     def conv_algo_name(self, w):
         return self.lib.tpuhip_conv2d_algo_name(w).decode()

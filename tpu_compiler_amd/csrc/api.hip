@@ -116,8 +116,7 @@ int tpuhip_memset(tpuhip_ctx *ctx, void *dptr, int value, size_t bytes) {
   const int threads = 256;
   size_t blocks = (bytes + threads - 1) / threads;
   if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)blocks), dim3(threads), 0, ctx->stream,
-                     (uint8_t *)dptr, (uint8_t)value, bytes);
+  launch(ctx, fill_bytes_kernel, dim3((unsigned)blocks), dim3(threads), (uint8_t *)dptr, (uint8_t)value, bytes);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -168,6 +167,14 @@ int tpuhip_event_elapsed_ms(tpuhip_ctx *ctx, void *start, void *stop, float *ms)
   TPUHIP_REQUIRE(ctx && start && stop && ms, "tpuhip_event_elapsed_ms: NULL argument");
   TPUHIP_CHECK_HIP(hipEventSynchronize((hipEvent_t)stop));
   TPUHIP_CHECK_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return TPUHIP_OK;
+}
+
+int tpuhip_ctx_set_kernel_events(tpuhip_ctx *ctx, void *start, void *stop) {
+  TPUHIP_REQUIRE(ctx, "tpuhip_ctx_set_kernel_events: NULL context");
+  TPUHIP_REQUIRE((start == nullptr) == (stop == nullptr), "set_kernel_events: pass both events or none");
+  ctx->prof_start = (hipEvent_t)start;
+  ctx->prof_stop = (hipEvent_t)stop;
   return TPUHIP_OK;
 }
 

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -17,6 +18,9 @@ struct tpuhip_ctx {
   bool owns_stream = false;
   int num_cu = 0;
   bool autotune = true;  // time the conv tile variants on a layer's first use
+  // when set, every kernel launch carries these events: they bracket the dispatch
+  // itself (begin / end of execution), not the gaps around it
+  hipEvent_t prof_start = nullptr, prof_stop = nullptr;
 };
 
 namespace tpuhip {
@@ -35,6 +39,17 @@ int set_error(int status, const char *fmt, ...) __attribute__((format(printf, 2,
   do {                                                                                  \
     if (!(cond)) return ::tpuhip::set_error(TPUHIP_ERR_INVALID, __VA_ARGS__);           \
   } while (0)
+
+// Launches on the context's stream; with profiling events set the dispatch records
+// its own begin / end timestamps into them.
+template <typename F, typename... Args>
+inline void launch(tpuhip_ctx *ctx, F kernel, dim3 grid, dim3 block, Args... args) {
+  if (ctx->prof_start)
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, ctx->stream, ctx->prof_start, ctx->prof_stop, 0,
+                          args...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, ctx->stream, args...);
+}
 
 inline int round_up(int v, int m) { return (v + m - 1) / m * m; }
 inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -70,6 +70,12 @@ struct ConvArgs {
   int npix;
   int lo;          // lower clamp bound: 0 with ReLU after saturation, else -128
   int relu_first;  // ReLU on the sum before requantisation (FC)
+  // optional fused eltwise add on the conv result (same shape and channel stride as y):
+  // add_dst = sat8(floor(relu?(add_src * add_m_src + y * add_m_conv) / 2^add_rshift + 0.5))
+  const int8_t *add_src;
+  int8_t *add_dst;
+  int add_m_src, add_m_conv, add_rshift, add_relu;
+  int store_y;     // 0: the conv result itself is not written (only the fused sum)
 };
 
 __device__ __forceinline__ int32_t epilogue(int32_t acc, int32_t bias, const QParam &p, int lo,
@@ -258,8 +264,27 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
   for (int j = 0; j < TN; ++j) {
     const int pix = pix_first + j * pix_stride;
     if (pix < a.npix) {
+      const int64_t off = (int64_t)pix * a.y_cs + oc;
       v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
-      *reinterpret_cast<v4i *>(a.y + (int64_t)pix * a.y_cs + oc) = o;
+      if (a.store_y) *reinterpret_cast<v4i *>(a.y + off) = o;
+      if (a.add_dst) {
+        // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
+        const v4i sv = *reinterpret_cast<const v4i *>(a.add_src + off);
+        const int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
+        v4i z;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          int32_t t[4];
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            int32_t sum = sbyte(sv[q], b) * a.add_m_src + sbyte(o[q], b) * a.add_m_conv;
+            if (a.add_relu) sum = max(sum, 0);
+            t[b] = (sum + rnd) >> a.add_rshift;
+          }
+          z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
+        }
+        *reinterpret_cast<v4i *>(a.add_dst + off) = z;
+      }
     }
   }
 }
@@ -679,20 +704,20 @@ const TileCfg kTiles[] = {
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
 template <bool FAST, bool UNI>
-void launch_mfma(int tile, dim3 grid, hipStream_t st, const ConvArgs &a) {
+void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
   switch (tile) {
-    case 0: hipLaunchKernelGGL((conv_mfma_kernel<128, 256, 2, 2, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 1: hipLaunchKernelGGL((conv_mfma_kernel<64, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((conv_mfma_kernel<64, 512, 1, 4, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 3: hipLaunchKernelGGL((conv_mfma_kernel<32, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((conv_mfma_kernel<128, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 5: hipLaunchKernelGGL((conv_mfma_kernel<64, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 6: hipLaunchKernelGGL((conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 7: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL((conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 9: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    case 10: hipLaunchKernelGGL((conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), 0, st, a); break;
-    default: hipLaunchKernelGGL((conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), 0, st, a); break;
+    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 2, FAST, UNI>), grid, dim3(256), a); break;
+    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
+    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 7: launch(ctx, (conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
+    case 8: launch(ctx, (conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
+    case 9: launch(ctx, (conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), a); break;
+    case 10: launch(ctx, (conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), a); break;
+    default: launch(ctx, (conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
   }
 }
 
@@ -821,6 +846,7 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
   a.npix = d.n * d.oh * d.ow;
   a.lo = (d.do_relu && !d.relu_first) ? 0 : -128;
   a.relu_first = (d.do_relu && d.relu_first) ? 1 : 0;
+  a.store_y = 1;
   if (w->algo == ALGO_MFMA) {
     const TileCfg &t = kTiles[w->tile];
     a.magic_c16 = (1u << 20) / (uint32_t)w->c16 + 1;
@@ -842,13 +868,13 @@ void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvA
   dim3 grid((unsigned)(a.tiles_per_xcd * 8));
   const bool uni = (w->c16 % 4) == 0;
   if (w->fast && uni)
-    launch_mfma<true, true>(w->tile, grid, ctx->stream, a);
+    launch_mfma<true, true>(ctx, w->tile, grid, a);
   else if (w->fast)
-    launch_mfma<true, false>(w->tile, grid, ctx->stream, a);
+    launch_mfma<true, false>(ctx, w->tile, grid, a);
   else if (uni)
-    launch_mfma<false, true>(w->tile, grid, ctx->stream, a);
+    launch_mfma<false, true>(ctx, w->tile, grid, a);
   else
-    launch_mfma<false, false>(w->tile, grid, ctx->stream, a);
+    launch_mfma<false, false>(ctx, w->tile, grid, a);
 }
 
 // Times every candidate tile on the layer's real buffers (the kernels are
@@ -1046,27 +1072,59 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
   return "?";
 }
 
-int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
-  TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_conv2d_i8: NULL argument");
+static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+                    const void *add_src, void *add_out, const tpuhip_fused_add *f) {
   if (w->algo == ALGO_MFMA && !w->tuned) {
     // first use: pick the tile by measurement (not capturable into a HIP graph)
-    if (int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, y)) return rc;
+    void *ty = y;
+    if (!ty) {   // tuning writes the plain conv result somewhere: borrow a scratch buffer
+      const size_t bytes = (size_t)w->d.n * w->d.oh * w->d.ow * w->d.y_cs;
+      if (int rc = tpuhip_malloc(ctx, bytes, &ty)) return rc;
+    }
+    int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, ty);
+    if (!y) tpuhip_free(ctx, ty);
+    if (rc) return rc;
   }
   ConvArgs a;
   fill_args(w, x, y, &a);
+  if (f && f->enable) {
+    a.add_src = (const int8_t *)add_src;
+    a.add_dst = (int8_t *)add_out;
+    a.add_m_src = f->m_src;
+    a.add_m_conv = f->m_conv;
+    a.add_rshift = f->rshift;
+    a.add_relu = f->do_relu ? 1 : 0;
+    a.store_y = y != nullptr;
+  }
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
     const int64_t total = (int64_t)a.npix * (a.ocw / 16);
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(total, 256), 1 << 20);
-    hipLaunchKernelGGL(conv_depthwise_kernel, dim3(blocks), dim3(256), 0, ctx->stream, a);
+    launch(ctx, conv_depthwise_kernel, dim3(blocks), dim3(256), a);
   } else {
     const int64_t total = (int64_t)a.npix * a.ocw;
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(total, 256), 1 << 20);
-    hipLaunchKernelGGL(conv_direct_kernel, dim3(blocks), dim3(256), 0, ctx->stream, a);
+    launch(ctx, conv_direct_kernel, dim3(blocks), dim3(256), a);
   }
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
+}
+
+int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
+  TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_conv2d_i8: NULL argument");
+  return run_conv(ctx, w, x, y, nullptr, nullptr, nullptr);
+}
+
+int tpuhip_conv2d_add_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+                         const void *add_src, void *add_out, const tpuhip_fused_add *f) {
+  TPUHIP_REQUIRE(ctx && w && x && add_src && add_out && f, "tpuhip_conv2d_add_i8: NULL argument");
+  TPUHIP_REQUIRE(w->algo == ALGO_MFMA, "conv2d_add: only dense convs on the MFMA path can fuse an add");
+  TPUHIP_REQUIRE(f->enable, "conv2d_add: fusion descriptor not enabled");
+  TPUHIP_REQUIRE(f->rshift >= 0 && f->rshift <= 30, "conv2d_add: rshift %d outside [0,30]", f->rshift);
+  TPUHIP_REQUIRE(f->m_src >= -128 && f->m_src <= 127 && f->m_conv >= -128 && f->m_conv <= 127,
+                 "conv2d_add: multipliers must be int8");
+  return run_conv(ctx, w, x, y, add_src, add_out, f);
 }
 
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,

@@ -250,8 +250,7 @@ int to_nhwc(tpuhip_ctx *ctx, const void *src, void *dst, int n, int c, int h, in
   if (int rc = check_layout_args(src, dst, n, c, h, w, cs)) return rc;
   const int64_t hw = (int64_t)h * w;
   dim3 grid((unsigned)ceil_div64(hw, 64), (unsigned)((cs + 63) / 64), (unsigned)n);
-  hipLaunchKernelGGL((nchw_to_nhwc_kernel<SRC>), grid, dim3(kThreads), 0, ctx->stream,
-                     (const SRC *)src, (int8_t *)dst, c, hw, cs);
+  launch(ctx, (nchw_to_nhwc_kernel<SRC>), grid, dim3(kThreads), (const SRC *)src, (int8_t *)dst, c, hw, cs);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -262,8 +261,7 @@ int to_nchw(tpuhip_ctx *ctx, const void *src, void *dst, int n, int c, int h, in
   if (int rc = check_layout_args(src, dst, n, c, h, w, cs)) return rc;
   const int64_t hw = (int64_t)h * w;
   dim3 grid((unsigned)ceil_div64(hw, 64), (unsigned)((c + 63) / 64), (unsigned)n);
-  hipLaunchKernelGGL((nhwc_to_nchw_kernel<DST>), grid, dim3(kThreads), 0, ctx->stream,
-                     (const int8_t *)src, (DST *)dst, c, hw, cs);
+  launch(ctx, (nhwc_to_nchw_kernel<DST>), grid, dim3(kThreads), (const int8_t *)src, (DST *)dst, c, hw, cs);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -305,11 +303,9 @@ int launch_lut(tpuhip_ctx *ctx, const void *x, void *y, const int8_t *table, int
                    (c % 16 == 0 || (coff + round_up(c, 16) <= y_cs));
   if (vec) {
     const int64_t total = pixels * ((c + 15) / 16);
-    hipLaunchKernelGGL(lut_vec_kernel, dim3(grid_for(total, kThreads * 4)), dim3(kThreads), 0,
-                       ctx->stream, a, t);
+    launch(ctx, lut_vec_kernel, dim3(grid_for(total, kThreads * 4)), dim3(kThreads), a, t);
   } else {
-    hipLaunchKernelGGL(lut_byte_kernel, dim3(grid_for(pixels * c, kThreads * 8)), dim3(kThreads),
-                       0, ctx->stream, a, t);
+    launch(ctx, lut_byte_kernel, dim3(grid_for(pixels * c, kThreads * 8)), dim3(kThreads), a, t);
   }
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
@@ -357,14 +353,14 @@ int tpuhip_eltwise_add_i8(tpuhip_ctx *ctx, const void *const *xs, int nin,
   a.n16 = (int64_t)(bytes / 16);
   const dim3 grid(grid_for(a.n16, kThreads * 2)), block(kThreads);
   switch (nin) {
-    case 1: hipLaunchKernelGGL(eltwise_add_kernel<1>, grid, block, 0, ctx->stream, a); break;
-    case 2: hipLaunchKernelGGL(eltwise_add_kernel<2>, grid, block, 0, ctx->stream, a); break;
-    case 3: hipLaunchKernelGGL(eltwise_add_kernel<3>, grid, block, 0, ctx->stream, a); break;
-    case 4: hipLaunchKernelGGL(eltwise_add_kernel<4>, grid, block, 0, ctx->stream, a); break;
-    case 5: hipLaunchKernelGGL(eltwise_add_kernel<5>, grid, block, 0, ctx->stream, a); break;
-    case 6: hipLaunchKernelGGL(eltwise_add_kernel<6>, grid, block, 0, ctx->stream, a); break;
-    case 7: hipLaunchKernelGGL(eltwise_add_kernel<7>, grid, block, 0, ctx->stream, a); break;
-    default: hipLaunchKernelGGL(eltwise_add_kernel<8>, grid, block, 0, ctx->stream, a); break;
+    case 1: launch(ctx, eltwise_add_kernel<1>, grid, block, a); break;
+    case 2: launch(ctx, eltwise_add_kernel<2>, grid, block, a); break;
+    case 3: launch(ctx, eltwise_add_kernel<3>, grid, block, a); break;
+    case 4: launch(ctx, eltwise_add_kernel<4>, grid, block, a); break;
+    case 5: launch(ctx, eltwise_add_kernel<5>, grid, block, a); break;
+    case 6: launch(ctx, eltwise_add_kernel<6>, grid, block, a); break;
+    case 7: launch(ctx, eltwise_add_kernel<7>, grid, block, a); break;
+    default: launch(ctx, eltwise_add_kernel<8>, grid, block, a); break;
   }
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
@@ -422,8 +418,7 @@ int tpuhip_relu_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t bytes) {
   TPUHIP_REQUIRE(bytes % 16 == 0, "relu: byte count %zu not a multiple of 16", bytes);
   if (bytes == 0) return TPUHIP_OK;
   const int64_t n16 = (int64_t)(bytes / 16);
-  hipLaunchKernelGGL(relu_kernel, dim3(grid_for(n16, kThreads * 2)), dim3(kThreads), 0,
-                     ctx->stream, (const v4i *)x, (v4i *)y, n16);
+  launch(ctx, relu_kernel, dim3(grid_for(n16, kThreads * 2)), dim3(kThreads), (const v4i *)x, (v4i *)y, n16);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -437,8 +432,7 @@ int tpuhip_upsample_nearest_i8(tpuhip_ctx *ctx, const void *x, void *y, int n, i
                  "upsample: bad channel strides %d / %d for %d channels", x_cs, y_cs, c);
   const int c16 = (c + 15) / 16;
   const int64_t total = (int64_t)n * ih * scale_h * iw * scale_w * c16;
-  hipLaunchKernelGGL(upsample_kernel, dim3(grid_for(total, kThreads * 2)), dim3(kThreads), 0,
-                     ctx->stream, (const int8_t *)x, (int8_t *)y, n, ih, iw, scale_h, scale_w, c16,
+  launch(ctx, upsample_kernel, dim3(grid_for(total, kThreads * 2)), dim3(kThreads), (const int8_t *)x, (int8_t *)y, n, ih, iw, scale_h, scale_w, c16,
                      x_cs, y_cs);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
@@ -509,8 +503,7 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
   if (axis == 1 && Cc % 16 != 0) {
     const int c1 = std::min(round_up(Cc, 16), y_cs);
     const int64_t total = (int64_t)N * H * W * (c1 - Cc);
-    hipLaunchKernelGGL(zero_channels_kernel, dim3(grid_for(total)), dim3(kThreads), 0, ctx->stream,
-                       (int8_t *)y, (int64_t)N * H * W, y_cs, Cc, c1);
+    launch(ctx, zero_channels_kernel, dim3(grid_for(total)), dim3(kThreads), (int8_t *)y, (int64_t)N * H * W, y_cs, Cc, c1);
     TPUHIP_CHECK_HIP(hipGetLastError());
   }
   return TPUHIP_OK;

@@ -320,7 +320,37 @@ Conv2DOpKernel::~Conv2DOpKernel() {
 }
 
 void Conv2DOpKernel::invoke() {
-  ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+  if (fused.enable)
+    ck(tpuhip_conv2d_add_i8(ctx, packed, input_data->data(), output_data->data(), add_src->data(),
+                            add_dst->data(), &fused),
+       name.c_str());
+  else
+    ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+}
+
+bool Conv2DOpKernel::can_fuse_add() const {
+  return std::string(tpuhip_conv2d_algo_name(packed)).rfind("mfma", 0) == 0;
+}
+
+void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift,
+                              bool relu) {
+  if (!src || !dst || src->slot_bytes() != output_data->slot_bytes() ||
+      dst->slot_bytes() != output_data->slot_bytes() || src->cs != output_data->cs ||
+      dst->cs != output_data->cs)
+    fail("Conv2D '" + name + "': fused add operands must match the conv result's shape");
+  add_src = src;
+  add_dst = dst;
+  fused.enable = 1;
+  fused.m_src = m_src;
+  fused.m_conv = m_conv;
+  fused.rshift = rshift;
+  fused.do_relu = relu ? 1 : 0;
+}
+
+void Conv2DOpKernel::clear_fusion() {
+  fused = tpuhip_fused_add{};
+  add_src.reset();
+  add_dst.reset();
 }
 
 const char *Conv2DOpKernel::algo_name() const { return tpuhip_conv2d_algo_name(packed); }
@@ -409,6 +439,7 @@ EltwiseAddOpKernel::EltwiseAddOpKernel(OpDesc &op, value_map_t &valueMapping,
 }
 
 void EltwiseAddOpKernel::invoke() {
+  if (fused_into_producer) return;   // the producing conv wrote this result already
   std::vector<const void *> ptrs;
   for (auto &t : inputs_data) ptrs.push_back(t->data());
   ck(tpuhip_eltwise_add_i8(ctx, ptrs.data(), (int)ptrs.size(), multiplier.data(), rshift,

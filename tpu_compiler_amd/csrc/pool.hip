@@ -146,7 +146,7 @@ int tpuhip_pool_max_i8(tpuhip_ctx *ctx, const tpuhip_pool_desc *d, const void *x
   TPUHIP_REQUIRE(ctx, "pool_max: NULL context");
   PoolArgs a;
   if (int rc = fill_args(d, x, y, &a)) return rc;
-  hipLaunchKernelGGL(pool_max_kernel, dim3(blocks_for(a)), dim3(256), 0, ctx->stream, a);
+  launch(ctx, pool_max_kernel, dim3(blocks_for(a)), dim3(256), a);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -160,7 +160,7 @@ int tpuhip_pool_avg_i8(tpuhip_ctx *ctx, const tpuhip_pool_desc *d, const void *x
   TPUHIP_REQUIRE((int64_t)d->kh * d->kw * 128 < (1 << 24), "pool_avg: window too large");
   a.mult = (float)multiplier;
   a.inv_pot = 1.0f / (float)(1 << rshift);
-  hipLaunchKernelGGL(pool_avg_kernel, dim3(blocks_for(a)), dim3(256), 0, ctx->stream, a);
+  launch(ctx, pool_avg_kernel, dim3(blocks_for(a)), dim3(256), a);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
