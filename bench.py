@@ -70,9 +70,11 @@ def main():
     graph_fn = graphs.CONFIGS[args.config]
     g = graph_fn()
     batch = g.input_op().shape[0]
-    tile_names = ["mfma_128x256", "mfma_64x256", "mfma_64x512", "mfma_32x256", "mfma_128x128",
-                  "mfma_64x128", "mfma_64x64"]
     if args.tiles:
+        from tpu_compiler_amd import capi
+        tile_names = []
+        while capi.bind().tpuhip_conv2d_tile_name(len(tile_names)):
+            tile_names.append(capi.bind().tpuhip_conv2d_tile_name(len(tile_names)).decode())
         for name, algo in json.load(open(args.tiles)).items():
             if algo in tile_names:
                 g.by_name[name].attrs["algo"] = 16 + tile_names.index(algo)

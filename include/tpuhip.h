@@ -146,6 +146,8 @@ int tpuhip_conv2d_add_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
                          const void *add_src, void *add_out, const tpuhip_fused_add *f);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
+/* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */
+const char *tpuhip_conv2d_tile_name(int tile);
 
 /* ---- FullyConnected ----------------------------------------------------- */
 

@@ -78,11 +78,13 @@ TILE_CASES = [
     (1, 40, 9, 9, 72, 3, 3, (2, 2), (1, 1, 1, 1), (1, 1), True),
     (3, 16, 5, 5, 16, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),      # one K step, tiny
     (1, 256, 6, 6, 300, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),     # 36 K steps
+    (2, 3, 20, 23, 40, 7, 7, (2, 2), (3, 3, 3, 3), (1, 1), True),      # 3 channels: 4-tap K packing
+    (1, 4, 11, 9, 24, 3, 3, (1, 1), (1, 1, 1, 1), (2, 1), False),
 ]
 
 
 @pytest.mark.parametrize("case", TILE_CASES)
-@pytest.mark.parametrize("tile", range(12))
+@pytest.mark.parametrize("tile", range(32))
 def test_conv_every_mfma_tile_variant(ctx, case, tile):
     n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
     rng = np.random.default_rng(ic * 7 + oc + tile)

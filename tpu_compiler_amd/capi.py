@@ -59,6 +59,7 @@ PROTOTYPES = {
     "tpuhip_conv2d_weights_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_conv2d_i8": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_conv2d_algo_name": (C.c_char_p, [C.c_void_p]),
+    "tpuhip_conv2d_tile_name": (C.c_char_p, [C.c_int]),
     "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,

@@ -38,6 +38,7 @@ struct tpuhip_conv_weights {
   int algo = ALGO_DIRECT;
   int tile = 0;          // MFMA tile variant
   int fast = 0;          // the overflow-free requant form is provably exact for this layer
+  bool smallc = false;   // ic <= 4: K packs 4 taps x 4 channels per 16-byte group (LDS kernels only)
   bool tuned = true;     // false: the tile is chosen by timing the candidates on first use
   std::vector<int8_t> host_filter;  // OIHW copy, kept while the layer can still be repacked
   int8_t *w = nullptr;   // packed filter
@@ -185,13 +186,13 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(ConvArgs a) {
 //
 // (icp = input channels rounded up to 16).  A workgroup of WM x WN waves owns a
 // tile of BM output channels x BN pixels; every wave owns (BM/WM) x (BN/WN) of it
-// as TM x TN blocks of 32x32 (v_mfma_i32_32x32x32_i8).  K is consumed 64 bytes per
+// as TM x TN blocks of 32x32 (v_mfma_i32_32x32x32_i8).  K is consumed BK bytes per
 // step.  Global loads run DEPTH steps ahead of the MFMAs in a ring of registers,
 // LDS is double-buffered, one barrier per step.
 //
-// LDS rows are 64 bytes (4 chunks of 16); the chunk index is XOR-swizzled with
-// (row >> 2) & 3 so that both the 16-byte stores of the loader and the 16-byte
-// fragment reads spread over all banks.
+// LDS rows are BK bytes (BK/16 chunks of 16); the chunk index is XOR-swizzled with
+// row bits chosen so that 16 consecutive rows of one chunk cover 256 distinct
+// bytes of bank space, for the loader's 16-byte stores and the fragment reads alike.
 //
 // The rows of a weight tile are stored permuted (see mfma_row_to_oc) so that in
 // the 32x32 result layout -- lane l holds column l & 31 and rows
@@ -291,6 +292,12 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
+// how a K group maps to filter taps (see load_tile)
+constexpr int kModeGeneral = 0;   // per-lane tap arithmetic
+constexpr int kModeUniform = 1;   // ic % (BK) == 0: all groups of a step in one tap, scalar arithmetic
+constexpr int kModeSmallC = 2;    // ic <= 4: four taps per 16-byte group
+
+
 // 16-byte load through a buffer descriptor: an offset at or beyond the
 // descriptor's size yields zeros, which is how padding taps, pixels past the end
 // of the tensor and K steps past the end of the filter are fed to the MFMAs
@@ -302,19 +309,26 @@ constexpr uint32_t kOobOffset = 0x7fffffffu;
 
 // UNI: the input channel count is a multiple of 64, so the four 16-byte K groups of
 // a step lie in one filter tap and all tap arithmetic is wave-uniform (scalar).
-template <int BM, int BN, int WM, int WN, int DEPTH, bool FAST, bool UNI>
-__global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
+// OCC: waves per SIMD the register allocation must allow (0 = whatever it takes)
+template <int BM, int BN, int WM, int WN, int BK, int DEPTH, int OCC, bool FAST, int MODE>
+__global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC > 0 ? OCC : 1))) void
+conv_mfma_kernel(ConvArgs a) {
+  constexpr bool UNI = MODE == kModeUniform;
+  constexpr bool SMALLC = MODE == kModeSmallC;
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32;  // 32x32 blocks per wave along oc
   constexpr int TN = BN / WN / 32;  // 32x32 blocks per wave along pixels
   static_assert(TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
-  constexpr int RP = NT / 4;                 // tile rows fetched per pass of the workgroup
+  constexpr int CH = BK / 16;                // 16-byte chunks per tile row (K bytes per step / 16)
+  constexpr int SW = CH == 4 ? 2 : CH == 8 ? 1 : 0;   // swizzle: chunk ^= (row >> SW) & (CH - 1)
+  static_assert(BK == 64 || BK == 128 || BK == 256, "K bytes per step");
+  constexpr int RP = NT / CH;                // tile rows fetched per pass of the workgroup
   constexpr int NW = (BM + RP - 1) / RP;     // 16-byte weight chunks per thread per step
   constexpr int NX = BN / RP;                // 16-byte activation chunks per thread per step
   static_assert(BN % RP == 0, "pixel tile must be a multiple of the loader pass");
-  static_assert(DEPTH == 2 || DEPTH == 4, "register ring depth");
+  static_assert(DEPTH % 2 == 0 && DEPTH >= 2 && DEPTH <= 12, "register ring depth");
 
-  __shared__ v4i lds[2][(BM + BN) * 4];
+  __shared__ v4i lds[2][(BM + BN) * CH];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -335,8 +349,8 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
 
   // ---- loader state: this thread fetches K-chunk kc of rows lrow + RP*s
-  const int kc = tid & 3;
-  const int lrow = tid >> 2;
+  const int kc = tid % CH;
+  const int lrow = tid / CH;
   int poff[NX];     // byte offset of (n, oh*sh - pt, ow*sw - pl, kc*16) in x (may lie before the image)
   int ih0[NX], iw0[NX];
   // (n, oh, ow) of the tile's first pixel: one generic division per workgroup ...
@@ -371,7 +385,7 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
   }
 
   v4i wreg[DEPTH][NW], xreg[DEPTH][NX];
-  const int nsteps = a.kp / 64;
+  const int nsteps = a.kp / BK;
 
   // fetch the tile of K step `step` into ring slot `slot`; no branches, no state.
   // A 16-byte K group kg = tap * c16 + cgrp with tap = tkh * kw + tkw; the divisions
@@ -381,9 +395,29 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
 #pragma unroll
     for (int s = 0; s < NW; ++s)
       wreg[slot][s] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
-          wrsrc, in_k ? woff[s] : kOobOffset, step * 64, 0);
-    if (UNI) {
-      const uint32_t kg0 = (uint32_t)(step * 4);
+          wrsrc, in_k ? woff[s] : kOobOffset, step * BK, 0);
+    if (SMALLC) {
+      // at most 4 input channels: a 16-byte K group is 4 filter taps x 4 channels, each
+      // tap one dword of its own pixel (K index = tap * 4 + c)
+      const int taps = a.kh * a.kw;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const uint32_t tap = (uint32_t)((step * CH + kc) * 4 + t);
+        const int tkh = (int)((tap * a.magic_kw) >> 20);
+        const int tkw = (int)tap - tkh * a.kw;
+        const int dh_off = (int)tap < taps ? tkh * a.dh : (1 << 28);
+        const int dw_off = tkw * a.dw;
+        const int tap_off = (dh_off * a.iw + dw_off) * a.x_cs;
+#pragma unroll
+        for (int s = 0; s < NX; ++s) {
+          const int ih = ih0[s] + dh_off, iw = iw0[s] + dw_off;
+          const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+          xreg[slot][s][t] = (int)__builtin_amdgcn_raw_buffer_load_b32(
+              xrsrc, ok ? (uint32_t)(poff[s] + tap_off) : kOobOffset, 0, 0);
+        }
+      }
+    } else if (UNI) {
+      const uint32_t kg0 = (uint32_t)(step * CH);
       const uint32_t tap = (kg0 * a.magic_c16) >> 20;
       const int cgrp0 = (int)(kg0 - tap * (uint32_t)a.c16);
       const int tkh = (int)((tap * a.magic_kw) >> 20);
@@ -399,7 +433,7 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
         xreg[slot][s] = buffer_load16(xrsrc, ok ? (uint32_t)(poff[s] + tap_off) : kOobOffset);
       }
     } else {
-      const uint32_t kg = (uint32_t)(step * 4 + kc);
+      const uint32_t kg = (uint32_t)(step * CH + kc);
       const uint32_t tap = (kg * a.magic_c16) >> 20;
       const int cgrp = (int)(kg - tap * (uint32_t)a.c16);
       const int tkh = (int)((tap * a.magic_kw) >> 20);
@@ -421,12 +455,12 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
 #pragma unroll
     for (int s = 0; s < NW; ++s) {
       const int r = lrow + RP * s;
-      if (BM % RP == 0 || r < BM) base[r * 4 + (kc ^ ((r >> 2) & 3))] = wreg[slot][s];
+      if (BM % RP == 0 || r < BM) base[r * CH + (kc ^ ((r >> SW) & (CH - 1)))] = wreg[slot][s];
     }
 #pragma unroll
     for (int s = 0; s < NX; ++s) {
       const int r = lrow + RP * s;
-      base[(BM + r) * 4 + (kc ^ ((r >> 2) & 3))] = xreg[slot][s];
+      base[(BM + r) * CH + (kc ^ ((r >> SW) & (CH - 1)))] = xreg[slot][s];
     }
   };
 
@@ -457,30 +491,50 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
   store_tile(0, 0);
   __syncthreads();
 
-  auto compute = [&](int buf) {
+  // MFMA fragments are double-buffered in registers: while the MFMAs of one 32-byte K
+  // slice run, the LDS reads of the next slice, the LDS writes of the next tile and the
+  // global loads of a later tile are issued in their shadow.  The first slice of a step
+  // is read right after the barrier that publishes its tile.
+  constexpr int KK = BK / 32;
+  v4i fa[2][TM], fb[2][TN];
+  auto read_frag = [&](int buf, int kk, int fs) {
     const v4i *wl = lds[buf];
-    const v4i *xl = lds[buf] + BM * 4;
+    const v4i *xl = lds[buf] + BM * CH;
+    const int chunk = kk * 2 + fk;
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      const int chunk = kk * 2 + fk;
-      v4i af[TM], bf[TN];
+    for (int i = 0; i < TM; ++i) {
+      const int r = (wm * TM + i) * 32 + frow;
+      fa[fs][i] = wl[r * CH + (chunk ^ ((r >> SW) & (CH - 1)))];
+    }
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int r = (wm * TM + i) * 32 + frow;
-        af[i] = wl[r * 4 + (chunk ^ ((r >> 2) & 3))];
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int r = (wn * TN + j) * 32 + frow;
-        bf[j] = xl[r * 4 + (chunk ^ ((r >> 2) & 3))];
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+    for (int j = 0; j < TN; ++j) {
+      const int r = (wn * TN + j) * 32 + frow;
+      fb[fs][j] = xl[r * CH + (chunk ^ ((r >> SW) & (CH - 1)))];
     }
   };
+  auto mfma_frag = [&](int fs) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[fs][i], fb[fs][j], acc[i][j], 0, 0, 0);
+  };
+  // one K step on LDS buffer d & 1; ring slot (d + 1) % DEPTH holds the next tile
+  auto step_body = [&](int d) {
+    const int buf = d & 1;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) read_frag(buf, kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_frag(kk & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk == 0) store_tile((d + 1) % DEPTH, buf ^ 1);
+    }
+    __syncthreads();
+    read_frag(buf ^ 1, 0, 0);
+  };
+  read_frag(0, 0, 0);
+
   // Whole groups of DEPTH steps: ring slots and LDS buffers are compile-time indices
   // (DEPTH is even, so buffer parity == slot parity) and the body has no branch.
   const int full = nsteps / DEPTH;
@@ -490,21 +544,14 @@ __global__ __launch_bounds__(WM *WN * 64) void conv_mfma_kernel(ConvArgs a) {
     for (int d = 0; d < DEPTH; ++d) {
       // slot d went to LDS one step ago: refill it with the tile DEPTH steps ahead
       load_tile(d, (g + 1) * DEPTH + d);
-      compute(d & 1);
-      store_tile((d + 1) % DEPTH, (d & 1) ^ 1);
-      __syncthreads();
+      step_body(d);
     }
   }
   // the last nsteps % DEPTH steps: their tiles are already in the ring / in LDS
   const int rem = nsteps - full * DEPTH;
 #pragma unroll
-  for (int d = 0; d < DEPTH - 1; ++d) {
-    if (d < rem) {
-      compute(d & 1);
-      store_tile((d + 1) % DEPTH, (d & 1) ^ 1);
-      __syncthreads();
-    }
-  }
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < rem) step_body(d);
 
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
@@ -677,6 +724,198 @@ conv_mfma_reg_kernel(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Split-K variant of the LDS-free kernel for layers with few output tiles and a
+// long K (late 3x3 and reduction 1x1 layers): the four waves of a workgroup share
+// one tile and take every fourth K step each, so four independent load -> MFMA
+// chains run per tile; the partial sums meet once in LDS.
+// ---------------------------------------------------------------------------
+template <int TM, int TN, int DEPTH, int OCC, bool FAST, bool UNI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+conv_mfma_splitk_kernel(ConvArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int logical_wg = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  const int wt = logical_wg;                   // the four waves share one tile and split K
+  if (wt >= a.n_tiles) return;                 // uniform over the workgroup
+  const int pix_tile = wt / a.n_oc_tiles;
+  const int oc_tile = wt - pix_tile * a.n_oc_tiles;
+  const int oc0 = oc_tile * (TM * 32);
+  const int pix0 = pix_tile * (TN * 32);
+
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  const int nsteps_all = a.kp / 64;
+  // wave w takes K steps w, w + 4, w + 8, ...
+  const int nsteps = (nsteps_all - wave + 3) / 4;
+
+  int poff[TN], ih0[TN], iw0[TN];
+  const int ow_first = pix0 % a.ow;
+  const int t_first = pix0 / a.ow;
+  const int oh_first = t_first % a.oh;
+  const int n_first = t_first / a.oh;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int delta = j * 32 + frow;
+    const bool pv = pix0 + delta < a.npix;
+    const uint32_t t1 = (uint32_t)(ow_first + delta);
+    const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
+    const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
+    const uint32_t t2 = (uint32_t)oh_first + q1;
+    const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
+    const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
+    const int n = n_first + (int)q2;
+    ih0[j] = pv ? oh * a.sh - a.pt : -(1 << 28);
+    iw0[j] = ow * a.sw - a.pl;
+    poff[j] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[j]) * a.x_cs + (UNI ? fk * 16 : 0);
+    asm volatile("" : "+v"(poff[j]), "+v"(ih0[j]), "+v"(iw0[j]));
+  }
+  // weight fragments: [oc block of 32][K step][kk][lane] x 16 bytes
+  uint32_t woff[TM];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    woff[i] = (uint32_t)(((oc0 / 32 + i) * nsteps_all) * 2048 + lane * 16);
+    asm volatile("" : "+v"(woff[i]));
+  }
+
+  v4i af[DEPTH][2][TM], bf[DEPTH][2][TN];
+
+  auto load_step = [&](int slot, int local_step) {
+    const int step = local_step * 4 + wave;
+    const bool in_k = step < nsteps_all;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[slot][kk][i] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+            wrsrc, in_k ? woff[i] : kOobOffset, step * 2048 + kk * 1024, 0);
+    if (UNI) {
+      const uint32_t kg0 = (uint32_t)(step * 4);
+      const uint32_t tap = (kg0 * a.magic_c16) >> 20;
+      const int cgrp0 = (int)(kg0 - tap * (uint32_t)a.c16);
+      const int tkh = (int)((tap * a.magic_kw) >> 20);
+      const int tkw = (int)tap - tkh * a.kw;
+      const int dh_off = (int)kg0 < a.k16 ? tkh * a.dh : (1 << 28);
+      const int dw_off = tkw * a.dw;
+      const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp0 * 16;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int ih = ih0[j] + dh_off, iw = iw0[j] + dw_off;
+        const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+        const uint32_t off = ok ? (uint32_t)(poff[j] + tap_off) : kOobOffset;
+        bf[slot][0][j] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 0, 0);
+        bf[slot][1][j] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 32, 0);
+      }
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const uint32_t kg = (uint32_t)(step * 4 + kk * 2 + fk);
+        const uint32_t tap = (kg * a.magic_c16) >> 20;
+        const int cgrp = (int)(kg - tap * (uint32_t)a.c16);
+        const int tkh = (int)((tap * a.magic_kw) >> 20);
+        const int tkw = (int)tap - tkh * a.kw;
+        const int dh_off = (int)kg < a.k16 ? tkh * a.dh : (1 << 28);
+        const int dw_off = tkw * a.dw;
+        const int tap_off = (tkh * a.dh * a.iw + dw_off) * a.x_cs + cgrp * 16;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int ih = ih0[j] + dh_off, iw = iw0[j] + dw_off;
+          const bool ok = ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+          bf[slot][kk][j] = buffer_load16(xrsrc, ok ? (uint32_t)(poff[j] + tap_off) : kOobOffset);
+        }
+      }
+    }
+  };
+
+  v16i acc[TM][TN];
+  const int ocw0 = oc0 + fk * 16 * TM;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v4i b = bp[q];
+      if (wave != 0) b = v4i{0, 0, 0, 0};
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j][q * 4 + 0] = b[0];
+        acc[i][j][q * 4 + 1] = b[1];
+        acc[i][j][q * 4 + 2] = b[2];
+        acc[i][j][q * 4 + 3] = b[3];
+      }
+    }
+  }
+
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
+
+  auto mfma_step = [&](int slot) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[slot][kk][i], bf[slot][kk][j],
+                                                            acc[i][j], 0, 0, 0);
+  };
+  // whole groups of DEPTH steps: branch-free body, ring slots are compile-time indices
+  const int full = nsteps / DEPTH;
+#pragma nounroll
+  for (int g = 0; g < full; ++g) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      mfma_step(d);
+      load_step(d, (g + 1) * DEPTH + d);
+    }
+  }
+  // the last nsteps % DEPTH steps are already in the ring
+  const int rem = nsteps - full * DEPTH;
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < rem) mfma_step(d);
+
+  // reduce the four partial sums through LDS: block b = i * TN + j is summed and
+  // finished (requantised, stored) by wave b % 4
+  constexpr int NB = TM * TN;
+  __shared__ v4i part[4 * NB * 4 * 64];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v4i v = {acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                 acc[i][j][q * 4 + 3]};
+        part[((wave * NB + i * TN + j) * 4 + q) * 64 + lane] = v;
+      }
+  __syncthreads();
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if ((b & 3) != wave) continue;
+    const int i = b / TN, j = b % TN;
+    v16i sum[1];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      v4i t = part[((0 * NB + b) * 4 + q) * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) t += part[((w * NB + b) * 4 + q) * 64 + lane];
+      sum[0][q * 4 + 0] = t[0];
+      sum[0][q * 4 + 1] = t[1];
+      sum[0][q * 4 + 2] = t[2];
+      sum[0][q * 4 + 3] = t[3];
+    }
+    const int oc = ocw0 + i * 16;
+    if (oc < a.ocw) epilogue_rows<1, FAST>(sum, a, oc, pix0 + j * 32 + frow, 32);
+  }
+}
+
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 namespace {
@@ -684,7 +923,8 @@ namespace {
 struct TileCfg {
   int bm, bn, wm, wn;
   const char *name;
-  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave
+  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave; 2: its split-K form
+  int bk;    // K bytes per step (0 = 64)
 };
 // wave tile = (bm/wm) x (bn/wn)
 const TileCfg kTiles[] = {
@@ -700,24 +940,66 @@ const TileCfg kTiles[] = {
     {64, 128, 1, 1, "mfma_reg_64x128", 1},  // 9
     {32, 32, 1, 1, "mfma_reg_32x32", 1},    // 10
     {64, 32, 1, 1, "mfma_reg_64x32", 1},    // 11
+    {64, 64, 2, 2, "mfma_64x64_k128", 0, 128},     // 12
+    {64, 64, 2, 2, "mfma_64x64_k256", 0, 256},     // 13
+    {64, 128, 2, 2, "mfma_64x128_k128", 0, 128},   // 14
+    {128, 128, 2, 2, "mfma_128x128_k128", 0, 128}, // 15
+    {64, 256, 1, 4, "mfma_64x256_k128", 0, 128},   // 16
+    {64, 64, 2, 2, "mfma_64x64_d8", 0, 64},        // 17: ring of 8 steps
+    {64, 128, 2, 2, "mfma_64x128_d8", 0, 64},      // 18
+    {64, 64, 2, 2, "mfma_64x64_k128_d6", 0, 128},  // 19
+    {128, 128, 2, 2, "mfma_128x128_d8", 0, 64},    // 20
+    {64, 64, 2, 2, "mfma_64x64_d12", 0, 64},       // 21
+    {64, 64, 1, 1, "mfma_splitk_64x64", 2},        // 22: one tile per workgroup, K split over 4 waves
+    {32, 64, 1, 1, "mfma_splitk_32x64", 2},        // 23
+    {32, 32, 1, 1, "mfma_splitk_32x32", 2},        // 24
+    {64, 32, 1, 1, "mfma_splitk_64x32", 2},        // 25
+    {64, 128, 2, 2, "mfma_64x128_o4", 0, 64},      // 26: 4 waves per SIMD
+    {64, 64, 2, 2, "mfma_64x64_o6", 0, 64},        // 27: 6 waves per SIMD
+    {128, 128, 2, 2, "mfma_128x128_o3", 0, 64},    // 28
+    {64, 256, 1, 4, "mfma_64x256_o3", 0, 64},      // 29
+    {32, 256, 1, 4, "mfma_32x256_o4", 0, 64},      // 30
+    {128, 256, 2, 2, "mfma_128x256_o2", 0, 64},    // 31
 };
+inline int tile_bk(const TileCfg &t) { return t.bk ? t.bk : 64; }
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
-template <bool FAST, bool UNI>
+template <bool FAST, int MODE>
 void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
+  constexpr bool UNI = MODE == kModeUniform;
   switch (tile) {
-    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 2, FAST, UNI>), grid, dim3(256), a); break;
-    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
-    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
-    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
-    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
-    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
-    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 64, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
     case 7: launch(ctx, (conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
     case 8: launch(ctx, (conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
     case 9: launch(ctx, (conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), a); break;
     case 10: launch(ctx, (conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), a); break;
-    default: launch(ctx, (conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
+    case 11: launch(ctx, (conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
+    case 12: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 13: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 256, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 14: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 15: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 16: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 17: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 18: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 19: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 6, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 20: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 21: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 12, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 22: launch(ctx, (conv_mfma_splitk_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
+    case 23: launch(ctx, (conv_mfma_splitk_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
+    case 24: launch(ctx, (conv_mfma_splitk_kernel<1, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
+    case 25: launch(ctx, (conv_mfma_splitk_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
+    case 26: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 4, FAST, MODE>), grid, dim3(256), a); break;
+    case 27: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 6, FAST, MODE>), grid, dim3(256), a); break;
+    case 28: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 3, FAST, MODE>), grid, dim3(256), a); break;
+    case 29: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 3, FAST, MODE>), grid, dim3(256), a); break;
+    case 30: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 4, FAST, MODE>), grid, dim3(256), a); break;
+    default: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 2, FAST, MODE>), grid, dim3(256), a); break;
   }
 }
 
@@ -731,7 +1013,7 @@ int pick_tile(const tpuhip_conv_desc &d, int k16, int num_cu) {
   int best_tile = 1;
   for (int t = 0; t < kNumTiles; ++t) {
     const TileCfg &c = kTiles[t];
-    if (c.reg) continue;
+    if (c.reg || c.bk || t > 6) continue;
     if (c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32)) continue;   // more than half the rows idle
     const int tm = c.bm / c.wm / 32, tn = c.bn / c.wn / 32;
     const int64_t wgs = ceil_div64(npix, c.bn) * ceil_div64(d.oc, c.bm);
@@ -784,6 +1066,10 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
   const int tm = t.bm / t.wm / 32;
   const int icp = round_up(d.ic, 16);
   const int ocp = round_up(d.oc, t.bm);
+  cw->smallc = d.ic <= 4 && !t.reg;
+  cw->c16 = icp / 16;
+  cw->k16 = cw->smallc ? (d.kh * d.kw * 4 + 15) / 16 : d.kh * d.kw * cw->c16;
+  cw->kp = round_up(cw->k16 * 16, tile_bk(t));
   std::vector<int8_t> packed((size_t)ocp * cw->kp, 0);
   const int8_t *filter = cw->host_filter.data();
   std::vector<int8_t> rowbuf((size_t)cw->kp);
@@ -794,9 +1080,10 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
     if (oc >= d.oc) continue;
     std::fill(rowbuf.begin(), rowbuf.end(), 0);
     const int8_t *src = filter + (size_t)oc * d.ic * d.kh * d.kw;
+    const int kstride = cw->smallc ? 4 : icp;   // channels per tap in the K order
     for (int c = 0; c < d.ic; ++c)
       for (int k = 0; k < d.kh * d.kw; ++k)
-        rowbuf[(size_t)k * icp + c] = src[(size_t)c * d.kh * d.kw + k];
+        rowbuf[(size_t)k * kstride + c] = src[(size_t)c * d.kh * d.kw + k];
     if (!t.reg) {
       memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
     } else {
@@ -823,6 +1110,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 
 bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
+  if (d.ic <= 4 && c.reg) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
 
@@ -858,7 +1146,7 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
     a.n_oc_tiles = w->ocp / t.bm;
     a.n_tiles = (int)(ceil_div64(a.npix, t.bn) * a.n_oc_tiles);
     // workgroups per XCD (a workgroup of the LDS-free kernel holds four wave tiles)
-    const int n_wgs = t.reg ? (a.n_tiles + 3) / 4 : a.n_tiles;
+    const int n_wgs = t.reg == 1 ? (a.n_tiles + 3) / 4 : a.n_tiles;
     a.tiles_per_xcd = (n_wgs + 7) / 8;
   }
   *out = a;
@@ -866,15 +1154,21 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
 
 void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvArgs &a) {
   dim3 grid((unsigned)(a.tiles_per_xcd * 8));
-  const bool uni = (w->c16 % 4) == 0;
-  if (w->fast && uni)
-    launch_mfma<true, true>(ctx, w->tile, grid, a);
-  else if (w->fast)
-    launch_mfma<true, false>(ctx, w->tile, grid, a);
-  else if (uni)
-    launch_mfma<false, true>(ctx, w->tile, grid, a);
-  else
-    launch_mfma<false, false>(ctx, w->tile, grid, a);
+  const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
+  if (w->smallc) {
+    if (w->fast)
+      launch_mfma<true, kModeSmallC>(ctx, w->tile, grid, a);
+    else
+      launch_mfma<false, kModeSmallC>(ctx, w->tile, grid, a);
+  } else if (w->fast && uni) {
+    launch_mfma<true, kModeUniform>(ctx, w->tile, grid, a);
+  } else if (w->fast) {
+    launch_mfma<true, kModeGeneral>(ctx, w->tile, grid, a);
+  } else if (uni) {
+    launch_mfma<false, kModeUniform>(ctx, w->tile, grid, a);
+  } else {
+    launch_mfma<false, kModeGeneral>(ctx, w->tile, grid, a);
+  }
 }
 
 // Times every candidate tile on the layer's real buffers (the kernels are
@@ -948,8 +1242,8 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   // the MFMA kernel locates a K group with multiply-shift divisions that are exact
   // for at most 4094 groups of at most 256 16-channel groups each
   const bool mfma_ok = dense && round_up(d.ic, 16) / 16 <= 256 &&
-                       (int64_t)d.kh * d.kw * (round_up(d.ic, 16) / 16) + 16 < 4095 &&
-                       (int64_t)round_up(d.oc, 128) * (d.kh * d.kw * round_up(d.ic, 16) + 64) <
+                       (int64_t)d.kh * d.kw * (round_up(d.ic, 16) / 16) + 128 < 4095 &&
+                       (int64_t)round_up(d.oc, 128) * (d.kh * d.kw * round_up(d.ic, 16) + 256) <
                            (1ll << 31);
   if (d.algo == ALGO_AUTO && algo == ALGO_MFMA && !mfma_ok) algo = ALGO_DIRECT;
   TPUHIP_REQUIRE(algo != ALGO_MFMA || mfma_ok,
@@ -963,10 +1257,8 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   std::vector<int8_t> packed;
   const size_t per_oc = (size_t)icg * d.kh * d.kw;
   if (algo == ALGO_MFMA) {
-    const int icp = round_up(d.ic, 16);
-    cw->c16 = icp / 16;
-    cw->k16 = d.kh * d.kw * cw->c16;
-    cw->kp = round_up(cw->k16 * 16, 64);
+    cw->c16 = round_up(d.ic, 16) / 16;
+    cw->k16 = d.kh * d.kw * cw->c16;   // refined per tile in pack_mfma_weights
     cw->host_filter.assign(filter, filter + (size_t)d.oc * per_oc);
     const int tile = forced_tile >= 0 ? forced_tile : pick_tile(d, cw->k16, ctx->num_cu);
     if (int rc = pack_mfma_weights(ctx, cw, tile)) {
@@ -1060,6 +1352,10 @@ int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w) {
   int rc4 = tpuhip_free(ctx, w->qplanes);
   delete w;
   return rc ? rc : rc2 ? rc2 : rc3 ? rc3 : rc4;
+}
+
+const char *tpuhip_conv2d_tile_name(int tile) {
+  return tile >= 0 && tile < kNumTiles ? kTiles[tile].name : nullptr;
 }
 
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {

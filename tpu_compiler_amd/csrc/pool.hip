@@ -111,6 +111,59 @@ __global__ __launch_bounds__(256) void pool_avg_kernel(PoolArgs a) {
   }
 }
 
+// Global / large-window average pooling: LANES lanes share one (pixel, 16-channel
+// group) output, each sums every LANES-th window position, and the partial sums
+// meet through wave shuffles.  Keeps enough loads in flight when there are few
+// outputs (a 7x7 global pool has 49 taps per output and only n*c/16 outputs).
+template <int LANES>
+__global__ __launch_bounds__(256) void pool_avg_split_kernel(PoolArgs a) {
+  const int64_t total = (int64_t)a.n * a.oh * a.ow * a.c16;
+  const int64_t gid = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / LANES;
+  const int sub = threadIdx.x % LANES;
+  const bool live = gid < total;
+  const int64_t i = live ? gid : 0;
+  const int cg = (int)(i % a.c16);
+  int64_t p = i / a.c16;
+  const int ow = (int)(p % a.ow);
+  p /= a.ow;
+  const int oh = (int)(p % a.oh);
+  const int b = (int)(p / a.oh);
+  int32_t sum[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) sum[k] = 0;
+  const int taps = a.kh * a.kw;
+  for (int t = sub; t < taps; t += LANES) {
+    const int kh = t / a.kw, kw = t - kh * a.kw;
+    const int ih = oh * a.sh - a.pt + kh, iw = ow * a.sw - a.pl + kw;
+    if (ih < 0 || ih >= a.ih || iw < 0 || iw >= a.iw) continue;
+    const v4i v = *reinterpret_cast<const v4i *>(
+        a.x + ((int64_t)(b * a.ih + ih) * a.iw + iw) * a.x_cs + cg * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) sum[q * 4 + k] += sb(v[q], k);
+  }
+#pragma unroll
+  for (int k = 0; k < 16; ++k)
+#pragma unroll
+    for (int off = LANES / 2; off > 0; off >>= 1) sum[k] += __shfl_xor(sum[k], off, LANES);
+  if (live && sub == 0) {
+    v4i out;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t w = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float prod = __fmul_rn((float)sum[q * 4 + k], a.mult);
+        const float quo = __fmul_rn(prod, a.inv_pot);
+        w |= ((uint32_t)saturate_int8_f(quo) & 0xffu) << (8 * k);
+      }
+      out[q] = (int)w;
+    }
+    *reinterpret_cast<v4i *>(a.y + ((int64_t)(b * a.oh + oh) * a.ow + ow) * a.y_cs + cg * 16) = out;
+  }
+}
+
 int fill_args(const tpuhip_pool_desc *d, const void *x, void *y, PoolArgs *a) {
   TPUHIP_REQUIRE(d && x && y, "pool: NULL argument");
   TPUHIP_REQUIRE(d->n > 0 && d->c > 0 && d->ih > 0 && d->iw > 0 && d->oh > 0 && d->ow > 0 &&
@@ -160,7 +213,13 @@ int tpuhip_pool_avg_i8(tpuhip_ctx *ctx, const tpuhip_pool_desc *d, const void *x
   TPUHIP_REQUIRE((int64_t)d->kh * d->kw * 128 < (1 << 24), "pool_avg: window too large");
   a.mult = (float)multiplier;
   a.inv_pot = 1.0f / (float)(1 << rshift);
-  launch(ctx, pool_avg_kernel, dim3(blocks_for(a)), dim3(256), a);
+  const int64_t outputs = (int64_t)a.n * a.oh * a.ow * a.c16;
+  if (d->kh * d->kw >= 16 && outputs < (1 << 16)) {
+    const unsigned blocks = (unsigned)((outputs * 8 + 255) / 256);
+    launch(ctx, pool_avg_split_kernel<8>, dim3(blocks), dim3(256), a);
+  } else {
+    launch(ctx, pool_avg_kernel, dim3(blocks_for(a)), dim3(256), a);
+  }
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
