@@ -10,6 +10,14 @@ from tpu_compiler_amd import capi
 pytestmark = pytest.mark.gpu
 
 
+def capi_tile_name(t):
+    name = capi.bind().tpuhip_conv2d_tile_name(t)
+    return name.decode() if name else None
+
+
+NUM_TILES = next(t for t in range(1024) if capi_tile_name(t) is None)
+
+
 @pytest.fixture(scope="module")
 def ctx():
     c = capi.Context(0)
@@ -83,8 +91,38 @@ TILE_CASES = [
 ]
 
 
+# large enough that a persistent workgroup walks several pixel tiles
+WALK_CASES = [
+    (32, 64, 56, 56, 64, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), True),
+    (13, 24, 67, 61, 80, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), False),    # ragged rows, general K mode
+    (6, 3, 150, 131, 32, 5, 5, (2, 2), (2, 2, 2, 2), (1, 1), True),     # 3 channels
+]
+PERSISTENT_TILES = [t for t in range(64) if (capi_tile_name(t) or "").startswith("mfma_p_")]
+
+
+@pytest.mark.parametrize("case", WALK_CASES)
+@pytest.mark.parametrize("tile", PERSISTENT_TILES)
+def test_conv_persistent_tiles_walk(ctx, case, tile):
+    n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
+    rng = np.random.default_rng(ic * 11 + oc + tile)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=16 + tile, stride=stride, pads=pads,
+                         dil=dil, do_relu=relu)
+    assert name.startswith("mfma_p_")
+    assert np.array_equal(got, want), "%s: %d mismatches" % (name, (got != want).sum())
+    rsh0 = rsh.copy()
+    rsh0[0] = 0     # the general requant form of the same tile
+    want = oracle_conv(x, w, bias, rsh0, mult, 1, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh0, mult, algo=16 + tile, stride=stride, pads=pads,
+                         dil=dil, do_relu=relu)
+    assert np.array_equal(got, want), "%s (general requant): %d mismatches" % (name, (got != want).sum())
+
+
 @pytest.mark.parametrize("case", TILE_CASES)
-@pytest.mark.parametrize("tile", range(32))
+@pytest.mark.parametrize("tile", range(NUM_TILES))
 def test_conv_every_mfma_tile_variant(ctx, case, tile):
     n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
     rng = np.random.default_rng(ic * 7 + oc + tile)

@@ -68,6 +68,9 @@ struct ConvArgs {
   uint32_t x_bytes, w_bytes;      // sizes behind x and w (buffer descriptors)
   uint32_t magic_ow, magic_oh;    // ceil(2^32 / d): x / d == umulhi(x, magic) for x, d < 2^16
   int n_oc_tiles, n_tiles, tiles_per_xcd;
+  // persistent kernels: workgroups per XCD (a multiple of n_oc_tiles) and the pixel
+  // advance between two tiles of one workgroup, split into (n, oh, ow) parts
+  int wgs_per_xcd, pstep_pix, pstep_n, pstep_oh, pstep_ow;
   int npix;
   int lo;          // lower clamp bound: 0 with ReLU after saturation, else -128
   int relu_first;  // ReLU on the sum before requantisation (FC)
@@ -240,13 +243,15 @@ __device__ __forceinline__ int32_t requant_core(int32_t v, int32_t mult, int32_t
 // per pixel.  Parameters are read four channels at a time to keep few registers live.
 template <int TN, bool FAST>
 __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
-                                              int pix_first, int pix_stride) {
+                                              const int32_t *pmult, const int32_t *pshift,
+                                              const int32_t *phpot, int pix_first,
+                                              int pix_stride) {
   uint32_t outw[TN][4];
 #pragma unroll
   for (int qd = 0; qd < 4; ++qd) {
-    const v4i m4 = *reinterpret_cast<const v4i *>(a.qmult + oc + qd * 4);
-    const v4i r4 = *reinterpret_cast<const v4i *>(a.qshift + oc + qd * 4);
-    const v4i h4 = *reinterpret_cast<const v4i *>(a.qhpot + oc + qd * 4);
+    const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
+    const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
+    const v4i h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       int32_t v0 = acc[j][qd * 4 + 0], v1 = acc[j][qd * 4 + 1], v2 = acc[j][qd * 4 + 2],
@@ -309,8 +314,14 @@ constexpr uint32_t kOobOffset = 0x7fffffffu;
 
 // UNI: the input channel count is a multiple of 64, so the four 16-byte K groups of
 // a step lie in one filter tap and all tap arithmetic is wave-uniform (scalar).
-// OCC: waves per SIMD the register allocation must allow (0 = whatever it takes)
-template <int BM, int BN, int WM, int WN, int BK, int DEPTH, int OCC, bool FAST, int MODE>
+// OCC: waves per SIMD the register allocation must allow (0 = whatever it takes).
+// PERSIST: a workgroup walks several pixel tiles of one output-channel tile.  The
+// launch holds about as many workgroups as fit on the chip at once; the requant
+// parameters of the channel tile sit in LDS, and the first K tiles of the next
+// pixel tile are fetched before the epilogue of the current one, so the global
+// latency at the head of a tile hides behind the VALU work at the tail of the last.
+template <int BM, int BN, int WM, int WN, int BK, int DEPTH, int OCC, bool PERSIST, bool FAST,
+          int MODE>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC > 0 ? OCC : 1))) void
 conv_mfma_kernel(ConvArgs a) {
   constexpr bool UNI = MODE == kModeUniform;
@@ -329,6 +340,8 @@ conv_mfma_kernel(ConvArgs a) {
   static_assert(DEPTH % 2 == 0 && DEPTH >= 2 && DEPTH <= 12, "register ring depth");
 
   __shared__ v4i lds[2][(BM + BN) * CH];
+  // bias | multiplier | rshift | 2^(rshift-1) of the workgroup's BM channels
+  __shared__ __attribute__((aligned(16))) int32_t qlds[PERSIST ? 4 * BM : 4];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -337,16 +350,26 @@ conv_mfma_kernel(ConvArgs a) {
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run
   // of tiles, output-channel tiles of one pixel tile next to each other, so that the
   // workgroups sharing activations (and writing the same output rows) share an L2.
-  const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  int ltile = (int)(blockIdx.x >> 3);                                   // tile index inside the XCD's run
+  int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + ltile;
   if (logical >= a.n_tiles) return;
   const int pix_tile = logical / a.n_oc_tiles;
-  const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;
-  const int pix0 = pix_tile * BN;
+  const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;   // the same for every tile of a walk
+  int pix0 = pix_tile * BN;
 
   const __amdgpu_buffer_rsrc_t xrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t wrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  if (PERSIST) {
+    for (int t = tid; t < BM; t += NT) {
+      qlds[t] = a.bias[oc0 + t];
+      qlds[BM + t] = a.qmult[oc0 + t];
+      qlds[2 * BM + t] = a.qshift[oc0 + t];
+      qlds[3 * BM + t] = a.qhpot[oc0 + t];
+    }
+  }
 
   // ---- loader state: this thread fetches K-chunk kc of rows lrow + RP*s
   const int kc = tid % CH;
@@ -354,28 +377,31 @@ conv_mfma_kernel(ConvArgs a) {
   int poff[NX];     // byte offset of (n, oh*sh - pt, ow*sw - pl, kc*16) in x (may lie before the image)
   int ih0[NX], iw0[NX];
   // (n, oh, ow) of the tile's first pixel: one generic division per workgroup ...
-  const int ow_first = pix0 % a.ow;
+  int ow_first = pix0 % a.ow;
   const int t_first = pix0 / a.ow;
-  const int oh_first = t_first % a.oh;
-  const int n_first = t_first / a.oh;
+  int oh_first = t_first % a.oh;
+  int n_first = t_first / a.oh;
+  auto setup_rows = [&]() {
 #pragma unroll
-  for (int s = 0; s < NX; ++s) {
-    // ... and exact multiply-high divisions of small numbers per row
-    const int delta = lrow + RP * s;
-    const bool pv = pix0 + delta < a.npix;
-    const uint32_t t1 = (uint32_t)(ow_first + delta);
-    const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
-    const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
-    const uint32_t t2 = (uint32_t)oh_first + q1;
-    const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
-    const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
-    const int n = n_first + (int)q2;
-    ih0[s] = pv ? oh * a.sh - a.pt : -(1 << 28);   // an invalid pixel never passes the bounds test
-    iw0[s] = ow * a.sw - a.pl;
-    poff[s] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[s]) * a.x_cs + (UNI ? kc * 16 : 0);
-    // keep the three values in registers instead of recomputing them every K step
-    asm volatile("" : "+v"(poff[s]), "+v"(ih0[s]), "+v"(iw0[s]));
-  }
+    for (int s = 0; s < NX; ++s) {
+      // ... and exact multiply-high divisions of small numbers per row
+      const int delta = lrow + RP * s;
+      const bool pv = pix0 + delta < a.npix;
+      const uint32_t t1 = (uint32_t)(ow_first + delta);
+      const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
+      const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
+      const uint32_t t2 = (uint32_t)oh_first + q1;
+      const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
+      const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
+      const int n = n_first + (int)q2;
+      ih0[s] = pv ? oh * a.sh - a.pt : -(1 << 28);   // an invalid pixel never passes the bounds test
+      iw0[s] = ow * a.sw - a.pl;
+      poff[s] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[s]) * a.x_cs + (UNI ? kc * 16 : 0);
+      // keep the three values in registers instead of recomputing them every K step
+      asm volatile("" : "+v"(poff[s]), "+v"(ih0[s]), "+v"(iw0[s]));
+    }
+  };
+  setup_rows();
   uint32_t woff[NW];
 #pragma unroll
   for (int s = 0; s < NW; ++s) {
@@ -466,35 +492,10 @@ conv_mfma_kernel(ConvArgs a) {
 
   const int frow = lane & 31;   // row inside a 32-row block
   const int fk = lane >> 5;     // which 16-byte half of a 32-byte MFMA K slice
+  const int lch0 = wm * TM * 32 + fk * 16 * TM;   // first of this lane's 16*TM channels in the tile
+  const int ocw0 = oc0 + lch0;
 
-  // accumulators start from the bias (the int32 add of the epilogue commutes with the sum)
   v16i acc[TM][TN];
-  const int ocw0 = oc0 + wm * TM * 32 + fk * 16 * TM;   // first of this lane's 16*TM channels
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const v4i b = bp[q];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        acc[i][j][q * 4 + 0] = b[0];
-        acc[i][j][q * 4 + 1] = b[1];
-        acc[i][j][q * 4 + 2] = b[2];
-        acc[i][j][q * 4 + 3] = b[3];
-      }
-    }
-  }
-
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
-  store_tile(0, 0);
-  __syncthreads();
-
-  // MFMA fragments are double-buffered in registers: while the MFMAs of one 32-byte K
-  // slice run, the LDS reads of the next slice, the LDS writes of the next tile and the
-  // global loads of a later tile are issued in their shadow.  The first slice of a step
-  // is read right after the barrier that publishes its tile.
   constexpr int KK = BK / 32;
   v4i fa[2][TM], fb[2][TN];
   auto read_frag = [&](int buf, int kk, int fs) {
@@ -519,7 +520,11 @@ conv_mfma_kernel(ConvArgs a) {
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[fs][i], fb[fs][j], acc[i][j], 0, 0, 0);
   };
-  // one K step on LDS buffer d & 1; ring slot (d + 1) % DEPTH holds the next tile
+  // one K step on LDS buffer d & 1; ring slot (d + 1) % DEPTH holds the next tile.
+  // MFMA fragments are double-buffered in registers: while the MFMAs of one 32-byte K
+  // slice run, the LDS reads of the next slice, the LDS writes of the next tile and the
+  // global loads of a later tile are issued in their shadow.  The first slice of a step
+  // is read right after the barrier that publishes its tile.
   auto step_body = [&](int d) {
     const int buf = d & 1;
 #pragma unroll
@@ -533,30 +538,87 @@ conv_mfma_kernel(ConvArgs a) {
     __syncthreads();
     read_frag(buf ^ 1, 0, 0);
   };
-  read_frag(0, 0, 0);
 
-  // Whole groups of DEPTH steps: ring slots and LDS buffers are compile-time indices
-  // (DEPTH is even, so buffer parity == slot parity) and the body has no branch.
-  const int full = nsteps / DEPTH;
-#pragma nounroll
-  for (int g = 0; g < full; ++g) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      // slot d went to LDS one step ago: refill it with the tile DEPTH steps ahead
-      load_tile(d, (g + 1) * DEPTH + d);
-      step_body(d);
+  for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
+  if (PERSIST) __syncthreads();   // publishes qlds
+
+  // After the last barrier of a tile no wave reads LDS data it still needs, so the
+  // first store of the next tile may overtake slower waves of the workgroup.
+  for (;;) {
+    // accumulators start from the bias (the int32 add of the epilogue commutes with the sum)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const v4i *bp = PERSIST ? reinterpret_cast<const v4i *>(qlds + lch0 + i * 16)
+                              : reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i b = bp[q];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j][q * 4 + 0] = b[0];
+          acc[i][j][q * 4 + 1] = b[1];
+          acc[i][j][q * 4 + 2] = b[2];
+          acc[i][j][q * 4 + 3] = b[3];
+        }
+      }
     }
-  }
-  // the last nsteps % DEPTH steps: their tiles are already in the ring / in LDS
-  const int rem = nsteps - full * DEPTH;
+    store_tile(0, 0);
+    __syncthreads();
+    read_frag(0, 0, 0);
+
+    // Whole groups of DEPTH steps: ring slots and LDS buffers are compile-time indices
+    // (DEPTH is even, so buffer parity == slot parity) and the body has no branch.
+    const int full = nsteps / DEPTH;
+#pragma nounroll
+    for (int g = 0; g < full; ++g) {
 #pragma unroll
-  for (int d = 0; d < DEPTH - 1; ++d)
-    if (d < rem) step_body(d);
+      for (int d = 0; d < DEPTH; ++d) {
+        // slot d went to LDS one step ago: refill it with the tile DEPTH steps ahead
+        load_tile(d, (g + 1) * DEPTH + d);
+        step_body(d);
+      }
+    }
+    // the last nsteps % DEPTH steps: their tiles are already in the ring / in LDS
+    const int rem = nsteps - full * DEPTH;
+#pragma unroll
+    for (int d = 0; d < DEPTH - 1; ++d)
+      if (d < rem) step_body(d);
+
+    const int pix_done = pix0;
+    bool more = false;
+    if (PERSIST) {
+      // next pixel tile of this workgroup: start its loads before the epilogue
+      ltile += a.wgs_per_xcd;
+      logical += a.wgs_per_xcd;
+      more = ltile < a.tiles_per_xcd && logical < a.n_tiles;
+      if (more) {
+        pix0 += a.pstep_pix;
+        ow_first += a.pstep_ow;
+        if (ow_first >= a.ow) { ow_first -= a.ow; ++oh_first; }
+        oh_first += a.pstep_oh;
+        if (oh_first >= a.oh) { oh_first -= a.oh; ++n_first; }
+        n_first += a.pstep_n;
+        setup_rows();
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
+      }
+    }
 
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int oc = ocw0 + i * 16;
-    if (oc < a.ocw) epilogue_rows<TN, FAST>(acc[i], a, oc, pix0 + wn * TN * 32 + frow, 32);
+    for (int i = 0; i < TM; ++i) {
+      const int oc = ocw0 + i * 16;
+      const int lc = lch0 + i * 16;
+      if (oc < a.ocw) {
+        if (PERSIST)
+          epilogue_rows<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc,
+                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32);
+        else
+          epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
+                                  pix_done + wn * TN * 32 + frow, 32);
+      }
+    }
+    if (!PERSIST || !more) break;
   }
 }
 
@@ -719,7 +781,8 @@ conv_mfma_reg_kernel(ConvArgs a) {
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int oc = ocw0 + i * 16;
-    if (oc < a.ocw) epilogue_rows<TN, FAST>(acc[i], a, oc, pix0 + frow, 32);
+    if (oc < a.ocw)
+      epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pix0 + frow, 32);
   }
 }
 
@@ -910,7 +973,9 @@ conv_mfma_splitk_kernel(ConvArgs a) {
       sum[0][q * 4 + 3] = t[3];
     }
     const int oc = ocw0 + i * 16;
-    if (oc < a.ocw) epilogue_rows<1, FAST>(sum, a, oc, pix0 + j * 32 + frow, 32);
+    if (oc < a.ocw)
+      epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
+                             pix0 + j * 32 + frow, 32);
   }
 }
 
@@ -923,7 +988,8 @@ namespace {
 struct TileCfg {
   int bm, bn, wm, wn;
   const char *name;
-  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave; 2: its split-K form
+  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave; 2: its split-K form;
+             // 3: the LDS kernel with persistent workgroups
   int bk;    // K bytes per step (0 = 64)
 };
 // wave tile = (bm/wm) x (bn/wn)
@@ -960,6 +1026,12 @@ const TileCfg kTiles[] = {
     {64, 256, 1, 4, "mfma_64x256_o3", 0, 64},      // 29
     {32, 256, 1, 4, "mfma_32x256_o4", 0, 64},      // 30
     {128, 256, 2, 2, "mfma_128x256_o2", 0, 64},    // 31
+    {64, 128, 2, 2, "mfma_p_64x128", 3, 64},       // 32: persistent walks over pixel tiles
+    {64, 64, 2, 2, "mfma_p_64x64", 3, 64},         // 33
+    {128, 128, 2, 2, "mfma_p_128x128", 3, 64},     // 34
+    {64, 256, 1, 4, "mfma_p_64x256", 3, 64},       // 35
+    {32, 256, 1, 4, "mfma_p_32x256", 3, 64},       // 36
+    {32, 128, 1, 4, "mfma_p_32x128", 3, 64},       // 37
 };
 inline int tile_bk(const TileCfg &t) { return t.bk ? t.bk : 64; }
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
@@ -968,39 +1040,84 @@ template <bool FAST, int MODE>
 void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
   constexpr bool UNI = MODE == kModeUniform;
   switch (tile) {
-    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 64, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 64, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
     case 7: launch(ctx, (conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
     case 8: launch(ctx, (conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
     case 9: launch(ctx, (conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), a); break;
     case 10: launch(ctx, (conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), a); break;
     case 11: launch(ctx, (conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 12: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 4, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 13: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 256, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 14: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 15: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 16: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 128, 2, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 17: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 18: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 19: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 6, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 20: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 8, 0, FAST, MODE>), grid, dim3(256), a); break;
-    case 21: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 12, 0, FAST, MODE>), grid, dim3(256), a); break;
+    case 12: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 13: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 256, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 14: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 15: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 16: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 17: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 18: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 19: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 6, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 20: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 21: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 12, 0, false, FAST, MODE>), grid, dim3(256), a); break;
     case 22: launch(ctx, (conv_mfma_splitk_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
     case 23: launch(ctx, (conv_mfma_splitk_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
     case 24: launch(ctx, (conv_mfma_splitk_kernel<1, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
     case 25: launch(ctx, (conv_mfma_splitk_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 26: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 4, FAST, MODE>), grid, dim3(256), a); break;
-    case 27: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 6, FAST, MODE>), grid, dim3(256), a); break;
-    case 28: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 3, FAST, MODE>), grid, dim3(256), a); break;
-    case 29: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 3, FAST, MODE>), grid, dim3(256), a); break;
-    case 30: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 4, FAST, MODE>), grid, dim3(256), a); break;
-    default: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 2, FAST, MODE>), grid, dim3(256), a); break;
+    case 26: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 4, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 27: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 6, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 28: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 3, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 29: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 3, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 30: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 4, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 31: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 2, false, FAST, MODE>), grid, dim3(256), a); break;
+    case 32: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 33: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 34: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 35: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 36: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
+    default: launch(ctx, (conv_mfma_kernel<32, 128, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
   }
+}
+
+// workgroups of persistent tile variant `tile` that fit on one CU at once
+template <bool FAST, int MODE>
+int persist_occupancy(int tile) {
+  int n = 0;
+  hipError_t e = hipErrorInvalidValue;
+  switch (tile) {
+    case 32: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>, 256, 0); break;
+    case 33: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 64, 2, 2, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+    case 34: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<128, 128, 2, 2, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+    case 35: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 256, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+    case 36: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 256, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+    case 37: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 128, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+  }
+  return e == hipSuccess && n > 0 ? n : 1;
+}
+
+// the (FAST, MODE) instantiation a prepacked conv dispatches to
+int conv_mode(const tpuhip_conv_weights *w) {
+  const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
+  return w->smallc ? kModeSmallC : uni ? kModeUniform : kModeGeneral;
+}
+
+int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
+  static int cache[kNumTiles][2][3];   // 0 = not asked yet
+  const int mode = conv_mode(w);
+  int &c = cache[w->tile][w->fast ? 1 : 0][mode];
+  if (c == 0) {
+    if (w->fast)
+      c = mode == kModeSmallC ? persist_occupancy<true, kModeSmallC>(w->tile)
+          : mode == kModeUniform ? persist_occupancy<true, kModeUniform>(w->tile)
+                                 : persist_occupancy<true, kModeGeneral>(w->tile);
+    else
+      c = mode == kModeSmallC ? persist_occupancy<false, kModeSmallC>(w->tile)
+          : mode == kModeUniform ? persist_occupancy<false, kModeUniform>(w->tile)
+                                 : persist_occupancy<false, kModeGeneral>(w->tile);
+  }
+  return c;
 }
 
 // Rough cost model (cycles) used to pick a tile: workgroup rounds over the CUs
@@ -1066,7 +1183,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
   const int tm = t.bm / t.wm / 32;
   const int icp = round_up(d.ic, 16);
   const int ocp = round_up(d.oc, t.bm);
-  cw->smallc = d.ic <= 4 && !t.reg;
+  cw->smallc = d.ic <= 4 && (t.reg == 0 || t.reg == 3);
   cw->c16 = icp / 16;
   cw->k16 = cw->smallc ? (d.kh * d.kw * 4 + 15) / 16 : d.kh * d.kw * cw->c16;
   cw->kp = round_up(cw->k16 * 16, tile_bk(t));
@@ -1084,7 +1201,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
     for (int c = 0; c < d.ic; ++c)
       for (int k = 0; k < d.kh * d.kw; ++k)
         rowbuf[(size_t)k * kstride + c] = src[(size_t)c * d.kh * d.kw + k];
-    if (!t.reg) {
+    if (t.reg == 0 || t.reg == 3) {
       memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
     } else {
       // fragment order: [row / 32][K step][kk][lane = (row & 31) + 32 * half][16 bytes]
@@ -1110,11 +1227,12 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 
 bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
-  if (d.ic <= 4 && c.reg) return false;   // prefer the 4-channel K packing of the LDS kernels
+  if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
 
-void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *out) {
+void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+               ConvArgs *out) {
   const tpuhip_conv_desc &d = w->d;
   ConvArgs a{};
   a.x = (const int8_t *)x;
@@ -1148,12 +1266,24 @@ void fill_args(const tpuhip_conv_weights *w, const void *x, void *y, ConvArgs *o
     // workgroups per XCD (a workgroup of the LDS-free kernel holds four wave tiles)
     const int n_wgs = t.reg == 1 ? (a.n_tiles + 3) / 4 : a.n_tiles;
     a.tiles_per_xcd = (n_wgs + 7) / 8;
+    a.wgs_per_xcd = a.tiles_per_xcd;
+    if (t.reg == 3) {
+      // every XCD owns a run of whole pixel tiles; a workgroup keeps its channel tile
+      const int n_pix_tiles = a.n_tiles / a.n_oc_tiles;
+      a.tiles_per_xcd = (n_pix_tiles + 7) / 8 * a.n_oc_tiles;
+      const int slots = std::max(1, ctx->num_cu / 8) * persist_wgs_per_cu(w);
+      a.wgs_per_xcd = std::min(a.tiles_per_xcd, std::max(1, slots / a.n_oc_tiles) * a.n_oc_tiles);
+      a.pstep_pix = a.wgs_per_xcd / a.n_oc_tiles * t.bn;
+      a.pstep_ow = a.pstep_pix % d.ow;
+      a.pstep_oh = a.pstep_pix / d.ow % d.oh;
+      a.pstep_n = a.pstep_pix / d.ow / d.oh;
+    }
   }
   *out = a;
 }
 
 void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvArgs &a) {
-  dim3 grid((unsigned)(a.tiles_per_xcd * 8));
+  dim3 grid((unsigned)(a.wgs_per_xcd * 8));
   const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
   if (w->smallc) {
     if (w->fast)
@@ -1185,7 +1315,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
-    fill_args(w, x, y, &a);
+    fill_args(ctx, w, x, y, &a);
     for (int i = 0; i < 2; ++i) launch_conv_mfma(ctx, w, a);
     hipEventRecord(e0, ctx->stream);
     for (int i = 0; i < 5; ++i) launch_conv_mfma(ctx, w, a);
@@ -1382,7 +1512,7 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     if (rc) return rc;
   }
   ConvArgs a;
-  fill_args(w, x, y, &a);
+  fill_args(ctx, w, x, y, &a);
   if (f && f->enable) {
     a.add_src = (const int8_t *)add_src;
     a.add_dst = (int8_t *)add_out;
