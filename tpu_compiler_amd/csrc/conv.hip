@@ -276,16 +276,22 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
       if (a.add_dst) {
         // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
         const v4i sv = *reinterpret_cast<const v4i *>(a.add_src + off);
+        // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
+        // unused byte lanes are zero), with the rounding term as its addend: adding
+        // 2^(r-1) before the ReLU gives the same quotient as after it.
         const int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
+        const int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
+        const int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
         v4i z;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           int32_t t[4];
 #pragma unroll
           for (int b = 0; b < 4; ++b) {
-            int32_t sum = sbyte(sv[q], b) * a.add_m_src + sbyte(o[q], b) * a.add_m_conv;
-            if (a.add_relu) sum = max(sum, 0);
-            t[b] = (sum + rnd) >> a.add_rshift;
+            const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[q],
+                                                        0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
+            const int32_t sum = __builtin_amdgcn_sdot4((int)pair, mpair, rnd, false);
+            t[b] = max(sum, floor_) >> a.add_rshift;
           }
           z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
         }
@@ -1073,11 +1079,11 @@ void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
     case 30: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 4, false, FAST, MODE>), grid, dim3(256), a); break;
     case 31: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 2, false, FAST, MODE>), grid, dim3(256), a); break;
     case 32: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 33: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 34: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 35: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 36: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
-    default: launch(ctx, (conv_mfma_kernel<32, 128, 1, 4, 64, 2, 0, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 33: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 2, 4, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 34: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 2, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 35: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 1, true, FAST, MODE>), grid, dim3(256), a); break;
+    case 36: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 2, true, FAST, MODE>), grid, dim3(256), a); break;
+    default: launch(ctx, (conv_mfma_kernel<32, 128, 1, 4, 64, 2, 3, true, FAST, MODE>), grid, dim3(256), a); break;
   }
 }
 
@@ -1088,12 +1094,14 @@ int persist_occupancy(int tile) {
   hipError_t e = hipErrorInvalidValue;
   switch (tile) {
     case 32: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>, 256, 0); break;
-    case 33: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 64, 2, 2, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
-    case 34: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<128, 128, 2, 2, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
-    case 35: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 256, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
-    case 36: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 256, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
-    case 37: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 128, 1, 4, 64, 2, 0, true, FAST, MODE>, 256, 0); break;
+    case 33: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 64, 2, 2, 64, 2, 4, true, FAST, MODE>, 256, 0); break;
+    case 34: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<128, 128, 2, 2, 64, 2, 2, true, FAST, MODE>, 256, 0); break;
+    case 35: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 256, 1, 4, 64, 2, 1, true, FAST, MODE>, 256, 0); break;
+    case 36: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 256, 1, 4, 64, 2, 2, true, FAST, MODE>, 256, 0); break;
+    case 37: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 128, 1, 4, 64, 2, 3, true, FAST, MODE>, 256, 0); break;
   }
+  if (getenv("TPUHIP_DEBUG")) fprintf(stderr, "persist_occupancy tile %d: rc %d n %d\n", tile, (int)e, n);
+  if (e != hipSuccess) (void)hipGetLastError();   // not sticky: clear it
   return e == hipSuccess && n > 0 ? n : 1;
 }
 
@@ -1303,7 +1311,23 @@ void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvA
 
 // Times every candidate tile on the layer's real buffers (the kernels are
 // idempotent and bit-identical across tiles) and keeps the fastest.
-int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *y) {
+void apply_fusion(ConvArgs *a, const void *y, const void *add_src, void *add_out,
+                  const tpuhip_fused_add *f) {
+  if (!f || !f->enable) return;
+  a->add_src = (const int8_t *)add_src;
+  a->add_dst = (int8_t *)add_out;
+  a->add_m_src = f->m_src;
+  a->add_m_conv = f->m_conv;
+  a->add_rshift = f->rshift;
+  a->add_relu = f->do_relu ? 1 : 0;
+  a->store_y = y != nullptr;
+}
+
+// The fused add (if any) is part of what is timed: it shifts the balance between
+// the tile shapes.  Every launch recomputes the same bytes, so repeating it is safe
+// as long as the sum is not written over its own input.
+int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *y,
+                  const void *add_src, void *add_out, const tpuhip_fused_add *f) {
   hipEvent_t e0, e1;
   TPUHIP_CHECK_HIP(hipEventCreate(&e0));
   TPUHIP_CHECK_HIP(hipEventCreate(&e1));
@@ -1316,13 +1340,18 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     if (rc) break;
     ConvArgs a;
     fill_args(ctx, w, x, y, &a);
+    apply_fusion(&a, y, add_src, add_out, f);
     for (int i = 0; i < 2; ++i) launch_conv_mfma(ctx, w, a);
     hipEventRecord(e0, ctx->stream);
     for (int i = 0; i < 5; ++i) launch_conv_mfma(ctx, w, a);
     hipEventRecord(e1, ctx->stream);
-    if (hipEventSynchronize(e1) != hipSuccess || hipGetLastError() != hipSuccess) {
-      rc = set_error(TPUHIP_ERR_HIP, "conv autotune: kernel launch failed");
-      break;
+    const hipError_t es = hipEventSynchronize(e1), el = hipGetLastError();
+    if (es != hipSuccess || el != hipSuccess) {
+      // a variant that cannot be launched is skipped; the layer fails only if none can
+      set_error(TPUHIP_ERR_HIP, "conv autotune: tile %s failed: %s", kTiles[t].name,
+                hipGetErrorString(es != hipSuccess ? es : el));
+      if (getenv("TPUHIP_DEBUG")) fprintf(stderr, "%s\n", tpuhip_last_error());
+      continue;
     }
     float ms = 0;
     hipEventElapsedTime(&ms, e0, e1);
@@ -1334,7 +1363,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
   hipEventDestroy(e0);
   hipEventDestroy(e1);
   if (rc) return rc;
-  if (best < 0) return set_error(TPUHIP_ERR_INVALID, "conv autotune: no candidate tile");
+  if (best < 0) return TPUHIP_ERR_HIP;   // the last launch error is still the message
   if (best != w->tile) rc = pack_mfma_weights(ctx, w, best);
   w->tuned = true;
   w->host_filter.clear();
@@ -1502,26 +1531,20 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
                     const void *add_src, void *add_out, const tpuhip_fused_add *f) {
   if (w->algo == ALGO_MFMA && !w->tuned) {
     // first use: pick the tile by measurement (not capturable into a HIP graph)
+    const bool fused = f && f->enable && add_out != add_src;
     void *ty = y;
-    if (!ty) {   // tuning writes the plain conv result somewhere: borrow a scratch buffer
+    if (!ty && !fused) {   // tuning writes the plain conv result somewhere: borrow a buffer
       const size_t bytes = (size_t)w->d.n * w->d.oh * w->d.ow * w->d.y_cs;
       if (int rc = tpuhip_malloc(ctx, bytes, &ty)) return rc;
     }
-    int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, ty);
-    if (!y) tpuhip_free(ctx, ty);
+    int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, ty, add_src, add_out,
+                           fused ? f : nullptr);
+    if (ty != y) tpuhip_free(ctx, ty);
     if (rc) return rc;
   }
   ConvArgs a;
   fill_args(ctx, w, x, y, &a);
-  if (f && f->enable) {
-    a.add_src = (const int8_t *)add_src;
-    a.add_dst = (int8_t *)add_out;
-    a.add_m_src = f->m_src;
-    a.add_m_conv = f->m_conv;
-    a.add_rshift = f->rshift;
-    a.add_relu = f->do_relu ? 1 : 0;
-    a.store_y = y != nullptr;
-  }
+  apply_fusion(&a, y, add_src, add_out, f);
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
