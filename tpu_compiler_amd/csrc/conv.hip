@@ -247,6 +247,15 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
                                               const int32_t *phpot, int pix_first,
                                               int pix_stride) {
   uint32_t outw[TN][4];
+  // the other operand of a fused add is fetched now and used after the requantisation
+  v4i sv[TN];
+  if (a.add_dst) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int pix = min(pix_first + j * pix_stride, a.npix - 1);
+      sv[j] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)pix * a.y_cs + oc);
+    }
+  }
 #pragma unroll
   for (int qd = 0; qd < 4; ++qd) {
     const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
@@ -275,7 +284,6 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
       if (a.store_y) *reinterpret_cast<v4i *>(a.y + off) = o;
       if (a.add_dst) {
         // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
-        const v4i sv = *reinterpret_cast<const v4i *>(a.add_src + off);
         // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
         // unused byte lanes are zero), with the rounding term as its addend: adding
         // 2^(r-1) before the ReLU gives the same quotient as after it.
@@ -288,7 +296,7 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
           int32_t t[4];
 #pragma unroll
           for (int b = 0; b < 4; ++b) {
-            const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[q],
+            const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[j][q],
                                                         0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
             const int32_t sum = __builtin_amdgcn_sdot4((int)pair, mpair, rnd, false);
             t[b] = max(sum, floor_) >> a.add_rshift;
