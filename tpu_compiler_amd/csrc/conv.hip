@@ -287,9 +287,11 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
         // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
         // unused byte lanes are zero), with the rounding term as its addend: adding
         // 2^(r-1) before the ReLU gives the same quotient as after it.
-        const int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
-        const int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
-        const int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
+        int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
+        int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
+        int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
+        // one scalar and one vector copy of the uniform operands, made once
+        asm volatile("" : "+s"(rnd), "+v"(mpair), "+s"(floor_));
         v4i z;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -298,7 +300,8 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
           for (int b = 0; b < 4; ++b) {
             const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[j][q],
                                                         0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
-            const int32_t sum = __builtin_amdgcn_sdot4((int)pair, mpair, rnd, false);
+            int32_t sum;   // the three-operand form: no copy of the addend into the result first
+            asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(sum) : "v"(pair), "v"(mpair), "s"(rnd));
             t[b] = max(sum, floor_) >> a.add_rshift;
           }
           z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
@@ -1002,114 +1005,87 @@ namespace {
 struct TileCfg {
   int bm, bn, wm, wn;
   const char *name;
-  int reg;   // 1: the LDS-free kernel, bm x bn is the tile of one wave; 2: its split-K form;
-             // 3: the LDS kernel with persistent workgroups
-  int bk;    // K bytes per step (0 = 64)
+  int reg;   // 0: LDS kernel, one tile per workgroup; 1: the LDS-free kernel, bm x bn is the
+             // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups
+  int bk;    // K bytes per step
 };
-// wave tile = (bm/wm) x (bn/wn)
+
+// The tile variants, in the order of their public index (conv desc algo = 16 + index).
+// LDS kernels: X(index, name, persistent, BM, BN, WM, WN, BK, ring depth, waves per SIMD)
+#define TPUHIP_LDS_TILES(X)                                     \
+  X(0, "mfma_p_64x128", true, 64, 128, 2, 2, 64, 2, 3)          \
+  X(1, "mfma_p_64x64", true, 64, 64, 2, 2, 64, 2, 4)            \
+  X(2, "mfma_p_128x128", true, 128, 128, 2, 2, 64, 2, 2)        \
+  X(3, "mfma_p_32x128", true, 32, 128, 1, 4, 64, 2, 3)          \
+  X(4, "mfma_p_64x256", true, 64, 256, 1, 4, 64, 2, 1)          \
+  X(5, "mfma_p_32x256", true, 32, 256, 1, 4, 64, 2, 2)          \
+  X(6, "mfma_p_64x64_k128", true, 64, 64, 2, 2, 128, 2, 3)      \
+  X(7, "mfma_p_64x64_k256", true, 64, 64, 2, 2, 256, 2, 2)      \
+  X(8, "mfma_p_64x128_k128", true, 64, 128, 2, 2, 128, 2, 2)    \
+  X(9, "mfma_64x64_k128", false, 64, 64, 2, 2, 128, 4, 0)       \
+  X(10, "mfma_64x64_k256", false, 64, 64, 2, 2, 256, 2, 0)      \
+  X(11, "mfma_64x128_k128", false, 64, 128, 2, 2, 128, 2, 0)    \
+  X(12, "mfma_64x64_k128_d6", false, 64, 64, 2, 2, 128, 6, 0)
+// LDS-free kernels: Y(index, name, split K, TM, TN, ring depth, waves per SIMD)
+#define TPUHIP_REG_TILES(Y)                        \
+  Y(13, "mfma_reg_32x64", false, 1, 2, 4, 3)       \
+  Y(14, "mfma_reg_32x32", false, 1, 1, 4, 5)       \
+  Y(15, "mfma_reg_64x64", false, 2, 2, 4, 2)       \
+  Y(16, "mfma_splitk_64x64", true, 2, 2, 4, 2)     \
+  Y(17, "mfma_splitk_32x64", true, 1, 2, 4, 3)
+
 const TileCfg kTiles[] = {
-    {128, 256, 2, 2, "mfma_128x256"},   // 0: waves of 64x128
-    {64, 256, 1, 4, "mfma_64x256"},     // 1: waves of 64x64
-    {64, 512, 1, 4, "mfma_64x512"},     // 2: waves of 64x128
-    {32, 256, 1, 4, "mfma_32x256"},     // 3: waves of 32x64
-    {128, 128, 2, 2, "mfma_128x128"},   // 4: waves of 64x64
-    {64, 128, 2, 2, "mfma_64x128"},     // 5: waves of 32x64
-    {64, 64, 2, 2, "mfma_64x64"},       // 6: waves of 32x32
-    {64, 64, 1, 1, "mfma_reg_64x64", 1},    // 7
-    {32, 64, 1, 1, "mfma_reg_32x64", 1},    // 8
-    {64, 128, 1, 1, "mfma_reg_64x128", 1},  // 9
-    {32, 32, 1, 1, "mfma_reg_32x32", 1},    // 10
-    {64, 32, 1, 1, "mfma_reg_64x32", 1},    // 11
-    {64, 64, 2, 2, "mfma_64x64_k128", 0, 128},     // 12
-    {64, 64, 2, 2, "mfma_64x64_k256", 0, 256},     // 13
-    {64, 128, 2, 2, "mfma_64x128_k128", 0, 128},   // 14
-    {128, 128, 2, 2, "mfma_128x128_k128", 0, 128}, // 15
-    {64, 256, 1, 4, "mfma_64x256_k128", 0, 128},   // 16
-    {64, 64, 2, 2, "mfma_64x64_d8", 0, 64},        // 17: ring of 8 steps
-    {64, 128, 2, 2, "mfma_64x128_d8", 0, 64},      // 18
-    {64, 64, 2, 2, "mfma_64x64_k128_d6", 0, 128},  // 19
-    {128, 128, 2, 2, "mfma_128x128_d8", 0, 64},    // 20
-    {64, 64, 2, 2, "mfma_64x64_d12", 0, 64},       // 21
-    {64, 64, 1, 1, "mfma_splitk_64x64", 2},        // 22: one tile per workgroup, K split over 4 waves
-    {32, 64, 1, 1, "mfma_splitk_32x64", 2},        // 23
-    {32, 32, 1, 1, "mfma_splitk_32x32", 2},        // 24
-    {64, 32, 1, 1, "mfma_splitk_64x32", 2},        // 25
-    {64, 128, 2, 2, "mfma_64x128_o4", 0, 64},      // 26: 4 waves per SIMD
-    {64, 64, 2, 2, "mfma_64x64_o6", 0, 64},        // 27: 6 waves per SIMD
-    {128, 128, 2, 2, "mfma_128x128_o3", 0, 64},    // 28
-    {64, 256, 1, 4, "mfma_64x256_o3", 0, 64},      // 29
-    {32, 256, 1, 4, "mfma_32x256_o4", 0, 64},      // 30
-    {128, 256, 2, 2, "mfma_128x256_o2", 0, 64},    // 31
-    {64, 128, 2, 2, "mfma_p_64x128", 3, 64},       // 32: persistent walks over pixel tiles
-    {64, 64, 2, 2, "mfma_p_64x64", 3, 64},         // 33
-    {128, 128, 2, 2, "mfma_p_128x128", 3, 64},     // 34
-    {64, 256, 1, 4, "mfma_p_64x256", 3, 64},       // 35
-    {32, 256, 1, 4, "mfma_p_32x256", 3, 64},       // 36
-    {32, 128, 1, 4, "mfma_p_32x128", 3, 64},       // 37
+#define X(i, name, P, BM, BN, WM, WN, BK, D, O) {BM, BN, WM, WN, name, P ? 3 : 0, BK},
+    TPUHIP_LDS_TILES(X)
+#undef X
+#define Y(i, name, SPLIT, TM, TN, D, O) {TM * 32, TN * 32, 1, 1, name, SPLIT ? 2 : 1, 64},
+    TPUHIP_REG_TILES(Y)
+#undef Y
 };
-inline int tile_bk(const TileCfg &t) { return t.bk ? t.bk : 64; }
+inline int tile_bk(const TileCfg &t) { return t.bk; }
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
+template <bool SPLIT, int TM, int TN, int D, int O, bool FAST, bool UNI>
+void launch_reg(tpuhip_ctx *ctx, dim3 grid, const ConvArgs &a) {
+  if constexpr (SPLIT)
+    launch(ctx, (conv_mfma_splitk_kernel<TM, TN, D, O, FAST, UNI>), grid, dim3(256), a);
+  else
+    launch(ctx, (conv_mfma_reg_kernel<TM, TN, D, O, FAST, UNI>), grid, dim3(256), a);
+}
 
 template <bool FAST, int MODE>
 void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
   constexpr bool UNI = MODE == kModeUniform;
   switch (tile) {
-    case 0: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 1: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 2: launch(ctx, (conv_mfma_kernel<64, 512, 1, 4, 64, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 3: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 4: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 5: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 6: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 7: launch(ctx, (conv_mfma_reg_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
-    case 8: launch(ctx, (conv_mfma_reg_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 9: launch(ctx, (conv_mfma_reg_kernel<2, 4, 2, 1, FAST, UNI>), grid, dim3(256), a); break;
-    case 10: launch(ctx, (conv_mfma_reg_kernel<1, 1, 4, 5, FAST, UNI>), grid, dim3(256), a); break;
-    case 11: launch(ctx, (conv_mfma_reg_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 12: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 4, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 13: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 256, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 14: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 15: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 16: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 128, 2, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 17: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 18: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 19: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 128, 6, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 20: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 8, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 21: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 12, 0, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 22: launch(ctx, (conv_mfma_splitk_kernel<2, 2, 4, 2, FAST, UNI>), grid, dim3(256), a); break;
-    case 23: launch(ctx, (conv_mfma_splitk_kernel<1, 2, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 24: launch(ctx, (conv_mfma_splitk_kernel<1, 1, 4, 4, FAST, UNI>), grid, dim3(256), a); break;
-    case 25: launch(ctx, (conv_mfma_splitk_kernel<2, 1, 4, 3, FAST, UNI>), grid, dim3(256), a); break;
-    case 26: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 4, 4, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 27: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 4, 6, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 28: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 3, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 29: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 3, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 30: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 4, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 31: launch(ctx, (conv_mfma_kernel<128, 256, 2, 2, 64, 2, 2, false, FAST, MODE>), grid, dim3(256), a); break;
-    case 32: launch(ctx, (conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 33: launch(ctx, (conv_mfma_kernel<64, 64, 2, 2, 64, 2, 4, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 34: launch(ctx, (conv_mfma_kernel<128, 128, 2, 2, 64, 2, 2, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 35: launch(ctx, (conv_mfma_kernel<64, 256, 1, 4, 64, 2, 1, true, FAST, MODE>), grid, dim3(256), a); break;
-    case 36: launch(ctx, (conv_mfma_kernel<32, 256, 1, 4, 64, 2, 2, true, FAST, MODE>), grid, dim3(256), a); break;
-    default: launch(ctx, (conv_mfma_kernel<32, 128, 1, 4, 64, 2, 3, true, FAST, MODE>), grid, dim3(256), a); break;
+#define X(i, name, P, BM, BN, WM, WN, BK, D, O)                                             \
+  case i:                                                                                   \
+    launch(ctx, (conv_mfma_kernel<BM, BN, WM, WN, BK, D, O, P, FAST, MODE>), grid,          \
+           dim3(WM * WN * 64), a);                                                          \
+    break;
+    TPUHIP_LDS_TILES(X)
+#undef X
+#define Y(i, name, SPLIT, TM, TN, D, O) \
+  case i: launch_reg<SPLIT, TM, TN, D, O, FAST, UNI>(ctx, grid, a); break;
+    TPUHIP_REG_TILES(Y)
+#undef Y
   }
 }
 
-// workgroups of persistent tile variant `tile` that fit on one CU at once
+// workgroups of LDS tile variant `tile` that fit on one CU at once
 template <bool FAST, int MODE>
 int persist_occupancy(int tile) {
   int n = 0;
   hipError_t e = hipErrorInvalidValue;
   switch (tile) {
-    case 32: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 128, 2, 2, 64, 2, 3, true, FAST, MODE>, 256, 0); break;
-    case 33: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 64, 2, 2, 64, 2, 4, true, FAST, MODE>, 256, 0); break;
-    case 34: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<128, 128, 2, 2, 64, 2, 2, true, FAST, MODE>, 256, 0); break;
-    case 35: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<64, 256, 1, 4, 64, 2, 1, true, FAST, MODE>, 256, 0); break;
-    case 36: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 256, 1, 4, 64, 2, 2, true, FAST, MODE>, 256, 0); break;
-    case 37: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_mfma_kernel<32, 128, 1, 4, 64, 2, 3, true, FAST, MODE>, 256, 0); break;
+#define X(i, name, P, BM, BN, WM, WN, BK, D, O)                                              \
+  case i:                                                                                    \
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(                                        \
+        &n, conv_mfma_kernel<BM, BN, WM, WN, BK, D, O, P, FAST, MODE>, WM * WN * 64, 0);     \
+    break;
+    TPUHIP_LDS_TILES(X)
+#undef X
   }
-  if (getenv("TPUHIP_DEBUG")) fprintf(stderr, "persist_occupancy tile %d: rc %d n %d\n", tile, (int)e, n);
-  if (e != hipSuccess) (void)hipGetLastError();   // not sticky: clear it
+  if (e != hipSuccess) (void)hipGetLastError();   // clear it: the caller falls back to 1
   return e == hipSuccess && n > 0 ? n : 1;
 }
 
@@ -1136,33 +1112,15 @@ int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
   return c;
 }
 
-// Rough cost model (cycles) used to pick a tile: workgroup rounds over the CUs
-// times the per-workgroup time (K steps bounded by MFMA issue or LDS reads, plus
-// the VALU epilogue), with two workgroups assumed to overlap on one CU.
+// Default tile when the variants are not timed on first use: the persistent tiles,
+// narrow in output channels for thin layers, wide in pixels when there are enough of
+// them to give every CU several tiles.
 int pick_tile(const tpuhip_conv_desc &d, int k16, int num_cu) {
+  (void)k16;
   const int64_t npix = (int64_t)d.n * d.oh * d.ow;
-  const int nsteps = (k16 * 16 + 63) / 64;
-  double best = 1e30;
-  int best_tile = 1;
-  for (int t = 0; t < kNumTiles; ++t) {
-    const TileCfg &c = kTiles[t];
-    if (c.reg || c.bk || t > 6) continue;
-    if (c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32)) continue;   // more than half the rows idle
-    const int tm = c.bm / c.wm / 32, tn = c.bn / c.wn / 32;
-    const int64_t wgs = ceil_div64(npix, c.bn) * ceil_div64(d.oc, c.bm);
-    const double mfma = tm * tn * 2 * 32.0;
-    const double ldsr = (tm + tn) * 2 * 8.0 * 4;          // four waves share the LDS port
-    const double step = std::max(std::max(mfma, ldsr), 160.0);
-    const double epi = tm * tn * 16 * 44.0;
-    const double per_wg = nsteps * step + epi + 1500.0;
-    const double rounds = std::ceil((double)wgs / (2.0 * num_cu));
-    const double cost = rounds * per_wg * (wgs < num_cu ? 1.0 : 1.0);
-    if (cost < best) {
-      best = cost;
-      best_tile = t;
-    }
-  }
-  return best_tile;
+  if (d.oc <= 32) return 3;
+  const int64_t tiles128 = ceil_div64(npix, 128) * ceil_div64(d.oc, 64);
+  return tiles128 >= 2 * (int64_t)num_cu ? 0 : 1;
 }
 
 int check_desc(const tpuhip_conv_desc &d) {
