@@ -150,6 +150,15 @@ def main():
                         "achieved": round(conv_ops / (conv_ms / 1e3) / 1e12, 2),
                         "frac": round(conv_ops / (conv_ms / 1e3) / 1e12 / PEAK_INT8_TOPS, 4),
                         "ms": round(conv_ms, 4)}}
+    # HBM bytes per launch of that kernel, from the committed rocprofv3 counter passes
+    # (FETCH_SIZE + WRITE_SIZE, scaled against a plain copy kernel) of this same workload
+    traffic_file = os.path.join(ROOT, "profiles", "resnet50_b32_bench_traffic.json")
+    if roofline and args.config == "cfg3" and os.path.exists(traffic_file):
+        t = json.load(open(traffic_file))["kernels"].get(dom_name)
+        if t:
+            roofline["traffic"] = int((t["fetch_KiB"] + t["write_KiB"]) * 1024)
+            roofline["traffic_unit"] = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/)"
+            roofline["algorithmic_bytes"] = int(dom["bytes"] / dom["launches"])
     if args.per_layer:
         for name, algo, ms in rows:
             op = g.by_name[name]

@@ -1034,16 +1034,27 @@ struct TileCfg {
   Y(16, "mfma_splitk_64x64", true, 2, 2, 4, 2)     \
   Y(17, "mfma_splitk_32x64", true, 1, 2, 4, 3)
 
-const TileCfg kTiles[] = {
-#define X(i, name, P, BM, BN, WM, WN, BK, D, O) {BM, BN, WM, WN, name, P ? 3 : 0, BK},
+struct TileTable {
+  TileCfg t[64];
+  int n = 0;
+  TileTable() {
+#define X(i, name, P, BM, BN, WM, WN, BK, D, O) \
+  t[i] = TileCfg{BM, BN, WM, WN, name, P ? 3 : 0, BK}; \
+  n = n > i ? n : i + 1;
     TPUHIP_LDS_TILES(X)
 #undef X
-#define Y(i, name, SPLIT, TM, TN, D, O) {TM * 32, TN * 32, 1, 1, name, SPLIT ? 2 : 1, 64},
+#define Y(i, name, SPLIT, TM, TN, D, O) \
+  t[i] = TileCfg{TM * 32, TN * 32, 1, 1, name, SPLIT ? 2 : 1, 64}; \
+  n = n > i ? n : i + 1;
     TPUHIP_REG_TILES(Y)
 #undef Y
+  }
 };
+const TileTable kTileTable;
+const TileCfg *const kTiles = kTileTable.t;
 inline int tile_bk(const TileCfg &t) { return t.bk; }
-constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+constexpr int kMaxTiles = 64;
+#define kNumTiles (kTileTable.n)
 
 template <bool SPLIT, int TM, int TN, int D, int O, bool FAST, bool UNI>
 void launch_reg(tpuhip_ctx *ctx, dim3 grid, const ConvArgs &a) {
@@ -1096,7 +1107,7 @@ int conv_mode(const tpuhip_conv_weights *w) {
 }
 
 int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
-  static int cache[kNumTiles][2][3];   // 0 = not asked yet
+  static int cache[kMaxTiles][2][3];   // 0 = not asked yet
   const int mode = conv_mode(w);
   int &c = cache[w->tile][w->fast ? 1 : 0][mode];
   if (c == 0) {
