@@ -56,6 +56,10 @@ def main():
     ap.add_argument("--save-tiles", default="", help="write the conv tile chosen for every layer")
     ap.add_argument("--tiles", default="", help="use the conv tiles recorded in this file instead "
                                                 "of timing the variants (repeatable profiling)")
+    ap.add_argument("--keep-all", action="store_true",
+                    help="write every tensor of the graph (the reference's get_all_tensor mode); "
+                         "by default the result of a conv that only feeds the add fused into it "
+                         "is not written")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write kernel (relu) so HBM "
                          "counters can be scaled against a kernel of known traffic")
@@ -79,6 +83,7 @@ def main():
             if algo in tile_names:
                 g.by_name[name].attrs["algo"] = 16 + tile_names.index(algo)
     m = module(device=0)
+    m.set_option("keep_all_tensors", 1 if args.keep_all else 0)
     m.load(g)
     m.set_tensor(g.input_op().name, g.input_op().data.astype(np.float32))
     lib, ctxh = m.lib, m.context_handle()
@@ -175,7 +180,9 @@ def main():
         "config": {"workload": "%s: %s INT8 graph, batch %d, %s input, random-init seeded weights"
                                % (args.config, g.name, batch,
                                   "x".join(str(v) for v in g.input_op().shape[1:])),
-                   "global_batch": batch},
+                   "global_batch": batch,
+                   "tensors_written": "all" if args.keep_all else
+                                      "all but the conv results consumed only by their fused add"},
         "tops": round(tops, 2),
         "ops_per_step": total_ops,
         "event_ms_per_step": round(ev_ms.value / args.steps, 4),

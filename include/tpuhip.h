@@ -255,6 +255,11 @@ int tpuhip_module_add_op(tpuhip_module *m, const tpuhip_op_desc *op);
 int tpuhip_module_set_returns(tpuhip_module *m, const char *const *names, int n);
 /* loadModule(module, target_op): builds / refreshes the kernel list; unchanged
  * kernels are kept (MlirModuleInterpreter.cpp:73-83, 118-350).  target_op may be NULL. */
+/* Options read at the next tpuhip_module_load: "fuse_eltwise" (default 1: an EltwiseAdd of a conv
+ * result runs in that conv's epilogue), "keep_all_tensors" (default 1: every tensor can be read back
+ * after an invoke, as with the reference's get_all_tensor; 0: the result of a conv whose only reader
+ * is the add fused into it is never written, and reading it back is an error). */
+int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value);
 int tpuhip_module_load(tpuhip_module *m, const char *target_op);
 /* setTensor / getTensor (:407-430) */
 int tpuhip_module_set_tensor(tpuhip_module *m, const char *name, const float *data, size_t count,

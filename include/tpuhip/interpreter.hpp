@@ -77,6 +77,7 @@ public:
 
   int32_t batch;
   int n = 1, c = 1, h = 1, w = 1;  // 4-d view of the shape (missing dims are 1)
+  bool materialized = true;        // false: no kernel writes this tensor (fused away)
   int cs = 16;                     // channel stride in bytes
   size_t slot_bytes() const { return (size_t)n * h * w * cs; }
   tpuhip_ctx *ctx() const { return ctx_; }
@@ -118,6 +119,7 @@ public:
   virtual void invoke() = 0;
 
   std::string get_name() { return name; }
+  const std::vector<Operand> &operands() const { return opdTensors; }
   SyncedDataShape get_shape() { return shape; }
   std::string get_data_type();
   void set_name(std::string n) { name = std::move(n); }
@@ -173,6 +175,9 @@ public:
   bool can_fuse_add() const;
   void fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift, bool relu);
   void clear_fusion();
+  // false: the conv result itself is not written, only the fused sum (set by the module
+  // interpreter when nothing else reads it and the caller asked for outputs only)
+  void set_store_result(bool store);
   SyncedData result() const { return output_data; }
 
 private:
@@ -180,6 +185,7 @@ private:
   SyncedData input_data, output_data;
   SyncedData add_src, add_dst;
   tpuhip_fused_add fused{};
+  bool store_result = true;
 };
 
 class FullyConnectedOpKernel : public CPUOpKernel {  // core/fullyconnected.cpp
@@ -351,6 +357,10 @@ public:
   tpuhip_ctx *context() const { return ctx_; }
   // conv + eltwise-add fusion (on by default; TPUHIP_FUSE=0 disables); applies at the next loadModule
   bool fuse_eltwise = true;
+  // true (default): every tensor of the graph can be read back after an invoke, like the
+  // reference.  false: the result of a conv whose only reader is the add fused into it is
+  // never written (reading it back is an error); applies at the next loadModule
+  bool keep_all_tensors = true;
 
   std::vector<std::pair<std::string, size_t>> input_details;
   std::vector<std::string> output_details;

@@ -145,6 +145,43 @@ def test_fusion_on_and_off_give_the_same_tensors(monkeypatch):
         m.close()
 
 
+def test_outputs_only_mode_skips_fused_conv_results_and_keeps_the_rest_exact():
+    g = graphs.cfg3_resnet50(batch=2, hw=96)
+    want = oracle_graph.run(g)
+    m = module()
+    m.set_option("keep_all_tensors", 0)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    adds = [op for op in g.ops if op.type == "tpu.eltwise_add"]
+    consumers = {}
+    for op in g.ops:
+        for i in op.inputs:
+            consumers.setdefault(i, []).append(op.name)
+    skipped = 0
+    for op in g.ops:
+        fused_away = (op.type == "tpu.conv_2d" and len(consumers.get(op.name, [])) == 1
+                      and g.by_name[consumers[op.name][0]].type == "tpu.eltwise_add"
+                      and g.by_name[consumers[op.name][0]].inputs[-1] == op.name)
+        if fused_away:
+            with pytest.raises(capi.TpuHipError, match="never written"):
+                m.get_tensor_i8(op.name)
+            skipped += 1
+        else:
+            assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    assert skipped == len(adds) == 16
+    with pytest.raises(capi.TpuHipError, match="unknown option"):
+        m.set_option("nope", 1)
+    # back to the default: everything readable again after a reload
+    m.set_option("keep_all_tensors", 1)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()
+
+
 def test_module_errors_are_reported():
     g = graphs.cfg1_single_conv()
     m = module()

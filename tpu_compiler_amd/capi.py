@@ -122,6 +122,7 @@ PROTOTYPES.update({
     "tpuhip_module_time_kernels": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float),
                                              C.c_int]),
     "tpuhip_module_ctx": (C.c_void_p, [C.c_void_p]),
+    "tpuhip_module_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
 })
 
 

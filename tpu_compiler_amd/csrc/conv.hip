@@ -379,13 +379,15 @@ conv_mfma_kernel(ConvArgs a) {
   const __amdgpu_buffer_rsrc_t wrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
 
-  if (PERSIST) {
-    for (int t = tid; t < BM; t += NT) {
-      qlds[t] = a.bias[oc0 + t];
-      qlds[BM + t] = a.qmult[oc0 + t];
-      qlds[2 * BM + t] = a.qshift[oc0 + t];
-      qlds[3 * BM + t] = a.qhpot[oc0 + t];
-    }
+  // requant parameters of the channel tile: fetched now, parked in LDS after the first
+  // tile loads have been issued (their latencies overlap instead of adding up)
+  static_assert(!PERSIST || BM <= NT, "one parameter row per thread");
+  int32_t qv[4] = {0, 0, 0, 0};
+  if (PERSIST && tid < BM) {
+    qv[0] = a.bias[oc0 + tid];
+    qv[1] = a.qmult[oc0 + tid];
+    qv[2] = a.qshift[oc0 + tid];
+    qv[3] = a.qhpot[oc0 + tid];
   }
 
   // ---- loader state: this thread fetches K-chunk kc of rows lrow + RP*s
@@ -558,7 +560,15 @@ conv_mfma_kernel(ConvArgs a) {
 
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
-  if (PERSIST) __syncthreads();   // publishes qlds
+  if (PERSIST) {
+    if (tid < BM) {
+      qlds[tid] = qv[0];
+      qlds[BM + tid] = qv[1];
+      qlds[2 * BM + tid] = qv[2];
+      qlds[3 * BM + tid] = qv[3];
+    }
+    __syncthreads();   // publishes qlds
+  }
 
   // After the last barrier of a tile no wave reads LDS data it still needs, so the
   // first store of the next tile may overtake slower waves of the workgroup.

@@ -3,6 +3,8 @@
 // lib/Dialect/TPU/Interpreter/MlirModuleInterpreter.cpp:73-457.
 #include "tpuhip/interpreter.hpp"
 
+#include <algorithm>
+
 #include <cstdio>
 #include <cstdlib>
 
@@ -58,6 +60,7 @@ void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
 void ModuleInterpreter::fuseKernels() {
   std::map<TensorData *, std::pair<int, Conv2DOpKernel *>> producer;   // tensor -> (position, conv)
   std::map<TensorData *, int> position;                               // tensor -> producing position
+  std::vector<Conv2DOpKernel *> fused_convs;
   int pos = 0;
   for (auto &k : kernel_list_) {
     if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) c->clear_fusion();
@@ -99,6 +102,19 @@ void ModuleInterpreter::fuseKernels() {
                    e->multipliers()[conv_idx], e->rshift_value(), e->relu());
     e->fused_into_producer = true;
     producer.erase(e->inputs()[conv_idx].get());   // one fusion per conv
+    fused_convs.push_back(conv);
+  }
+  if (keep_all_tensors) return;
+  // outputs only: a fused conv whose result has no reader but the add, and is not a
+  // module output, need not write it
+  std::map<TensorData *, int> readers;
+  for (auto &k : kernel_list_)
+    for (auto &opd : k->operands())
+      if (opd.act) ++readers[opd.act.get()];
+  for (Conv2DOpKernel *conv : fused_convs) {
+    const bool is_output =
+        std::find(output_details.begin(), output_details.end(), conv->name) != output_details.end();
+    if (!is_output && readers[conv->result().get()] == 1) conv->set_store_result(false);
   }
 }
 

@@ -121,6 +121,9 @@ void TensorData::assign(const float *first, size_t num, int32_t bidx) {
 }
 
 std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
+  if (!materialized)
+    fail("TensorData::tensor: this tensor is fused into its consumer and never written "
+         "(load the module with keep_all_tensors to read it)");
   if (bidx < 0 || bidx >= batch) fail("TensorData::tensor: slot out of range");
   auto out = std::make_shared<std::vector<float>>(size_);
   void *tmp = nullptr;
@@ -134,6 +137,9 @@ std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
 }
 
 void TensorData::read_i8(int8_t *dst, size_t num, int32_t bidx) const {
+  if (!materialized)
+    fail("TensorData::read_i8: this tensor is fused into its consumer and never written "
+         "(load the module with keep_all_tensors to read it)");
   if (num != size_) fail("TensorData::read_i8: size mismatch");
   if (bidx < 0 || bidx >= batch) fail("TensorData::read_i8: slot out of range");
   void *tmp = nullptr;
@@ -321,7 +327,8 @@ Conv2DOpKernel::~Conv2DOpKernel() {
 
 void Conv2DOpKernel::invoke() {
   if (fused.enable)
-    ck(tpuhip_conv2d_add_i8(ctx, packed, input_data->data(), output_data->data(), add_src->data(),
+    ck(tpuhip_conv2d_add_i8(ctx, packed, input_data->data(),
+                            store_result ? output_data->data() : nullptr, add_src->data(),
                             add_dst->data(), &fused),
        name.c_str());
   else
@@ -347,7 +354,15 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
   fused.do_relu = relu ? 1 : 0;
 }
 
+void Conv2DOpKernel::set_store_result(bool store) {
+  if (!store && !fused.enable) fail("Conv2D '" + name + "': only a fused conv may drop its own result");
+  store_result = store;
+  output_data->materialized = store;
+}
+
 void Conv2DOpKernel::clear_fusion() {
+  store_result = true;
+  output_data->materialized = true;
   fused = tpuhip_fused_add{};
   add_src.reset();
   add_dst.reset();

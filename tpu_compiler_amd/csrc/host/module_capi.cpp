@@ -81,6 +81,18 @@ int tpuhip_module_set_returns(tpuhip_module *m, const char *const *names, int n)
   })
 }
 
+int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value) {
+  GUARD(m, {
+    const std::string k = key ? key : "";
+    if (k == "fuse_eltwise")
+      m->interp->fuse_eltwise = value != 0;
+    else if (k == "keep_all_tensors")
+      m->interp->keep_all_tensors = value != 0;
+    else
+      throw std::runtime_error("tpuhip_module_set_option: unknown option '" + k + "'");
+  })
+}
+
 int tpuhip_module_load(tpuhip_module *m, const char *target_op) {
   GUARD(m, {
     m->interp->loadModule(m->desc, target_op ? target_op : "");

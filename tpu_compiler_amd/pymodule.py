@@ -94,6 +94,10 @@ class module:
         self._ck(self.lib.tpuhip_module_set_returns(self.h, ra, len(rets)))
         self._ck(self.lib.tpuhip_module_load(self.h, target_op.encode() if target_op else None))
 
+    def set_option(self, key, value):
+        """Options read at the next load(): "fuse_eltwise", "keep_all_tensors" (both default 1)."""
+        self._ck(self.lib.tpuhip_module_set_option(self.h, key.encode(), int(value)))
+
     # -- details ------------------------------------------------------------
     def get_input_details(self):
         out = {}
