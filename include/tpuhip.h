@@ -144,6 +144,23 @@ typedef struct {
 } tpuhip_fused_add;
 int tpuhip_conv2d_add_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                          const void *add_src, void *add_out, const tpuhip_fused_add *f);
+/* General form of what can ride in a dense conv's epilogue, in this order:
+ *   z0 = conv result                          -> y        (if not NULL)
+ *   z1 = lut ? lut[(uint8_t)z0] : z0          -> lut_out  (if not NULL)   [LutOpKernel and its
+ *        subclasses: core/activation.cpp:47-53, 126-153; core/clip.cpp:29-40]
+ *   z2 = add.enable ? EltwiseAdd(add_src, z1) -> add_out                  [core/eltwise.cpp:52-85]
+ * lut is a HOST table of 256 int8 entries indexed by the two's-complement byte of the input (passed by
+ * value to the kernel).  Only the LDS kernel variants can apply a table; the variant is chosen among them
+ * when the first use of the layer is this call. */
+typedef struct tpuhip_conv_post {
+  const int8_t *lut;
+  void *lut_out;
+  tpuhip_fused_add add;
+  const void *add_src;
+  void *add_out;
+} tpuhip_conv_post;
+int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+                          const tpuhip_conv_post *post);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */

@@ -174,6 +174,15 @@ public:
   // interpreter arranges this (it also silences the eltwise kernel).
   bool can_fuse_add() const;
   void fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift, bool relu);
+  // Fold a 256-entry table op on this conv's result (Lut / LeakyRelu / Clip kernels) into
+  // the epilogue, ahead of a fused add: invoke() then also writes dst = table[result].
+  bool can_fuse_lut() const;
+  void fuse_lut(const int8_t *table, SyncedData dst);
+  bool has_fused_lut() const { return lut_dst != nullptr; }
+  bool has_fused_add() const { return fused.enable != 0; }
+  // false: table[result] is not written (only the sum fused behind it)
+  void set_store_lut(bool store);
+  SyncedData final_result() const { return lut_dst ? lut_dst : output_data; }
   void clear_fusion();
   // false: the conv result itself is not written, only the fused sum (set by the module
   // interpreter when nothing else reads it and the caller asked for outputs only)
@@ -186,6 +195,9 @@ private:
   SyncedData add_src, add_dst;
   tpuhip_fused_add fused{};
   bool store_result = true;
+  SyncedData lut_dst;
+  int8_t lut_table[256];
+  bool store_lut = true;
 };
 
 class FullyConnectedOpKernel : public CPUOpKernel {  // core/fullyconnected.cpp
@@ -245,6 +257,10 @@ public:
   LutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
   void invoke() override;
   int8_t table[256];
+  // set by the module interpreter when the producing conv applies the table itself
+  bool fused_into_producer = false;
+  SyncedData input() const { return input_data; }
+  SyncedData result() const { return output_data; }
 
 protected:
   SyncedData input_data, output_data;

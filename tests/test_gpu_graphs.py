@@ -145,6 +145,36 @@ def test_fusion_on_and_off_give_the_same_tensors(monkeypatch):
         m.close()
 
 
+@pytest.mark.parametrize("builder,kw", [(graphs.cfg5_yolo_v3, dict(batch=1, hw=96)),
+                                        (graphs.cfg4_mobilenet_v2, dict(batch=2, hw=64)),
+                                        (graphs.cfg2_mobilenet_block, dict(batch=1))])
+def test_table_fusion_on_off_and_outputs_only_agree_with_the_oracle(monkeypatch, builder, kw):
+    """leaky-relu / clip tables ride in the producing conv; every variant gives the oracle's bytes"""
+    g = builder(**kw)
+    want = oracle_graph.run(g)
+    for fuse, keep in (("1", 1), ("0", 1), ("1", 0)):
+        monkeypatch.setenv("TPUHIP_FUSE", fuse)
+        m = module()
+        m.set_option("keep_all_tensors", keep)
+        m.load(g)
+        m.set_tensor("input", g.input_op().data.astype(np.float32))
+        m.invoke()
+        launched = [a for _, a in m.kernels()]
+        checked = 0
+        for op in g.ops:
+            try:
+                got = m.get_tensor_i8(op.name)
+            except capi.TpuHipError as e:
+                assert keep == 0 and "never written" in str(e), (op.name, str(e))
+                continue
+            assert np.array_equal(got, want[op.name].reshape(op.shape)), (fuse, keep, op.name)
+            checked += 1
+        for name in g.outputs:
+            assert np.array_equal(m.get_tensor_i8(name), want[name].reshape(g.by_name[name].shape))
+        assert checked == len(g.ops) if keep else checked < len(g.ops)
+        m.close()
+
+
 def test_outputs_only_mode_skips_fused_conv_results_and_keeps_the_rest_exact():
     g = graphs.cfg3_resnet50(batch=2, hw=96)
     want = oracle_graph.run(g)

@@ -231,7 +231,7 @@ def test_conv_requant_edge_parameters(ctx, algo):
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("tile", [1, 4, 5, 6, 7, 10])
+@pytest.mark.parametrize("tile", [0, 2, 7, 9, 13, 16])   # persistent, wide K, one-tile, LDS-free, split K
 @pytest.mark.parametrize("relu,rs,keep_y", [(True, 6, True), (False, 0, True), (True, 9, False)])
 def test_conv_with_fused_eltwise_add(ctx, tile, relu, rs, keep_y):
     """conv + EltwiseAdd in one kernel == the two ops run one after the other"""
@@ -255,6 +255,56 @@ def test_conv_with_fused_eltwise_add(ctx, tile, relu, rs, keep_y):
         assert np.array_equal(ctx.to_nchw(yt), y_ref)
     else:
         assert (ctx.raw(yt) == 0x55).all()      # the conv result was not written
+    ctx.conv_weights_destroy(wh)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 3, 6, 9, 12])      # the variants with an LDS epilogue
+@pytest.mark.parametrize("with_add,keep_y,keep_lut", [(False, True, True), (False, False, True),
+                                                      (True, True, True), (True, False, False)])
+def test_conv_with_fused_table_and_add(ctx, tile, with_add, keep_y, keep_lut):
+    """conv -> 256-entry table -> EltwiseAdd in one kernel == the three ops one after the other"""
+    rng = np.random.default_rng(tile * 17 + with_add * 5 + keep_y)
+    x = rnd_i8(rng, (2, 48, 13, 11))
+    w = rnd_w(rng, (72, 48, 3, 3))                # 72 channels: 8 pad channels in the last group
+    bias, rsh, mult = rnd_params(rng, 72)
+    table = rnd_i8(rng, 256)
+    table[0] = 77                                  # pad channels must stay 0 all the same
+    other = rnd_i8(rng, (2, 72, 13, 11))
+    y_ref = oracle_conv(x, w, bias, rsh, mult, 1, (1, 1), (1, 1, 1, 1))
+    t_ref = O.lut_i8(y_ref, table)
+    z_ref = O.eltwise_add_i8([other, t_ref], [37, 51], [6], True)
+    d = conv_desc(x.shape, w.shape, pads=(1, 1, 1, 1), algo=16 + tile)
+    xt, ot = ctx.from_nchw(x), ctx.from_nchw(other)
+    yt, tt, zt = ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape)
+    for t in (yt, tt, zt):
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, t.ptr, 0x55, t.nbytes))
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    ctx.conv_post(wh, xt, yt if keep_y else None, table, tt if keep_lut else None,
+                  (ot, zt, 37, 51, 6, True) if with_add else None)
+    if keep_y:
+        assert np.array_equal(ctx.to_nchw(yt), y_ref)
+    else:
+        assert (ctx.raw(yt) == 0x55).all()
+    if keep_lut:
+        assert np.array_equal(ctx.to_nchw(tt), t_ref)
+        assert not ctx.raw(tt)[..., 72:].any()
+    else:
+        assert (ctx.raw(tt) == 0x55).all()
+    if with_add:
+        assert np.array_equal(ctx.to_nchw(zt), z_ref)
+        assert not ctx.raw(zt)[..., 72:].any()
+    ctx.conv_weights_destroy(wh)
+
+
+def test_conv_table_fusion_needs_an_lds_variant(ctx):
+    d = conv_desc((1, 32, 6, 6), (32, 32, 1, 1), algo=16 + 13)      # LDS-free variant
+    wh = ctx.conv_prepack(d, np.ones((32, 32, 1, 1), np.int8), None, np.full(32, 1 << 30, np.int32),
+                          np.full(32, 8, np.int32))
+    xt, yt = ctx.tensor((1, 32, 6, 6)), ctx.tensor((1, 32, 6, 6))
+    with pytest.raises(capi.TpuHipError, match="cannot fuse a table"):
+        ctx.conv_post(wh, xt, yt, np.zeros(256, np.int8), yt)
+    with pytest.raises(capi.TpuHipError, match="nothing would be written"):
+        ctx.conv_post(wh, xt, None)
     ctx.conv_weights_destroy(wh)
 
 

@@ -20,6 +20,11 @@ class FusedAdd(C.Structure):
     _fields_ = [(k, C.c_int) for k in ("enable", "m_src", "m_conv", "rshift", "do_relu")]
 
 
+class ConvPost(C.Structure):
+    _fields_ = [("lut", C.c_void_p), ("lut_out", C.c_void_p), ("add", FusedAdd),
+                ("add_src", C.c_void_p), ("add_out", C.c_void_p)]
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
@@ -61,6 +66,7 @@ PROTOTYPES = {
     "tpuhip_conv2d_algo_name": (C.c_char_p, [C.c_void_p]),
     "tpuhip_conv2d_tile_name": (C.c_char_p, [C.c_int]),
     "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
+    "tpuhip_conv2d_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost)]),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
                                                                    c_void_pp]),
@@ -290,6 +296,22 @@ class Context:
         f = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(do_relu))
         self._ck(self.lib.tpuhip_conv2d_add_i8(self.h, w, x.ptr, None if y is None else y.ptr,
                                                add_src.ptr, add_out.ptr, C.byref(f)))
+
+    def conv_post(self, w, x, y=None, table=None, lut_out=None, add=None):
+        """conv, then the optional table, then the optional add = (src, out, m_src, m_conv, rshift, relu)"""
+        p = ConvPost()
+        t = None
+        if table is not None:
+            t = np.ascontiguousarray(table, dtype=np.int8)
+            assert t.size == 256
+            p.lut = t.ctypes.data
+            p.lut_out = None if lut_out is None else lut_out.ptr
+        if add is not None:
+            src, out, m_src, m_conv, rshift, relu = add
+            p.add = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(relu))
+            p.add_src, p.add_out = src.ptr, out.ptr
+        self._ck(self.lib.tpuhip_conv2d_post_i8(self.h, w, x.ptr, None if y is None else y.ptr,
+                                                C.byref(p)))
 
     def conv_algo_name(self, w):
         return self.lib.tpuhip_conv2d_algo_name(w).decode()

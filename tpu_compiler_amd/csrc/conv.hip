@@ -79,7 +79,12 @@ struct ConvArgs {
   const int8_t *add_src;
   int8_t *add_dst;
   int add_m_src, add_m_conv, add_rshift, add_relu;
-  int store_y;     // 0: the conv result itself is not written (only the fused sum)
+  int store_y;     // 0: the conv result itself is not written (only what is fused behind it)
+  // optional fused 256-entry table on the conv result, applied before the fused add:
+  // lut_dst (may be null) receives table[y]; the add then takes table[y]
+  int has_lut;
+  int8_t *lut_dst;
+  Table256 lut;
 };
 
 __device__ __forceinline__ int32_t epilogue(int32_t acc, int32_t bias, const QParam &p, int lo,
@@ -245,7 +250,7 @@ template <int TN, bool FAST>
 __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
                                               const int32_t *pmult, const int32_t *pshift,
                                               const int32_t *phpot, int pix_first,
-                                              int pix_stride) {
+                                              int pix_stride, const uint8_t *lut = nullptr) {
   uint32_t outw[TN][4];
   // the other operand of a fused add is fetched now and used after the requantisation
   v4i sv[TN];
@@ -282,6 +287,21 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
       const int64_t off = (int64_t)pix * a.y_cs + oc;
       v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
       if (a.store_y) *reinterpret_cast<v4i *>(a.y + off) = o;
+      if (lut) {
+        // table lookup per byte (index = the two's-complement byte); the 256-byte table
+        // covers each LDS bank once, so any 64 indices are conflict-free.  Pad channels
+        // stay zero whatever table[0] is.
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t wd = (uint32_t)o[q];
+          const uint32_t r = (uint32_t)lut[wd & 255u] | ((uint32_t)lut[(wd >> 8) & 255u] << 8) |
+                             ((uint32_t)lut[(wd >> 16) & 255u] << 16) | ((uint32_t)lut[wd >> 24] << 24);
+          const int valid = a.oc - (oc + q * 4);   // channels of this dword that exist
+          const uint32_t mask = valid >= 4 ? 0xffffffffu : valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
+          o[q] = (int)(r & mask);
+        }
+        if (a.lut_dst) *reinterpret_cast<v4i *>(a.lut_dst + off) = o;
+      }
       if (a.add_dst) {
         // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
         // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
@@ -359,6 +379,7 @@ conv_mfma_kernel(ConvArgs a) {
   __shared__ v4i lds[2][(BM + BN) * CH];
   // bias | multiplier | rshift | 2^(rshift-1) of the workgroup's BM channels
   __shared__ __attribute__((aligned(16))) int32_t qlds[PERSIST ? 4 * BM : 4];
+  __shared__ uint32_t lutw[64];   // fused table (published by the first barrier of the K loop)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -379,6 +400,8 @@ conv_mfma_kernel(ConvArgs a) {
   const __amdgpu_buffer_rsrc_t wrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
 
+  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
   // requant parameters of the channel tile: fetched now, parked in LDS after the first
   // tile loads have been issued (their latencies overlap instead of adding up)
   static_assert(!PERSIST || BM <= NT, "one parameter row per thread");
@@ -639,10 +662,10 @@ conv_mfma_kernel(ConvArgs a) {
       if (oc < a.ocw) {
         if (PERSIST)
           epilogue_rows<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc,
-                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32);
+                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32, lut);
         else
           epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
-                                  pix_done + wn * TN * 32 + frow, 32);
+                                  pix_done + wn * TN * 32 + frow, 32, lut);
       }
     }
     if (!PERSIST || !more) break;
@@ -1220,6 +1243,9 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
   return TPUHIP_OK;
 }
 
+// the fused table lives in the LDS of the LDS kernels
+bool tile_has_lds_epilogue(int t) { return kTiles[t].reg == 0 || kTiles[t].reg == 3; }
+
 bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
   if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
@@ -1298,15 +1324,30 @@ void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvA
 
 // Times every candidate tile on the layer's real buffers (the kernels are
 // idempotent and bit-identical across tiles) and keeps the fastest.
-void apply_fusion(ConvArgs *a, const void *y, const void *add_src, void *add_out,
-                  const tpuhip_fused_add *f) {
-  if (!f || !f->enable) return;
-  a->add_src = (const int8_t *)add_src;
-  a->add_dst = (int8_t *)add_out;
-  a->add_m_src = f->m_src;
-  a->add_m_conv = f->m_conv;
-  a->add_rshift = f->rshift;
-  a->add_relu = f->do_relu ? 1 : 0;
+// what runs behind the requantisation in the epilogue
+struct PostOps {
+  const int8_t *lut = nullptr;   // host table, 256 entries
+  void *lut_out = nullptr;
+  const tpuhip_fused_add *f = nullptr;
+  const void *add_src = nullptr;
+  void *add_out = nullptr;
+  bool has_add() const { return f && f->enable; }
+};
+
+void apply_fusion(ConvArgs *a, const void *y, const PostOps &p) {
+  if (p.lut) {
+    a->has_lut = 1;
+    a->lut_dst = (int8_t *)p.lut_out;
+    memcpy(a->lut.w, p.lut, 256);
+  }
+  if (p.has_add()) {
+    a->add_src = (const int8_t *)p.add_src;
+    a->add_dst = (int8_t *)p.add_out;
+    a->add_m_src = p.f->m_src;
+    a->add_m_conv = p.f->m_conv;
+    a->add_rshift = p.f->rshift;
+    a->add_relu = p.f->do_relu ? 1 : 0;
+  }
   a->store_y = y != nullptr;
 }
 
@@ -1314,7 +1355,7 @@ void apply_fusion(ConvArgs *a, const void *y, const void *add_src, void *add_out
 // the tile shapes.  Every launch recomputes the same bytes, so repeating it is safe
 // as long as the sum is not written over its own input.
 int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *y,
-                  const void *add_src, void *add_out, const tpuhip_fused_add *f) {
+                  const PostOps &post) {
   hipEvent_t e0, e1;
   TPUHIP_CHECK_HIP(hipEventCreate(&e0));
   TPUHIP_CHECK_HIP(hipEventCreate(&e1));
@@ -1323,11 +1364,12 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
   int rc = TPUHIP_OK;
   for (int t = 0; t < kNumTiles && !rc; ++t) {
     if (!tile_is_candidate(w->d, t)) continue;
+    if (post.lut && !tile_has_lds_epilogue(t)) continue;
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
     fill_args(ctx, w, x, y, &a);
-    apply_fusion(&a, y, add_src, add_out, f);
+    apply_fusion(&a, y, post);
     for (int i = 0; i < 2; ++i) launch_conv_mfma(ctx, w, a);
     hipEventRecord(e0, ctx->stream);
     for (int i = 0; i < 5; ++i) launch_conv_mfma(ctx, w, a);
@@ -1515,23 +1557,27 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
 }
 
 static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
-                    const void *add_src, void *add_out, const tpuhip_fused_add *f) {
+                    const PostOps &post) {
   if (w->algo == ALGO_MFMA && !w->tuned) {
-    // first use: pick the tile by measurement (not capturable into a HIP graph)
-    const bool fused = f && f->enable && add_out != add_src;
+    // first use: pick the tile by measurement (not capturable into a HIP graph).  The
+    // fused work is timed with it unless the sum would overwrite its own operand.
+    PostOps tp = post;
+    if (tp.has_add() && tp.add_out == tp.add_src) tp.f = nullptr;
     void *ty = y;
-    if (!ty && !fused) {   // tuning writes the plain conv result somewhere: borrow a buffer
+    if (!ty && !tp.has_add() && !(tp.lut && tp.lut_out)) {
+      // tuning writes the plain conv result somewhere: borrow a buffer
       const size_t bytes = (size_t)w->d.n * w->d.oh * w->d.ow * w->d.y_cs;
       if (int rc = tpuhip_malloc(ctx, bytes, &ty)) return rc;
     }
-    int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, ty, add_src, add_out,
-                           fused ? f : nullptr);
+    int rc = autotune_mfma(ctx, const_cast<tpuhip_conv_weights *>(w), x, ty, tp);
     if (ty != y) tpuhip_free(ctx, ty);
     if (rc) return rc;
   }
+  TPUHIP_REQUIRE(!post.lut || (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
+                 "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
   ConvArgs a;
   fill_args(ctx, w, x, y, &a);
-  apply_fusion(&a, y, add_src, add_out, f);
+  apply_fusion(&a, y, post);
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
@@ -1549,18 +1595,48 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
 
 int tpuhip_conv2d_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_conv2d_i8: NULL argument");
-  return run_conv(ctx, w, x, y, nullptr, nullptr, nullptr);
+  return run_conv(ctx, w, x, y, PostOps{});
+}
+
+static int check_fused_add(const tpuhip_conv_weights *w, const void *add_src, const void *add_out,
+                           const tpuhip_fused_add *f) {
+  TPUHIP_REQUIRE(add_src && add_out, "conv2d fused add: NULL operand");
+  TPUHIP_REQUIRE(w->algo == ALGO_MFMA, "conv2d fused add: only dense convs on the MFMA path can fuse an add");
+  TPUHIP_REQUIRE(f->rshift >= 0 && f->rshift <= 30, "conv2d fused add: rshift %d outside [0,30]", f->rshift);
+  TPUHIP_REQUIRE(f->m_src >= -128 && f->m_src <= 127 && f->m_conv >= -128 && f->m_conv <= 127,
+                 "conv2d fused add: multipliers must be int8");
+  return TPUHIP_OK;
 }
 
 int tpuhip_conv2d_add_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                          const void *add_src, void *add_out, const tpuhip_fused_add *f) {
-  TPUHIP_REQUIRE(ctx && w && x && add_src && add_out && f, "tpuhip_conv2d_add_i8: NULL argument");
-  TPUHIP_REQUIRE(w->algo == ALGO_MFMA, "conv2d_add: only dense convs on the MFMA path can fuse an add");
+  TPUHIP_REQUIRE(ctx && w && x && f, "tpuhip_conv2d_add_i8: NULL argument");
   TPUHIP_REQUIRE(f->enable, "conv2d_add: fusion descriptor not enabled");
-  TPUHIP_REQUIRE(f->rshift >= 0 && f->rshift <= 30, "conv2d_add: rshift %d outside [0,30]", f->rshift);
-  TPUHIP_REQUIRE(f->m_src >= -128 && f->m_src <= 127 && f->m_conv >= -128 && f->m_conv <= 127,
-                 "conv2d_add: multipliers must be int8");
-  return run_conv(ctx, w, x, y, add_src, add_out, f);
+  if (int rc = check_fused_add(w, add_src, add_out, f)) return rc;
+  PostOps p;
+  p.f = f;
+  p.add_src = add_src;
+  p.add_out = add_out;
+  return run_conv(ctx, w, x, y, p);
+}
+
+int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
+                          const tpuhip_conv_post *post) {
+  TPUHIP_REQUIRE(ctx && w && x && post, "tpuhip_conv2d_post_i8: NULL argument");
+  PostOps p;
+  if (post->lut) {
+    TPUHIP_REQUIRE(w->algo == ALGO_MFMA, "conv2d_post: only dense convs on the MFMA path can fuse a table");
+    p.lut = post->lut;
+    p.lut_out = post->lut_out;
+  }
+  if (post->add.enable) {
+    if (int rc = check_fused_add(w, post->add_src, post->add_out, &post->add)) return rc;
+    p.f = &post->add;
+    p.add_src = post->add_src;
+    p.add_out = post->add_out;
+  }
+  TPUHIP_REQUIRE(y || p.lut_out || p.add_out, "conv2d_post: nothing would be written");
+  return run_conv(ctx, w, x, y, p);
 }
 
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,

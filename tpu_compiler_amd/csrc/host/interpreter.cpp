@@ -53,18 +53,21 @@ void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
   fuseKernels();
 }
 
-// A two-input EltwiseAdd whose later-produced input comes from a dense conv is
-// computed in that conv's epilogue (same bytes, one kernel and one read of the conv
-// result fewer).  Recomputed from scratch on every load so that rebuilt kernels
-// never keep stale links.
+// Work that rides in a dense conv's epilogue instead of running as a kernel of its own
+// (same bytes, fewer launches and fewer passes over the tensors):
+//  * a table op (Lut / LeakyRelu / Clip) whose input is the conv result;
+//  * a two-input EltwiseAdd whose later-produced input is the conv's final result
+//    (after the fused table, if any).
+// Recomputed from scratch on every load so that rebuilt kernels never keep stale links.
 void ModuleInterpreter::fuseKernels() {
-  std::map<TensorData *, std::pair<int, Conv2DOpKernel *>> producer;   // tensor -> (position, conv)
+  std::map<TensorData *, std::pair<int, Conv2DOpKernel *>> producer;   // final result -> (position, conv)
   std::map<TensorData *, int> position;                               // tensor -> producing position
   std::vector<Conv2DOpKernel *> fused_convs;
   int pos = 0;
   for (auto &k : kernel_list_) {
     if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) c->clear_fusion();
     if (auto *e = dynamic_cast<EltwiseAddOpKernel *>(k.get())) e->fused_into_producer = false;
+    if (auto *l = dynamic_cast<LutOpKernel *>(k.get())) l->fused_into_producer = false;
   }
   const char *env = getenv("TPUHIP_FUSE");
   if (!fuse_eltwise || (env && atoi(env) == 0)) return;
@@ -73,6 +76,20 @@ void ModuleInterpreter::fuseKernels() {
     if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) {
       producer[c->result().get()] = {pos, c};
       position[c->result().get()] = pos;
+      continue;
+    }
+    if (auto *l = dynamic_cast<LutOpKernel *>(k.get())) {
+      position[l->result().get()] = pos;
+      auto it = producer.find(l->input().get());
+      if (it == producer.end() || !it->second.second->can_fuse_lut()) continue;
+      Conv2DOpKernel *conv = it->second.second;
+      if (conv->result().get() != l->input().get()) continue;
+      const int conv_pos = it->second.first;
+      conv->fuse_lut(l->table, l->result());
+      l->fused_into_producer = true;
+      producer.erase(it);
+      producer[l->result().get()] = {conv_pos, conv};   // an add may follow the table
+      fused_convs.push_back(conv);
       continue;
     }
     auto *e = dynamic_cast<EltwiseAddOpKernel *>(k.get());
@@ -101,20 +118,30 @@ void ModuleInterpreter::fuseKernels() {
     conv->fuse_add(e->inputs()[1 - conv_idx], e->result(), e->multipliers()[1 - conv_idx],
                    e->multipliers()[conv_idx], e->rshift_value(), e->relu());
     e->fused_into_producer = true;
-    producer.erase(e->inputs()[conv_idx].get());   // one fusion per conv
-    fused_convs.push_back(conv);
+    producer.erase(e->inputs()[conv_idx].get());   // one add per conv
+    if (std::find(fused_convs.begin(), fused_convs.end(), conv) == fused_convs.end())
+      fused_convs.push_back(conv);
   }
   if (keep_all_tensors) return;
-  // outputs only: a fused conv whose result has no reader but the add, and is not a
-  // module output, need not write it
+  // outputs only: an intermediate of a fused chain that nothing else reads, and that is
+  // not a module output, need not be written
   std::map<TensorData *, int> readers;
+  std::map<TensorData *, std::string> tensor_name;
   for (auto &k : kernel_list_)
     for (auto &opd : k->operands())
       if (opd.act) ++readers[opd.act.get()];
+  for (auto &kv : activationMapping) tensor_name[kv.second.get()] = kv.first;
+  auto droppable = [&](TensorData *t) {
+    const bool is_output = std::find(output_details.begin(), output_details.end(),
+                                     tensor_name[t]) != output_details.end();
+    return !is_output && readers[t] == 1;
+  };
   for (Conv2DOpKernel *conv : fused_convs) {
-    const bool is_output =
-        std::find(output_details.begin(), output_details.end(), conv->name) != output_details.end();
-    if (!is_output && readers[conv->result().get()] == 1) conv->set_store_result(false);
+    // the one reader of the conv result is the fused table op or the fused add
+    if (droppable(conv->result().get())) conv->set_store_result(false);
+    if (conv->has_fused_lut() && conv->final_result().get() != conv->result().get() &&
+        conv->has_fused_add() && droppable(conv->final_result().get()))
+      conv->set_store_lut(false);
   }
 }
 
@@ -302,7 +329,9 @@ std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_
     std::vector<bool> launched(nk, false);
     for (auto &krnl : kernel_list_) {
       auto *el = dynamic_cast<EltwiseAddOpKernel *>(krnl.get());
-      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) || (el && el->fused_into_producer));
+      auto *lu = dynamic_cast<LutOpKernel *>(krnl.get());
+      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) ||
+                          (el && el->fused_into_producer) || (lu && lu->fused_into_producer));
       if (runs) ck(tpuhip_ctx_set_kernel_events(ctx_, e0[i], e1[i]), "timeKernels");
       krnl->invoke();
       launched[i] = runs;

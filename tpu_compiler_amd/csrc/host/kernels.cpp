@@ -326,13 +326,23 @@ Conv2DOpKernel::~Conv2DOpKernel() {
 }
 
 void Conv2DOpKernel::invoke() {
-  if (fused.enable)
-    ck(tpuhip_conv2d_add_i8(ctx, packed, input_data->data(),
-                            store_result ? output_data->data() : nullptr, add_src->data(),
-                            add_dst->data(), &fused),
-       name.c_str());
-  else
+  if (!fused.enable && !lut_dst) {
     ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+    return;
+  }
+  tpuhip_conv_post post{};
+  if (lut_dst) {
+    post.lut = lut_table;
+    post.lut_out = store_lut ? lut_dst->data() : nullptr;
+  }
+  if (fused.enable) {
+    post.add = fused;
+    post.add_src = add_src->data();
+    post.add_out = add_dst->data();
+  }
+  ck(tpuhip_conv2d_post_i8(ctx, packed, input_data->data(),
+                           store_result ? output_data->data() : nullptr, &post),
+     name.c_str());
 }
 
 bool Conv2DOpKernel::can_fuse_add() const {
@@ -354,8 +364,26 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
   fused.do_relu = relu ? 1 : 0;
 }
 
+bool Conv2DOpKernel::can_fuse_lut() const { return can_fuse_add() && !lut_dst && !fused.enable; }
+
+void Conv2DOpKernel::fuse_lut(const int8_t *table, SyncedData dst) {
+  if (!dst || dst->slot_bytes() != output_data->slot_bytes() || dst->cs != output_data->cs)
+    fail("Conv2D '" + name + "': a fused table's result must match the conv result's shape");
+  memcpy(lut_table, table, 256);
+  lut_dst = dst;
+  store_lut = true;
+}
+
+void Conv2DOpKernel::set_store_lut(bool store) {
+  if (!lut_dst || (!store && !fused.enable))
+    fail("Conv2D '" + name + "': only a table with an add fused behind it may go unwritten");
+  store_lut = store;
+  lut_dst->materialized = store;
+}
+
 void Conv2DOpKernel::set_store_result(bool store) {
-  if (!store && !fused.enable) fail("Conv2D '" + name + "': only a fused conv may drop its own result");
+  if (!store && !fused.enable && !lut_dst)
+    fail("Conv2D '" + name + "': only a fused conv may drop its own result");
   store_result = store;
   output_data->materialized = store;
 }
@@ -363,6 +391,9 @@ void Conv2DOpKernel::set_store_result(bool store) {
 void Conv2DOpKernel::clear_fusion() {
   store_result = true;
   output_data->materialized = true;
+  if (lut_dst) lut_dst->materialized = true;
+  lut_dst.reset();
+  store_lut = true;
   fused = tpuhip_fused_add{};
   add_src.reset();
   add_dst.reset();
@@ -526,6 +557,7 @@ LutOpKernel::LutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &we
 }
 
 void LutOpKernel::invoke() {
+  if (fused_into_producer) return;   // the conv that produces the input applies the table
   ck(tpuhip_lut_i8(ctx, input_data->data(), output_data->data(), table,
                    (size_t)input_data->n * input_data->h * input_data->w, input_data->c,
                    input_data->cs),
