@@ -164,6 +164,9 @@ DEPTHWISE = [
     (1, 24, 9, 9, 3, (1, 1), (1, 1, 1, 1), False),       # 24 channels: padded group
     (1, 32, 12, 12, 5, (1, 1), (2, 2, 2, 2), False),
     (1, 16, 7, 7, 7, (1, 1), (0, 0, 0, 0), False),       # global depthwise
+    (1, 48, 10, 9, 2, (1, 1), (0, 1, 0, 1), True),       # 2x2: a single tap group
+    (16, 96, 112, 112, 3, (1, 1), (1, 1, 1, 1), True),   # more pixels than lanes: every lane walks
+    (3, 40, 23, 17, 3, (2, 1), (1, 1, 1, 1), False),     # mixed strides, ragged everything
 ]
 
 
@@ -180,6 +183,31 @@ def test_conv_depthwise(ctx, case, algo):
                          do_relu=relu)
     assert np.array_equal(got, want), name
     assert len(np.unique(want)) > 8
+
+
+def test_conv_depthwise_dilated_general_requant_and_fused_table(ctx):
+    rng = np.random.default_rng(77)
+    x = rnd_i8(rng, (2, 40, 14, 13))
+    w = rnd_w(rng, (40, 1, 3, 3), 24)
+    bias, rsh, mult = rnd_params(rng, 40, 5, 12, 2048)
+    rsh[3] = 0                                         # forces the general rounding form
+    want = oracle_conv(x, w, bias, rsh, mult, 40, (1, 1), (2, 2, 2, 2), (2, 2), (0, 0), True)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, g=40, pads=(2, 2, 2, 2), dil=(2, 2), do_relu=True)
+    assert name == "depthwise" and np.array_equal(got, want)
+    # the same layer with a table behind it, in one kernel
+    table = rnd_i8(rng, 256)
+    table[0] = -5
+    d = conv_desc(x.shape, w.shape, g=40, pads=(2, 2, 2, 2), dil=(2, 2), do_relu=True)
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    xt, yt, tt = ctx.from_nchw(x), ctx.tensor(want.shape), ctx.tensor(want.shape)
+    ctx.conv_post(wh, xt, yt, table, tt)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert np.array_equal(ctx.to_nchw(tt), O.lut_i8(want, table))
+    assert not ctx.raw(tt)[..., 40:].any()
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.conv_post(wh, xt, None, table, tt)
+    assert (ctx.raw(yt) == 0x55).all()
+    ctx.conv_weights_destroy(wh)
 
 
 def test_conv_grouped_and_inserted_zeros_direct(ctx):

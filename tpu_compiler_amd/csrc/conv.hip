@@ -133,58 +133,8 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(ConvArgs a) {
   }
 }
 
-// ---------------------------------------------------------------------------
-// depthwise kernel: one thread per (pixel, 16-channel group).  Filter layout
-// [kh][kw][ocw] (channel fastest, zero in the pad channels).
-// ---------------------------------------------------------------------------
 __device__ __forceinline__ int32_t sbyte(int32_t word, int i) {
   return (int32_t)(int8_t)(word >> (8 * i));
-}
-
-__global__ __launch_bounds__(256) void conv_depthwise_kernel(ConvArgs a) {
-  const int c16 = a.ocw >> 4;
-  const int64_t total = (int64_t)a.npix * c16;
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (int64_t)gridDim.x * blockDim.x) {
-    const int cg = (int)(idx % c16);
-    const int pix = (int)(idx / c16);
-    const int ow = pix % a.ow;
-    const int oh = (pix / a.ow) % a.oh;
-    const int n = pix / (a.ow * a.oh);
-    int32_t acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0;
-    for (int kh = 0; kh < a.kh; ++kh) {
-      const int ih = oh * a.sh - a.pt + kh * a.dh;
-      if (ih < 0 || ih >= a.ih) continue;
-      for (int kw = 0; kw < a.kw; ++kw) {
-        const int iw = ow * a.sw - a.pl + kw * a.dw;
-        if (iw < 0 || iw >= a.iw) continue;
-        const v4i xv = *reinterpret_cast<const v4i *>(
-            a.x + ((int64_t)(n * a.ih + ih) * a.iw + iw) * a.x_cs + cg * 16);
-        const v4i wv = *reinterpret_cast<const v4i *>(
-            a.w + ((int64_t)(kh * a.kw + kw)) * a.ocw + cg * 16);
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int b = 0; b < 4; ++b) acc[q * 4 + b] += sbyte(xv[q], b) * sbyte(wv[q], b);
-      }
-    }
-    v4i out;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      uint32_t word = 0;
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int c = cg * 16 + q * 4 + b;
-        int32_t v = 0;
-        if (c < a.oc) v = epilogue(acc[q * 4 + b], a.bias[c], a.qp[c], a.lo, a.relu_first);
-        word |= ((uint32_t)v & 0xffu) << (8 * b);
-      }
-      out[q] = (int)word;
-    }
-    *reinterpret_cast<v4i *>(a.y + (int64_t)pix * a.y_cs + cg * 16) = out;
-  }
 }
 
 // ---------------------------------------------------------------------------
@@ -348,6 +298,141 @@ __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32
   return (v4i)__builtin_amdgcn_raw_buffer_load_b128(rsrc, offset, 0, 0);
 }
 constexpr uint32_t kOobOffset = 0x7fffffffu;
+
+// ---------------------------------------------------------------------------
+// depthwise kernel (g == ic == oc).  A lane owns 16 channels and walks pixels with a
+// fixed stride, so its filter taps and requant parameters stay in registers.  The
+// multiply-adds run as 4 x int8 dot products over FOUR TAPS of one channel: the four
+// 16-byte loads of a tap group are byte-transposed (8 v_perm per 4 channels) into one
+// dword per channel, and the filter is stored the same way, [tap group][channel] ->
+// 4 taps.  Taps outside the image read zeros through the buffer descriptor.
+// G = tap groups held in registers (kh*kw <= 4*G); G == 0 streams the filter instead.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void transpose4x4_bytes(uint32_t t0, uint32_t t1, uint32_t t2,
+                                                   uint32_t t3, uint32_t (&c)[4]) {
+  const uint32_t ab_lo = __builtin_amdgcn_perm(t1, t0, 0x05010400u);   // a0 b0 a1 b1
+  const uint32_t ab_hi = __builtin_amdgcn_perm(t1, t0, 0x07030602u);   // a2 b2 a3 b3
+  const uint32_t cd_lo = __builtin_amdgcn_perm(t3, t2, 0x05010400u);
+  const uint32_t cd_hi = __builtin_amdgcn_perm(t3, t2, 0x07030602u);
+  c[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);             // a0 b0 c0 d0
+  c[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);
+  c[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);
+  c[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);
+}
+
+template <int G, bool FAST>
+__global__ __launch_bounds__(256) void conv_depthwise_kernel(ConvArgs a) {
+  __shared__ uint32_t lutw[64];
+  if (a.has_lut) {
+    if (threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+    __syncthreads();
+  }
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  const int c16 = a.ocw >> 4;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int nslots = (int)(((int64_t)gridDim.x * blockDim.x) / c16);   // pixels in flight
+  const int cg = (int)(gid % c16);
+  int pix = (int)(gid / c16);
+  if (pix >= nslots) return;
+  const int groups = (a.kh * a.kw + 3) >> 2;
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+
+  // per-channel constants of this lane's 16 channels
+  v4i wq[G > 0 ? G : 1][4], bias4[4], mult4[4], shift4[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    bias4[q] = *reinterpret_cast<const v4i *>(a.bias + cg * 16 + q * 4);
+    mult4[q] = *reinterpret_cast<const v4i *>(a.qmult + cg * 16 + q * 4);
+    shift4[q] = *reinterpret_cast<const v4i *>(a.qshift + cg * 16 + q * 4);
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+      wq[g][q] = *reinterpret_cast<const v4i *>(a.w + ((int64_t)g * a.ocw + cg * 16 + q * 4) * 4);
+  }
+
+  // (n, oh, ow) of the lane's pixel, advanced by the walk's stride with carries
+  int ow = pix % a.ow;
+  int oh = (pix / a.ow) % a.oh;
+  int n = pix / (a.ow * a.oh);
+  const int d_ow = nslots % a.ow, d_oh = (nslots / a.ow) % a.oh, d_n = nslots / (a.ow * a.oh);
+
+  for (; pix < a.npix; pix += nslots) {
+    const int ihb = oh * a.sh - a.pt, iwb = ow * a.sw - a.pl;
+    const int base = ((n * a.ih + ihb) * a.iw + iwb) * a.x_cs + cg * 16;
+    int32_t acc[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[q * 4 + i] = bias4[q][i];
+    auto tap_group = [&](int g, const v4i (&wg)[4]) {
+      v4i t[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t tap = (uint32_t)(g * 4 + k);
+        const int tkh = (int)((tap * a.magic_kw) >> 20);
+        const int tkw = (int)tap - tkh * a.kw;
+        const int ih = ihb + tkh * a.dh, iw = iwb + tkw * a.dw;
+        const bool ok = ((int)tap < a.kh * a.kw) & ((unsigned)ih < (unsigned)a.ih) &
+                        ((unsigned)iw < (unsigned)a.iw);
+        t[k] = buffer_load16(xrsrc, ok ? (uint32_t)(base + (tkh * a.dh * a.iw + tkw * a.dw) * a.x_cs)
+                                       : kOobOffset);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        uint32_t c[4];
+        transpose4x4_bytes((uint32_t)t[0][q], (uint32_t)t[1][q], (uint32_t)t[2][q], (uint32_t)t[3][q], c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc[q * 4 + i] = __builtin_amdgcn_sdot4((int)c[i], wg[q][i], acc[q * 4 + i], false);
+      }
+    };
+    if (G > 0) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) tap_group(g, wq[g]);
+    } else {
+      for (int g = 0; g < groups; ++g) {
+        v4i wg[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          wg[q] = *reinterpret_cast<const v4i *>(a.w + ((int64_t)g * a.ocw + cg * 16 + q * 4) * 4);
+        tap_group(g, wg);
+      }
+    }
+    v4i o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int32_t r[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int32_t v = acc[q * 4 + i];
+        if (a.relu_first) v = max(v, 0);
+        const int32_t e = shift4[q][i];
+        r[i] = requant_core<FAST>(v, mult4[q][i], e, (int32_t)((1u << e) >> 1));
+      }
+      o[q] = (int)pack_sat4(r[0], r[1], r[2], r[3], a.lo);
+    }
+    const int64_t off = (int64_t)pix * a.y_cs + cg * 16;
+    if (a.store_y) *reinterpret_cast<v4i *>(a.y + off) = o;
+    if (lut) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t wd = (uint32_t)o[q];
+        const uint32_t r = (uint32_t)lut[wd & 255u] | ((uint32_t)lut[(wd >> 8) & 255u] << 8) |
+                           ((uint32_t)lut[(wd >> 16) & 255u] << 16) | ((uint32_t)lut[wd >> 24] << 24);
+        const int valid = a.oc - (cg * 16 + q * 4);
+        const uint32_t mask = valid >= 4 ? 0xffffffffu : valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
+        o[q] = (int)(r & mask);
+      }
+      if (a.lut_dst) *reinterpret_cast<v4i *>(a.lut_dst + off) = o;
+    }
+    ow += d_ow;
+    if (ow >= a.ow) { ow -= a.ow; ++oh; }
+    oh += d_oh;
+    if (oh >= a.oh) { oh -= a.oh; ++n; }
+    n += d_n;
+  }
+}
+
 
 // UNI: the input channel count is a multiple of 64, so the four 16-byte K groups of
 // a step lie in one filter tap and all tap arithmetic is wave-uniform (scalar).
@@ -1274,11 +1359,11 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.lo = (d.do_relu && !d.relu_first) ? 0 : -128;
   a.relu_first = (d.do_relu && d.relu_first) ? 1 : 0;
   a.store_y = 1;
+  a.magic_kw = (1u << 20) / (uint32_t)d.kw + 1;
+  a.x_bytes = (uint32_t)((int64_t)d.n * d.ih * d.iw * d.x_cs);
   if (w->algo == ALGO_MFMA) {
     const TileCfg &t = kTiles[w->tile];
     a.magic_c16 = (1u << 20) / (uint32_t)w->c16 + 1;
-    a.magic_kw = (1u << 20) / (uint32_t)d.kw + 1;
-    a.x_bytes = (uint32_t)((int64_t)d.n * d.ih * d.iw * d.x_cs);
     a.w_bytes = (uint32_t)((int64_t)w->ocp * w->kp);
     a.magic_ow = d.ow > 1 ? (uint32_t)(((1ull << 32) + d.ow - 1) / (uint64_t)d.ow) : 0;
     a.magic_oh = d.oh > 1 ? (uint32_t)(((1ull << 32) + d.oh - 1) / (uint64_t)d.oh) : 0;
@@ -1459,13 +1544,13 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
       cw->host_filter.shrink_to_fit();
     }
   } else if (algo == ALGO_DEPTHWISE) {
+    // [tap group][channel][4 taps]: one dword per channel and group of four taps
     cw->ocp = round_up(d.oc, 16);
-    packed.assign((size_t)d.kh * d.kw * cw->ocp, 0);
+    const int groups = std::max(3, (d.kh * d.kw + 3) / 4);   // the kernel holds three groups in registers
+    packed.assign((size_t)groups * cw->ocp * 4, 0);
     for (int c = 0; c < d.oc; ++c)
-      for (int kh = 0; kh < d.kh; ++kh)
-        for (int kw = 0; kw < d.kw; ++kw)
-          packed[(size_t)(kh * d.kw + kw) * cw->ocp + c] =
-              filter[((size_t)c * d.kh + kh) * d.kw + kw];
+      for (int tap = 0; tap < d.kh * d.kw; ++tap)
+        packed[((size_t)(tap / 4) * cw->ocp + c) * 4 + tap % 4] = filter[(size_t)c * d.kh * d.kw + tap];
   } else {
     cw->ocp = d.oc;
     packed.assign((size_t)d.oc * d.kh * d.kw * icg, 0);
@@ -1512,7 +1597,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   if (!rc) rc = tpuhip_malloc(ctx, qp.size() * sizeof(QParam), (void **)&cw->qp);
   if (!rc) rc = tpuhip_upload(ctx, cw->bias, b32.data(), b32.size() * sizeof(int32_t));
   if (!rc) rc = tpuhip_upload(ctx, cw->qp, qp.data(), qp.size() * sizeof(QParam));
-  if (!rc && algo == ALGO_MFMA) {
+  if (!rc && (algo == ALGO_MFMA || algo == ALGO_DEPTHWISE)) {
     std::vector<int32_t> planes(3 * nparam);
     for (size_t i = 0; i < nparam; ++i) {
       planes[i] = qp[i].mult;
@@ -1573,7 +1658,8 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     if (ty != y) tpuhip_free(ctx, ty);
     if (rc) return rc;
   }
-  TPUHIP_REQUIRE(!post.lut || (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
+  TPUHIP_REQUIRE(!post.lut || w->algo == ALGO_DEPTHWISE ||
+                     (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
                  "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
   ConvArgs a;
   fill_args(ctx, w, x, y, &a);
@@ -1581,9 +1667,19 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
+    // enough lanes to fill the chip a few times over; every lane then walks pixels
     const int64_t total = (int64_t)a.npix * (a.ocw / 16);
-    const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(total, 256), 1 << 20);
-    launch(ctx, conv_depthwise_kernel, dim3(blocks), dim3(256), a);
+    const unsigned blocks =
+        (unsigned)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(total, 256), (int64_t)ctx->num_cu * 16));
+    const int groups = (a.kh * a.kw + 3) / 4;
+    const dim3 grid(blocks), block(256);
+    if (groups <= 3) {
+      if (w->fast) launch(ctx, (conv_depthwise_kernel<3, true>), grid, block, a);
+      else launch(ctx, (conv_depthwise_kernel<3, false>), grid, block, a);
+    } else {
+      if (w->fast) launch(ctx, (conv_depthwise_kernel<0, true>), grid, block, a);
+      else launch(ctx, (conv_depthwise_kernel<0, false>), grid, block, a);
+    }
   } else {
     const int64_t total = (int64_t)a.npix * a.ocw;
     const unsigned blocks = (unsigned)std::min<int64_t>(ceil_div64(total, 256), 1 << 20);
@@ -1625,7 +1721,8 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
   TPUHIP_REQUIRE(ctx && w && x && post, "tpuhip_conv2d_post_i8: NULL argument");
   PostOps p;
   if (post->lut) {
-    TPUHIP_REQUIRE(w->algo == ALGO_MFMA, "conv2d_post: only dense convs on the MFMA path can fuse a table");
+    TPUHIP_REQUIRE(w->algo == ALGO_MFMA || w->algo == ALGO_DEPTHWISE,
+                   "conv2d_post: only dense convs on the MFMA path and depthwise convs can fuse a table");
     p.lut = post->lut;
     p.lut_out = post->lut_out;
   }

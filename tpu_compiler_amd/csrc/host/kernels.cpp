@@ -364,7 +364,10 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
   fused.do_relu = relu ? 1 : 0;
 }
 
-bool Conv2DOpKernel::can_fuse_lut() const { return can_fuse_add() && !lut_dst && !fused.enable; }
+bool Conv2DOpKernel::can_fuse_lut() const {
+  const std::string algo = tpuhip_conv2d_algo_name(packed);
+  return (algo.rfind("mfma", 0) == 0 || algo == "depthwise") && !lut_dst && !fused.enable;
+}
 
 void Conv2DOpKernel::fuse_lut(const int8_t *table, SyncedData dst) {
   if (!dst || dst->slot_bytes() != output_data->slot_bytes() || dst->cs != output_data->cs)
