@@ -1667,10 +1667,11 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
-    // enough lanes to fill the chip a few times over; every lane then walks pixels
+    // as many workgroups as are resident at once (3 per CU at this register count): every
+    // lane then walks pixels and its filter / parameter loads are paid once (measured best)
     const int64_t total = (int64_t)a.npix * (a.ocw / 16);
     const unsigned blocks =
-        (unsigned)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(total, 256), (int64_t)ctx->num_cu * 16));
+        (unsigned)std::max<int64_t>(1, std::min<int64_t>(ceil_div64(total, 256), (int64_t)ctx->num_cu * 3));
     const int groups = (a.kh * a.kw + 3) / 4;
     const dim3 grid(blocks), block(256);
     if (groups <= 3) {
