@@ -186,6 +186,28 @@ int tpuhip_eltwise_add_i8(tpuhip_ctx *ctx, const void *const *xs, int nin,
                           const int8_t *multiplier, int rshift, int do_relu, void *y,
                           size_t bytes);
 
+/* ---- two-input elementwise ops with broadcasting ------------------------------
+ * Replaces the INT8 branches of EltwiseMaxOpKernel / EltwiseMinOpKernel / EltwiseMulOpKernel
+ * (core/eltwise.cpp:143-189, 233-279, 324-347) and BroadcastAddOpKernel / BroadcastMulOpKernel /
+ * BroadcastSubOpKernel (core/broadcast.cpp:45-154).  Every dimension of an operand equals the
+ * output's or is 1.  add / sub / max / min: sat8(floor(relu?(op(x0*m0, x1*m1)) / 2^rshift + 0.5));
+ * mul: qdm(relu?(x0*x1), rshift, multiplier).  m0, m1 are the int8-converted multipliers,
+ * multiplier the uint32-converted one (as int32), rshift the uint32-converted shift. */
+enum { TPUHIP_BIN_ADD = 0, TPUHIP_BIN_SUB = 1, TPUHIP_BIN_MAX = 2, TPUHIP_BIN_MIN = 3, TPUHIP_BIN_MUL = 4 };
+typedef struct tpuhip_binary_desc {
+  int op;
+  int n, c, h, w;       /* output */
+  int n0, c0, h0, w0;   /* operand 0 */
+  int n1, c1, h1, w1;   /* operand 1 */
+  int m0, m1;
+  int32_t multiplier;
+  int rshift;
+  int do_relu;
+  int x0_cs, x1_cs, y_cs;
+} tpuhip_binary_desc;
+int tpuhip_binary_i8(tpuhip_ctx *ctx, const tpuhip_binary_desc *d, const void *x0, const void *x1,
+                     void *y);
+
 /* ---- Pooling -------------------------------------------------------------- */
 
 /* Field meaning follows parsePoolParam (TPUOperationSupport.cpp:479-522). */

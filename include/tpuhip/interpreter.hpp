@@ -234,6 +234,36 @@ private:
   bool do_relu = false;
 };
 
+// Two-input elementwise ops.  The Eltwise* classes take same-shape inputs followed by
+// [n+0]quant_scale [n+1]zeropoint [n+2]rshift [n+3]multiplier (core/eltwise.cpp:102-126);
+// the Broadcast* classes two inputs whose dimensions are the result's or 1, followed by
+// [2]scale [3]zeropoint [4]rshift [5]multiplier (core/broadcast.cpp:9-43).
+class BinaryOpKernel : public CPUOpKernel {
+public:
+  void invoke() override;
+
+protected:
+  BinaryOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping, int op_code,
+                 bool broadcast, const char *what);
+  tpuhip_binary_desc desc{};
+  SyncedData in0, in1, output_data;
+};
+
+#define TPUHIP_BINARY_KERNEL(Class, Name, code, bcast)                                        \
+  class Class : public BinaryOpKernel {                                                       \
+  public:                                                                                     \
+    static constexpr const char *OpName = Name;                                               \
+    Class(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)                 \
+        : BinaryOpKernel(op, valueMapping, weightMapping, code, bcast, Name) {}               \
+  };
+TPUHIP_BINARY_KERNEL(EltwiseMaxOpKernel, "CPUEltwiseMaxOp", TPUHIP_BIN_MAX, false)   // eltwise.cpp:102
+TPUHIP_BINARY_KERNEL(EltwiseMinOpKernel, "CPUEltwiseMinOp", TPUHIP_BIN_MIN, false)   // eltwise.cpp:192
+TPUHIP_BINARY_KERNEL(EltwiseMulOpKernel, "CPUEltwiseMulOp", TPUHIP_BIN_MUL, false)   // eltwise.cpp:282
+TPUHIP_BINARY_KERNEL(BroadcastAddOpKernel, "CPUBroadcastAddOp", TPUHIP_BIN_ADD, true)   // broadcast.cpp:45
+TPUHIP_BINARY_KERNEL(BroadcastMulOpKernel, "CPUBroadcastMulOp", TPUHIP_BIN_MUL, true)   // broadcast.cpp:90
+TPUHIP_BINARY_KERNEL(BroadcastSubOpKernel, "CPUBroadcastSubOp", TPUHIP_BIN_SUB, true)   // broadcast.cpp:117
+#undef TPUHIP_BINARY_KERNEL
+
 class PoolingOpKernel : public CPUOpKernel {  // core/pooling.cpp
 public:
   static constexpr const char *OpName = "CPUPoolingOp";

@@ -291,6 +291,46 @@ void orc_eltwise_add_i8(const int8_t *const *xs, int nin, const float *multiplie
   }
 }
 
+/* broadcast.cpp:60-75 index arithmetic; eltwise.cpp i8_invoke bodies for the
+ * same-shape case (every n_i == n etc.). */
+int orc_binary_i8(const int8_t *x0, const int8_t *x1, int8_t *y, const orc_binary_desc *d,
+                  const float *multiplier, float rshift) {
+  const uint32_t rs = orc_f2u32(rshift);
+  const uint32_t mq = orc_f2u32(multiplier[0]);
+  if (d->op == ORC_BIN_MUL && rs == 0 && mq == 0) return -1;
+  const int8_t m0 = d->op == ORC_BIN_MUL ? 0 : (int8_t)(int)multiplier[0];
+  const int8_t m1 = d->op == ORC_BIN_MUL ? 0 : (int8_t)(int)multiplier[1];
+#pragma omp parallel for collapse(2)
+  for (int n = 0; n < d->n; ++n)
+    for (int c = 0; c < d->c; ++c)
+      for (int h = 0; h < d->h; ++h)
+        for (int w = 0; w < d->w; ++w) {
+          const int64_t i0 = (((int64_t)(d->n0 == 1 ? 0 : n) * d->c0 + (d->c0 == 1 ? 0 : c)) * d->h0 +
+                              (d->h0 == 1 ? 0 : h)) * d->w0 + (d->w0 == 1 ? 0 : w);
+          const int64_t i1 = (((int64_t)(d->n1 == 1 ? 0 : n) * d->c1 + (d->c1 == 1 ? 0 : c)) * d->h1 +
+                              (d->h1 == 1 ? 0 : h)) * d->w1 + (d->w1 == 1 ? 0 : w);
+          const int64_t o = (((int64_t)n * d->c + c) * d->h + h) * d->w + w;
+          float a = (float)x0[i0], b = (float)x1[i1], v;
+          if (d->op == ORC_BIN_MUL) {
+            v = a * b;
+            if (d->do_relu) v = v > 0 ? v : 0;
+            y[o] = orc_apply_mult_rshift_sat8_f(v, rs, mq, 1);
+            continue;
+          }
+          a *= m0;
+          b *= m1;
+          switch (d->op) {
+            case ORC_BIN_ADD: v = a + b; break;
+            case ORC_BIN_SUB: v = a - b; break;
+            case ORC_BIN_MAX: v = a > b ? a : b; break;
+            default: v = a < b ? a : b; break;
+          }
+          if (d->do_relu) v = v > 0 ? v : 0;
+          y[o] = orc_apply_rshift_sat8(v, rs);
+        }
+  return 0;
+}
+
 /* ------------------------------------------------------------------------- */
 /* pooling                                                                    */
 /* ------------------------------------------------------------------------- */

@@ -91,6 +91,24 @@ int64_t orc_fc_guard(const int8_t *x, const int8_t *w, const float *bias, int ba
 void orc_eltwise_add_i8(const int8_t *const *xs, int nin, const float *multiplier,
                         const float *rshift, int do_relu, int8_t *y, size_t count);
 
+/* ---- two-input elementwise ops with broadcasting ----
+ * core/eltwise.cpp:143-189 (Max), 233-279 (Min), 324-347 (Mul) and core/broadcast.cpp:45-154
+ * (BroadcastAdd / Mul / Sub).  Every dimension of an operand equals the output's or is 1.
+ * add/sub/max/min: each input times (int8_t)multiplier[i] in float, combined, ReLU, then
+ * v / 2^rshift and floor(. + 0.5), saturate.  mul: product, ReLU, qdm requant with
+ * (uint32)rshift, (uint32)multiplier[0].  Returns -1 for the one case with no int8 meaning:
+ * an eltwise mul with rshift == 0 and multiplier == 0 (the reference leaves the raw product). */
+enum { ORC_BIN_ADD = 0, ORC_BIN_SUB = 1, ORC_BIN_MAX = 2, ORC_BIN_MIN = 3, ORC_BIN_MUL = 4 };
+typedef struct {
+  int op;
+  int n, c, h, w;       /* output */
+  int n0, c0, h0, w0;   /* operand 0 */
+  int n1, c1, h1, w1;   /* operand 1 */
+  int do_relu;
+} orc_binary_desc;
+int orc_binary_i8(const int8_t *x0, const int8_t *x1, int8_t *y, const orc_binary_desc *d,
+                  const float *multiplier, float rshift);
+
 /* ---- pooling: core/pooling.cpp:89-160 (normal path only) ---- */
 typedef struct {
   int n, c, ih, iw, oh, ow, kh, kw, sh, sw, pt, pb, pl, pr;

@@ -20,6 +20,11 @@ def _conv(op, x):
                        op.weights["multiplier"], d), d, w
 
 
+_BINARY = {"tpu.eltwise_max": O.BIN_MAX, "tpu.eltwise_min": O.BIN_MIN, "tpu.eltwise_mul": O.BIN_MUL,
+           "tpu.broadcast_add": O.BIN_ADD, "tpu.broadcast_sub": O.BIN_SUB,
+           "tpu.broadcast_mul": O.BIN_MUL}
+
+
 def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=None):
     """Returns {name: int8 NCHW array}.  batch_slice selects images (ops are
     independent across the batch, which is also how the reference runs a batch:
@@ -50,6 +55,12 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
         elif t == "tpu.eltwise_add":
             y = O.eltwise_add_i8(ins, op.weights["multiplier"], op.weights["rshift"],
                                  bool(op.attrs["do_relu"]))
+        elif t in _BINARY:
+            def nchw(a):
+                return a.reshape(a.shape + (1,) * (4 - a.ndim))
+            y = O.binary_i8(_BINARY[t], nchw(ins[0]), nchw(ins[1]), op.weights["multiplier"],
+                            op.weights["rshift"][0], bool(op.attrs.get("do_relu", 0)))
+            y = y.reshape(op.shape)
         elif t in ("tpu.pool_max_2d", "tpu.pool_avg_2d"):
             a = op.attrs
             d = O.make_pool_desc(ins[0].shape, (int(a["kernel_h"]), int(a["kernel_w"])),

@@ -26,6 +26,14 @@ class PoolDesc(C.Structure):
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr")]
 
 
+class BinaryDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in (
+        "op", "n", "c", "h", "w", "n0", "c0", "h0", "w0", "n1", "c1", "h1", "w1", "do_relu")]
+
+
+BIN_ADD, BIN_SUB, BIN_MAX, BIN_MIN, BIN_MUL = range(5)
+
+
 def build():
     subprocess.check_call(["make", "-s", "-C", ORACLE_DIR])
 
@@ -61,6 +69,8 @@ def _load():
     lib.orc_fc_guard.argtypes = [i8p, i8p, f32p] + [C.c_int] * 4
     lib.orc_eltwise_add_i8.argtypes = [C.POINTER(i8p), C.c_int, f32p, f32p, C.c_int, i8p,
                                        C.c_size_t]
+    lib.orc_binary_i8.restype = C.c_int
+    lib.orc_binary_i8.argtypes = [i8p, i8p, i8p, C.POINTER(BinaryDesc), f32p, C.c_float]
     lib.orc_pool_max_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc)]
     lib.orc_pool_avg_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc), C.c_float, C.c_float]
     lib.orc_leaky_relu_i8.argtypes = [i8p, i8p, C.c_size_t] + [C.c_float] * 4
@@ -178,6 +188,20 @@ def eltwise_add_i8(xs, multiplier, rshift, do_relu):
     m, r = _f32(multiplier), _f32(rshift)
     lib.orc_eltwise_add_i8(_ptr_array(xs), len(xs), _p(m, C.c_float), _p(r, C.c_float),
                            int(do_relu), _p(y, C.c_int8), xs[0].size)
+    return y
+
+
+def binary_i8(op, x0, x1, multiplier, rshift, do_relu=False):
+    """two-input elementwise op with broadcasting; x0, x1 4-d NCHW int8 (dims 1 broadcast)"""
+    x0, x1 = _i8(x0), _i8(x1)
+    out = tuple(max(a, b) for a, b in zip(x0.shape, x1.shape))
+    d = BinaryDesc(op, *out, *x0.shape, *x1.shape, int(do_relu))
+    y = np.empty(out, np.int8)
+    m = _f32(multiplier)
+    rc = lib.orc_binary_i8(_p(x0, C.c_int8), _p(x1, C.c_int8), _p(y, C.c_int8), C.byref(d),
+                           _p(m, C.c_float), float(rshift))
+    if rc != 0:
+        raise ValueError("orc_binary_i8: no int8 meaning (mul with rshift 0 and multiplier 0)")
     return y
 
 

@@ -264,3 +264,42 @@ def test_lut_activation_and_general_reshape():
     assert np.array_equal(m.get_tensor_i8("flat"), sig.reshape(2, -1))
     assert np.array_equal(m.get_tensor_i8("back"), sig.reshape(2, 8, 25, 6))
     m.close()
+
+
+def test_graph_with_elementwise_family_matches_the_oracle():
+    """a squeeze-excite shaped graph: conv pair -> max / min / mul -> global average ->
+    1x1 conv gate -> broadcast mul / add / sub with the feature map"""
+    b = graphs.Builder("se_block", graphs.BASE_SEED + 77, 2, (6, 12))
+    x = b.input("input", 24, 12, 10)
+    c1 = b.conv("c1", x, 40, 3, relu=True)
+    c2 = b.conv("c2", x, 40, 3, relu=False)
+    g = b.g
+    shp = g.by_name[c1].shape
+    f32 = lambda *v: np.array(v, np.float32)
+
+    def binop(t, name, srcs, shape, mult, rshift, relu=0):
+        g.add(graphs.Op(t, name, srcs, shape, dict(do_relu=relu),
+                        dict(rshift=f32(rshift), multiplier=f32(*mult)), "RSHIFT_AND_M_I8"))
+        return name
+
+    mx = binop("tpu.eltwise_max", "mx", [c1, c2], shp, (3, 2), 1)
+    mn = binop("tpu.eltwise_min", "mn", [c1, c2], shp, (1, 1), 0, relu=1)
+    ml = binop("tpu.eltwise_mul", "ml", [mx, mn], shp, (1518500250,), 6)
+    g.add(graphs.Op("tpu.pool_avg_2d", "gap", ["ml"], (shp[0], shp[1], 1, 1),
+                    dict(kernel_h=shp[2], kernel_w=shp[3], stride_h=1, stride_w=1, padding_t=0,
+                         padding_b=0, padding_l=0, padding_r=0, do_relu=0),
+                    dict(rshift=f32(7), multiplier=f32(2)), "RSHIFT_AND_M_I8"))
+    pooled = "gap"
+    gate = binop("tpu.broadcast_mul", "gate", [mx, pooled], shp, (1 << 30,), 5)
+    ba = binop("tpu.broadcast_add", "badd", [gate, pooled], shp, (2, 3), 2, relu=1)
+    bs = binop("tpu.broadcast_sub", "bsub", [pooled, ba], shp, (9, 5), 1)
+    g.outputs = [bs]
+    want = oracle_graph.run(g)
+    m = module()
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    assert len(np.unique(want[bs])) > 8
+    m.close()

@@ -503,3 +503,43 @@ def test_layout_round_trip_and_float_edge(ctx):
     dst = ctx.malloc(xf.nbytes)
     ctx._ck(ctx.lib.tpuhip_nhwc_i8_to_nchw_f32(ctx.h, t2.ptr, dst, n, c, h, w, t2.cs))
     assert np.array_equal(ctx.download(dst, x.shape, np.float32), xf)
+
+
+BINARY_SHAPES = [((2, 40, 9, 7), (2, 40, 9, 7)),      # same shape (the Eltwise* ops)
+                 ((2, 40, 9, 7), (1, 40, 1, 1)),      # per-channel operand (scale-like)
+                 ((2, 40, 9, 7), (2, 1, 9, 7)),       # one channel repeated over all
+                 ((1, 1, 9, 1), (2, 40, 1, 7)),       # both operands broadcast
+                 ((2, 40, 1, 1), (2, 40, 9, 7)),      # squeeze-excite gate times feature map
+                 ((3, 16, 4, 4), (1, 1, 1, 1))]       # scalar
+
+
+@pytest.mark.parametrize("shapes", BINARY_SHAPES)
+@pytest.mark.parametrize("op", [capi.BIN_ADD, capi.BIN_SUB, capi.BIN_MAX, capi.BIN_MIN, capi.BIN_MUL])
+@pytest.mark.parametrize("relu", [False, True])
+def test_binary_ops_with_broadcast(ctx, shapes, op, relu):
+    rng = np.random.default_rng(op * 13 + len(shapes[0]) + relu)
+    a, b = rnd_i8(rng, shapes[0]), rnd_i8(rng, shapes[1])
+    out_shape = tuple(max(p, q) for p, q in zip(*shapes))
+    at, bt, yt = ctx.from_nchw(a), ctx.from_nchw(b), ctx.tensor(out_shape)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    if op == capi.BIN_MUL:
+        for mult, r in [(1 << 30, 7), (1518500250, 6), ((1 << 31) - 128, 14), (1 << 30, 0)]:
+            want = O.binary_i8(op, a, b, [float(mult)], r, relu)
+            ctx.binary(op, at, bt, yt, multiplier=f2i32(np.float32(mult)), rshift=r, do_relu=relu)
+            assert np.array_equal(ctx.to_nchw(yt), want), (mult, r)
+    else:
+        for m0, m1, r in [(1, 1, 0), (3, -2, 1), (127, 127, 7), (-128, 77, 8), (90, 45, 30)]:
+            want = O.binary_i8(op, a, b, [m0, m1], r, relu)
+            ctx.binary(op, at, bt, yt, m0=m0, m1=m1, rshift=r, do_relu=relu)
+            assert np.array_equal(ctx.to_nchw(yt), want), (m0, m1, r)
+    assert not ctx.raw(yt)[..., out_shape[1]:].any()        # pad channels written as zero
+
+
+def test_binary_rejects_bad_arguments(ctx):
+    a, b = ctx.tensor((1, 16, 4, 4)), ctx.tensor((1, 8, 4, 4))
+    with pytest.raises(capi.TpuHipError, match="neither 1 nor"):
+        ctx.binary(capi.BIN_ADD, a, b, a)
+    with pytest.raises(capi.TpuHipError, match="no int8 meaning"):
+        ctx.binary(capi.BIN_MUL, a, a, a, multiplier=0, rshift=0)
+    with pytest.raises(capi.TpuHipError, match="int8"):
+        ctx.binary(capi.BIN_MAX, a, a, a, m0=300)

@@ -25,6 +25,15 @@ class ConvPost(C.Structure):
                 ("add_src", C.c_void_p), ("add_out", C.c_void_p)]
 
 
+class BinaryDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in (
+        "op", "n", "c", "h", "w", "n0", "c0", "h0", "w0", "n1", "c1", "h1", "w1", "m0", "m1")] + \
+        [("multiplier", C.c_int32)] + [(k, C.c_int) for k in ("rshift", "do_relu", "x0_cs", "x1_cs", "y_cs")]
+
+
+BIN_ADD, BIN_SUB, BIN_MAX, BIN_MIN, BIN_MUL = range(5)
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
@@ -67,6 +76,7 @@ PROTOTYPES = {
     "tpuhip_conv2d_tile_name": (C.c_char_p, [C.c_int]),
     "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
     "tpuhip_conv2d_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost)]),
+    "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
                                                                    c_void_pp]),
@@ -321,6 +331,14 @@ class Context:
         m = np.ascontiguousarray(mult, dtype=np.int8)
         self._ck(self.lib.tpuhip_eltwise_add_i8(self.h, ptrs, len(xs), m.ctypes.data, int(rshift),
                                                 int(do_relu), y.ptr, y.nbytes))
+
+    def binary(self, op, x0, x1, y, m0=1, m1=1, multiplier=0, rshift=0, do_relu=False):
+        """x0, x1, y: device tensors made by tensor()/from_nchw() (logical NCHW shapes)"""
+        s0, s1, so = x0.shape, x1.shape, y.shape
+        d = BinaryDesc(op, so[0], so[1], so[2], so[3], s0[0], s0[1], s0[2], s0[3],
+                       s1[0], s1[1], s1[2], s1[3], int(m0), int(m1), int(multiplier), int(rshift),
+                       int(do_relu), x0.cs, x1.cs, y.cs)
+        self._ck(self.lib.tpuhip_binary_i8(self.h, C.byref(d), x0.ptr, x1.ptr, y.ptr))
 
     def pool_max(self, d, x, y):
         self._ck(self.lib.tpuhip_pool_max_i8(self.h, C.byref(d), x.ptr, y.ptr))

@@ -203,6 +203,18 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<FullyConnectedOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.eltwise_add") {
       krnl = std::make_shared<EltwiseAddOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.eltwise_max") {
+      krnl = std::make_shared<EltwiseMaxOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.eltwise_min") {
+      krnl = std::make_shared<EltwiseMinOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.eltwise_mul") {
+      krnl = std::make_shared<EltwiseMulOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.broadcast_add") {
+      krnl = std::make_shared<BroadcastAddOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.broadcast_mul") {
+      krnl = std::make_shared<BroadcastMulOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.broadcast_sub") {
+      krnl = std::make_shared<BroadcastSubOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.pool_avg_2d" || t == "tpu.pool_max_2d") {
       krnl = std::make_shared<PoolingOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.leaky_relu") {

@@ -497,6 +497,48 @@ void EltwiseAddOpKernel::invoke() {
 }
 
 // ---------------------------------------------------------------------------
+// EltwiseMax / Min / Mul (core/eltwise.cpp:102-347), BroadcastAdd / Mul / Sub
+// (core/broadcast.cpp:9-154)
+// ---------------------------------------------------------------------------
+BinaryOpKernel::BinaryOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+                               int op_code, bool broadcast, const char *what)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8(what);
+  const std::string who = std::string(what) + " '" + name + "'";
+  if (opdTensors.size() != 6) fail(who + ": expected two inputs + 4 quantization operands");
+  if (op.param_type == "NONE") fail(who + ": the unquantized (fp32) fallback is not implemented");
+  in0 = opdTensors[0].act;
+  in1 = opdTensors[1].act;
+  output_data = resTensor;
+  if (!in0 || !in1) fail(who + ": both inputs must be activations");
+  auto quant_rshift = opdTensors[4].weight;
+  auto quant_multiplier = opdTensors[5].weight;
+  if (!quant_rshift || !quant_multiplier || quant_rshift->size() < 1 || quant_multiplier->size() < 1)
+    fail(who + ": rshift / multiplier missing");
+  tpuhip_binary_desc &d = desc;
+  d.op = op_code;
+  d.do_relu = op.attr("do_relu", 0) != 0;
+  d.n = output_data->n; d.c = output_data->c; d.h = output_data->h; d.w = output_data->w;
+  d.n0 = in0->n; d.c0 = in0->c; d.h0 = in0->h; d.w0 = in0->w;
+  d.n1 = in1->n; d.c1 = in1->c; d.h1 = in1->h; d.w1 = in1->w;
+  d.x0_cs = in0->cs; d.x1_cs = in1->cs; d.y_cs = output_data->cs;
+  if (!broadcast && (in0->size() != output_data->size() || in1->size() != output_data->size()))
+    fail(who + ": input shapes differ from the result's");
+  d.rshift = (int)f2u32(quant_rshift->at(0));
+  if (op_code == TPUHIP_BIN_MUL) {
+    d.multiplier = (int32_t)f2u32(quant_multiplier->at(0));   // eltwise.cpp:341-343, broadcast.cpp:110
+  } else {
+    if (quant_multiplier->size() < 2) fail(who + ": one multiplier per input needed");
+    d.m0 = f2i8(quant_multiplier->at(0));                      // eltwise.cpp:160, broadcast.cpp:53
+    d.m1 = f2i8(quant_multiplier->at(1));
+  }
+}
+
+void BinaryOpKernel::invoke() {
+  ck(tpuhip_binary_i8(ctx, &desc, in0->data(), in1->data(), output_data->data()), name.c_str());
+}
+
+// ---------------------------------------------------------------------------
 // Pooling (core/pooling.cpp:33-160)
 // ---------------------------------------------------------------------------
 PoolingOpKernel::PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)

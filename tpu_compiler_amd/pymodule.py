@@ -19,6 +19,12 @@ _WEIGHT_OPERANDS = {
     "tpu.conv_2d": ["filter", "bias", None, None, "rshift", "multiplier"],
     "tpu.fully_connected": ["filter", "bias", None, None, "rshift", "multiplier"],
     "tpu.eltwise_add": [None, None, "rshift", "multiplier"],
+    "tpu.eltwise_max": [None, None, "rshift", "multiplier"],
+    "tpu.eltwise_min": [None, None, "rshift", "multiplier"],
+    "tpu.eltwise_mul": [None, None, "rshift", "multiplier"],
+    "tpu.broadcast_add": [None, None, "rshift", "multiplier"],
+    "tpu.broadcast_mul": [None, None, "rshift", "multiplier"],
+    "tpu.broadcast_sub": [None, None, "rshift", "multiplier"],
     "tpu.pool_avg_2d": [None, None, "rshift", "multiplier"],
     "tpu.pool_max_2d": [],
     "tpu.leaky_relu": [None, None, None, None, "rshift_pos", "multiplier_pos", "rshift_neg",
