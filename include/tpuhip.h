@@ -245,6 +245,14 @@ int tpuhip_clip_table(float min, float max, uint32_t rshift, uint32_t multiplier
 /* Replaces ReluOpKernel::invoke (core/activation.cpp:155-164). */
 int tpuhip_relu_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t bytes);
 
+/* One table per channel: y[.., c] = tables[c * 256 + (uint8_t)x[.., c]]; tables is DEVICE memory
+ * (c * 256 bytes).  With tpuhip_prelu_tables (host) it replaces PReluOpKernel::invoke, INT8 branch
+ * (core/activation.cpp:185-224): slope holds the c float-stored int8 slopes. */
+int tpuhip_lut_per_channel_i8(tpuhip_ctx *ctx, const void *x, void *y, const void *tables,
+                              size_t pixels, int c, int cs);
+int tpuhip_prelu_tables(const float *slope, int c, uint32_t rshift_pos, uint32_t multiplier_pos,
+                        uint32_t rshift_neg, int8_t *tables /* c * 256 */);
+
 /* ---- Upsample, Concat ----------------------------------------------------- */
 
 /* Replaces UpsampleOpKernel::invoke (core/upsample.cpp:20-41), nearest. */

@@ -308,6 +308,20 @@ public:
   ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
 };
 
+// operands: [0]input [1]slope (c values) [2..5]unused [6]rshift_pos [7]multiplier_pos
+// [8]rshift_neg (core/activation.cpp:165-183).  Realised as one 256-entry table per channel.
+class PReluOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPUPReluOp";
+  PReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~PReluOpKernel() override;
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+  void *tables = nullptr;   // device, c * 256 bytes
+};
+
 class ReluOpKernel : public CPUOpKernel {  // core/activation.cpp:155-164
 public:
   static constexpr const char *OpName = "CPUReluOp";

@@ -412,6 +412,26 @@ void orc_leaky_relu_i8(const int8_t *x, int8_t *y, size_t count, float rshift_po
   }
 }
 
+/* activation.cpp:185-224.  First pass: x > 0 keeps x, else slope[channel] * x (float).
+ * Second pass: x > 0 -> float overload, non-qdm, multiplier converted implicitly from
+ * float to uint32; else applyRShiftAndSaturateInt8. */
+void orc_prelu_i8(const int8_t *x, int8_t *y, int n, int c, int hw, const float *slope,
+                  float rshift_pos, float multiplier_pos, float rshift_neg) {
+#pragma omp parallel for collapse(2)
+  for (int b = 0; b < n; ++b)
+    for (int ch = 0; ch < c; ++ch) {
+      const size_t base = ((size_t)b * c + ch) * hw;
+      for (int i = 0; i < hw; ++i) {
+        const float in = (float)x[base + i];
+        if (in > 0)
+          y[base + i] = orc_apply_mult_rshift_sat8_f(in, orc_f2u32(rshift_pos),
+                                                     orc_f2u32(multiplier_pos), 0);
+        else
+          y[base + i] = orc_apply_rshift_sat8(slope[ch] * in, orc_f2u32(rshift_neg));
+      }
+    }
+}
+
 /* activation.cpp:47-53: y0_table_op->at((unsigned char)input).  float ->
  * unsigned char of a negative value keeps the low byte on x86-64 gcc, i.e. the
  * index is the two's-complement byte of the int8 input. */

@@ -121,6 +121,10 @@ void orc_pool_avg_i8(const int8_t *x, int8_t *y, const orc_pool_desc *d, float r
 /* :126-153 */
 void orc_leaky_relu_i8(const int8_t *x, int8_t *y, size_t count, float rshift_pos,
                        float multiplier_pos, float rshift_neg, float multiplier_neg);
+/* :185-224 PRelu: x > 0 -> non-qdm (x * multiplier_pos) / 2^rshift_pos; else slope[c] * x then
+ * / 2^rshift_neg; both floor(. + 0.5), saturate.  slope holds c floats. */
+void orc_prelu_i8(const int8_t *x, int8_t *y, int n, int c, int hw, const float *slope,
+                  float rshift_pos, float multiplier_pos, float rshift_neg);
 /* :47-53 and siblings: y = table[(unsigned char)x]; table holds 256 floats */
 void orc_lut_i8(const int8_t *x, int8_t *y, size_t count, const float *table256);
 /* :155-164 + core/internal.cpp:13-18 */

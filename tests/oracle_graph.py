@@ -75,6 +75,10 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             w = op.weights
             y = O.leaky_relu_i8(ins[0], w["rshift_pos"][0], w["multiplier_pos"][0],
                                 w["rshift_neg"][0], w["multiplier_neg"][0])
+        elif t == "tpu.prelu":
+            w = op.weights
+            y = O.prelu_i8(ins[0], w["slope"], w["rshift_pos"][0], w["multiplier_pos"][0],
+                           w["rshift_neg"][0])
         elif t == "tpu.clip":
             y = O.clip_i8(ins[0], op.attrs["min"], op.attrs["max"], op.weights["rshift"][0],
                           op.weights["multiplier"][0])

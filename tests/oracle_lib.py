@@ -74,6 +74,7 @@ def _load():
     lib.orc_pool_max_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc)]
     lib.orc_pool_avg_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc), C.c_float, C.c_float]
     lib.orc_leaky_relu_i8.argtypes = [i8p, i8p, C.c_size_t] + [C.c_float] * 4
+    lib.orc_prelu_i8.argtypes = [i8p, i8p, C.c_int, C.c_int, C.c_int, f32p] + [C.c_float] * 3
     lib.orc_lut_i8.argtypes = [i8p, i8p, C.c_size_t, f32p]
     lib.orc_relu_i8.argtypes = [i8p, i8p, C.c_size_t]
     lib.orc_clip_i8.argtypes = [i8p, i8p, C.c_size_t] + [C.c_float] * 4
@@ -188,6 +189,16 @@ def eltwise_add_i8(xs, multiplier, rshift, do_relu):
     m, r = _f32(multiplier), _f32(rshift)
     lib.orc_eltwise_add_i8(_ptr_array(xs), len(xs), _p(m, C.c_float), _p(r, C.c_float),
                            int(do_relu), _p(y, C.c_int8), xs[0].size)
+    return y
+
+
+def prelu_i8(x, slope, rshift_pos, multiplier_pos, rshift_neg):
+    x = _i8(x)
+    n, c = x.shape[0], x.shape[1]
+    y = np.empty(x.shape, np.int8)
+    sl = _f32(slope)
+    lib.orc_prelu_i8(_p(x, C.c_int8), _p(y, C.c_int8), n, c, x.size // (n * c), _p(sl, C.c_float),
+                     float(rshift_pos), float(multiplier_pos), float(rshift_neg))
     return y
 
 

@@ -282,8 +282,12 @@ def test_graph_with_elementwise_family_matches_the_oracle():
                         dict(rshift=f32(rshift), multiplier=f32(*mult)), "RSHIFT_AND_M_I8"))
         return name
 
+    slope = (np.arange(shp[1]) % 23 - 7).astype(np.float32)
+    g.add(graphs.Op("tpu.prelu", "pr", [c2], shp, {},
+                    dict(slope=slope, rshift_pos=f32(1), multiplier_pos=f32(3), rshift_neg=f32(3)),
+                    "RSHIFT_AND_M_I8"))
     mx = binop("tpu.eltwise_max", "mx", [c1, c2], shp, (3, 2), 1)
-    mn = binop("tpu.eltwise_min", "mn", [c1, c2], shp, (1, 1), 0, relu=1)
+    mn = binop("tpu.eltwise_min", "mn", [c1, "pr"], shp, (1, 1), 0, relu=1)
     ml = binop("tpu.eltwise_mul", "ml", [mx, mn], shp, (1518500250,), 6)
     g.add(graphs.Op("tpu.pool_avg_2d", "gap", ["ml"], (shp[0], shp[1], 1, 1),
                     dict(kernel_h=shp[2], kernel_w=shp[3], stride_h=1, stride_w=1, padding_t=0,

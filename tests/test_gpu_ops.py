@@ -543,3 +543,17 @@ def test_binary_rejects_bad_arguments(ctx):
         ctx.binary(capi.BIN_MUL, a, a, a, multiplier=0, rshift=0)
     with pytest.raises(capi.TpuHipError, match="int8"):
         ctx.binary(capi.BIN_MAX, a, a, a, m0=300)
+
+
+@pytest.mark.parametrize("shape", [(2, 7, 256, 1), (3, 40, 9, 11), (1, 130, 5, 5)])
+def test_prelu_per_channel_tables(ctx, shape):
+    rng = np.random.default_rng(shape[1])
+    x = rnd_i8(rng, shape)
+    if shape[2] == 256:
+        x[...] = np.arange(-128, 128, dtype=np.int8).reshape(1, 1, 256, 1)    # every input value
+    slope = rng.integers(-128, 128, shape[1]).astype(np.float32)
+    xt, yt = ctx.from_nchw(x), ctx.tensor(shape)
+    for mp, rp, rn in [(1, 0, 0), (3, 1, 2), (200, 7, 5)]:
+        ctx.prelu(xt, yt, slope, rp, mp, rn)
+        assert np.array_equal(ctx.to_nchw(yt), O.prelu_i8(x, slope, rp, mp, rn)), (mp, rp, rn)
+        assert not ctx.raw(yt)[..., shape[1]:].any()

@@ -88,3 +88,18 @@ def test_mul_without_requant_is_refused():
     a = np.ones((1, 1, 1, 1), np.int8)
     with pytest.raises(ValueError):
         O.binary_i8(O.BIN_MUL, a, a, [0.0], 0)
+
+
+def test_prelu_matches_exact_arithmetic_for_every_input_value():
+    """every int8 input on every channel: x > 0 -> nearest(x * m / 2^rp), else nearest(slope * x / 2^rn),
+    ties toward +inf, saturated"""
+    c = 7
+    slope = np.array([-128, -3, -1, 0, 1, 55, 127], np.float32)
+    x = np.tile(np.arange(-128, 128, dtype=np.int8).reshape(1, 1, 256, 1), (2, c, 1, 1))
+    for mp, rp, rn in [(1, 0, 0), (3, 1, 2), (200, 7, 5), (77, 4, 6)]:
+        got = O.prelu_i8(x, slope, rp, mp, rn)
+        for ch in range(c):
+            for v in range(-128, 128):
+                want = (sat8(nearest_ties_up(Fraction(v * mp, 1 << rp))) if v > 0 else
+                        sat8(nearest_ties_up(Fraction(int(slope[ch]) * v, 1 << rn))))
+                assert got[1, ch, v + 128, 0] == want, (mp, rp, rn, ch, v)

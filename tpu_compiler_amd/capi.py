@@ -76,6 +76,9 @@ PROTOTYPES = {
     "tpuhip_conv2d_tile_name": (C.c_char_p, [C.c_int]),
     "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
     "tpuhip_conv2d_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost)]),
+    "tpuhip_lut_per_channel_i8": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t, C.c_int, C.c_int]),
+    "tpuhip_prelu_tables": (C.c_int, [C.POINTER(C.c_float), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32,
+                                      C.POINTER(C.c_int8)]),
     "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
@@ -331,6 +334,19 @@ class Context:
         m = np.ascontiguousarray(mult, dtype=np.int8)
         self._ck(self.lib.tpuhip_eltwise_add_i8(self.h, ptrs, len(xs), m.ctypes.data, int(rshift),
                                                 int(do_relu), y.ptr, y.nbytes))
+
+    def prelu(self, x, y, slope, rshift_pos, multiplier_pos, rshift_neg):
+        c = x.shape[1]
+        sl = np.ascontiguousarray(slope, dtype=np.float32)
+        tables = np.empty(c * 256, np.int8)
+        self._ck(self.lib.tpuhip_prelu_tables(sl.ctypes.data_as(C.POINTER(C.c_float)), c,
+                                              int(rshift_pos), int(multiplier_pos), int(rshift_neg),
+                                              tables.ctypes.data_as(C.POINTER(C.c_int8))))
+        dev = self.malloc(tables.nbytes)
+        self.upload(dev, tables)
+        self._ck(self.lib.tpuhip_lut_per_channel_i8(self.h, x.ptr, y.ptr, dev, x.pixels, c, x.cs))
+        self.sync()
+        self.free(dev)
 
     def binary(self, op, x0, x1, y, m0=1, m1=1, multiplier=0, rshift=0, do_relu=False):
         """x0, x1, y: device tensors made by tensor()/from_nchw() (logical NCHW shapes)"""

@@ -66,6 +66,36 @@ __global__ __launch_bounds__(kThreads) void eltwise_add_kernel(EltArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// one 256-entry table per channel (PRelu's per-channel slope, core/activation.cpp:185-224):
+// y[pixel][c] = tables[c][(unsigned char)x[pixel][c]].  One lane = 16 channels of a pixel;
+// the tables (c * 256 bytes) stay in the caches.  Pad channels are written as zero.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kThreads) void lut_per_channel_kernel(const int8_t *x, int8_t *y,
+                                                                   const uint8_t *tables,
+                                                                   int64_t total, int c, int cs) {
+  const int c16 = cs >> 4;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int cg = (int)(i % c16);
+    const v4i in = reinterpret_cast<const v4i *>(x)[i];
+    v4i out;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int ch = cg * 16 + q * 4 + b;
+        const uint32_t idx = ((uint32_t)in[q] >> (8 * b)) & 255u;
+        const uint32_t r = ch < c ? tables[(size_t)ch * 256 + idx] : 0u;
+        word |= r << (8 * b);
+      }
+      out[q] = (int)word;
+    }
+    reinterpret_cast<v4i *>(y)[i] = out;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // table ops: y = table[(unsigned char)x] (core/activation.cpp:47-53).  The table
 // arrives by value in the kernel arguments and is spread into LDS once per
 // workgroup; pad channels are forced to zero.
@@ -372,6 +402,41 @@ int tpuhip_lut_i8(tpuhip_ctx *ctx, const void *x, void *y, const int8_t *table25
   TPUHIP_REQUIRE(c > 0 && cs >= c && cs % 16 == 0, "lut: bad channels %d / stride %d", c, cs);
   if (pixels == 0) return TPUHIP_OK;
   return launch_lut(ctx, x, y, table256, (int64_t)pixels, c, cs, cs, 0);
+}
+
+int tpuhip_lut_per_channel_i8(tpuhip_ctx *ctx, const void *x, void *y, const void *tables,
+                              size_t pixels, int c, int cs) {
+  TPUHIP_REQUIRE(ctx && x && y && tables, "lut_per_channel: NULL argument");
+  TPUHIP_REQUIRE(c > 0 && cs >= c && cs % 16 == 0, "lut_per_channel: bad channels %d / stride %d", c, cs);
+  if (pixels == 0) return TPUHIP_OK;
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  const int64_t total = (int64_t)pixels * (cs / 16);
+  launch(ctx, lut_per_channel_kernel, dim3(grid_for(total, kThreads * 2)), dim3(kThreads),
+         (const int8_t *)x, (int8_t *)y, (const uint8_t *)tables, total, c, cs);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
+int tpuhip_prelu_tables(const float *slope, int c, uint32_t rshift_pos, uint32_t multiplier_pos,
+                        uint32_t rshift_neg, int8_t *tables) {
+  TPUHIP_REQUIRE(slope && tables && c > 0, "prelu_tables: bad argument");
+  TPUHIP_REQUIRE(rshift_pos <= 30 && rshift_neg <= 30, "prelu: rshift outside [0,30]");
+  // PReluOpKernel::invoke (core/activation.cpp:185-224) for each channel and each of the 256 inputs
+  for (int ch = 0; ch < c; ++ch)
+    for (int v = -128; v <= 127; ++v) {
+      int8_t out;
+      if (v > 0) {
+        out = host_mult_rshift_sat8((float)v, rshift_pos, multiplier_pos);
+      } else {
+        volatile float prod = slope[ch] * (float)v;
+        volatile float quo = prod / (float)(1 << rshift_neg);
+        double s = std::floor((double)quo + 0.5);
+        s = s > 127.0 ? 127.0 : s < -128.0 ? -128.0 : s;
+        out = (int8_t)(int)s;
+      }
+      tables[(size_t)ch * 256 + (uint8_t)(int8_t)v] = out;
+    }
+  return TPUHIP_OK;
 }
 
 int tpuhip_leaky_relu_table(uint32_t rshift_pos, uint32_t multiplier_pos, uint32_t rshift_neg,

@@ -219,6 +219,8 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<PoolingOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.leaky_relu") {
       krnl = std::make_shared<LeakyReluOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.prelu") {
+      krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {
       krnl = std::make_shared<ClipOpKernel>(*op, valueMapping, weightMapping);
     } else if (is_lut_op(t)) {

@@ -609,6 +609,39 @@ void LutOpKernel::invoke() {
      name.c_str());
 }
 
+PReluOpKernel::PReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("PRelu");
+  if (opdTensors.size() < 9) fail("PRelu '" + name + "': expected 9 operands");
+  input_data = opdTensors[0].act;
+  output_data = resTensor;
+  auto slope = opdTensors[1].weight;
+  if (!input_data || !slope) fail("PRelu '" + name + "': input / slope missing");
+  if (input_data->size() != output_data->size()) fail("PRelu '" + name + "': shape mismatch");
+  if ((int)slope->size() < input_data->c) fail("PRelu '" + name + "': one slope per channel needed");
+  for (int i = 6; i <= 8; ++i)
+    if (!opdTensors[i].weight) fail("PRelu '" + name + "': rshift / multiplier operand missing");
+  std::vector<int8_t> host((size_t)input_data->c * 256);
+  // rshift operands cast explicitly, the multiplier converted implicitly (activation.cpp:211-217)
+  ck(tpuhip_prelu_tables(slope->data.data(), input_data->c, f2u32(opdTensors[6].weight->at(0)),
+                         f2u32(opdTensors[7].weight->at(0)), f2u32(opdTensors[8].weight->at(0)),
+                         host.data()),
+     name.c_str());
+  ck(tpuhip_malloc(ctx, host.size(), &tables), name.c_str());
+  ck(tpuhip_upload(ctx, tables, host.data(), host.size()), name.c_str());
+}
+
+PReluOpKernel::~PReluOpKernel() {
+  if (tables) tpuhip_free(ctx, tables);
+}
+
+void PReluOpKernel::invoke() {
+  ck(tpuhip_lut_per_channel_i8(ctx, input_data->data(), output_data->data(), tables,
+                               (size_t)input_data->n * input_data->h * input_data->w,
+                               input_data->c, input_data->cs),
+     name.c_str());
+}
+
 LeakyReluOpKernel::LeakyReluOpKernel(OpDesc &op, value_map_t &valueMapping,
                                      weight_map_t &weightMapping)
     : LutOpKernel(op, valueMapping, weightMapping) {

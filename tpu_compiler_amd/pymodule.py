@@ -29,6 +29,7 @@ _WEIGHT_OPERANDS = {
     "tpu.pool_max_2d": [],
     "tpu.leaky_relu": [None, None, None, None, "rshift_pos", "multiplier_pos", "rshift_neg",
                        "multiplier_neg"],
+    "tpu.prelu": ["slope", None, None, None, None, "rshift_pos", "multiplier_pos", "rshift_neg"],
     "tpu.clip": [None, None, "rshift", "multiplier"],
     "tpu.lut": ["table", None],
     "tpu.relu": [],
