@@ -267,6 +267,35 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
                      const int *in_cs, int axis, const uint32_t *rshift,
                      const uint32_t *multiplier, int do_relu, void *y, int y_cs);
 
+/* ---- pure data movement, 4-d shapes -----------------------------------------
+ * Replaces PadOpKernel, CropOpKernel, PermuteOpKernel, ReorgOpKernel, TileOpKernel,
+ * ReverseOpKernel, ShuffleChannelOpKernel, DepthToSpaceOpKernel (core/pad.cpp:114-141,
+ * crop.cpp:44-92, permute.cpp:8-44, reorg.cpp:20-42, tile.cpp:24-42, reverse.cpp:19-42,
+ * shuffle_channel.cpp:21-48, depthtospace.cpp:8-80).  p[]:
+ *   PAD_CONST / PAD_EDGE  p[0..3] pads at the beginning of n,c,h,w, p[4..7] at the end (constant
+ *                         mode: negative = cut; the padding is 0: the reference never reads
+ *                         const_val; edge mode: h and w only)
+ *   CROP                  p[0..3] crop_offset, p[4..7] steps
+ *   PERMUTE               p[0..3] order (output dimension k is input dimension order[k])
+ *   REORG                 p[0] stride
+ *   TILE                  p[0] axis, p[1] tiles
+ *   REVERSE               p[0] axis
+ *   SHUFFLE_CHANNEL       p[0] group
+ *   DEPTH_TO_SPACE        p[0] upscale factor, p[1] 1 = "DCR" mode, 0 = CRD */
+enum {
+  TPUHIP_MOVE_PAD_CONST = 0, TPUHIP_MOVE_PAD_EDGE = 1, TPUHIP_MOVE_CROP = 2, TPUHIP_MOVE_PERMUTE = 3,
+  TPUHIP_MOVE_REORG = 4, TPUHIP_MOVE_TILE = 5, TPUHIP_MOVE_REVERSE = 6,
+  TPUHIP_MOVE_SHUFFLE_CHANNEL = 7, TPUHIP_MOVE_DEPTH_TO_SPACE = 8
+};
+typedef struct tpuhip_move_desc {
+  int kind;
+  int in, ic, ih, iw;   /* input */
+  int on, oc, oh, ow;   /* output */
+  int x_cs, y_cs;
+  int p[8];
+} tpuhip_move_desc;
+int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y);
+
 /* ---- module interpreter ------------------------------------------------------ */
 
 /* Flat view of the C++ ModuleInterpreter (include/tpuhip/interpreter.hpp), which

@@ -358,6 +358,35 @@ private:
   SyncedData output_data;
 };
 
+// Pure data movement (4-d shapes).  Array attributes arrive as numbered scalars:
+// pads0..7 + mode_edge (PadOp: pads, mode == "edge"), crop_offset0..3 + steps0..3 (CropOp),
+// order0..3 (PermuteOp), stride (ReorgOp), axis + tiles (TileOp), axis (ReverseOp),
+// group (ShuffleChannelOp), upscale_factor + mode_dcr (DepthToSpaceOp, mode == "DCR").
+class MoveOpKernel : public CPUOpKernel {
+public:
+  void invoke() override;
+
+protected:
+  MoveOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping, const char *what);
+  tpuhip_move_desc desc{};
+  SyncedData input_data, output_data;
+};
+#define TPUHIP_MOVE_KERNEL(Class, Name)                                         \
+  class Class : public MoveOpKernel {                                           \
+  public:                                                                       \
+    static constexpr const char *OpName = Name;                                 \
+    Class(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);  \
+  };
+TPUHIP_MOVE_KERNEL(PadOpKernel, "CPUPadOp")                          // core/pad.cpp:114-141
+TPUHIP_MOVE_KERNEL(CropOpKernel, "CPUCropOp")                        // core/crop.cpp:34-92
+TPUHIP_MOVE_KERNEL(PermuteOpKernel, "CPUPermuteOp")                  // core/permute.cpp:35-44
+TPUHIP_MOVE_KERNEL(ReorgOpKernel, "CPUReorgOp")                      // core/reorg.cpp:8-42
+TPUHIP_MOVE_KERNEL(TileOpKernel, "CPUTileOp")                        // core/tile.cpp:8-42
+TPUHIP_MOVE_KERNEL(ReverseOpKernel, "CPUReverseOp")                  // core/reverse.cpp:7-42
+TPUHIP_MOVE_KERNEL(ShuffleChannelOpKernel, "CPUShuffleChannelOp")    // core/shuffle_channel.cpp:7-48
+TPUHIP_MOVE_KERNEL(DepthToSpaceOpKernel, "CPUPixelShuffleOp")        // core/depthtospace.cpp:60-80
+#undef TPUHIP_MOVE_KERNEL
+
 // tpu.reshape whose source and result are not the same bytes in channels-last
 // order (the reference aliases the NCHW buffer: MlirModuleInterpreter.cpp:331-338).
 class ReshapeOpKernel : public CPUOpKernel {

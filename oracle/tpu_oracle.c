@@ -510,3 +510,139 @@ void orc_concat_i8(const int8_t *const *xs, int nin, const int64_t *shapes, int 
       if (y[i] < 0) y[i] = 0;
   }
 }
+
+/* ------------------------------------------------------------------------- */
+/* pure data movement                                                         */
+/* ------------------------------------------------------------------------- */
+
+/* pad.cpp: constant mode copies rows of the (possibly cut) input into the result buffer and
+ * touches nothing else: const_val is parsed (:119) and passed down (:139) but never read, so
+ * the padding keeps the zeros the result tensor was created with (cpukernel.cpp:75-80).
+ * Edge mode replicates the border (h and w only, asserted). */
+void orc_pad_i8(const int8_t *x, int8_t *y, const int64_t *is, const int *pads, int edge_mode) {
+  const int8_t const_val = 0;
+  const int in = (int)is[0], ic = (int)is[1], ih = (int)is[2], iw = (int)is[3];
+  const int on = pads[0] + pads[4] + in, oc = pads[1] + pads[5] + ic;
+  const int oh = pads[2] + pads[6] + ih, ow = pads[3] + pads[7] + iw;
+  for (int64_t i = 0; i < (int64_t)on * oc * oh * ow; ++i) y[i] = const_val;
+  if (edge_mode) {
+    for (int n = 0; n < in; ++n)
+      for (int c = 0; c < ic; ++c)
+        for (int h = 0; h < oh; ++h)
+          for (int w = 0; w < ow; ++w) {
+            int sh = h - pads[2], sw = w - pads[3];
+            sh = sh < 0 ? 0 : sh >= ih ? ih - 1 : sh;
+            sw = sw < 0 ? 0 : sw >= iw ? iw - 1 : sw;
+            y[(((int64_t)n * oc + c) * oh + h) * ow + w] = x[(((int64_t)n * ic + c) * ih + sh) * iw + sw];
+          }
+    return;
+  }
+  const int s_n = pads[0] < 0 ? -pads[0] : 0, s_c = pads[1] < 0 ? -pads[1] : 0;
+  const int s_h = pads[2] < 0 ? -pads[2] : 0, s_w = pads[3] < 0 ? -pads[3] : 0;
+  const int e_n = pads[4] < 0 ? in + pads[4] : in, e_c = pads[5] < 0 ? ic + pads[5] : ic;
+  const int e_h = pads[6] < 0 ? ih + pads[6] : ih, e_w = pads[7] < 0 ? iw + pads[7] : iw;
+  const int b_n = pads[0] < 0 ? 0 : pads[0], b_c = pads[1] < 0 ? 0 : pads[1];
+  const int b_h = pads[2] < 0 ? 0 : pads[2], b_w = pads[3] < 0 ? 0 : pads[3];
+  for (int n = s_n; n < e_n; ++n)
+    for (int c = s_c; c < e_c; ++c)
+      for (int h = s_h; h < e_h; ++h)
+        for (int w = s_w; w < e_w; ++w)
+          y[((((int64_t)(n - s_n + b_n)) * oc + (c - s_c + b_c)) * oh + (h - s_h + b_h)) * ow +
+            (w - s_w + b_w)] = x[(((int64_t)n * ic + c) * ih + h) * iw + w];
+}
+
+void orc_crop_i8(const int8_t *x, int8_t *y, const int64_t *is, const int64_t *os, const int *off,
+                 const int *st) {
+  for (int64_t n = 0; n < os[0]; ++n)
+    for (int64_t c = 0; c < os[1]; ++c)
+      for (int64_t h = 0; h < os[2]; ++h)
+        for (int64_t w = 0; w < os[3]; ++w) {
+          const int64_t a = n * st[0] + off[0], b = c * st[1] + off[1], d = h * st[2] + off[2],
+                        e = w * st[3] + off[3];
+          y[((n * os[1] + c) * os[2] + h) * os[3] + w] = x[((a * is[1] + b) * is[2] + d) * is[3] + e];
+        }
+}
+
+void orc_permute_i8(const int8_t *x, int8_t *y, const int64_t *is, const int *order) {
+  for (int64_t n = 0; n < is[0]; ++n)
+    for (int64_t c = 0; c < is[1]; ++c)
+      for (int64_t h = 0; h < is[2]; ++h)
+        for (int64_t w = 0; w < is[3]; ++w) {
+          const int64_t cur[4] = {n, c, h, w};
+          const int64_t in_idx = w + h * is[3] + c * is[2] * is[3] + n * is[1] * is[2] * is[3];
+          const int64_t out_idx = cur[order[3]] + cur[order[2]] * is[order[3]] +
+                                  cur[order[1]] * is[order[3]] * is[order[2]] +
+                                  cur[order[0]] * is[order[3]] * is[order[2]] * is[order[1]];
+          y[out_idx] = x[in_idx];
+        }
+}
+
+void orc_reorg_i8(const int8_t *x, int8_t *y, const int64_t *is, int stride) {
+  const int n = (int)is[0], in_c = (int)is[1], in_h = (int)is[2], in_w = (int)is[3];
+  const int out_c = in_c * stride * stride, out_h = in_h / stride, out_w = in_w / stride;
+  for (int b = 0; b < n; b++)
+    for (int k = 0; k < out_c; k++)
+      for (int j = 0; j < out_h; j++)
+        for (int i = 0; i < out_w; i++) {
+          const int64_t in_index = i + out_w * (j + out_h * (k + (int64_t)out_c * b));
+          const int c2 = k % in_c, offset = k / in_c;
+          const int w2 = i * stride + offset % stride, h2 = j * stride + offset / stride;
+          const int64_t out_index = w2 + in_w * (h2 + in_h * (c2 + (int64_t)in_c * b));
+          y[in_index] = x[out_index];
+        }
+}
+
+void orc_tile_i8(const int8_t *x, int8_t *y, const int64_t *is, int axis, int tiles) {
+  int64_t outer = 1, inner = 1;
+  for (int i = 0; i < axis; ++i) outer *= is[i];
+  for (int i = axis; i < 4; ++i) inner *= is[i];
+  for (int64_t o = 0; o < outer; ++o)
+    for (int t = 0; t < tiles; ++t)
+      memcpy(y + o * tiles * inner + t * inner, x + o * inner, (size_t)inner);
+}
+
+void orc_reverse_i8(const int8_t *x, int8_t *y, const int64_t *s, int axis) {
+  const int64_t stride[4] = {s[1] * s[2] * s[3], s[2] * s[3], s[3], 1};
+  for (int64_t n = 0; n < s[0]; ++n)
+    for (int64_t c = 0; c < s[1]; ++c)
+      for (int64_t h = 0; h < s[2]; ++h)
+        for (int64_t w = 0; w < s[3]; ++w) {
+          int64_t src[4] = {n, c, h, w}, dst[4] = {n, c, h, w};
+          dst[axis] = s[axis] - src[axis] - 1;
+          y[dst[0] * stride[0] + dst[1] * stride[1] + dst[2] * stride[2] + dst[3]] =
+              x[src[0] * stride[0] + src[1] * stride[1] + src[2] * stride[2] + src[3]];
+        }
+}
+
+void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *s, int group) {
+  const int64_t frame = s[2] * s[3], batch = frame * s[1];
+  const int col = (int)(s[1] / group);
+  for (int64_t i = 0; i < s[0]; ++i)
+    for (int j = 0; j < group; ++j)
+      for (int k = 0; k < col; ++k)
+        memcpy(y + i * batch + ((int64_t)k * group + j) * frame,
+               x + i * batch + ((int64_t)j * col + k) * frame, (size_t)frame);
+}
+
+void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *is, int r, int dcr_mode) {
+  const int in = (int)is[0], ic = (int)is[1], ih = (int)is[2], iw = (int)is[3];
+  const int oc = ic / (r * r), oh = ih * r, ow = iw * r;
+  int64_t i_index = 0;
+  for (int n = 0; n < in; n++)
+    for (int c = 0; c < ic; c++)
+      for (int h = 0; h < ih; h++)
+        for (int w = 0; w < iw; w++) {
+          int new_c, new_h, new_w;
+          if (dcr_mode) {
+            new_c = c % oc;
+            new_h = h * r + (c / oc) / r;
+            new_w = w * r + ((c / oc) % r);
+          } else {
+            new_c = c / (r * r);
+            new_h = h * r + (c / r) % r;
+            new_w = w * r + (c % (r * r)) % r;
+          }
+          y[(int64_t)n * oc * oh * ow + (int64_t)new_c * oh * ow + (int64_t)new_h * ow + new_w] =
+              x[i_index++];
+        }
+}

@@ -142,6 +142,28 @@ void orc_upsample_i8(const int8_t *x, int8_t *y, int n, int c, int ih, int iw, i
 void orc_concat_i8(const int8_t *const *xs, int nin, const int64_t *shapes, int ndim, int axis,
                    const float *rshift, const float *multiplier, int do_relu, int8_t *y);
 
+/* ---- pure data movement (no INT8-specific branch in the reference), 4-d shapes ---- */
+/* core/pad.cpp:62-112 (constant mode; negative pads cut) and :7-60 (edge mode, h/w only).
+ * pads = {n,c,h,w begin, n,c,h,w end}.  The reference never reads const_val: constant
+ * padding is the zero of the freshly created result tensor. */
+void orc_pad_i8(const int8_t *x, int8_t *y, const int64_t *ishape, const int *pads, int edge_mode);
+/* core/crop.cpp:44-92: y[o] = x[o * steps + offset] per dimension */
+void orc_crop_i8(const int8_t *x, int8_t *y, const int64_t *ishape, const int64_t *oshape,
+                 const int *offset, const int *steps);
+/* core/permute.cpp:8-33: output dimension k is input dimension order[k] */
+void orc_permute_i8(const int8_t *x, int8_t *y, const int64_t *ishape, const int *order);
+/* core/reorg.cpp:20-42 */
+void orc_reorg_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int stride);
+/* core/tile.cpp:24-42: the block from `axis` on is repeated `tiles` times */
+void orc_tile_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int axis, int tiles);
+/* core/reverse.cpp:19-42 */
+void orc_reverse_i8(const int8_t *x, int8_t *y, const int64_t *shape, int axis);
+/* core/shuffle_channel.cpp:21-48 */
+void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, int group);
+/* core/depthtospace.cpp:8-58 (pixelshuffle), dcr_mode as in :60 */
+void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int upscale,
+                           int dcr_mode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,13 @@ _BINARY = {"tpu.eltwise_max": O.BIN_MAX, "tpu.eltwise_min": O.BIN_MIN, "tpu.eltw
            "tpu.broadcast_mul": O.BIN_MUL}
 
 
+_MOVES = {"tpu.pad": ("pad_const", ["pads*"]), "tpu.crop": ("crop", ["crop_offset*", "steps*"]),
+          "tpu.permute": ("permute", ["order*"]), "tpu.reorg": ("reorg", ["stride"]),
+          "tpu.tile": ("tile", ["axis", "tiles"]), "tpu.reverse": ("reverse", ["axis"]),
+          "tpu.shuffle_channel": ("shuffle_channel", ["group"]),
+          "tpu.pixelshuffle": ("depth_to_space", ["upscale_factor", "mode_dcr"])}
+
+
 def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=None):
     """Returns {name: int8 NCHW array}.  batch_slice selects images (ops are
     independent across the batch, which is also how the reference runs a batch:
@@ -75,6 +82,19 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             w = op.weights
             y = O.leaky_relu_i8(ins[0], w["rshift_pos"][0], w["multiplier_pos"][0],
                                 w["rshift_neg"][0], w["multiplier_neg"][0])
+        elif t in _MOVES:
+            a = op.attrs
+            kind, keys = _MOVES[t]
+            if t == "tpu.pad" and a.get("mode_edge", 0):
+                kind = "pad_edge"
+            params = []
+            for k in keys:
+                if k.endswith("*"):
+                    base, cnt, dflt = k[:-1], (8 if k.startswith("pads") else 4), (1 if k.startswith("steps") else 0)
+                    params += [int(a.get(base + str(i), dflt)) for i in range(cnt)]
+                else:
+                    params.append(int(a.get(k, 0)))
+            y = O.move_i8(kind, ins[0], params, op.shape)
         elif t == "tpu.prelu":
             w = op.weights
             y = O.prelu_i8(ins[0], w["slope"], w["rshift_pos"][0], w["multiplier_pos"][0],

@@ -71,6 +71,15 @@ def _load():
                                        C.c_size_t]
     lib.orc_binary_i8.restype = C.c_int
     lib.orc_binary_i8.argtypes = [i8p, i8p, i8p, C.POINTER(BinaryDesc), f32p, C.c_float]
+    i64p, ip = C.POINTER(C.c_int64), C.POINTER(C.c_int)
+    lib.orc_pad_i8.argtypes = [i8p, i8p, i64p, ip, C.c_int]
+    lib.orc_crop_i8.argtypes = [i8p, i8p, i64p, i64p, ip, ip]
+    lib.orc_permute_i8.argtypes = [i8p, i8p, i64p, ip]
+    lib.orc_reorg_i8.argtypes = [i8p, i8p, i64p, C.c_int]
+    lib.orc_tile_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
+    lib.orc_reverse_i8.argtypes = [i8p, i8p, i64p, C.c_int]
+    lib.orc_shuffle_channel_i8.argtypes = [i8p, i8p, i64p, C.c_int]
+    lib.orc_depth_to_space_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_pool_max_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc)]
     lib.orc_pool_avg_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc), C.c_float, C.c_float]
     lib.orc_leaky_relu_i8.argtypes = [i8p, i8p, C.c_size_t] + [C.c_float] * 4
@@ -190,6 +199,58 @@ def eltwise_add_i8(xs, multiplier, rshift, do_relu):
     lib.orc_eltwise_add_i8(_ptr_array(xs), len(xs), _p(m, C.c_float), _p(r, C.c_float),
                            int(do_relu), _p(y, C.c_int8), xs[0].size)
     return y
+
+
+def _shape64(shape):
+    return (C.c_int64 * 4)(*shape)
+
+
+def _ints(v):
+    return (C.c_int * len(v))(*[int(a) for a in v])
+
+
+def move_i8(kind, x, params, out_shape=None):
+    """the data movement ops by name: pad_const, pad_edge, crop, permute, reorg, tile, reverse,
+    shuffle_channel, depth_to_space (params as in the C ABI's tpuhip_move_desc.p)"""
+    x = _i8(x)
+    s, p = x.shape, [int(v) for v in params]
+    if kind in ("pad_const", "pad_edge"):
+        out = tuple(s[k] + p[k] + p[4 + k] for k in range(4))
+    elif kind == "crop":
+        out = tuple(out_shape)
+    elif kind == "permute":
+        out = tuple(s[p[k]] for k in range(4))
+    elif kind == "reorg":
+        out = (s[0], s[1] * p[0] * p[0], s[2] // p[0], s[3] // p[0])
+    elif kind == "tile":
+        out = tuple(s[k] * (p[1] if k == p[0] else 1) for k in range(4))
+    elif kind in ("reverse", "shuffle_channel"):
+        out = s
+    else:
+        out = (s[0], s[1] // (p[0] * p[0]), s[2] * p[0], s[3] * p[0])
+    y = np.empty(out, np.int8)
+    xp, yp = _p(x, C.c_int8), _p(y, C.c_int8)
+    if kind in ("pad_const", "pad_edge"):
+        lib.orc_pad_i8(xp, yp, _shape64(s), _ints(p[:8]), int(kind == "pad_edge"))
+    elif kind == "crop":
+        lib.orc_crop_i8(xp, yp, _shape64(s), _shape64(out), _ints(p[:4]), _ints(p[4:8]))
+    elif kind == "permute":
+        lib.orc_permute_i8(xp, yp, _shape64(s), _ints(p[:4]))
+    elif kind == "reorg":
+        lib.orc_reorg_i8(xp, yp, _shape64(s), p[0])
+    elif kind == "tile":
+        lib.orc_tile_i8(xp, yp, _shape64(s), p[0], p[1])
+    elif kind == "reverse":
+        lib.orc_reverse_i8(xp, yp, _shape64(s), p[0])
+    elif kind == "shuffle_channel":
+        lib.orc_shuffle_channel_i8(xp, yp, _shape64(s), p[0])
+    else:
+        lib.orc_depth_to_space_i8(xp, yp, _shape64(s), p[0], p[1])
+    return y
+
+
+MOVE_KINDS = ["pad_const", "pad_edge", "crop", "permute", "reorg", "tile", "reverse",
+              "shuffle_channel", "depth_to_space"]
 
 
 def prelu_i8(x, slope, rshift_pos, multiplier_pos, rshift_neg):

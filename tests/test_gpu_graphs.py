@@ -307,3 +307,39 @@ def test_graph_with_elementwise_family_matches_the_oracle():
         assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
     assert len(np.unique(want[bs])) > 8
     m.close()
+
+
+def test_graph_with_data_movement_ops_matches_the_oracle():
+    b = graphs.Builder("movers", graphs.BASE_SEED + 78, 2, (6, 12))
+    x = b.input("input", 12, 8, 6)
+    c1 = b.conv("c1", x, 36, 3, relu=True)
+    g = b.g
+
+    def mv(t, name, src, shape, **attrs):
+        g.add(graphs.Op(t, name, [src], shape, attrs))
+        return name
+
+    n = 2
+    p = mv("tpu.pad", "pad", c1, (n, 36, 11, 9), pads0=0, pads1=0, pads2=1, pads3=2, pads4=0, pads5=0,
+           pads6=2, pads7=1)
+    pe = mv("tpu.pad", "pad_edge", c1, (n, 36, 10, 8), mode_edge=1, pads0=0, pads1=0, pads2=1, pads3=1,
+            pads4=0, pads5=0, pads6=1, pads7=1)
+    cr = mv("tpu.crop", "crop", p, (n, 20, 8, 6), crop_offset0=0, crop_offset1=4, crop_offset2=1,
+            crop_offset3=2)
+    pm = mv("tpu.permute", "perm", cr, (n, 8, 6, 20), order0=0, order1=2, order2=3, order3=1)
+    ro = mv("tpu.reorg", "reorg", c1, (n, 144, 4, 3), stride=2)
+    d2s = mv("tpu.pixelshuffle", "d2s", ro, (n, 36, 8, 6), upscale_factor=2, mode_dcr=1)
+    tl = mv("tpu.tile", "tile", d2s, (n, 36, 8, 18), axis=3, tiles=3)
+    rv = mv("tpu.reverse", "rev", tl, (n, 36, 8, 18), axis=2)
+    sh = mv("tpu.shuffle_channel", "shuf", rv, (n, 36, 8, 18), group=4)
+    g.outputs = [pm, pe, sh]
+    want = oracle_graph.run(g)
+    # DCR depth-to-space undoes a reorg (both put the block offset outermost in the channels)
+    assert np.array_equal(want["d2s"], want["c1"])
+    m = module()
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()

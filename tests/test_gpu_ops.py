@@ -557,3 +557,47 @@ def test_prelu_per_channel_tables(ctx, shape):
         ctx.prelu(xt, yt, slope, rp, mp, rn)
         assert np.array_equal(ctx.to_nchw(yt), O.prelu_i8(x, slope, rp, mp, rn)), (mp, rp, rn)
         assert not ctx.raw(yt)[..., shape[1]:].any()
+
+
+MOVES = [
+    ("pad_const", (2, 20, 5, 4), [0, 1, 2, 3, 1, 0, 4, 1], None),
+    ("pad_const", (2, 20, 5, 4), [0, -1, 2, -2, 0, 1, -1, 0], None),
+    ("pad_edge", (2, 20, 5, 4), [0, 0, 2, 1, 0, 0, 3, 4], None),
+    ("crop", (3, 37, 9, 8), [1, 2, 0, 3, 1, 1, 1, 1], (2, 30, 9, 5)),
+    ("crop", (3, 37, 9, 8), [0, 1, 2, 0, 2, 3, 2, 4], (2, 12, 4, 2)),
+    ("permute", (2, 3, 18, 4), [0, 2, 3, 1], None),
+    ("permute", (2, 19, 5, 4), [0, 3, 1, 2], None),
+    ("permute", (4, 3, 5, 33), [3, 2, 1, 0], None),
+    ("reorg", (2, 24, 6, 4), [2], None),
+    ("tile", (2, 20, 5, 4), [1, 3], None),
+    ("tile", (2, 20, 5, 4), [3, 2], None),
+    ("reverse", (2, 20, 5, 4), [1], None),
+    ("reverse", (2, 20, 5, 4), [2], None),
+    ("shuffle_channel", (2, 24, 3, 4), [3], None),
+    ("depth_to_space", (2, 36, 3, 4), [3, 0], None),
+    ("depth_to_space", (2, 64, 3, 4), [2, 1], None),
+]
+
+
+@pytest.mark.parametrize("kind,shape,params,out_shape", MOVES)
+def test_data_movement_ops(ctx, kind, shape, params, out_shape):
+    rng = np.random.default_rng(len(kind) + shape[1])
+    x = rnd_i8(rng, shape)
+    want = O.move_i8(kind, x, params, out_shape)
+    xt, yt = ctx.from_nchw(x), ctx.tensor(want.shape)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.move(O.MOVE_KINDS.index(kind), xt, yt, params)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., want.shape[1]:].any()
+
+
+def test_data_movement_rejects_bad_arguments(ctx):
+    x, y = ctx.tensor((1, 16, 4, 4)), ctx.tensor((1, 16, 4, 4))
+    with pytest.raises(capi.TpuHipError, match="reads past"):
+        ctx.move(capi.MOVE_CROP, x, y, [0, 1, 0, 0, 1, 1, 1, 1])
+    with pytest.raises(capi.TpuHipError, match="permutation"):
+        ctx.move(capi.MOVE_PERMUTE, x, y, [0, 1, 2, 2])
+    with pytest.raises(capi.TpuHipError, match="group"):
+        ctx.move(capi.MOVE_SHUFFLE_CHANNEL, x, y, [5])
+    with pytest.raises(capi.TpuHipError, match="expected"):
+        ctx.move(capi.MOVE_PAD_CONST, x, y, [0, 0, 1, 0, 0, 0, 0, 0])

@@ -1,0 +1,75 @@
+"""Pins the oracle's data movement ops against numpy / torch routines that define the same
+rearrangements independently (np.pad, slicing, transpose, tile, flip, reshape chains,
+torch.pixel_shuffle)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle_lib as O
+
+
+def rnd(shape, seed=0):
+    return np.random.default_rng(seed).integers(-128, 128, shape).astype(np.int8)
+
+
+def test_pad_constant_is_zero_padding_and_negative_pads_cut():
+    x = rnd((2, 3, 5, 4))
+    got = O.move_i8("pad_const", x, [0, 1, 2, 3, 1, 0, 4, 1])
+    assert np.array_equal(got, np.pad(x, [(0, 1), (1, 0), (2, 4), (3, 1)]))
+    got = O.move_i8("pad_const", x, [0, -1, 2, -2, 0, 1, -1, 0])     # cut c at the front, w twice, h at the end
+    want = np.pad(x[:, 1:, :4, 2:], [(0, 0), (0, 1), (2, 0), (0, 0)])
+    assert np.array_equal(got, want)
+
+
+def test_pad_edge_replicates_borders():
+    x = rnd((2, 3, 5, 4), 1)
+    got = O.move_i8("pad_edge", x, [0, 0, 2, 1, 0, 0, 3, 4])
+    assert np.array_equal(got, np.pad(x, [(0, 0), (0, 0), (2, 3), (1, 4)], mode="edge"))
+
+
+def test_crop_with_offsets_and_steps():
+    x = rnd((3, 7, 9, 8), 2)
+    got = O.move_i8("crop", x, [1, 2, 0, 3, 1, 1, 1, 1], out_shape=(2, 4, 9, 5))
+    assert np.array_equal(got, x[1:3, 2:6, :, 3:8])
+    got = O.move_i8("crop", x, [0, 1, 2, 0, 2, 3, 2, 4], out_shape=(2, 2, 4, 2))
+    assert np.array_equal(got, x[0::2, 1::3, 2::2, 0::4][:2, :2, :4, :2])
+
+
+@pytest.mark.parametrize("order", [(0, 2, 3, 1), (0, 3, 1, 2), (1, 0, 2, 3), (3, 2, 1, 0), (0, 1, 3, 2)])
+def test_permute_is_numpy_transpose(order):
+    x = rnd((2, 3, 5, 4), 3)
+    assert np.array_equal(O.move_i8("permute", x, order), np.transpose(x, order))
+
+
+def test_reorg_is_space_to_depth_with_the_block_offset_outermost():
+    x = rnd((2, 3, 6, 4), 4)
+    b, c, h, w = x.shape
+    s = 2
+    want = x.reshape(b, c, h // s, s, w // s, s).transpose(0, 3, 5, 1, 2, 4).reshape(b, s * s * c, h // s, w // s)
+    assert np.array_equal(O.move_i8("reorg", x, [s]), want)
+
+
+@pytest.mark.parametrize("axis", [0, 1, 2, 3])
+def test_tile_and_reverse(axis):
+    x = rnd((2, 3, 5, 4), 5)
+    reps = [1, 1, 1, 1]
+    reps[axis] = 3
+    assert np.array_equal(O.move_i8("tile", x, [axis, 3]), np.tile(x, reps))
+    assert np.array_equal(O.move_i8("reverse", x, [axis]), np.flip(x, axis))
+
+
+def test_shuffle_channel_is_group_transpose():
+    x = rnd((2, 12, 3, 4), 6)
+    g = 3
+    want = x.reshape(2, g, 12 // g, 3, 4).transpose(0, 2, 1, 3, 4).reshape(x.shape)
+    assert np.array_equal(O.move_i8("shuffle_channel", x, [g]), want)
+
+
+def test_depth_to_space_both_modes():
+    x = rnd((2, 12, 3, 4), 7)
+    r = 2
+    crd = torch.pixel_shuffle(torch.from_numpy(x.astype(np.int32)), r).numpy().astype(np.int8)
+    assert np.array_equal(O.move_i8("depth_to_space", x, [r, 0]), crd)
+    b, c, h, w = x.shape
+    dcr = x.reshape(b, r, r, c // (r * r), h, w).transpose(0, 3, 4, 1, 5, 2).reshape(b, c // (r * r), h * r, w * r)
+    assert np.array_equal(O.move_i8("depth_to_space", x, [r, 1]), dcr)

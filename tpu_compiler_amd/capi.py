@@ -34,6 +34,15 @@ class BinaryDesc(C.Structure):
 BIN_ADD, BIN_SUB, BIN_MAX, BIN_MIN, BIN_MUL = range(5)
 
 
+class MoveDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in ("kind", "in_", "ic", "ih", "iw", "on", "oc", "oh", "ow",
+                                       "x_cs", "y_cs")] + [("p", C.c_int * 8)]
+
+
+(MOVE_PAD_CONST, MOVE_PAD_EDGE, MOVE_CROP, MOVE_PERMUTE, MOVE_REORG, MOVE_TILE, MOVE_REVERSE,
+ MOVE_SHUFFLE_CHANNEL, MOVE_DEPTH_TO_SPACE) = range(9)
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
@@ -79,6 +88,7 @@ PROTOTYPES = {
     "tpuhip_lut_per_channel_i8": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t, C.c_int, C.c_int]),
     "tpuhip_prelu_tables": (C.c_int, [C.POINTER(C.c_float), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32,
                                       C.POINTER(C.c_int8)]),
+    "tpuhip_move_i8": (C.c_int, [C.c_void_p, C.POINTER(MoveDesc), C.c_void_p, C.c_void_p]),
     "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
@@ -334,6 +344,11 @@ class Context:
         m = np.ascontiguousarray(mult, dtype=np.int8)
         self._ck(self.lib.tpuhip_eltwise_add_i8(self.h, ptrs, len(xs), m.ctypes.data, int(rshift),
                                                 int(do_relu), y.ptr, y.nbytes))
+
+    def move(self, kind, x, y, params):
+        p = (C.c_int * 8)(*(list(params) + [0] * (8 - len(params))))
+        d = MoveDesc(kind, *x.shape, *y.shape, x.cs, y.cs, p)
+        self._ck(self.lib.tpuhip_move_i8(self.h, C.byref(d), x.ptr, y.ptr))
 
     def prelu(self, x, y, slope, rshift_pos, multiplier_pos, rshift_neg):
         c = x.shape[1]

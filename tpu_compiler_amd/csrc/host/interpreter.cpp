@@ -219,6 +219,22 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<PoolingOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.leaky_relu") {
       krnl = std::make_shared<LeakyReluOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.pad") {
+      krnl = std::make_shared<PadOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.crop") {
+      krnl = std::make_shared<CropOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.permute") {
+      krnl = std::make_shared<PermuteOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.reorg") {
+      krnl = std::make_shared<ReorgOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.tile") {
+      krnl = std::make_shared<TileOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.reverse") {
+      krnl = std::make_shared<ReverseOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.shuffle_channel") {
+      krnl = std::make_shared<ShuffleChannelOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.pixelshuffle") {
+      krnl = std::make_shared<DepthToSpaceOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.prelu") {
       krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {

@@ -539,6 +539,76 @@ void BinaryOpKernel::invoke() {
 }
 
 // ---------------------------------------------------------------------------
+// Pad, Crop, Permute, Reorg, Tile, Reverse, ShuffleChannel, DepthToSpace
+// ---------------------------------------------------------------------------
+MoveOpKernel::MoveOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+                           const char *what)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8(what);
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail(std::string(what) + " '" + name + "': input missing");
+  if (op.operands.empty() || valueMapping.shapes[op.operands[0]].size() != 4 || shape.size() != 4)
+    fail(std::string(what) + " '" + name + "': only 4-d shapes are supported");
+  tpuhip_move_desc &d = desc;
+  d.in = input_data->n; d.ic = input_data->c; d.ih = input_data->h; d.iw = input_data->w;
+  d.on = output_data->n; d.oc = output_data->c; d.oh = output_data->h; d.ow = output_data->w;
+  d.x_cs = input_data->cs;
+  d.y_cs = output_data->cs;
+}
+
+void MoveOpKernel::invoke() {
+  ck(tpuhip_move_i8(ctx, &desc, input_data->data(), output_data->data()), name.c_str());
+}
+
+static void numbered(const OpDesc &op, const char *base, int count, int *out, double dflt, bool required) {
+  for (int i = 0; i < count; ++i) {
+    const std::string key = base + std::to_string(i);
+    out[i] = (int)(required ? op.attr(key) : op.attr(key, dflt));
+  }
+}
+
+PadOpKernel::PadOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Pad") {
+  desc.kind = op.attr("mode_edge", 0) != 0 ? TPUHIP_MOVE_PAD_EDGE : TPUHIP_MOVE_PAD_CONST;
+  numbered(op, "pads", 8, desc.p, 0, true);
+}
+CropOpKernel::CropOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Crop") {
+  desc.kind = TPUHIP_MOVE_CROP;
+  numbered(op, "crop_offset", 4, desc.p, 0, true);
+  numbered(op, "steps", 4, desc.p + 4, 1, false);   // steps default to 1 (parseCropParam)
+}
+PermuteOpKernel::PermuteOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "Permute") {
+  desc.kind = TPUHIP_MOVE_PERMUTE;
+  numbered(op, "order", 4, desc.p, 0, true);
+}
+ReorgOpKernel::ReorgOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Reorg") {
+  desc.kind = TPUHIP_MOVE_REORG;
+  desc.p[0] = (int)op.attr("stride");
+}
+TileOpKernel::TileOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Tile") {
+  desc.kind = TPUHIP_MOVE_TILE;
+  desc.p[0] = (int)op.attr("axis");
+  desc.p[1] = (int)op.attr("tiles");
+}
+ReverseOpKernel::ReverseOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "Reverse") {
+  desc.kind = TPUHIP_MOVE_REVERSE;
+  desc.p[0] = (int)op.attr("axis");
+}
+ShuffleChannelOpKernel::ShuffleChannelOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "ShuffleChannel") {
+  desc.kind = TPUHIP_MOVE_SHUFFLE_CHANNEL;
+  desc.p[0] = (int)op.attr("group");
+}
+DepthToSpaceOpKernel::DepthToSpaceOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "DepthToSpace") {
+  desc.kind = TPUHIP_MOVE_DEPTH_TO_SPACE;
+  desc.p[0] = (int)op.attr("upscale_factor");
+  desc.p[1] = op.attr("mode_dcr", 0) != 0 ? 1 : 0;
+}
+
+// ---------------------------------------------------------------------------
 // Pooling (core/pooling.cpp:33-160)
 // ---------------------------------------------------------------------------
 PoolingOpKernel::PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)

@@ -1,0 +1,227 @@
+// Pure data movement on int8 channels-last tensors: Pad, Crop, Permute, Reorg, Tile,
+// Reverse, ShuffleChannel, DepthToSpace (core/pad.cpp, crop.cpp, permute.cpp, reorg.cpp,
+// tile.cpp, reverse.cpp, shuffle_channel.cpp, depthtospace.cpp).  Each is an index map from
+// the logical (n, c, h, w) of an output element to that of its source; one kernel
+// evaluates the map per element and moves the byte.  A lane produces four consecutive
+// output channels of a pixel (one dword store); pad channels are written as zero.
+#include "common.hpp"
+
+using namespace tpuhip;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct MoveArgs {
+  const int8_t *x;
+  int8_t *y;
+  int kind;
+  int in, ic, ih, iw, ics;
+  int on, oc, oh, ow, ocs;
+  int p[12];
+  int64_t total;   // output pixels * (ocs / 4)
+};
+
+// source of output element o = (n, c, h, w); false: the element is padding (zero)
+__device__ __forceinline__ bool source_of(const MoveArgs &a, const int (&o)[4], int (&s)[4]) {
+  switch (a.kind) {
+    case TPUHIP_MOVE_PAD_CONST: {
+      // p[0..3] where the first kept input element lands, p[4..7] its index, p[8..11] end of
+      // the kept input range
+      bool inside = true;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        s[d] = o[d] - a.p[d] + a.p[4 + d];
+        inside = inside && s[d] >= a.p[4 + d] && s[d] < a.p[8 + d];
+      }
+      return inside;
+    }
+    case TPUHIP_MOVE_PAD_EDGE:
+      s[0] = o[0];
+      s[1] = o[1];
+      s[2] = min(max(o[2] - a.p[2], 0), a.ih - 1);
+      s[3] = min(max(o[3] - a.p[3], 0), a.iw - 1);
+      return true;
+    case TPUHIP_MOVE_CROP:
+#pragma unroll
+      for (int d = 0; d < 4; ++d) s[d] = o[d] * a.p[4 + d] + a.p[d];
+      return true;
+    case TPUHIP_MOVE_PERMUTE:
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        // output dimension d is input dimension p[d]
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (a.p[d] == k) s[k] = o[d];
+      }
+      return true;
+    case TPUHIP_MOVE_REORG: {
+      const int st = a.p[0], off = o[1] / a.ic;
+      s[0] = o[0];
+      s[1] = o[1] - off * a.ic;
+      s[2] = o[2] * st + off / st;
+      s[3] = o[3] * st + off % st;
+      return true;
+    }
+    case TPUHIP_MOVE_TILE: {
+      const int dims[4] = {a.in, a.ic, a.ih, a.iw};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) s[d] = a.p[0] == d ? o[d] % dims[d] : o[d];
+      return true;
+    }
+    case TPUHIP_MOVE_REVERSE: {
+      const int dims[4] = {a.in, a.ic, a.ih, a.iw};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) s[d] = a.p[0] == d ? dims[d] - 1 - o[d] : o[d];
+      return true;
+    }
+    case TPUHIP_MOVE_SHUFFLE_CHANNEL: {
+      const int group = a.p[0], col = a.ic / group;
+      s[0] = o[0];
+      s[1] = (o[1] % group) * col + o[1] / group;
+      s[2] = o[2];
+      s[3] = o[3];
+      return true;
+    }
+    default: {   // TPUHIP_MOVE_DEPTH_TO_SPACE: p[0] = upscale factor, p[1] = DCR mode
+      const int r = a.p[0];
+      const int dh = o[2] % r, dw = o[3] % r;
+      s[0] = o[0];
+      s[1] = a.p[1] ? (dh * r + dw) * a.oc + o[1] : o[1] * r * r + dh * r + dw;
+      s[2] = o[2] / r;
+      s[3] = o[3] / r;
+      return true;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void move_kernel(MoveArgs a) {
+  const int c4 = a.ocs >> 2;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int cq = (int)(i % c4);
+    const int pix = (int)(i / c4);
+    const int w = pix % a.ow;
+    const int h = (pix / a.ow) % a.oh;
+    const int n = pix / (a.ow * a.oh);
+    uint32_t word = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int c = cq * 4 + b;
+      if (c >= a.oc) continue;
+      const int o[4] = {n, c, h, w};
+      int s[4] = {0, 0, 0, 0};
+      if (!source_of(a, o, s)) continue;
+      const int8_t v = a.x[((int64_t)(s[0] * a.ih + s[2]) * a.iw + s[3]) * a.ics + s[1]];
+      word |= (uint32_t)(uint8_t)v << (8 * b);
+    }
+    *reinterpret_cast<uint32_t *>(a.y + (int64_t)pix * a.ocs + cq * 4) = word;
+  }
+}
+
+}  // namespace
+
+extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
+  TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");
+  TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_DEPTH_TO_SPACE,
+                 "move: unknown kind %d", d->kind);
+  TPUHIP_REQUIRE(d->in > 0 && d->ic > 0 && d->ih > 0 && d->iw > 0 && d->on > 0 && d->oc > 0 &&
+                     d->oh > 0 && d->ow > 0,
+                 "move: non-positive dimension");
+  TPUHIP_REQUIRE(d->x_cs >= d->ic && d->x_cs % 16 == 0 && d->y_cs >= d->oc && d->y_cs % 16 == 0,
+                 "move: channel strides must be multiples of 16 covering the channels");
+  TPUHIP_REQUIRE((int64_t)d->in * d->ih * d->iw * d->x_cs < (1ll << 31) &&
+                     (int64_t)d->on * d->oh * d->ow < (1ll << 31),
+                 "move: tensor too large");
+  const int is[4] = {d->in, d->ic, d->ih, d->iw}, os[4] = {d->on, d->oc, d->oh, d->ow};
+  const int *p = d->p;
+  MoveArgs a{};
+  // every kind: check that the map stays inside the input for every output element
+  switch (d->kind) {
+    case TPUHIP_MOVE_PAD_CONST:
+      // p[0..3] pads at the beginning, p[4..7] at the end (negative: cut), as the op's attribute
+      for (int k = 0; k < 4; ++k) {
+        TPUHIP_REQUIRE(os[k] == is[k] + p[k] + p[4 + k], "pad: output dimension %d is %d, expected %d",
+                       k, os[k], is[k] + p[k] + p[4 + k]);
+        a.p[k] = p[k] < 0 ? 0 : p[k];
+        a.p[4 + k] = p[k] < 0 ? -p[k] : 0;
+        a.p[8 + k] = p[4 + k] < 0 ? is[k] + p[4 + k] : is[k];
+        TPUHIP_REQUIRE(a.p[4 + k] <= a.p[8 + k], "pad: dimension %d is cut away entirely", k);
+      }
+      break;
+    case TPUHIP_MOVE_PAD_EDGE:
+      TPUHIP_REQUIRE(p[0] == 0 && p[1] == 0 && p[4] == 0 && p[5] == 0, "pad: edge mode pads h and w only");
+      TPUHIP_REQUIRE(p[2] >= 0 && p[3] >= 0 && p[6] >= 0 && p[7] >= 0, "pad: edge mode needs pads >= 0");
+      for (int k = 0; k < 4; ++k) {
+        TPUHIP_REQUIRE(os[k] == is[k] + p[k] + p[4 + k], "pad: output dimension %d is %d, expected %d",
+                       k, os[k], is[k] + p[k] + p[4 + k]);
+        a.p[k] = p[k];
+      }
+      break;
+    case TPUHIP_MOVE_CROP:
+      // p[0..3] offsets, p[4..7] steps
+      for (int k = 0; k < 4; ++k) {
+        TPUHIP_REQUIRE(p[k] >= 0 && p[4 + k] >= 1 && (int64_t)(os[k] - 1) * p[4 + k] + p[k] < is[k],
+                       "crop: dimension %d reads past the input", k);
+        a.p[k] = p[k];
+        a.p[4 + k] = p[4 + k];
+      }
+      break;
+    case TPUHIP_MOVE_PERMUTE: {
+      int seen = 0;
+      for (int k = 0; k < 4; ++k) {
+        TPUHIP_REQUIRE(p[k] >= 0 && p[k] < 4, "permute: order[%d] = %d", k, p[k]);
+        seen |= 1 << p[k];
+        TPUHIP_REQUIRE(os[k] == is[p[k]], "permute: output dimension %d is %d, expected %d", k, os[k],
+                       is[p[k]]);
+        a.p[k] = p[k];
+      }
+      TPUHIP_REQUIRE(seen == 15, "permute: order is not a permutation");
+      break;
+    }
+    case TPUHIP_MOVE_REORG:
+      TPUHIP_REQUIRE(p[0] >= 1 && is[2] % p[0] == 0 && is[3] % p[0] == 0, "reorg: bad stride %d", p[0]);
+      TPUHIP_REQUIRE(os[0] == is[0] && os[1] == is[1] * p[0] * p[0] && os[2] == is[2] / p[0] &&
+                         os[3] == is[3] / p[0],
+                     "reorg: output shape does not match");
+      a.p[0] = p[0];
+      break;
+    case TPUHIP_MOVE_TILE:
+      TPUHIP_REQUIRE(p[0] >= 0 && p[0] < 4 && p[1] >= 1, "tile: bad axis %d / tiles %d", p[0], p[1]);
+      for (int k = 0; k < 4; ++k)
+        TPUHIP_REQUIRE(os[k] == (k == p[0] ? is[k] * p[1] : is[k]), "tile: output dimension %d is %d", k,
+                       os[k]);
+      a.p[0] = p[0];
+      break;
+    case TPUHIP_MOVE_REVERSE:
+      TPUHIP_REQUIRE(p[0] >= 0 && p[0] < 4, "reverse: bad axis %d", p[0]);
+      for (int k = 0; k < 4; ++k) TPUHIP_REQUIRE(os[k] == is[k], "reverse: shapes differ");
+      a.p[0] = p[0];
+      break;
+    case TPUHIP_MOVE_SHUFFLE_CHANNEL:
+      TPUHIP_REQUIRE(p[0] >= 1 && is[1] % p[0] == 0, "shuffle_channel: wrong group size, c=%d, group=%d",
+                     is[1], p[0]);
+      for (int k = 0; k < 4; ++k) TPUHIP_REQUIRE(os[k] == is[k], "shuffle_channel: shapes differ");
+      a.p[0] = p[0];
+      break;
+    default:
+      TPUHIP_REQUIRE(p[0] >= 1 && is[1] % (p[0] * p[0]) == 0, "depth_to_space: bad upscale factor %d", p[0]);
+      TPUHIP_REQUIRE(os[0] == is[0] && os[1] == is[1] / (p[0] * p[0]) && os[2] == is[2] * p[0] &&
+                         os[3] == is[3] * p[0],
+                     "depth_to_space: output shape does not match");
+      a.p[0] = p[0];
+      a.p[1] = p[1] ? 1 : 0;
+      break;
+  }
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  a.x = (const int8_t *)x; a.y = (int8_t *)y;
+  a.kind = d->kind;
+  a.in = d->in; a.ic = d->ic; a.ih = d->ih; a.iw = d->iw; a.ics = d->x_cs;
+  a.on = d->on; a.oc = d->oc; a.oh = d->oh; a.ow = d->ow; a.ocs = d->y_cs;
+  a.total = (int64_t)d->on * d->oh * d->ow * (d->y_cs / 4);
+  const unsigned blocks = (unsigned)std::max<int64_t>(
+      1, std::min<int64_t>(ceil_div64(a.total, kThreads), (int64_t)ctx->num_cu * 32));
+  launch(ctx, move_kernel, dim3(blocks), dim3(kThreads), a);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
