@@ -164,7 +164,8 @@ public:
 class Conv2DOpKernel : public CPUOpKernel {  // core/conv.cpp
 public:
   static constexpr const char *OpName = "CPUConv2DOp";
-  Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+      : Conv2DOpKernel(op, valueMapping, weightMapping, false) {}
   ~Conv2DOpKernel() override;
   void invoke() override;
   const char *algo_name() const;
@@ -189,6 +190,11 @@ public:
   void set_store_result(bool store);
   SyncedData result() const { return output_data; }
 
+protected:
+  // transposed: the attributes describe a DeConv2D; it runs as a stride-1 conv over the
+  // zero-inserted input with the filter flipped
+  Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping, bool transposed);
+
 private:
   tpuhip_conv_weights *packed = nullptr;
   SyncedData input_data, output_data;
@@ -198,6 +204,14 @@ private:
   SyncedData lut_dst;
   int8_t lut_table[256];
   bool store_lut = true;
+};
+
+// core/deconv.cpp:7-73, same operands and epilogue as Conv2D
+class DeConv2DOpKernel : public Conv2DOpKernel {
+public:
+  static constexpr const char *OpName = "CPUDeConv2DOp";
+  DeConv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+      : Conv2DOpKernel(op, valueMapping, weightMapping, true) {}
 };
 
 class FullyConnectedOpKernel : public CPUOpKernel {  // core/fullyconnected.cpp

@@ -646,3 +646,44 @@ void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *is, int r,
               x[i_index++];
         }
 }
+
+/* ------------------------------------------------------------------------- */
+/* transposed convolution                                                     */
+/* ------------------------------------------------------------------------- */
+void orc_deconv2d_acc(const int8_t *x, const int8_t *w, int32_t *acc, const orc_conv_desc *d) {
+  const int icg = d->ic / d->g, ocg = d->oc / d->g;
+  memset(acc, 0, sizeof(int32_t) * (size_t)d->n * d->oc * d->oh * d->ow);
+#pragma omp parallel for collapse(2)
+  for (int n = 0; n < d->n; ++n)
+    for (int oc = 0; oc < d->oc; ++oc) {
+      const int g = oc / ocg;
+      int32_t *ap = acc + ((size_t)n * d->oc + oc) * d->oh * d->ow;
+      for (int c = 0; c < icg; ++c) {
+        const int8_t *xp = x + ((size_t)n * d->ic + g * icg + c) * d->ih * d->iw;
+        const int8_t *wp = w + ((size_t)oc * icg + c) * d->kh * d->kw;
+        for (int ih = 0; ih < d->ih; ++ih)
+          for (int iw = 0; iw < d->iw; ++iw) {
+            const int32_t xv = xp[ih * d->iw + iw];
+            for (int kh = 0; kh < d->kh; ++kh) {
+              const int oh = ih * d->sh + kh * d->dh - d->pt;
+              if (oh < 0 || oh >= d->oh) continue;
+              for (int kw = 0; kw < d->kw; ++kw) {
+                const int ow = iw * d->sw + kw * d->dw - d->pl;
+                if (ow < 0 || ow >= d->ow) continue;
+                ap[oh * d->ow + ow] += xv * (int32_t)wp[kh * d->kw + kw];
+              }
+            }
+          }
+      }
+    }
+}
+
+void orc_deconv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                     const float *multiplier, int8_t *y, const orc_conv_desc *d) {
+  const size_t count = (size_t)d->n * d->oc * d->oh * d->ow;
+  int32_t *acc = (int32_t *)malloc(count * sizeof(int32_t));
+  orc_deconv2d_acc(x, w, acc, d);
+  orc_requant_per_channel(acc, y, d->with_bias ? bias : NULL, d->do_relu, d->n, d->oc,
+                          (int64_t)d->oh * d->ow, rshift, multiplier);
+  free(acc);
+}

@@ -79,6 +79,15 @@ void orc_requant_per_channel(const int32_t *acc, int8_t *y, const float *bias, i
 void orc_conv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
                    const float *multiplier, int8_t *y, const orc_conv_desc *d);
 
+/* ---- transposed convolution: core/deconv.cpp:56-73 over MKLDeconv
+ * (NativeCpuImplementation.h:194-280: deconvolution_direct, filter oihw / goihw with o = this
+ * op's output channels).  Every input pixel scatters into the outputs
+ * (ih*sh + kh*dh - pt, iw*sw + kw*dw - pl); then the conv's per-channel epilogue.
+ * d uses the deconvolution's own stride / padding / dilation; ins_* are ignored. ---- */
+void orc_deconv2d_acc(const int8_t *x, const int8_t *w, int32_t *acc, const orc_conv_desc *d);
+void orc_deconv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                     const float *multiplier, int8_t *y, const orc_conv_desc *d);
+
 /* ---- fully connected: core/fullyconnected.cpp:44-91 (no transposes), one
  * rshift / multiplier per batch matmul.  x: batch*m*k, w: batch*n*k,
  * bias: batch*n or NULL, y: batch*m*n ---- */

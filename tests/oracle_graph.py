@@ -50,6 +50,19 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             if guards is not None:
                 guards[op.name] = O.conv2d_guard(ins[0], w, d) + int(
                     np.abs(op.weights["bias"]).max())
+        elif t == "tpu.deconv_2d":
+            a = op.attrs
+            w = op.weights["filter"].astype(np.int8)
+            g_ = int(a.get("group", 1))
+            w = w.reshape(op.shape[1], ins[0].shape[1] // g_, int(a["kernel_h"]), int(a["kernel_w"]))
+            d = O.make_deconv_desc(ins[0].shape, w.shape, g_, (int(a["stride_h"]), int(a["stride_w"])),
+                                   (int(a["padding_t"]), int(a["padding_b"]), int(a["padding_l"]),
+                                    int(a["padding_r"])),
+                                   (int(a.get("dilation_h", 1)), int(a.get("dilation_w", 1))),
+                                   (op.shape[2], op.shape[3]), bool(a.get("do_relu", 0)),
+                                   bool(a.get("with_bias", 1)))
+            y = O.deconv2d_i8(ins[0], w, op.weights.get("bias"), op.weights["rshift"],
+                              op.weights["multiplier"], d)
         elif t == "tpu.fully_connected":
             x = ins[0].reshape(ins[0].shape[0], -1)
             w = op.weights["filter"].astype(np.int8)

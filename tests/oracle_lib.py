@@ -64,6 +64,8 @@ def _load():
     lib.orc_requant_per_channel.argtypes = [i32p, i8p, f32p, C.c_int, C.c_int64, C.c_int64,
                                             C.c_int64, f32p, f32p]
     lib.orc_conv2d_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p, C.POINTER(ConvDesc)]
+    lib.orc_deconv2d_acc.argtypes = [i8p, i8p, i32p, C.POINTER(ConvDesc)]
+    lib.orc_deconv2d_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p, C.POINTER(ConvDesc)]
     lib.orc_fc_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p] + [C.c_int] * 5
     lib.orc_fc_guard.restype = C.c_int64
     lib.orc_fc_guard.argtypes = [i8p, i8p, f32p] + [C.c_int] * 4
@@ -198,6 +200,31 @@ def eltwise_add_i8(xs, multiplier, rshift, do_relu):
     m, r = _f32(multiplier), _f32(rshift)
     lib.orc_eltwise_add_i8(_ptr_array(xs), len(xs), _p(m, C.c_float), _p(r, C.c_float),
                            int(do_relu), _p(y, C.c_int8), xs[0].size)
+    return y
+
+
+def make_deconv_desc(x_shape, w_shape, g, stride, pads, dil, out_hw, do_relu=False, with_bias=True):
+    """w_shape = (oc, ic // g, kh, kw); out_hw is the op's result size"""
+    n, ic, ih, iw = x_shape
+    return ConvDesc(n, ic, ih, iw, w_shape[0], out_hw[0], out_hw[1], g, w_shape[2], w_shape[3],
+                    stride[0], stride[1], pads[0], pads[1], pads[2], pads[3], dil[0], dil[1], 0, 0,
+                    int(do_relu), int(with_bias))
+
+
+def deconv2d_acc(x, w, d):
+    x, w = _i8(x), _i8(w)
+    acc = np.empty((d.n, d.oc, d.oh, d.ow), np.int32)
+    lib.orc_deconv2d_acc(_p(x, C.c_int8), _p(w, C.c_int8), _p(acc, C.c_int32), C.byref(d))
+    return acc
+
+
+def deconv2d_i8(x, w, bias, rshift, multiplier, d):
+    x, w = _i8(x), _i8(w)
+    y = np.empty((d.n, d.oc, d.oh, d.ow), np.int8)
+    b = _f32(bias) if bias is not None else None
+    lib.orc_deconv2d_i8(_p(x, C.c_int8), _p(w, C.c_int8), _p(b, C.c_float) if b is not None else None,
+                        _p(_f32(rshift), C.c_float), _p(_f32(multiplier), C.c_float),
+                        _p(y, C.c_int8), C.byref(d))
     return y
 
 

@@ -343,3 +343,37 @@ def test_graph_with_data_movement_ops_matches_the_oracle():
     for op in g.ops:
         assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
     m.close()
+
+
+@pytest.mark.parametrize("cfg", [
+    # ic, ih, iw, oc, k, stride, pads(t,b,l,r), dil, groups, out_hw
+    (24, 7, 6, 40, 3, (2, 2), (1, 1, 1, 1), (1, 1), 1, (14, 12)),     # output_padding 1
+    (16, 5, 9, 24, 4, (2, 3), (1, 1, 2, 2), (1, 1), 2, (10, 24)),
+    (20, 6, 6, 20, 3, (1, 1), (0, 0, 0, 0), (2, 2), 20, (10, 10)),    # depthwise, dilated
+    (12, 8, 5, 18, 2, (2, 2), (0, 0, 0, 0), (1, 1), 1, (16, 10)),     # the 2x upsampling deconv
+])
+def test_deconv_graph_matches_the_oracle(cfg):
+    ic, ih, iw, oc, k, stride, pads, dil, grp, out_hw = cfg
+    rng = np.random.default_rng(ic + oc + k)
+    g = graphs.Graph("deconv", 1)
+    x = rng.integers(-128, 128, (2, ic, ih, iw)).astype(np.int8)
+    inp = g.add(graphs.Op("tpu.input", "input", [], x.shape))
+    inp.data = x
+    w = np.clip(np.rint(rng.normal(0, 30, (oc, ic // grp, k, k))), -127, 127).astype(np.float32)
+    bias = rng.integers(-2000, 2000, oc).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, oc) * 128).astype(np.float32)
+    rsh = rng.integers(5, 12, oc).astype(np.float32)
+    g.add(graphs.Op("tpu.deconv_2d", "up", ["input"], (2, oc) + out_hw,
+                    dict(kernel_h=k, kernel_w=k, stride_h=stride[0], stride_w=stride[1],
+                         padding_t=pads[0], padding_b=pads[1], padding_l=pads[2], padding_r=pads[3],
+                         dilation_h=dil[0], dilation_w=dil[1], group=grp, with_bias=1, do_relu=1),
+                    dict(filter=w.ravel(), bias=bias, rshift=rsh, multiplier=mult), "RSHIFT_AND_M_I32"))
+    g.outputs = ["up"]
+    want = oracle_graph.run(g)
+    m = module()
+    m.load(g)
+    m.set_tensor("input", x.astype(np.float32))
+    m.invoke()
+    assert np.array_equal(m.get_tensor_i8("up"), want["up"])
+    assert len(np.unique(want["up"])) > 8
+    m.close()

@@ -73,3 +73,24 @@ def test_depth_to_space_both_modes():
     b, c, h, w = x.shape
     dcr = x.reshape(b, r, r, c // (r * r), h, w).transpose(0, 3, 4, 1, 5, 2).reshape(b, c // (r * r), h * r, w * r)
     assert np.array_equal(O.move_i8("depth_to_space", x, [r, 1]), dcr)
+
+
+@pytest.mark.parametrize("cfg", [
+    # n, ic, ih, iw, oc, k, stride, pads(t,b,l,r), dil, groups, output_padding
+    (2, 6, 5, 4, 8, 3, (2, 2), (1, 1, 1, 1), (1, 1), 1, (1, 1)),
+    (1, 4, 7, 6, 6, 4, (2, 3), (1, 1, 2, 2), (1, 1), 2, (0, 1)),
+    (2, 5, 4, 4, 5, 3, (1, 1), (0, 0, 0, 0), (2, 2), 5, (0, 0)),
+    (1, 3, 6, 5, 7, 2, (2, 2), (0, 0, 0, 0), (1, 1), 1, (0, 0)),
+])
+def test_deconv_accumulators_equal_torch_conv_transpose(cfg):
+    n, ic, ih, iw, oc, k, stride, pads, dil, g, opad = cfg
+    rng = np.random.default_rng(ic + oc)
+    x = rng.integers(-128, 128, (n, ic, ih, iw)).astype(np.int8)
+    w = rng.integers(-127, 128, (oc, ic // g, k, k)).astype(np.int8)       # oihw / goihw
+    # torch wants (ic, oc // g, kh, kw)
+    wt = w.reshape(g, oc // g, ic // g, k, k).transpose(0, 2, 1, 3, 4).reshape(ic, oc // g, k, k)
+    want = torch.nn.functional.conv_transpose2d(
+        torch.from_numpy(x.astype(np.float64)), torch.from_numpy(wt.astype(np.float64)), None, stride,
+        (pads[0], pads[2]), opad, g, dil).numpy()
+    d = O.make_deconv_desc(x.shape, w.shape, g, stride, pads, dil, want.shape[2:])
+    assert np.array_equal(O.deconv2d_acc(x, w, d), want.astype(np.int64))

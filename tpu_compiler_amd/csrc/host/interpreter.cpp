@@ -199,6 +199,8 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<InputOpKernel>(*op, valueMapping, weightMapping, input_details);
     } else if (t == "tpu.conv_2d") {
       krnl = std::make_shared<Conv2DOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.deconv_2d") {
+      krnl = std::make_shared<DeConv2DOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.fully_connected") {
       krnl = std::make_shared<FullyConnectedOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.eltwise_add") {

@@ -5,6 +5,7 @@
 // through the C ABI.
 #include "tpuhip/interpreter.hpp"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -257,7 +258,8 @@ void InputOpKernel::set_tensor(const std::vector<float> &data) {
 // ---------------------------------------------------------------------------
 // Conv2D (core/conv.cpp:11-104)
 // ---------------------------------------------------------------------------
-Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
+                               bool transposed)
     : CPUOpKernel(op, valueMapping, weightMapping) {
   require_int8("Conv2D");
   if (opdTensors.size() != 7) fail("Conv2D '" + name + "': expected 7 operands");
@@ -304,6 +306,24 @@ Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
     fail("Conv2D '" + name + "': rshift / multiplier need one entry per output channel");
   std::vector<int8_t> w8(fsz);
   for (size_t i = 0; i < fsz; ++i) w8[i] = weight_to_i8(filter->at(i), name, "filter");
+  if (transposed) {
+    // out(oh) = sum x(ih) * w(kh) over ih*sh + kh*dh - pt == oh (MKLDeconv,
+    // NativeCpuImplementation.h:194-280) == a stride-1 conv of the input with sh-1 zeros
+    // between its rows, the filter flipped, padded by (kh-1)*dh - pt at the top
+    if (d.ins_h || d.ins_w) fail("DeConv2D '" + name + "': inserted zeros are not an attribute of a deconv");
+    const int pt = (d.kh - 1) * d.dh - d.pt, pl = (d.kw - 1) * d.dw - d.pl;
+    if (pt < 0 || pl < 0) fail("DeConv2D '" + name + "': padding larger than the kernel extent");
+    const int ihd = (d.ih - 1) * d.sh + 1, iwd = (d.iw - 1) * d.sw + 1;
+    d.ins_h = d.sh - 1;
+    d.ins_w = d.sw - 1;
+    d.sh = d.sw = 1;
+    d.pt = pt;
+    d.pl = pl;
+    d.pb = std::max(0, d.oh + d.dh * (d.kh - 1) - ihd - pt);
+    d.pr = std::max(0, d.ow + d.dw * (d.kw - 1) - iwd - pl);
+    const size_t plane = (size_t)d.kh * d.kw;
+    for (size_t f = 0; f < fsz; f += plane) std::reverse(w8.begin() + f, w8.begin() + f + plane);
+  }
   std::vector<int32_t> b32, m32((size_t)d.oc), r32((size_t)d.oc);
   // without with_bias the epilogue adds a zero tensor (conv.cpp:59-61)
   if (d.with_bias) {

@@ -17,6 +17,7 @@ from . import capi
 # activation inputs; None marks an operand the INT8 path leaves empty
 _WEIGHT_OPERANDS = {
     "tpu.conv_2d": ["filter", "bias", None, None, "rshift", "multiplier"],
+    "tpu.deconv_2d": ["filter", "bias", None, None, "rshift", "multiplier"],
     "tpu.fully_connected": ["filter", "bias", None, None, "rshift", "multiplier"],
     "tpu.eltwise_add": [None, None, "rshift", "multiplier"],
     "tpu.eltwise_max": [None, None, "rshift", "multiplier"],
