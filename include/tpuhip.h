@@ -296,6 +296,15 @@ typedef struct tpuhip_move_desc {
 } tpuhip_move_desc;
 int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y);
 
+/* ---- QuantOp at the graph edges -------------------------------------------
+ * Replaces QuantOpKernel::invoke (core/quant.cpp:133-166) for the two conversions an INT8 graph
+ * has: fp32 -> int8 right after an input (round(src * scale), half away from zero, clamped,
+ * :20-30) and int8 -> fp32 (BF16(src * BF16(scale)), :108-116).  The fp32 side is NCHW. */
+int tpuhip_quant_f32_to_i8(tpuhip_ctx *ctx, const void *x_nchw_f32, void *y, int n, int c, int h,
+                           int w, int cs, float scale);
+int tpuhip_dequant_i8_to_f32(tpuhip_ctx *ctx, const void *x, void *y_nchw_f32, int n, int c, int h,
+                             int w, int cs, float scale);
+
 /* ---- module interpreter ------------------------------------------------------ */
 
 /* Flat view of the C++ ModuleInterpreter (include/tpuhip/interpreter.hpp), which

@@ -54,12 +54,14 @@ struct WeightData {
   float at(size_t i) const { return data.at(i); }
 };
 
-// An activation tensor: `batch` slots of one int8 channels-last image set in HBM.
+// An activation tensor: `batch` slots of one int8 channels-last image set in HBM -- or, at
+// the graph edges only (an fp32 input before its QuantOp, the result of a dequantising
+// QuantOp), of float NCHW data like the reference's tensors.
 // Mirrors mlir::TensorData (cpukernel.h:15-78): size(), set_batch_idx(),
 // assign(), tensor(bidx).
 class TensorData {
 public:
-  TensorData(tpuhip_ctx *ctx, int32_t batch, const SyncedDataShape &shape);
+  TensorData(tpuhip_ctx *ctx, int32_t batch, const SyncedDataShape &shape, bool f32 = false);
   ~TensorData();
   TensorData(const TensorData &) = delete;
   TensorData &operator=(const TensorData &) = delete;
@@ -79,7 +81,8 @@ public:
   int n = 1, c = 1, h = 1, w = 1;  // 4-d view of the shape (missing dims are 1)
   bool materialized = true;        // false: no kernel writes this tensor (fused away)
   int cs = 16;                     // channel stride in bytes
-  size_t slot_bytes() const { return (size_t)n * h * w * cs; }
+  bool f32 = false;                // float NCHW instead of int8 channels-last
+  size_t slot_bytes() const { return f32 ? size_ * sizeof(float) : (size_t)n * h * w * cs; }
   tpuhip_ctx *ctx() const { return ctx_; }
 
 private:
@@ -334,6 +337,19 @@ public:
 private:
   SyncedData input_data, output_data;
   void *tables = nullptr;   // device, c * 256 bytes
+};
+
+// core/quant.cpp:118-166.  The result type is the op's quant mode ("INT8" or "NONE"); the
+// source type is that of the operand tensor.  attrs: scale.
+class QuantOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPUQuantOp";
+  QuantOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+  float scale = 1.0f;
 };
 
 class ReluOpKernel : public CPUOpKernel {  // core/activation.cpp:155-164

@@ -687,3 +687,42 @@ void orc_deconv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const 
                           (int64_t)d->oh * d->ow, rshift, multiplier);
   free(acc);
 }
+
+/* ------------------------------------------------------------------------- */
+/* QuantOp                                                                    */
+/* ------------------------------------------------------------------------- */
+
+/* QuantizationArithmetic.cpp:873-913, 958-964 */
+float orc_bf16(float src, int rounding) {
+  uint32_t u;
+  memcpy(&u, &src, 4);
+  uint16_t h;
+  if (rounding) {
+    const uint32_t lsb = (u >> 16) & 1;
+    u += 0x7fff + lsb;
+    h = (uint16_t)(u >> 16);
+    if ((h & 0x7f80) == 0x7f80) h = 0x7f7f;
+  } else {
+    h = (uint16_t)(u >> 16);
+  }
+  const uint32_t o = (uint32_t)h << 16;
+  float dst;
+  memcpy(&dst, &o, 4);
+  return dst;
+}
+
+/* quant.cpp:20-30 */
+void orc_quant_f32_to_i8(const float *src, int8_t *dst, size_t count, float scale) {
+  for (size_t i = 0; i < count; ++i) {
+    const float r = roundf(src[i] * scale);
+    int val = r > 127.0f ? 127 : r < -128.0f ? -128 : (int)r;   /* the int conversion of the */
+    dst[i] = (int8_t)val;                                       /* reference, made total      */
+  }
+}
+
+/* quant.cpp:108-116 with zero_point == 0 */
+void orc_dequant_i8_to_f32(const int8_t *src, float *dst, size_t count, float scale) {
+  const float s = orc_bf16(scale, 1);
+  for (size_t i = 0; i < count; ++i)
+    dst[i] = orc_bf16(orc_bf16((float)src[i] + 0, 0) * s, 1);
+}

@@ -151,6 +151,14 @@ void orc_upsample_i8(const int8_t *x, int8_t *y, int n, int c, int ih, int iw, i
 void orc_concat_i8(const int8_t *const *xs, int nin, const int64_t *shapes, int ndim, int axis,
                    const float *rshift, const float *multiplier, int do_relu, int8_t *y);
 
+/* ---- QuantOp at the graph edges: core/quant.cpp:9-32 (fp32 -> int8 right after an input:
+ * round(src * scale), half away from zero, clamped; zero_point is 0, :138) and :108-124
+ * (int8 -> fp32, always the TPU-aligned form: BF16(BF16(src) * BF16(scale)) with the
+ * round-to-nearest-even BF16 of QuantizationArithmetic.cpp:873-913, infinity clipped). ---- */
+void orc_quant_f32_to_i8(const float *src, int8_t *dst, size_t count, float scale);
+void orc_dequant_i8_to_f32(const int8_t *src, float *dst, size_t count, float scale);
+float orc_bf16(float src, int rounding);
+
 /* ---- pure data movement (no INT8-specific branch in the reference), 4-d shapes ---- */
 /* core/pad.cpp:62-112 (constant mode; negative pads cut) and :7-60 (edge mode, h/w only).
  * pads = {n,c,h,w begin, n,c,h,w end}.  The reference never reads const_val: constant

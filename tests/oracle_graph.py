@@ -108,6 +108,11 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
                 else:
                     params.append(int(a.get(k, 0)))
             y = O.move_i8(kind, ins[0], params, op.shape)
+        elif t == "tpu.quant":
+            if op.quant == "INT8":
+                y = O.quant_f32_to_i8(ins[0], op.attrs["scale"])
+            else:
+                y = O.dequant_i8_to_f32(ins[0], op.attrs["scale"])
         elif t == "tpu.prelu":
             w = op.weights
             y = O.prelu_i8(ins[0], w["slope"], w["rshift_pos"][0], w["multiplier_pos"][0],

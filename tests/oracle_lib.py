@@ -66,6 +66,10 @@ def _load():
     lib.orc_conv2d_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p, C.POINTER(ConvDesc)]
     lib.orc_deconv2d_acc.argtypes = [i8p, i8p, i32p, C.POINTER(ConvDesc)]
     lib.orc_deconv2d_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p, C.POINTER(ConvDesc)]
+    lib.orc_quant_f32_to_i8.argtypes = [f32p, i8p, C.c_size_t, C.c_float]
+    lib.orc_dequant_i8_to_f32.argtypes = [i8p, f32p, C.c_size_t, C.c_float]
+    lib.orc_bf16.restype = C.c_float
+    lib.orc_bf16.argtypes = [C.c_float, C.c_int]
     lib.orc_fc_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p] + [C.c_int] * 5
     lib.orc_fc_guard.restype = C.c_int64
     lib.orc_fc_guard.argtypes = [i8p, i8p, f32p] + [C.c_int] * 4
@@ -225,6 +229,20 @@ def deconv2d_i8(x, w, bias, rshift, multiplier, d):
     lib.orc_deconv2d_i8(_p(x, C.c_int8), _p(w, C.c_int8), _p(b, C.c_float) if b is not None else None,
                         _p(_f32(rshift), C.c_float), _p(_f32(multiplier), C.c_float),
                         _p(y, C.c_int8), C.byref(d))
+    return y
+
+
+def quant_f32_to_i8(x, scale):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty(x.shape, np.int8)
+    lib.orc_quant_f32_to_i8(_p(x, C.c_float), _p(y, C.c_int8), x.size, float(scale))
+    return y
+
+
+def dequant_i8_to_f32(x, scale):
+    x = _i8(x)
+    y = np.empty(x.shape, np.float32)
+    lib.orc_dequant_i8_to_f32(_p(x, C.c_int8), _p(y, C.c_float), x.size, float(scale))
     return y
 
 

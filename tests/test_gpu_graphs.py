@@ -377,3 +377,52 @@ def test_deconv_graph_matches_the_oracle(cfg):
     assert np.array_equal(m.get_tensor_i8("up"), want["up"])
     assert len(np.unique(want["up"])) > 8
     m.close()
+
+
+def test_graph_with_fp32_edges_quantizes_and_dequantizes_like_the_oracle():
+    """fp32 input -> QuantOp -> conv -> conv -> QuantOp -> fp32 output"""
+    rng = np.random.default_rng(5)
+    b = graphs.Builder("edges", graphs.BASE_SEED + 79, 3, (6, 12))
+    x8 = b.input("x8", 20, 9, 7)                 # calibrates the convs; replaced by the quant op below
+    c1 = b.conv("c1", x8, 32, 3, relu=True)
+    c2 = b.conv("c2", c1, 24, 1, relu=False)
+    g = b.g
+    # put an fp32 input and a QuantOp in front, a dequantising QuantOp behind
+    shape = g.by_name["x8"].shape
+    xf = rng.normal(0, 1.2, shape).astype(np.float32)
+    xf.flat[:8] = [0.5 / 31.75, -0.5 / 31.75, 1.5 / 31.75, 4.1, -4.1, 100.0, -100.0, 0.0]
+    fin = graphs.Op("tpu.input", "input", [], shape)
+    fin.quant = "NONE"
+    fin.data = xf
+    q = graphs.Op("tpu.quant", "x8", ["input"], shape, dict(scale=31.75))
+    old = g.ops[0]
+    g.ops[0:1] = [fin, q]
+    g.by_name["input"] = fin
+    g.by_name["x8"] = q
+    dq = graphs.Op("tpu.quant", "out", [c2], g.by_name[c2].shape, dict(scale=0.0207))
+    dq.quant = "NONE"
+    g.add(dq)
+    g.outputs = ["out"]
+    want = oracle_graph.run(g)
+    assert want["out"].dtype == np.float32 and want["x8"].dtype == np.int8
+    m = module()
+    m.load(g)
+    m.set_tensor("input", xf)
+    m.invoke()
+    assert np.array_equal(m.get_tensor("input"), xf)
+    for name in ("x8", c1, c2):
+        assert np.array_equal(m.get_tensor_i8(name), want[name]), name
+    got = m.get_tensor("out")
+    assert got.dtype == np.float32 and np.array_equal(got, want["out"])
+    assert len(np.unique(got)) > 8
+    with pytest.raises(capi.TpuHipError, match="fp32"):
+        m.get_tensor_i8("out")
+    m.close()
+    # an INT8 op fed with fp32 data is refused
+    g2 = graphs.Graph("bad", 1)
+    i2 = g2.add(graphs.Op("tpu.input", "input", [], (1, 16, 4, 4)))
+    i2.quant = "NONE"
+    i2.data = np.zeros((1, 16, 4, 4), np.float32)
+    g2.add(graphs.Op("tpu.relu", "r", ["input"], (1, 16, 4, 4)))
+    with pytest.raises(capi.TpuHipError, match="QuantOp in front"):
+        module().load(g2)

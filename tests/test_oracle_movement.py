@@ -94,3 +94,37 @@ def test_deconv_accumulators_equal_torch_conv_transpose(cfg):
         (pads[0], pads[2]), opad, g, dil).numpy()
     d = O.make_deconv_desc(x.shape, w.shape, g, stride, pads, dil, want.shape[2:])
     assert np.array_equal(O.deconv2d_acc(x, w, d), want.astype(np.int64))
+
+
+def test_bf16_rounding_is_round_to_nearest_even_like_torch():
+    rng = np.random.default_rng(11)
+    vals = np.concatenate([rng.normal(0, 50, 4000), rng.normal(0, 1e-3, 500), [0.0, 1.0, -1.0, 3.140625,
+                           1.00390625, 1.01171875, 255.5, -255.5, 65504.0]]).astype(np.float32)
+    want = torch.from_numpy(vals).to(torch.bfloat16).to(torch.float32).numpy()
+    got = np.array([O.lib.orc_bf16(float(v), 1) for v in vals], np.float32)
+    assert np.array_equal(got, want)
+    # truncation mode keeps the high 16 bits
+    assert O.lib.orc_bf16(1.01171875, 0) == 1.0078125
+
+
+def test_quantize_rounds_half_away_from_zero_and_saturates():
+    from fractions import Fraction
+    rng = np.random.default_rng(12)
+    x = np.concatenate([rng.normal(0, 2, 3000), [0.5, -0.5, 1.5, -1.5, 2.5, 126.5, 127.49, 127.5, -128.5,
+                        -129.0, 1e6, -1e6, 0.0]]).astype(np.float32)
+    for scale in (1.0, 0.37, 63.5, 127.0 / 2.64):
+        got = O.quant_f32_to_i8(x, scale)
+        prod = x * np.float32(scale)                       # the float32 product the reference forms
+        for v, g in zip(prod, got):
+            f = Fraction(float(v))
+            r = int(abs(f) + Fraction(1, 2))               # nearest, ties away from zero
+            r = r if f >= 0 else -r
+            assert g == max(-128, min(127, r)), (float(v), scale)
+
+
+def test_dequantize_is_bf16_of_value_times_bf16_scale():
+    x = np.arange(-128, 128, dtype=np.int8)
+    for scale in (1.0, 0.0207, 2.64 / 127.0, 3.7):
+        s = torch.tensor(scale, dtype=torch.float32).to(torch.bfloat16).to(torch.float32)
+        want = (torch.from_numpy(x.astype(np.float32)) * s).to(torch.bfloat16).to(torch.float32).numpy()
+        assert np.array_equal(O.dequant_i8_to_f32(x, scale), want)

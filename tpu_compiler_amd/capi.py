@@ -88,6 +88,8 @@ PROTOTYPES = {
     "tpuhip_lut_per_channel_i8": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t, C.c_int, C.c_int]),
     "tpuhip_prelu_tables": (C.c_int, [C.POINTER(C.c_float), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32,
                                       C.POINTER(C.c_int8)]),
+    "tpuhip_quant_f32_to_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5 + [C.c_float]),
+    "tpuhip_dequant_i8_to_f32": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5 + [C.c_float]),
     "tpuhip_move_i8": (C.c_int, [C.c_void_p, C.POINTER(MoveDesc), C.c_void_p, C.c_void_p]),
     "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,

@@ -237,6 +237,8 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<ShuffleChannelOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.pixelshuffle") {
       krnl = std::make_shared<DepthToSpaceOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.quant") {
+      krnl = std::make_shared<QuantOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.prelu") {
       krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {

@@ -84,8 +84,8 @@ std::string OpDesc::signature() const {
 // ---------------------------------------------------------------------------
 // TensorData
 // ---------------------------------------------------------------------------
-TensorData::TensorData(tpuhip_ctx *ctx, int32_t batch_, const SyncedDataShape &shape)
-    : batch(batch_), ctx_(ctx) {
+TensorData::TensorData(tpuhip_ctx *ctx, int32_t batch_, const SyncedDataShape &shape, bool f32_)
+    : batch(batch_), f32(f32_), ctx_(ctx) {
   if (batch < 1) fail("TensorData: batch < 1");
   view4(shape, &n, &c, &h, &w);
   cs = tpuhip_channel_stride(c);
@@ -107,6 +107,11 @@ void TensorData::set_batch_idx(int32_t bidx) {
 void TensorData::assign(const float *first, size_t num, int32_t bidx) {
   if (num != size_) fail("TensorData::assign: size mismatch");
   if (bidx < 0 || bidx >= batch) fail("TensorData::assign: slot out of range");
+  if (f32) {
+    ck(tpuhip_upload(ctx_, (char *)base_ + slot_bytes() * (size_t)bidx, first, num * sizeof(float)),
+       "TensorData::assign");
+    return;
+  }
   for (size_t i = 0; i < num; ++i)
     if (!(first[i] >= -128.0f && first[i] <= 127.0f) || first[i] != std::nearbyint(first[i]))
       fail("TensorData::assign: element " + std::to_string(i) + " = " + std::to_string(first[i]) +
@@ -127,6 +132,12 @@ std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
          "(load the module with keep_all_tensors to read it)");
   if (bidx < 0 || bidx >= batch) fail("TensorData::tensor: slot out of range");
   auto out = std::make_shared<std::vector<float>>(size_);
+  if (f32) {
+    ck(tpuhip_download(ctx_, out->data(), (char *)base_ + slot_bytes() * (size_t)bidx,
+                       size_ * sizeof(float)),
+       "TensorData::tensor");
+    return out;
+  }
   void *tmp = nullptr;
   ck(tpuhip_malloc(ctx_, size_ * sizeof(float), &tmp), "TensorData::tensor");
   int rc = tpuhip_nhwc_i8_to_nchw_f32(ctx_, (char *)base_ + slot_bytes() * (size_t)bidx, tmp, n, c,
@@ -141,6 +152,7 @@ void TensorData::read_i8(int8_t *dst, size_t num, int32_t bidx) const {
   if (!materialized)
     fail("TensorData::read_i8: this tensor is fused into its consumer and never written "
          "(load the module with keep_all_tensors to read it)");
+  if (f32) fail("TensorData::read_i8: this tensor holds fp32 data");
   if (num != size_) fail("TensorData::read_i8: size mismatch");
   if (bidx < 0 || bidx >= batch) fail("TensorData::read_i8: slot out of range");
   void *tmp = nullptr;
@@ -229,7 +241,12 @@ void CPUOpKernel::assignOperandTensors(OpDesc &op_, const value_map_t &valueMapp
 }
 
 void CPUOpKernel::assignResultTensor(OpDesc &op_, value_map_t &valueMapping) {
-  resTensor = std::make_shared<TensorData>(ctx, max_batch_size, op_.shape);
+  // fp32 results exist only where the reference's graphs have them next to INT8 ops: the
+  // network input and the dequantising QuantOp
+  const bool f32 = datatype == DataType::FP32;
+  if (f32 && op_.type != "tpu.input" && op_.type != "tpu.quant")
+    fail(op_.type + " '" + op_.name + "': only the INT8 path is implemented on the GPU");
+  resTensor = std::make_shared<TensorData>(ctx, max_batch_size, op_.shape, f32);
   valueMapping[op_.name] = resTensor;
   valueMapping.shapes[op_.name] = op_.shape;
 }
@@ -237,6 +254,9 @@ void CPUOpKernel::assignResultTensor(OpDesc &op_, value_map_t &valueMapping) {
 void CPUOpKernel::require_int8(const char *what) const {
   if (datatype != DataType::INT8)
     fail(std::string(what) + " '" + name + "': only the INT8 path is implemented on the GPU");
+  for (auto &opd : opdTensors)
+    if (opd.act && opd.act->f32)
+      fail(std::string(what) + " '" + name + "': an fp32 operand needs a QuantOp in front");
 }
 
 // ---------------------------------------------------------------------------
@@ -697,6 +717,29 @@ void LutOpKernel::invoke() {
                    (size_t)input_data->n * input_data->h * input_data->w, input_data->c,
                    input_data->cs),
      name.c_str());
+}
+
+QuantOpKernel::QuantOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail("Quant '" + name + "': input missing");
+  if (input_data->size() != output_data->size()) fail("Quant '" + name + "': shape mismatch");
+  if (input_data->f32 == output_data->f32)
+    fail("Quant '" + name + "': only fp32 -> INT8 and INT8 -> fp32 are implemented");
+  scale = (float)op.attr("scale");
+}
+
+void QuantOpKernel::invoke() {
+  const TensorData &q = input_data->f32 ? *output_data : *input_data;   // the int8 side
+  if (input_data->f32)
+    ck(tpuhip_quant_f32_to_i8(ctx, input_data->data(), output_data->data(), q.n, q.c, q.h, q.w, q.cs,
+                              scale),
+       name.c_str());
+  else
+    ck(tpuhip_dequant_i8_to_f32(ctx, input_data->data(), output_data->data(), q.n, q.c, q.h, q.w,
+                                q.cs, scale),
+       name.c_str());
 }
 
 PReluOpKernel::PReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)

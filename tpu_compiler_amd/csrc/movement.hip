@@ -6,6 +6,8 @@
 // output channels of a pixel (one dword store); pad channels are written as zero.
 #include "common.hpp"
 
+#include <cstring>
+
 using namespace tpuhip;
 
 namespace {
@@ -119,7 +121,86 @@ __global__ __launch_bounds__(kThreads) void move_kernel(MoveArgs a) {
   }
 }
 
+// QuantOp at the graph edges (core/quant.cpp).  The float side is NCHW like the reference's
+// tensors, the int8 side channels-last: the layout change rides along.
+__device__ __forceinline__ float bf16_rne(float v) {   // QuantizationArithmetic.cpp:893-905
+  uint32_t u = __float_as_uint(v);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  uint32_t h = u >> 16;
+  if ((h & 0x7f80u) == 0x7f80u) h = 0x7f7fu;
+  return __uint_as_float(h << 16);
+}
+
+__global__ __launch_bounds__(kThreads) void quant_f32_to_i8_kernel(const float *x, int8_t *y, int n,
+                                                                   int c, int h, int w, int cs,
+                                                                   float scale) {
+  const int64_t total = (int64_t)n * h * w * cs;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int ch = (int)(i % cs);
+    const int64_t pix = i / cs;
+    int8_t out = 0;
+    if (ch < c) {
+      const int iw = (int)(pix % w), ih = (int)((pix / w) % h), in = (int)(pix / ((int64_t)w * h));
+      const float v = x[(((int64_t)in * c + ch) * h + ih) * w + iw];
+      const float r = roundf(__fmul_rn(v, scale));   // std::round: half away from zero
+      out = (int8_t)(r > 127.0f ? 127 : r < -128.0f ? -128 : (int)r);
+    }
+    y[i] = out;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void dequant_i8_to_f32_kernel(const int8_t *x, float *y,
+                                                                     int n, int c, int h, int w,
+                                                                     int cs, float scale_bf16) {
+  const int64_t total = (int64_t)n * c * h * w;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int iw = (int)(i % w), ih = (int)((i / w) % h);
+    const int ch = (int)((i / ((int64_t)w * h)) % c), in = (int)(i / ((int64_t)w * h * c));
+    const float v = (float)x[(((int64_t)in * h + ih) * w + iw) * cs + ch];   // exact in bf16
+    y[i] = bf16_rne(__fmul_rn(v, scale_bf16));
+  }
+}
+
 }  // namespace
+
+extern "C" int tpuhip_quant_f32_to_i8(tpuhip_ctx *ctx, const void *x_nchw_f32, void *y, int n, int c,
+                                      int h, int w, int cs, float scale) {
+  TPUHIP_REQUIRE(ctx && x_nchw_f32 && y, "quant: NULL argument");
+  TPUHIP_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && cs >= c && cs % 16 == 0, "quant: bad shape");
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  const int64_t total = (int64_t)n * h * w * cs;
+  const unsigned blocks = (unsigned)std::max<int64_t>(
+      1, std::min<int64_t>(ceil_div64(total, kThreads), (int64_t)ctx->num_cu * 32));
+  launch(ctx, quant_f32_to_i8_kernel, dim3(blocks), dim3(kThreads), (const float *)x_nchw_f32,
+         (int8_t *)y, n, c, h, w, cs, scale);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
+extern "C" int tpuhip_dequant_i8_to_f32(tpuhip_ctx *ctx, const void *x, void *y_nchw_f32, int n, int c,
+                                        int h, int w, int cs, float scale) {
+  TPUHIP_REQUIRE(ctx && x && y_nchw_f32, "dequant: NULL argument");
+  TPUHIP_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && cs >= c && cs % 16 == 0, "dequant: bad shape");
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  // scale = BF16(scale) on the host (quant.cpp:110), same rounding as the device function
+  uint32_t u;
+  memcpy(&u, &scale, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  uint32_t hbits = u >> 16;
+  if ((hbits & 0x7f80u) == 0x7f80u) hbits = 0x7f7fu;
+  hbits <<= 16;
+  float sb;
+  memcpy(&sb, &hbits, 4);
+  const int64_t total = (int64_t)n * c * h * w;
+  const unsigned blocks = (unsigned)std::max<int64_t>(
+      1, std::min<int64_t>(ceil_div64(total, kThreads), (int64_t)ctx->num_cu * 32));
+  launch(ctx, dequant_i8_to_f32_kernel, dim3(blocks), dim3(kThreads), (const int8_t *)x,
+         (float *)y_nchw_f32, n, c, h, w, cs, sb);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
 
 extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");

@@ -34,6 +34,9 @@ _WEIGHT_OPERANDS = {
     "tpu.clip": [None, None, "rshift", "multiplier"],
     "tpu.lut": ["table", None],
     "tpu.relu": [],
+    "tpu.quant": [],
+    "tpu.pad": [], "tpu.crop": [], "tpu.permute": [], "tpu.reorg": [], "tpu.tile": [],
+    "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [],
     "tpu.upsample": [],
     "tpu.concat": [None, None, "rshift", "multiplier"],
     "tpu.reshape": [],
