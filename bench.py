@@ -164,12 +164,22 @@ def main():
             roofline["traffic"] = int((t["fetch_KiB"] + t["write_KiB"]) * 1024)
             roofline["traffic_unit"] = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, profiles/)"
             roofline["algorithmic_bytes"] = int(dom["bytes"] / dom["launches"])
+    # bandwidth-bound ops: algorithmic bytes (int8 inputs + output once) over their time
+    hbm_bytes = hbm_ms = 0.0
+    for name, algo, ms in rows:
+        op = g.by_name[name]
+        if op.type in ("tpu.conv_2d", "tpu.fully_connected", "tpu.input") or ms <= 0:
+            continue
+        hbm_bytes += sum(int(np.prod(g.by_name[i].shape)) for i in op.inputs) + int(np.prod(op.shape))
+        hbm_ms += ms
     if args.per_layer:
         for name, algo, ms in rows:
             op = g.by_name[name]
             macs = getattr(op, "macs", 0)
-            print("%-22s %-18s %-14s %9.2f us %8.1f TOP/s" %
-                  (name, op.type, algo, ms * 1e3, 2 * macs / (ms / 1e3) / 1e12 if ms > 0 else 0),
+            nbytes = sum(int(np.prod(g.by_name[i].shape)) for i in op.inputs) + int(np.prod(op.shape))
+            print("%-22s %-18s %-18s %9.2f us %8.1f TOP/s %8.1f GB/s" %
+                  (name, op.type, algo, ms * 1e3, 2 * macs / (ms / 1e3) / 1e12 if ms > 0 else 0,
+                   nbytes / (ms / 1e3) / 1e9 if ms > 0 else 0),
                   file=sys.stderr)
 
     out = {
@@ -187,6 +197,9 @@ def main():
         "ops_per_step": total_ops,
         "event_ms_per_step": round(ev_ms.value / args.steps, 4),
         "roofline": roofline,
+        "hbm_bound_ops": None if hbm_ms <= 0 else {
+            "achieved": round(hbm_bytes / (hbm_ms / 1e3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(hbm_bytes / (hbm_ms / 1e3) / 1e9 / PEAK_HBM_GBS, 4), "ms": round(hbm_ms, 4)},
     }
     if not args.no_cpu_baseline:
         sample = {"cfg1": 8, "cfg2": 8, "cfg3": 8, "cfg4": 16, "cfg5": 1}[args.config]
