@@ -171,7 +171,7 @@ DEPTHWISE = [
 
 
 @pytest.mark.parametrize("case", DEPTHWISE)
-@pytest.mark.parametrize("algo", [capi.ALGO_DEPTHWISE, capi.ALGO_DIRECT])
+@pytest.mark.parametrize("algo", [capi.ALGO_DEPTHWISE, capi.ALGO_DEPTHWISE_DOT, capi.ALGO_DIRECT])
 def test_conv_depthwise(ctx, case, algo):
     n, c, ih, iw, k, stride, pads, relu = case
     rng = np.random.default_rng(c + k)
@@ -185,19 +185,21 @@ def test_conv_depthwise(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
-def test_conv_depthwise_dilated_general_requant_and_fused_table(ctx):
+@pytest.mark.parametrize("algo", [capi.ALGO_DEPTHWISE, capi.ALGO_DEPTHWISE_DOT])
+def test_conv_depthwise_dilated_general_requant_and_fused_table(ctx, algo):
     rng = np.random.default_rng(77)
     x = rnd_i8(rng, (2, 40, 14, 13))
     w = rnd_w(rng, (40, 1, 3, 3), 24)
     bias, rsh, mult = rnd_params(rng, 40, 5, 12, 2048)
     rsh[3] = 0                                         # forces the general rounding form
     want = oracle_conv(x, w, bias, rsh, mult, 40, (1, 1), (2, 2, 2, 2), (2, 2), (0, 0), True)
-    got, name = run_conv(ctx, x, w, bias, rsh, mult, g=40, pads=(2, 2, 2, 2), dil=(2, 2), do_relu=True)
-    assert name == "depthwise" and np.array_equal(got, want)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=algo, g=40, pads=(2, 2, 2, 2), dil=(2, 2),
+                         do_relu=True)
+    assert name.startswith("depthwise") and np.array_equal(got, want)
     # the same layer with a table behind it, in one kernel
     table = rnd_i8(rng, 256)
     table[0] = -5
-    d = conv_desc(x.shape, w.shape, g=40, pads=(2, 2, 2, 2), dil=(2, 2), do_relu=True)
+    d = conv_desc(x.shape, w.shape, g=40, pads=(2, 2, 2, 2), dil=(2, 2), do_relu=True, algo=algo)
     wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
     xt, yt, tt = ctx.from_nchw(x), ctx.tensor(want.shape), ctx.tensor(want.shape)
     ctx.conv_post(wh, xt, yt, table, tt)

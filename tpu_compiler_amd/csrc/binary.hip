@@ -34,6 +34,9 @@ __device__ __forceinline__ v4i load_operand(const int8_t *x, int pix, int cs, in
   return *reinterpret_cast<const v4i *>(x + (int64_t)pix * cs + cg * 16);
 }
 
+// PIXELWISE: neither operand repeats along n, h or w, so both read the output's pixel and
+// the index arithmetic below disappears (a channel count of 1 may still repeat).
+template <bool PIXELWISE>
 __global__ __launch_bounds__(kThreads) void binary_kernel(BinArgs a) {
   const int c16 = a.cs >> 4;
   const int32_t rnd = a.rshift > 0 ? (1 << (a.rshift - 1)) : 0;
@@ -42,11 +45,14 @@ __global__ __launch_bounds__(kThreads) void binary_kernel(BinArgs a) {
        i += (int64_t)gridDim.x * blockDim.x) {
     const int cg = (int)(i % c16);
     const int pix = (int)(i / c16);
-    const int w = pix % a.w;
-    const int h = (pix / a.w) % a.h;
-    const int n = pix / (a.w * a.h);
-    const int p0 = ((a.n0 == 1 ? 0 : n) * a.h0 + (a.h0 == 1 ? 0 : h)) * a.w0 + (a.w0 == 1 ? 0 : w);
-    const int p1 = ((a.n1 == 1 ? 0 : n) * a.h1 + (a.h1 == 1 ? 0 : h)) * a.w1 + (a.w1 == 1 ? 0 : w);
+    int p0 = pix, p1 = pix;
+    if (!PIXELWISE) {
+      const int w = pix % a.w;
+      const int h = (pix / a.w) % a.h;
+      const int n = pix / (a.w * a.h);
+      p0 = ((a.n0 == 1 ? 0 : n) * a.h0 + (a.h0 == 1 ? 0 : h)) * a.w0 + (a.w0 == 1 ? 0 : w);
+      p1 = ((a.n1 == 1 ? 0 : n) * a.h1 + (a.h1 == 1 ? 0 : h)) * a.w1 + (a.w1 == 1 ? 0 : w);
+    }
     const v4i v0 = load_operand(a.x0, p0, a.cs0, a.c0, cg);
     const v4i v1 = load_operand(a.x1, p1, a.cs1, a.c1, cg);
     v4i out;
@@ -120,7 +126,12 @@ extern "C" int tpuhip_binary_i8(tpuhip_ctx *ctx, const tpuhip_binary_desc *d, co
   a.total = (int64_t)d->n * d->h * d->w * (d->y_cs / 16);
   const unsigned blocks = (unsigned)std::max<int64_t>(
       1, std::min<int64_t>(ceil_div64(a.total, kThreads), (int64_t)ctx->num_cu * 32));
-  launch(ctx, binary_kernel, dim3(blocks), dim3(kThreads), a);
+  const bool pixelwise = d->n0 == d->n && d->h0 == d->h && d->w0 == d->w && d->n1 == d->n &&
+                         d->h1 == d->h && d->w1 == d->w;
+  if (pixelwise)
+    launch(ctx, binary_kernel<true>, dim3(blocks), dim3(kThreads), a);
+  else
+    launch(ctx, binary_kernel<false>, dim3(blocks), dim3(kThreads), a);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }

@@ -23,7 +23,7 @@ using namespace tpuhip;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3 };
+enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3, ALGO_DEPTHWISE_DOT = 4 };
 
 // per-channel requantisation record
 struct __attribute__((aligned(16))) QParam {
@@ -754,6 +754,98 @@ conv_mfma_kernel(ConvArgs a) {
       }
     }
     if (!PERSIST || !more) break;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// depthwise on the matrix cores.  A depthwise tap is a 32x32 DIAGONAL matrix times
+// the 32 channels x 32 pixels activation block: D[c][pix] += W_t[c][c] * X_t[pix][c],
+// one v_mfma_i32_32x32x32_i8 per tap (K = the 32 channels).  31/32 of the multiplies
+// hit zeros, but the matrix pipe is otherwise idle here and the vector ALU, which the
+// per-byte multiply-adds of the scalar form saturate, is left with the requantisation
+// alone.  The B fragment of a tap is exactly a channels-last load (lane: pixel l & 31,
+// 16 channels from 16*(l >> 5)); the diagonal A fragments are built on the host, rows
+// permuted so that a lane's 16 results are 16 consecutive channels.  A wave keeps its
+// 32-channel block and walks 32-pixel blocks.
+// REGW: kh*kw <= 9 and the nine A fragments stay in registers.
+// ---------------------------------------------------------------------------
+template <bool FAST, bool REGW>
+__global__ __launch_bounds__(256) void conv_depthwise_mfma_kernel(ConvArgs a) {
+  __shared__ uint32_t lutw[64];
+  if (a.has_lut) {
+    if (threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+    __syncthreads();
+  }
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  const int lane = threadIdx.x & 63;
+  const int frow = lane & 31, fk = lane >> 5;
+  const int n_cb = (a.ocw + 31) >> 5;
+  const int n_pb = (a.npix + 31) >> 5;
+  const int gw = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+  const int nslots = (int)(gridDim.x * 4) / n_cb;     // pixel blocks in flight (>= 1)
+  const int cb = gw % n_cb;
+  int pb = gw / n_cb;
+  if (pb >= nslots) return;                           // no barrier below
+  const int oc = cb * 32 + fk * 16;                   // this lane's 16 channels
+  const bool ch_ok = oc < a.ocw;
+  const int taps = a.kh * a.kw;
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + (size_t)cb * taps * 64 + lane;
+  v4i areg[REGW ? 9 : 1];
+  if (REGW) {
+#pragma unroll
+    for (int t = 0; t < 9; ++t) areg[t] = t < taps ? afrag[t * 64] : v4i{0, 0, 0, 0};
+  }
+
+  int pix = pb * 32 + frow;
+  int ow = pix % a.ow;
+  int oh = (pix / a.ow) % a.oh;
+  int n = pix / (a.ow * a.oh);
+  const int step = nslots * 32;
+  const int d_ow = step % a.ow, d_oh = (step / a.ow) % a.oh, d_n = step / (a.ow * a.oh);
+
+  for (; pb < n_pb; pb += nslots) {
+    const bool pv = (pix < a.npix) & ch_ok;
+    const int ihb = oh * a.sh - a.pt, iwb = ow * a.sw - a.pl;
+    const int base = ((n * a.ih + ihb) * a.iw + iwb) * a.x_cs + oc;
+    v16i acc[1];
+    {
+      const v4i *bp = reinterpret_cast<const v4i *>(a.bias + (ch_ok ? oc : 0));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i b = bp[q];
+        acc[0][q * 4 + 0] = b[0]; acc[0][q * 4 + 1] = b[1];
+        acc[0][q * 4 + 2] = b[2]; acc[0][q * 4 + 3] = b[3];
+      }
+    }
+    auto tap_load = [&](int t) {
+      const int tkh = (int)(((uint32_t)t * a.magic_kw) >> 20);
+      const int tkw = t - tkh * a.kw;
+      const int ih = ihb + tkh * a.dh, iw = iwb + tkw * a.dw;
+      const bool ok = pv & (t < taps) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+      return buffer_load16(xrsrc, ok ? (uint32_t)(base + (tkh * a.dh * a.iw + tkw * a.dw) * a.x_cs)
+                                     : kOobOffset);
+    };
+    if (REGW) {
+      v4i bt[9];
+#pragma unroll
+      for (int t = 0; t < 9; ++t) bt[t] = tap_load(t);
+#pragma unroll
+      for (int t = 0; t < 9; ++t)
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[t], bt[t], acc[0], 0, 0, 0);
+    } else {
+      for (int t = 0; t < taps; ++t)
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[t * 64], tap_load(t), acc[0], 0, 0, 0);
+    }
+    if (ch_ok)
+      epilogue_rows<1, FAST>(acc, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pix, 32, lut);
+    pix += step;
+    ow += d_ow;
+    if (ow >= a.ow) { ow -= a.ow; ++oh; }
+    oh += d_oh;
+    if (oh >= a.oh) { oh -= a.oh; ++n; }
+    n += d_n;
   }
 }
 
@@ -1511,7 +1603,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
     TPUHIP_REQUIRE(forced_tile < kNumTiles, "conv: unknown MFMA tile %d", forced_tile);
   }
   if (algo == ALGO_AUTO) algo = dense ? ALGO_MFMA : depthwise ? ALGO_DEPTHWISE : ALGO_DIRECT;
-  TPUHIP_REQUIRE(algo >= ALGO_DIRECT && algo <= ALGO_DEPTHWISE, "conv: unknown algo %d", d.algo);
+  TPUHIP_REQUIRE(algo >= ALGO_DIRECT && algo <= ALGO_DEPTHWISE_DOT, "conv: unknown algo %d", d.algo);
   // the MFMA kernel locates a K group with multiply-shift divisions that are exact
   // for at most 4094 groups of at most 256 16-channel groups each
   const bool mfma_ok = dense && round_up(d.ic, 16) / 16 <= 256 &&
@@ -1521,7 +1613,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   if (d.algo == ALGO_AUTO && algo == ALGO_MFMA && !mfma_ok) algo = ALGO_DIRECT;
   TPUHIP_REQUIRE(algo != ALGO_MFMA || mfma_ok,
                  "conv: MFMA path needs g == 1, no inserted zeros, ic <= 4096 and K < 65000");
-  TPUHIP_REQUIRE(algo != ALGO_DEPTHWISE || depthwise,
+  TPUHIP_REQUIRE((algo != ALGO_DEPTHWISE && algo != ALGO_DEPTHWISE_DOT) || depthwise,
                  "conv: depthwise path needs g == ic == oc and no inserted zeros");
 
   auto *cw = new tpuhip_conv_weights();
@@ -1544,6 +1636,21 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
       cw->host_filter.shrink_to_fit();
     }
   } else if (algo == ALGO_DEPTHWISE) {
+    // diagonal MFMA A fragments: [32-channel block][tap][lane][16 bytes]; lane l holds row
+    // l & 31 (channel mfma_row_to_oc(row) of the block), K bytes 16*(l >> 5) .. +15
+    cw->ocp = round_up(d.oc, 16);
+    const int taps = d.kh * d.kw, n_cb = (cw->ocp + 31) / 32;
+    packed.assign((size_t)n_cb * taps * 1024, 0);
+    for (int cb = 0; cb < n_cb; ++cb)
+      for (int t = 0; t < taps; ++t)
+        for (int lane = 0; lane < 64; ++lane) {
+          const int ch_in_block = mfma_row_to_oc(lane & 31, 1);
+          const int ch = cb * 32 + ch_in_block;
+          const int j = ch_in_block - 16 * (lane >> 5);
+          if (ch < d.oc && j >= 0 && j < 16)
+            packed[((size_t)(cb * taps + t) * 64 + lane) * 16 + j] = filter[(size_t)ch * taps + t];
+        }
+  } else if (algo == ALGO_DEPTHWISE_DOT) {
     // [tap group][channel][4 taps]: one dword per channel and group of four taps
     cw->ocp = round_up(d.oc, 16);
     const int groups = std::max(3, (d.kh * d.kw + 3) / 4);   // the kernel holds three groups in registers
@@ -1597,7 +1704,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   if (!rc) rc = tpuhip_malloc(ctx, qp.size() * sizeof(QParam), (void **)&cw->qp);
   if (!rc) rc = tpuhip_upload(ctx, cw->bias, b32.data(), b32.size() * sizeof(int32_t));
   if (!rc) rc = tpuhip_upload(ctx, cw->qp, qp.data(), qp.size() * sizeof(QParam));
-  if (!rc && (algo == ALGO_MFMA || algo == ALGO_DEPTHWISE)) {
+  if (!rc && (algo == ALGO_MFMA || algo == ALGO_DEPTHWISE || algo == ALGO_DEPTHWISE_DOT)) {
     std::vector<int32_t> planes(3 * nparam);
     for (size_t i = 0; i < nparam; ++i) {
       planes[i] = qp[i].mult;
@@ -1636,6 +1743,7 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
   switch (w->algo) {
     case ALGO_DIRECT: return "direct";
     case ALGO_DEPTHWISE: return "depthwise";
+    case ALGO_DEPTHWISE_DOT: return "depthwise_dot";
     case ALGO_MFMA: return kTiles[w->tile].name;
   }
   return "?";
@@ -1658,7 +1766,7 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     if (ty != y) tpuhip_free(ctx, ty);
     if (rc) return rc;
   }
-  TPUHIP_REQUIRE(!post.lut || w->algo == ALGO_DEPTHWISE ||
+  TPUHIP_REQUIRE(!post.lut || w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT ||
                      (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
                  "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
   ConvArgs a;
@@ -1667,6 +1775,22 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
   if (w->algo == ALGO_MFMA) {
     launch_conv_mfma(ctx, w, a);
   } else if (w->algo == ALGO_DEPTHWISE) {
+    // one wave per (32-channel block, 32-pixel block); a resident set of workgroups, each
+    // wave walking pixel blocks of its channel block
+    const int n_cb = (a.ocw + 31) / 32, n_pb = (a.npix + 31) / 32;
+    const int64_t waves = (int64_t)n_cb * n_pb;
+    const unsigned blocks = (unsigned)std::max<int64_t>(
+        (n_cb + 3) / 4, std::min<int64_t>(ceil_div64(waves, 4), (int64_t)ctx->num_cu * 3));
+    const dim3 grid(blocks), block(256);
+    const bool regw = a.kh * a.kw <= 9;
+    if (w->fast) {
+      if (regw) launch(ctx, (conv_depthwise_mfma_kernel<true, true>), grid, block, a);
+      else launch(ctx, (conv_depthwise_mfma_kernel<true, false>), grid, block, a);
+    } else {
+      if (regw) launch(ctx, (conv_depthwise_mfma_kernel<false, true>), grid, block, a);
+      else launch(ctx, (conv_depthwise_mfma_kernel<false, false>), grid, block, a);
+    }
+  } else if (w->algo == ALGO_DEPTHWISE_DOT) {
     // as many workgroups as are resident at once (3 per CU at this register count): every
     // lane then walks pixels and its filter / parameter loads are paid once (measured best)
     const int64_t total = (int64_t)a.npix * (a.ocw / 16);
@@ -1722,7 +1846,7 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
   TPUHIP_REQUIRE(ctx && w && x && post, "tpuhip_conv2d_post_i8: NULL argument");
   PostOps p;
   if (post->lut) {
-    TPUHIP_REQUIRE(w->algo == ALGO_MFMA || w->algo == ALGO_DEPTHWISE,
+    TPUHIP_REQUIRE(w->algo == ALGO_MFMA || w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT,
                    "conv2d_post: only dense convs on the MFMA path and depthwise convs can fuse a table");
     p.lut = post->lut;
     p.lut_out = post->lut_out;
