@@ -770,22 +770,31 @@ conv_mfma_kernel(ConvArgs a) {
 // REGW: kh*kw <= 9 and the nine A fragments stay in registers.
 // ---------------------------------------------------------------------------
 template <bool FAST, bool REGW>
-__global__ __launch_bounds__(256) void conv_depthwise_mfma_kernel(ConvArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(REGW ? 3 : 4, REGW ? 3 : 4))) void
+conv_depthwise_mfma_kernel(ConvArgs a) {
   __shared__ uint32_t lutw[64];
-  if (a.has_lut) {
-    if (threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
-    __syncthreads();
-  }
-  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  __shared__ int32_t qlds[4][4][32];                  // per wave: bias, mult, shift, hpot
   const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int frow = lane & 31, fk = lane >> 5;
   const int n_cb = (a.ocw + 31) >> 5;
   const int n_pb = (a.npix + 31) >> 5;
-  const int gw = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+  const int gw = (int)blockIdx.x * 4 + wave;
   const int nslots = (int)(gridDim.x * 4) / n_cb;     // pixel blocks in flight (>= 1)
   const int cb = gw % n_cb;
   int pb = gw / n_cb;
+  // a wave's parameters never change: they live in LDS, whose reads do not queue behind
+  // the activation loads in flight (the parameter arrays are padded past the last block)
+  {
+    const int32_t *src = fk == 0 ? a.bias : a.qmult;
+    const int32_t *src2 = fk == 0 ? a.qshift : a.qhpot;
+    qlds[wave][fk][frow] = src[cb * 32 + frow];
+    qlds[wave][2 + fk][frow] = src2[cb * 32 + frow];
+  }
+  if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+  __syncthreads();
   if (pb >= nslots) return;                           // no barrier below
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
   const int oc = cb * 32 + fk * 16;                   // this lane's 16 channels
   const bool ch_ok = oc < a.ocw;
   const int taps = a.kh * a.kw;
@@ -797,6 +806,8 @@ __global__ __launch_bounds__(256) void conv_depthwise_mfma_kernel(ConvArgs a) {
 #pragma unroll
     for (int t = 0; t < 9; ++t) areg[t] = t < taps ? afrag[t * 64] : v4i{0, 0, 0, 0};
   }
+  const int32_t *pbias = &qlds[wave][0][fk * 16], *pmult = &qlds[wave][1][fk * 16];
+  const int32_t *pshift = &qlds[wave][2][fk * 16], *phpot = &qlds[wave][3][fk * 16];
 
   int pix = pb * 32 + frow;
   int ow = pix % a.ow;
@@ -805,47 +816,64 @@ __global__ __launch_bounds__(256) void conv_depthwise_mfma_kernel(ConvArgs a) {
   const int step = nslots * 32;
   const int d_ow = step % a.ow, d_oh = (step / a.ow) % a.oh, d_n = step / (a.ow * a.oh);
 
-  for (; pb < n_pb; pb += nslots) {
-    const bool pv = (pix < a.npix) & ch_ok;
+  auto tap_load = [&](int t) {
+    const int tkh = (int)(((uint32_t)t * a.magic_kw) >> 20);
+    const int tkw = t - tkh * a.kw;
     const int ihb = oh * a.sh - a.pt, iwb = ow * a.sw - a.pl;
-    const int base = ((n * a.ih + ihb) * a.iw + iwb) * a.x_cs + oc;
-    v16i acc[1];
-    {
-      const v4i *bp = reinterpret_cast<const v4i *>(a.bias + (ch_ok ? oc : 0));
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const v4i b = bp[q];
-        acc[0][q * 4 + 0] = b[0]; acc[0][q * 4 + 1] = b[1];
-        acc[0][q * 4 + 2] = b[2]; acc[0][q * 4 + 3] = b[3];
-      }
-    }
-    auto tap_load = [&](int t) {
-      const int tkh = (int)(((uint32_t)t * a.magic_kw) >> 20);
-      const int tkw = t - tkh * a.kw;
-      const int ih = ihb + tkh * a.dh, iw = iwb + tkw * a.dw;
-      const bool ok = pv & (t < taps) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
-      return buffer_load16(xrsrc, ok ? (uint32_t)(base + (tkh * a.dh * a.iw + tkw * a.dw) * a.x_cs)
-                                     : kOobOffset);
-    };
-    if (REGW) {
-      v4i bt[9];
-#pragma unroll
-      for (int t = 0; t < 9; ++t) bt[t] = tap_load(t);
-#pragma unroll
-      for (int t = 0; t < 9; ++t)
-        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[t], bt[t], acc[0], 0, 0, 0);
-    } else {
-      for (int t = 0; t < taps; ++t)
-        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[t * 64], tap_load(t), acc[0], 0, 0, 0);
-    }
-    if (ch_ok)
-      epilogue_rows<1, FAST>(acc, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pix, 32, lut);
+    const int ih = ihb + tkh * a.dh, iw = iwb + tkw * a.dw;
+    const bool ok = (pix < a.npix) & ch_ok & (t < taps) & ((unsigned)ih < (unsigned)a.ih) &
+                    ((unsigned)iw < (unsigned)a.iw);
+    return buffer_load16(xrsrc, ok ? (uint32_t)(((n * a.ih + ih) * a.iw + iw) * a.x_cs + oc)
+                                   : kOobOffset);
+  };
+  auto advance = [&]() {
+    pb += nslots;
     pix += step;
     ow += d_ow;
     if (ow >= a.ow) { ow -= a.ow; ++oh; }
     oh += d_oh;
     if (oh >= a.oh) { oh -= a.oh; ++n; }
     n += d_n;
+  };
+  auto bias_acc = [&](v16i &acc) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4i b = *reinterpret_cast<const v4i *>(pbias + q * 4);
+      acc[q * 4 + 0] = b[0]; acc[q * 4 + 1] = b[1]; acc[q * 4 + 2] = b[2]; acc[q * 4 + 3] = b[3];
+    }
+  };
+
+  if (REGW) {
+    // the nine operands of the NEXT pixel block are requested before the epilogue of this
+    // one, into the registers the MFMAs have just consumed
+    v4i bt[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) bt[t] = tap_load(t);
+    for (;;) {
+      v16i acc[1];
+      bias_acc(acc[0]);
+#pragma unroll
+      for (int t = 0; t < 9; ++t)
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[t], bt[t], acc[0], 0, 0, 0);
+      const int pix_done = pix;
+      advance();
+      const bool more = pb < n_pb;
+      if (more) {
+#pragma unroll
+        for (int t = 0; t < 9; ++t) bt[t] = tap_load(t);
+      }
+      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix_done, 32, lut);
+      if (!more) break;
+    }
+  } else {
+    for (; pb < n_pb;) {
+      v16i acc[1];
+      bias_acc(acc[0]);
+      for (int t = 0; t < taps; ++t)
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[t * 64], tap_load(t), acc[0], 0, 0, 0);
+      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix, 32, lut);
+      advance();
+    }
   }
 }
 
