@@ -82,6 +82,7 @@ public:
   bool materialized = true;        // false: no kernel writes this tensor (fused away)
   int cs = 16;                     // channel stride in bytes
   bool f32 = false;                // float NCHW instead of int8 channels-last
+  bool is_unsigned = false;        // the bytes hold 0..255 (UINT8 tensors: image data in front of a ScaleLut)
   size_t slot_bytes() const { return f32 ? size_ * sizeof(float) : (size_t)n * h * w * cs; }
   tpuhip_ctx *ctx() const { return ctx_; }
 
@@ -332,6 +333,22 @@ public:
   static constexpr const char *OpName = "CPUPReluOp";
   PReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
   ~PReluOpKernel() override;
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+  void *tables = nullptr;   // device, c * 256 bytes
+};
+
+// core/scale_lut.cpp:7-31: y[n,c,h,w] = table[c * 256 + x[n,c,h,w]], operands [0]input
+// [1]table (1 x c x 16 x 16, built by quantizeInt8ScaleLutOps, QuantizeInt8.cpp:623-657, for
+// inputs 0..255).  The input must be a UINT8 tensor: with a negative x the reference's index
+// lands in the previous channel's table, or throws for channel 0.
+class ScaleLutOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPUScaleLutOp";
+  ScaleLutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~ScaleLutOpKernel() override;
   void invoke() override;
 
 private:

@@ -432,6 +432,20 @@ void orc_prelu_i8(const int8_t *x, int8_t *y, int n, int c, int hw, const float 
     }
 }
 
+/* scale_lut.cpp:15-31: table->at((int)(ci * 256 + x)) with x the float-stored input, which
+ * the quantizer defines for inputs 0..255 (QuantizeInt8.cpp:623-657): x is a uint8 tensor. */
+void orc_scale_lut_u8(const uint8_t *x, int8_t *y, int n, int c, int hw, const float *table) {
+#pragma omp parallel for collapse(2)
+  for (int b = 0; b < n; ++b)
+    for (int ch = 0; ch < c; ++ch) {
+      const size_t base = ((size_t)b * c + ch) * hw;
+      for (int i = 0; i < hw; ++i) {
+        const float in = (float)x[base + i];
+        y[base + i] = (int8_t)table[(int)(ch * 256 + in)];
+      }
+    }
+}
+
 /* activation.cpp:47-53: y0_table_op->at((unsigned char)input).  float ->
  * unsigned char of a negative value keeps the low byte on x86-64 gcc, i.e. the
  * index is the two's-complement byte of the int8 input. */

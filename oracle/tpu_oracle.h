@@ -135,6 +135,7 @@ void orc_leaky_relu_i8(const int8_t *x, int8_t *y, size_t count, float rshift_po
 void orc_prelu_i8(const int8_t *x, int8_t *y, int n, int c, int hw, const float *slope,
                   float rshift_pos, float multiplier_pos, float rshift_neg);
 /* :47-53 and siblings: y = table[(unsigned char)x]; table holds 256 floats */
+void orc_scale_lut_u8(const uint8_t *x, int8_t *y, int n, int c, int hw, const float *table);
 void orc_lut_i8(const int8_t *x, int8_t *y, size_t count, const float *table256);
 /* :155-164 + core/internal.cpp:13-18 */
 void orc_relu_i8(const int8_t *x, int8_t *y, size_t count);

@@ -113,6 +113,8 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
                 y = O.quant_f32_to_i8(ins[0], op.attrs["scale"])
             else:
                 y = O.dequant_i8_to_f32(ins[0], op.attrs["scale"])
+        elif t == "tpu.scale_lut":
+            y = O.scale_lut_u8(ins[0], op.weights["table"])
         elif t == "tpu.prelu":
             w = op.weights
             y = O.prelu_i8(ins[0], w["slope"], w["rshift_pos"][0], w["multiplier_pos"][0],

@@ -308,6 +308,17 @@ def prelu_i8(x, slope, rshift_pos, multiplier_pos, rshift_neg):
     return y
 
 
+def scale_lut_u8(x, table):
+    """x: uint8 NCHW; table: c * 256 float-stored int8 entries"""
+    x = np.ascontiguousarray(x, np.uint8)
+    n, c = x.shape[0], x.shape[1]
+    t = _f32(table)
+    assert t.size >= c * 256
+    y = np.empty(x.shape, np.int8)
+    lib.orc_scale_lut_u8(_p(x, C.c_uint8), _p(y, C.c_int8), n, c, x.size // (n * c), _p(t, C.c_float))
+    return y
+
+
 def binary_i8(op, x0, x1, multiplier, rshift, do_relu=False):
     """two-input elementwise op with broadcasting; x0, x1 4-d NCHW int8 (dims 1 broadcast)"""
     x0, x1 = _i8(x0), _i8(x1)

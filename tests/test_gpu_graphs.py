@@ -345,6 +345,57 @@ def test_graph_with_data_movement_ops_matches_the_oracle():
     m.close()
 
 
+def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle():
+    """uint8 image -> ScaleLut (per-channel 256-entry tables) -> conv"""
+    rng = np.random.default_rng(6)
+    b = graphs.Builder("scale_lut", graphs.BASE_SEED + 80, 2, (6, 12))
+    x8 = b.input("x8", 3, 20, 18)                # calibrates the conv; replaced below
+    c1 = b.conv("c1", x8, 24, 3, relu=True)
+    g = b.g
+    shape = g.by_name["x8"].shape
+    img = rng.integers(0, 256, shape).astype(np.uint8)
+    img.flat[:4] = [0, 127, 128, 255]
+    idx = np.arange(256)
+    scale, bias = np.array([0.9, 1.0, 0.4]), np.array([-110.0, -128.0, 11.0])
+    table = np.clip(np.floor(idx[None] * scale[:, None] + bias[:, None] + 0.5), -128, 127)
+    fin = graphs.Op("tpu.input", "input", [], shape)
+    fin.quant = "UINT8"
+    fin.data = img
+    sl = graphs.Op("tpu.scale_lut", "x8", ["input"], shape, {},
+                   dict(table=table.astype(np.float32).reshape(-1)))
+    g.ops[0:1] = [fin, sl]
+    g.by_name["input"] = fin
+    g.by_name["x8"] = sl
+    g.outputs = [c1]
+    want = oracle_graph.run(g)
+    assert np.array_equal(want["x8"][:, 1], (img[:, 1].astype(np.int16) - 128).astype(np.int8))
+    m = module()
+    m.load(g)
+    m.set_tensor("input", img.astype(np.float32))
+    m.invoke()
+    assert np.array_equal(m.get_tensor("input"), img.astype(np.float32))
+    for name in ("x8", c1):
+        assert np.array_equal(m.get_tensor_i8(name), want[name]), name
+    assert len(np.unique(want[c1])) > 8
+    with pytest.raises(capi.TpuHipError, match="not a uint8 value"):
+        m.set_tensor("input", img.astype(np.float32) - 1.0)
+    m.close()
+    # a signed tensor in front of a ScaleLut, and a UINT8 tensor in front of anything else, are refused
+    g2 = graphs.Graph("bad", 1)
+    g2.add(graphs.Op("tpu.input", "input", [], (1, 3, 4, 4))).data = np.zeros((1, 3, 4, 4), np.int8)
+    g2.add(graphs.Op("tpu.scale_lut", "s", ["input"], (1, 3, 4, 4), {},
+                     dict(table=np.zeros(768, np.float32))))
+    with pytest.raises(capi.TpuHipError, match="UINT8 tensor"):
+        module().load(g2)
+    g3 = graphs.Graph("bad", 1)
+    i3 = g3.add(graphs.Op("tpu.input", "input", [], (1, 16, 4, 4)))
+    i3.quant = "UINT8"
+    i3.data = np.zeros((1, 16, 4, 4), np.uint8)
+    g3.add(graphs.Op("tpu.relu", "r", ["input"], (1, 16, 4, 4)))
+    with pytest.raises(capi.TpuHipError, match="only read by ScaleLut"):
+        module().load(g3)
+
+
 @pytest.mark.parametrize("cfg", [
     # ic, ih, iw, oc, k, stride, pads(t,b,l,r), dil, groups, out_hw
     (24, 7, 6, 40, 3, (2, 2), (1, 1, 1, 1), (1, 1), 1, (14, 12)),     # output_padding 1

@@ -103,3 +103,20 @@ def test_prelu_matches_exact_arithmetic_for_every_input_value():
                 want = (sat8(nearest_ties_up(Fraction(v * mp, 1 << rp))) if v > 0 else
                         sat8(nearest_ties_up(Fraction(int(slope[ch]) * v, 1 << rn))))
                 assert got[1, ch, v + 128, 0] == want, (mp, rp, rn, ch, v)
+
+
+def test_scale_lut_reads_each_channels_table_at_the_unsigned_value():
+    """every uint8 value on every channel equals plain numpy indexing table[c, x]; the tables are
+    built the way the quantizer builds them (saturated nearest of idx * scale + bias)"""
+    c = 5
+    scale = np.array([0.5, 1.0, 0.017, 2.0, 0.25])
+    bias = np.array([-64.0, -128.0, 3.0, -300.0, 0.4])
+    idx = np.arange(256)
+    table = np.clip(np.floor(idx[None, :] * scale[:, None] + bias[:, None] + 0.5), -128, 127).astype(np.float32)
+    x = np.tile(idx.astype(np.uint8).reshape(1, 1, 16, 16), (2, c, 1, 1))
+    x[1] = x[1, :, ::-1, ::-1]
+    got = O.scale_lut_u8(x, table.reshape(-1))
+    want = table.astype(np.int8)[np.arange(c)[None, :, None, None], x.astype(np.int64)]
+    assert got.dtype == np.int8 and np.array_equal(got, want)
+    # channel 1 is the identity shifted by 128: the unsigned byte reinterpreted as int8
+    assert np.array_equal(got[:, 1], (x[:, 1].astype(np.int16) - 128).astype(np.int8))

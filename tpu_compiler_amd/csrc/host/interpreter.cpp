@@ -239,6 +239,8 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<DepthToSpaceOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.quant") {
       krnl = std::make_shared<QuantOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.scale_lut") {
+      krnl = std::make_shared<ScaleLutOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.prelu") {
       krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {

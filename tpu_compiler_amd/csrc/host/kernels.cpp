@@ -112,10 +112,18 @@ void TensorData::assign(const float *first, size_t num, int32_t bidx) {
        "TensorData::assign");
     return;
   }
+  const float lo = is_unsigned ? 0.0f : -128.0f, hi = is_unsigned ? 255.0f : 127.0f;
   for (size_t i = 0; i < num; ++i)
-    if (!(first[i] >= -128.0f && first[i] <= 127.0f) || first[i] != std::nearbyint(first[i]))
+    if (!(first[i] >= lo && first[i] <= hi) || first[i] != std::nearbyint(first[i]))
       fail("TensorData::assign: element " + std::to_string(i) + " = " + std::to_string(first[i]) +
-           " is not an int8 value");
+           (is_unsigned ? " is not a uint8 value" : " is not an int8 value"));
+  std::vector<float> wrapped;   // 128..255 travel as the int8 value with the same byte
+  if (is_unsigned) {
+    wrapped.assign(first, first + num);
+    for (auto &v : wrapped)
+      if (v >= 128.0f) v -= 256.0f;
+    first = wrapped.data();
+  }
   void *tmp = nullptr;
   ck(tpuhip_malloc(ctx_, num * sizeof(float), &tmp), "TensorData::assign");
   int rc = tpuhip_upload(ctx_, tmp, first, num * sizeof(float));
@@ -145,6 +153,9 @@ std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
   if (!rc) rc = tpuhip_download(ctx_, out->data(), tmp, size_ * sizeof(float));
   tpuhip_free(ctx_, tmp);
   ck(rc, "TensorData::tensor");
+  if (is_unsigned)
+    for (auto &v : *out)
+      if (v < 0.0f) v += 256.0f;
   return out;
 }
 
@@ -247,6 +258,7 @@ void CPUOpKernel::assignResultTensor(OpDesc &op_, value_map_t &valueMapping) {
   if (f32 && op_.type != "tpu.input" && op_.type != "tpu.quant")
     fail(op_.type + " '" + op_.name + "': only the INT8 path is implemented on the GPU");
   resTensor = std::make_shared<TensorData>(ctx, max_batch_size, op_.shape, f32);
+  resTensor->is_unsigned = !f32 && op_.quant == "UINT8";
   valueMapping[op_.name] = resTensor;
   valueMapping.shapes[op_.name] = op_.shape;
 }
@@ -254,9 +266,14 @@ void CPUOpKernel::assignResultTensor(OpDesc &op_, value_map_t &valueMapping) {
 void CPUOpKernel::require_int8(const char *what) const {
   if (datatype != DataType::INT8)
     fail(std::string(what) + " '" + name + "': only the INT8 path is implemented on the GPU");
-  for (auto &opd : opdTensors)
+  for (auto &opd : opdTensors) {
     if (opd.act && opd.act->f32)
       fail(std::string(what) + " '" + name + "': an fp32 operand needs a QuantOp in front");
+    if (opd.act && opd.act->is_unsigned)
+      fail(std::string(what) + " '" + name + "': a UINT8 operand is only read by ScaleLut");
+  }
+  if (resTensor && resTensor->is_unsigned)
+    fail(std::string(what) + " '" + name + "': UINT8 results exist only for the network input");
 }
 
 // ---------------------------------------------------------------------------
@@ -769,6 +786,43 @@ PReluOpKernel::~PReluOpKernel() {
 }
 
 void PReluOpKernel::invoke() {
+  ck(tpuhip_lut_per_channel_i8(ctx, input_data->data(), output_data->data(), tables,
+                               (size_t)input_data->n * input_data->h * input_data->w,
+                               input_data->c, input_data->cs),
+     name.c_str());
+}
+
+// ---------------------------------------------------------------------------
+// ScaleLut (core/scale_lut.cpp:7-31)
+// ---------------------------------------------------------------------------
+ScaleLutOpKernel::ScaleLutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  if (datatype != DataType::INT8 || resTensor->is_unsigned)
+    fail("ScaleLut '" + name + "': the result is an INT8 tensor");
+  if (opdTensors.size() < 2) fail("ScaleLut '" + name + "': expected 2 operands");
+  input_data = opdTensors[0].act;
+  output_data = resTensor;
+  auto table = opdTensors[1].weight;
+  if (!input_data || !table) fail("ScaleLut '" + name + "': input / table missing");
+  if (input_data->f32) fail("ScaleLut '" + name + "': an fp32 operand needs a QuantOp in front");
+  if (!input_data->is_unsigned)
+    fail("ScaleLut '" + name + "': the input must be a UINT8 tensor (a negative value would index "
+         "the previous channel's table in the reference)");
+  if (input_data->size() != output_data->size() || input_data->c != output_data->c)
+    fail("ScaleLut '" + name + "': shape mismatch");
+  const size_t need = (size_t)input_data->c * 256;
+  if (table->size() < need) fail("ScaleLut '" + name + "': the table needs 256 entries per channel");
+  std::vector<int8_t> host(need);
+  for (size_t i = 0; i < need; ++i) host[i] = weight_to_i8(table->at(i), name, "table");
+  ck(tpuhip_malloc(ctx, host.size(), &tables), name.c_str());
+  ck(tpuhip_upload(ctx, tables, host.data(), host.size()), name.c_str());
+}
+
+ScaleLutOpKernel::~ScaleLutOpKernel() {
+  if (tables) tpuhip_free(ctx, tables);
+}
+
+void ScaleLutOpKernel::invoke() {
   ck(tpuhip_lut_per_channel_i8(ctx, input_data->data(), output_data->data(), tables,
                                (size_t)input_data->n * input_data->h * input_data->w,
                                input_data->c, input_data->cs),

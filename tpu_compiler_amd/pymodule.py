@@ -33,6 +33,7 @@ _WEIGHT_OPERANDS = {
     "tpu.prelu": ["slope", None, None, None, None, "rshift_pos", "multiplier_pos", "rshift_neg"],
     "tpu.clip": [None, None, "rshift", "multiplier"],
     "tpu.lut": ["table", None],
+    "tpu.scale_lut": ["table"],
     "tpu.relu": [],
     "tpu.quant": [],
     "tpu.pad": [], "tpu.crop": [], "tpu.permute": [], "tpu.reorg": [], "tpu.tile": [],
