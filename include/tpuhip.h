@@ -377,6 +377,47 @@ const char *tpuhip_module_kernel_algo(tpuhip_module *m, int i);
 int tpuhip_module_time_kernels(tpuhip_module *m, int bidx, int iters, float *ms, int capacity);
 tpuhip_ctx *tpuhip_module_ctx(tpuhip_module *m);
 
+/* ---- Modules and tensors in the reference's file formats ------------------- */
+
+/* Replaces py_module::load (bindings/python/pymlir.cpp, load / parseMLIRInput) and the first half
+ * of tpuc-interpreter's main (tools/tpuc-interpreter/tpuc-interpreter.cpp): parses a TPU-dialect
+ * .mlir file in the generic textual form, reads every tpu.load_weight from the .npz its
+ * tpu.weight_file names (MlirModuleInterpreter::updateWeightMap, MlirModuleInterpreter.cpp:352-369)
+ * and builds the kernels (loadModule).  The weight file is looked up as written, then beside
+ * the .mlir. */
+int tpuhip_module_load_mlir(tpuhip_module *m, const char *mlir_path, const char *target_op);
+/* py_module::getWeightFilePath / op_info (pymlir.cpp parseMLIRInfo): name, op type, quant mode */
+const char *tpuhip_module_weight_file(tpuhip_module *m);
+int tpuhip_module_num_ops(tpuhip_module *m);
+int tpuhip_module_op_info(tpuhip_module *m, int i, const char **name, const char **type,
+                          const char **quant);
+/* The whole of tpuc-interpreter's main: `<mlir> --tensor-in <npz> [--tensor-out <npz>]
+ * [--dump-all-tensor <npz>]`; NULL, "" or "-" leaves an output file out. */
+int tpuhip_module_interpret_files(tpuhip_module *m, const char *mlir_path, const char *tensor_in,
+                                  const char *tensor_out, const char *dump_all_tensor);
+/* Parses only (no GPU, no weights): one text line per weight, op and return value, for tools
+ * and tests.  Writes at most capacity bytes (NUL-terminated); *needed gets the full size. */
+int tpuhip_mlir_describe(const char *mlir_path, char *buf, size_t capacity, size_t *needed);
+
+/* TensorFile (include/tpuc/Support/TensorFile.h:83-319): an .npz of arrays keyed by name, held in
+ * memory and written back as a whole by keep().  mode 0 = openInputTensorFile (read only, must
+ * exist), 1 = openOutputTensorFile (starts empty), 2 = read what exists and allow changes. */
+typedef struct tpuhip_npz tpuhip_npz;
+int tpuhip_npz_open(const char *filename, int mode, tpuhip_npz **out);
+int tpuhip_npz_close(tpuhip_npz *f);
+int tpuhip_npz_count(tpuhip_npz *f);
+const char *tpuhip_npz_name(tpuhip_npz *f, int i);
+/* shape (up to 8 dims), numpy kind character ('f', 'i', 'u', 'b') and bytes per element */
+int tpuhip_npz_info(tpuhip_npz *f, const char *name, int64_t *dims8, int *ndim, char *kind,
+                    int *word_size);
+/* readTensor<float>(name, data, count): float32 of exactly count elements, else an error */
+int tpuhip_npz_read_f32(tpuhip_npz *f, const char *name, float *dst, size_t count);
+/* addTensor: an error if the name is already used */
+int tpuhip_npz_add_f32(tpuhip_npz *f, const char *name, const float *data, const int64_t *dims,
+                       int ndim);
+int tpuhip_npz_delete(tpuhip_npz *f, const char *name);
+int tpuhip_npz_keep(tpuhip_npz *f);
+
 #ifdef __cplusplus
 }
 #endif

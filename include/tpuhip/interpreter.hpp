@@ -470,6 +470,13 @@ public:
 
   void loadModule(ModuleDesc &module, std::string target_op);
   void loadModule(ModuleDesc &module) { loadModule(module, ""); }
+  // module.load(filename) of pymlir / the first half of tpuc-interpreter's main: parse the
+  // TPU-dialect text, read the weights its tpu.weight_file names, build the kernels
+  void loadModuleFile(const std::string &mlir_path, std::string target_op = "");
+  const std::string &weightFilePath() const { return weight_file_path_; }
+  // name, op type, quant mode of every op of the loaded file (pymlir's op_info)
+  struct OpInfo { std::string name, type, quant; };
+  const std::vector<OpInfo> &opInfo() const { return op_info_; }
   void fastInvokeAllBatch(std::string name, int32_t batch);
   void invokeTo(std::string name, int32_t bidx);
   void invoke(int32_t bidx) { invokeTo("", bidx); }
@@ -511,6 +518,13 @@ private:
   tpuhip_ctx *ctx_ = nullptr;
   kernel_map_t kernel_map_;
   kernel_list_t kernel_list_;
+  std::string weight_file_path_;
+  std::vector<OpInfo> op_info_;
 };
+
+// tools/tpuc-interpreter/tpuc-interpreter.cpp main(): `mlir --tensor-in in.npz [--tensor-out
+// out.npz] [--dump-all-tensor all.npz]`; "" or "-" leaves a file out.
+void interpretFiles(ModuleInterpreter &interp, const std::string &mlir_path, const std::string &tensor_in,
+                    const std::string &tensor_out, const std::string &dump_all_tensor);
 
 }  // namespace tpuhip

@@ -1,6 +1,8 @@
 """GPU parity on whole graphs through the module API (C++ op classes +
 ModuleInterpreter behind the C ABI): every tensor of every layer must equal the
 oracle's, for the five benchmark configurations at their full sizes."""
+import os
+
 import numpy as np
 import pytest
 
@@ -8,6 +10,47 @@ import oracle_graph
 from tpu_compiler_amd import capi, graphs, module
 
 pytestmark = pytest.mark.gpu
+
+
+def check_through_files(g, x, want, tmp_path):
+    """the same graph as files: written as TPU-dialect text + weight .npz, loaded by name like
+    pymlir's module.load, and run the way the tpuc-interpreter tool runs (.npz in, .npz out)"""
+    from tpu_compiler_amd import mlir_text
+    path = tmp_path / (g.name + ".mlir")
+    wfile = mlir_text.write_mlir(g, path)
+    m = module()
+    m.load(str(path))
+    assert m.get_weight_file_path() == os.path.basename(wfile)
+    assert [(i["name"], i["type"], i["quant"]) for i in m.op_info] == [(o.name, o.type, o.quant) for o in g.ops]
+    assert list(m.get_output_details()) == list(g.outputs)
+    m.set_tensor(g.input_op().name, np.asarray(x, np.float32))
+    m.invoke()
+    for op in g.ops:
+        w = want[op.name].reshape(op.shape)
+        got = m.get_tensor(op.name) if w.dtype == np.float32 or op.quant == "UINT8" else m.get_tensor_i8(op.name)
+        assert np.array_equal(got, w.astype(got.dtype)), op.name
+    m.close()
+    np.savez(tmp_path / "in.npz", **{g.input_op().name: np.asarray(x, np.float32)})
+    m = module()
+    m.interpret_files(path, tmp_path / "in.npz", tmp_path / "out.npz", tmp_path / "all.npz")
+    m.close()
+    with np.load(tmp_path / "out.npz") as z:
+        assert sorted(z.files) == sorted(g.outputs)
+        for name in g.outputs:
+            assert z[name].dtype == np.float32 and z[name].shape == tuple(g.by_name[name].shape)
+            assert np.array_equal(z[name], want[name].reshape(z[name].shape).astype(np.float32)), name
+    with np.load(tmp_path / "all.npz") as z:
+        assert sorted(z.files) == sorted(o.name for o in g.ops)
+        for op in g.ops:
+            assert np.array_equal(z[op.name], want[op.name].reshape(op.shape).astype(np.float32)), op.name
+
+
+@pytest.mark.parametrize("cfg,kw", [("cfg1", {}), ("cfg2", dict(batch=2)), ("cfg3", dict(batch=1, hw=96)),
+                                    ("cfg4", dict(batch=2, hw=96)), ("cfg5", dict(batch=1, hw=96))])
+def test_configurations_loaded_from_files_match_the_oracle(tmp_path, cfg, kw):
+    g = graphs.CONFIGS[cfg](**kw)
+    x = g.input_op().data
+    check_through_files(g, x, oracle_graph.run(g), tmp_path)
 
 
 def run_and_compare(g, check_stats=True):
@@ -266,7 +309,7 @@ def test_lut_activation_and_general_reshape():
     m.close()
 
 
-def test_graph_with_elementwise_family_matches_the_oracle():
+def test_graph_with_elementwise_family_matches_the_oracle(tmp_path):
     """a squeeze-excite shaped graph: conv pair -> max / min / mul -> global average ->
     1x1 conv gate -> broadcast mul / add / sub with the feature map"""
     b = graphs.Builder("se_block", graphs.BASE_SEED + 77, 2, (6, 12))
@@ -307,9 +350,10 @@ def test_graph_with_elementwise_family_matches_the_oracle():
         assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
     assert len(np.unique(want[bs])) > 8
     m.close()
+    check_through_files(g, g.input_op().data, want, tmp_path)
 
 
-def test_graph_with_data_movement_ops_matches_the_oracle():
+def test_graph_with_data_movement_ops_matches_the_oracle(tmp_path):
     b = graphs.Builder("movers", graphs.BASE_SEED + 78, 2, (6, 12))
     x = b.input("input", 12, 8, 6)
     c1 = b.conv("c1", x, 36, 3, relu=True)
@@ -343,9 +387,10 @@ def test_graph_with_data_movement_ops_matches_the_oracle():
     for op in g.ops:
         assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
     m.close()
+    check_through_files(g, g.input_op().data, want, tmp_path)
 
 
-def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle():
+def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle(tmp_path):
     """uint8 image -> ScaleLut (per-channel 256-entry tables) -> conv"""
     rng = np.random.default_rng(6)
     b = graphs.Builder("scale_lut", graphs.BASE_SEED + 80, 2, (6, 12))
@@ -380,6 +425,7 @@ def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle():
     with pytest.raises(capi.TpuHipError, match="not a uint8 value"):
         m.set_tensor("input", img.astype(np.float32) - 1.0)
     m.close()
+    check_through_files(g, img, want, tmp_path)
     # a signed tensor in front of a ScaleLut, and a UINT8 tensor in front of anything else, are refused
     g2 = graphs.Graph("bad", 1)
     g2.add(graphs.Op("tpu.input", "input", [], (1, 3, 4, 4))).data = np.zeros((1, 3, 4, 4), np.int8)
@@ -430,7 +476,7 @@ def test_deconv_graph_matches_the_oracle(cfg):
     m.close()
 
 
-def test_graph_with_fp32_edges_quantizes_and_dequantizes_like_the_oracle():
+def test_graph_with_fp32_edges_quantizes_and_dequantizes_like_the_oracle(tmp_path):
     """fp32 input -> QuantOp -> conv -> conv -> QuantOp -> fp32 output"""
     rng = np.random.default_rng(5)
     b = graphs.Builder("edges", graphs.BASE_SEED + 79, 3, (6, 12))
@@ -469,6 +515,7 @@ def test_graph_with_fp32_edges_quantizes_and_dequantizes_like_the_oracle():
     with pytest.raises(capi.TpuHipError, match="fp32"):
         m.get_tensor_i8("out")
     m.close()
+    check_through_files(g, xf, want, tmp_path)
     # an INT8 op fed with fp32 data is refused
     g2 = graphs.Graph("bad", 1)
     i2 = g2.add(graphs.Op("tpu.input", "input", [], (1, 16, 4, 4)))

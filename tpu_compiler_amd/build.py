@@ -34,7 +34,7 @@ def build(verbose=True):
     for s in sources():
         # .cpp host files are compiled as HIP too so they can include the runtime headers
         cmd += ["-x", "hip", s]
-    cmd += ["-o", LIB]
+    cmd += ["-lz", "-o", LIB]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

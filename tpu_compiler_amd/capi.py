@@ -154,6 +154,24 @@ PROTOTYPES.update({
                                              C.c_int]),
     "tpuhip_module_ctx": (C.c_void_p, [C.c_void_p]),
     "tpuhip_module_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
+    "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
+    "tpuhip_module_weight_file": (C.c_char_p, [C.c_void_p]),
+    "tpuhip_module_num_ops": (C.c_int, [C.c_void_p]),
+    "tpuhip_module_op_info": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(C.c_char_p),
+                                        C.POINTER(C.c_char_p), C.POINTER(C.c_char_p)]),
+    "tpuhip_module_interpret_files": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p, C.c_char_p,
+                                                C.c_char_p]),
+    "tpuhip_mlir_describe": (C.c_int, [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]),
+    "tpuhip_npz_open": (C.c_int, [C.c_char_p, C.c_int, C.POINTER(C.c_void_p)]),
+    "tpuhip_npz_close": (C.c_int, [C.c_void_p]),
+    "tpuhip_npz_count": (C.c_int, [C.c_void_p]),
+    "tpuhip_npz_name": (C.c_char_p, [C.c_void_p, C.c_int]),
+    "tpuhip_npz_info": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_int64), C.POINTER(C.c_int),
+                                  C.POINTER(C.c_char), C.POINTER(C.c_int)]),
+    "tpuhip_npz_read_f32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]),
+    "tpuhip_npz_add_f32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int]),
+    "tpuhip_npz_delete": (C.c_int, [C.c_void_p, C.c_char_p]),
+    "tpuhip_npz_keep": (C.c_int, [C.c_void_p]),
 })
 
 
@@ -175,6 +193,59 @@ def bind(lib=None, prototypes=None):
 def check(lib, status):
     if status != 0:
         raise TpuHipError(status, lib.tpuhip_last_error().decode())
+
+
+def mlir_describe(path, lib=None):
+    """what the reader understood of a TPU-dialect .mlir file, one line per weight / op / return
+    (parses only: no GPU, no weight file)"""
+    lib = lib or bind()
+    need = C.c_size_t(0)
+    check(lib, lib.tpuhip_mlir_describe(str(path).encode(), None, 0, C.byref(need)))
+    buf = C.create_string_buffer(need.value)
+    check(lib, lib.tpuhip_mlir_describe(str(path).encode(), buf, need.value, None))
+    return buf.value.decode()
+
+
+class TensorFile:
+    """include/tpuc/Support/TensorFile.h: an .npz of arrays keyed by name.  mode "r" = read only,
+    "w" = start empty, "a" = read what exists and allow changes; keep() writes the file."""
+
+    def __init__(self, filename, mode="r", lib=None):
+        self.lib = lib or bind()
+        self.h = C.c_void_p()
+        check(self.lib, self.lib.tpuhip_npz_open(str(filename).encode(), {"r": 0, "w": 1, "a": 2}[mode],
+                                                 C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            self.lib.tpuhip_npz_close(self.h)
+            self.h = None
+
+    def names(self):
+        return [self.lib.tpuhip_npz_name(self.h, i).decode() for i in range(self.lib.tpuhip_npz_count(self.h))]
+
+    def info(self, name):
+        dims, nd, kind, ws = (C.c_int64 * 8)(), C.c_int(0), C.c_char(b"?"), C.c_int(0)
+        check(self.lib, self.lib.tpuhip_npz_info(self.h, name.encode(), dims, C.byref(nd), C.byref(kind),
+                                                 C.byref(ws)))
+        return tuple(dims[i] for i in range(nd.value)), kind.value.decode(), ws.value
+
+    def read(self, name):
+        shape, _, _ = self.info(name)
+        out = np.empty(shape, np.float32)
+        check(self.lib, self.lib.tpuhip_npz_read_f32(self.h, name.encode(), out.ctypes.data, out.size))
+        return out
+
+    def add(self, name, array):
+        a = np.asarray(array, dtype=np.float32, order="C")    # keeps a 0-d array 0-d
+        dims = (C.c_int64 * max(a.ndim, 1))(*a.shape)
+        check(self.lib, self.lib.tpuhip_npz_add_f32(self.h, name.encode(), a.ctypes.data, dims, a.ndim))
+
+    def delete(self, name):
+        check(self.lib, self.lib.tpuhip_npz_delete(self.h, name.encode()))
+
+    def keep(self):
+        check(self.lib, self.lib.tpuhip_npz_keep(self.h))
 
 
 def channel_stride(c):

@@ -3,10 +3,18 @@
 #include <cstring>
 
 #include "tpuhip/interpreter.hpp"
+#include "tpuhip/mlir_text.hpp"
+#include "tpuhip/tensor_file.hpp"
 
 namespace tpuhip {
 int set_error(int status, const char *fmt, ...);
+MlirModule readMlirFile(const std::string &mlir_path);
 }
+
+struct tpuhip_npz {
+  std::unique_ptr<tpuhip::TensorFile> file;
+  std::vector<std::string> names;
+};
 
 struct tpuhip_module {
   std::unique_ptr<tpuhip::ModuleInterpreter> interp;
@@ -210,5 +218,124 @@ int tpuhip_module_time_kernels(tpuhip_module *m, int bidx, int iters, float *ms,
 }
 
 tpuhip_ctx *tpuhip_module_ctx(tpuhip_module *m) { return m ? m->interp->context() : nullptr; }
+
+// ---- modules and tensors in files --------------------------------------------
+
+int tpuhip_module_load_mlir(tpuhip_module *m, const char *mlir_path, const char *target_op) {
+  GUARD(m, {
+    if (!mlir_path) throw std::runtime_error("load_mlir: NULL path");
+    m->interp->loadModuleFile(mlir_path, target_op ? target_op : "");
+    m->tensor_names = m->interp->getAllTensorName();
+  })
+}
+
+const char *tpuhip_module_weight_file(tpuhip_module *m) {
+  return m ? m->interp->weightFilePath().c_str() : nullptr;
+}
+
+int tpuhip_module_num_ops(tpuhip_module *m) { return m ? (int)m->interp->opInfo().size() : 0; }
+
+int tpuhip_module_op_info(tpuhip_module *m, int i, const char **name, const char **type, const char **quant) {
+  GUARD(m, {
+    auto &info = m->interp->opInfo();
+    if (i < 0 || i >= (int)info.size()) throw std::runtime_error("op_info: index out of range");
+    if (name) *name = info[i].name.c_str();
+    if (type) *type = info[i].type.c_str();
+    if (quant) *quant = info[i].quant.c_str();
+  })
+}
+
+int tpuhip_module_interpret_files(tpuhip_module *m, const char *mlir_path, const char *tensor_in,
+                                  const char *tensor_out, const char *dump_all_tensor) {
+  GUARD(m, {
+    if (!mlir_path || !tensor_in) throw std::runtime_error("interpret_files: NULL path");
+    interpretFiles(*m->interp, mlir_path, tensor_in, tensor_out ? tensor_out : "",
+                   dump_all_tensor ? dump_all_tensor : "");
+    m->tensor_names = m->interp->getAllTensorName();
+  })
+}
+
+int tpuhip_mlir_describe(const char *mlir_path, char *buf, size_t capacity, size_t *needed) {
+  try {
+    if (!mlir_path) throw std::runtime_error("mlir_describe: NULL path");
+    const std::string text = describeModule(readMlirFile(mlir_path));
+    if (needed) *needed = text.size() + 1;
+    if (buf && capacity) {
+      const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+      std::memcpy(buf, text.data(), n);
+      buf[n] = '\0';
+    }
+  } catch (const std::exception &e) {
+    return set_error(TPUHIP_ERR_INVALID, "%s", e.what());
+  }
+  return TPUHIP_OK;
+}
+
+int tpuhip_npz_open(const char *filename, int mode, tpuhip_npz **out) {
+  if (!filename || !out) return set_error(TPUHIP_ERR_INVALID, "tpuhip_npz_open: NULL argument");
+  try {
+    auto *f = new tpuhip_npz();
+    // 0: read only (must exist), 1: new empty file, 2: read what exists and allow changes
+    f->file.reset(new TensorFile(filename, mode == 0, mode == 1));
+    f->names = f->file->names();
+    *out = f;
+  } catch (const std::exception &e) {
+    return set_error(TPUHIP_ERR_INVALID, "%s", e.what());
+  }
+  return TPUHIP_OK;
+}
+
+int tpuhip_npz_close(tpuhip_npz *f) {
+  delete f;
+  return TPUHIP_OK;
+}
+
+int tpuhip_npz_count(tpuhip_npz *f) { return f ? (int)f->names.size() : 0; }
+
+const char *tpuhip_npz_name(tpuhip_npz *f, int i) {
+  return f && i >= 0 && i < (int)f->names.size() ? f->names[i].c_str() : nullptr;
+}
+
+int tpuhip_npz_info(tpuhip_npz *f, const char *name, int64_t *dims8, int *ndim, char *kind, int *word_size) {
+  GUARD(f, {
+    auto *a = f->file->find(name ? name : "");
+    if (!a) throw std::runtime_error(std::string("failed to find tensor ") + (name ? name : "(null)"));
+    if (a->shape.size() > 8) throw std::runtime_error("npz_info: more than 8 dimensions");
+    if (ndim) *ndim = (int)a->shape.size();
+    if (dims8) for (size_t i = 0; i < a->shape.size(); ++i) dims8[i] = a->shape[i];
+    if (kind) *kind = a->kind;
+    if (word_size) *word_size = a->word_size;
+  })
+}
+
+int tpuhip_npz_read_f32(tpuhip_npz *f, const char *name, float *dst, size_t count) {
+  GUARD(f, {
+    if (!name || (!dst && count)) throw std::runtime_error("npz_read_f32: NULL argument");
+    if (!f->file->readTensor(name, dst, count)) {
+      if (!f->file->find(name)) throw std::runtime_error(std::string("failed to find tensor ") + name + " to read");
+      throw std::runtime_error(std::string("size does not match for tensor ") + name);
+    }
+  })
+}
+
+int tpuhip_npz_add_f32(tpuhip_npz *f, const char *name, const float *data, const int64_t *dims, int ndim) {
+  GUARD(f, {
+    if (!name || !dims || ndim < 0) throw std::runtime_error("npz_add_f32: bad argument");
+    std::vector<int64_t> shape(dims, dims + ndim);
+    if (!f->file->addTensor(name, data, shape))
+      throw std::runtime_error(std::string("failed to add tensor ") + name + ", already exist");
+    f->names = f->file->names();
+  })
+}
+
+int tpuhip_npz_delete(tpuhip_npz *f, const char *name) {
+  GUARD(f, {
+    if (!f->file->deleteTensor(name ? name : ""))
+      throw std::runtime_error(std::string("failed to find tensor ") + (name ? name : "(null)") + " to delete");
+    f->names = f->file->names();
+  })
+}
+
+int tpuhip_npz_keep(tpuhip_npz *f) { GUARD(f, f->file->keep()) }
 
 }  // extern "C"

@@ -8,6 +8,7 @@ Tensors cross this API as float32 NCHW arrays holding integers, like the
 reference's; `get_tensor_i8` is the cheaper int8 view of the same data.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -72,7 +73,19 @@ class module:
 
     # -- loading ----------------------------------------------------------
     def load(self, graph, target_op=""):
-        """updateWeightMap + loadModule for `graph` (pymlir.cpp:99-122)."""
+        """updateWeightMap + loadModule (pymlir.cpp:99-122) for a TPU-dialect .mlir file given by
+        name, like pymlir, or for a graph object built in Python."""
+        if isinstance(graph, (str, os.PathLike)):
+            self.graph = None
+            self._ck(self.lib.tpuhip_module_load_mlir(self.h, os.fspath(graph).encode(),
+                                                      target_op.encode() if target_op else None))
+            self.op_info = []
+            n, t, q = C.c_char_p(), C.c_char_p(), C.c_char_p()
+            for i in range(self.lib.tpuhip_module_num_ops(self.h)):
+                self._ck(self.lib.tpuhip_module_op_info(self.h, i, C.byref(n), C.byref(t), C.byref(q)))
+                self.op_info.append({"name": n.value.decode(), "type": t.value.decode(),
+                                     "quant": q.value.decode()})
+            return
         self.graph = graph
         self._ck(self.lib.tpuhip_module_clear_ops(self.h))
         self.op_info = []
@@ -105,6 +118,16 @@ class module:
         ra = (C.c_char_p * max(len(rets), 1))(*rets)
         self._ck(self.lib.tpuhip_module_set_returns(self.h, ra, len(rets)))
         self._ck(self.lib.tpuhip_module_load(self.h, target_op.encode() if target_op else None))
+
+    def get_weight_file_path(self):
+        return (self.lib.tpuhip_module_weight_file(self.h) or b"").decode()
+
+    def interpret_files(self, mlir_path, tensor_in, tensor_out=None, dump_all_tensor=None):
+        """the tpuc-interpreter tool: <mlir> --tensor-in <npz> [--tensor-out <npz>]
+        [--dump-all-tensor <npz>]"""
+        enc = lambda p: os.fspath(p).encode() if p else None
+        self._ck(self.lib.tpuhip_module_interpret_files(self.h, enc(mlir_path), enc(tensor_in),
+                                                        enc(tensor_out), enc(dump_all_tensor)))
 
     def set_option(self, key, value):
         """Options read at the next load(): "fuse_eltwise", "keep_all_tensors" (both default 1)."""
