@@ -112,7 +112,10 @@ typedef struct {
   int with_bias;
   int x_cs, y_cs;    /* channel strides of input / output */
   int relu_first;    /* 0: ReLU after saturation (conv); 1: ReLU on the sum before requant (FC) */
-  int algo;          /* 0 auto, 1 direct (one thread per output), 2 MFMA implicit GEMM, 3 depthwise */
+  int algo;          /* 0 auto, 1 direct (one thread per output), 2 MFMA implicit GEMM, 3 depthwise
+                        (one diagonal MFMA per tap), 4 depthwise with per-byte dot products,
+                        5 stem (at most 4 input and 64 output channels: input rows staged once in
+                        LDS, one MFMA K step per filter row), 16 + t: MFMA tile variant t */
 } tpuhip_conv_desc;
 
 typedef struct tpuhip_conv_weights tpuhip_conv_weights;

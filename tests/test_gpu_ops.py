@@ -80,6 +80,66 @@ def test_conv_dense(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
+# n, ic, ih, iw, oc, kh, kw, stride, pads, relu: at most 4 input channels, at most 64 output channels
+STEM_CASES = [
+    (2, 3, 64, 64, 64, 7, 7, (2, 2), (3, 3, 3, 3), True),        # ResNet-50 conv1 at a smaller size
+    (3, 3, 40, 300, 32, 3, 3, (2, 2), (1, 1, 1, 1), True),       # 150 pixels per row: two segments
+    (2, 3, 19, 141, 32, 3, 3, (1, 1), (1, 1, 1, 1), False),      # stride 1, ragged second segment
+    (70, 3, 9, 12, 24, 3, 3, (1, 1), (1, 1, 1, 1), True),        # many tiny tiles: the workgroups walk
+    (1, 1, 30, 31, 16, 5, 5, (1, 2), (2, 2, 2, 2), False),       # one channel, mixed strides
+    (2, 4, 12, 20, 48, 2, 8, (1, 1), (0, 1, 3, 4), False),       # four channels, kw = 8, asymmetric pads
+    (1, 2, 17, 9, 64, 7, 1, (3, 1), (3, 3, 0, 0), True),         # kw = 1, stride_h 3
+    (2, 3, 21, 21, 40, 4, 6, (2, 2), (1, 2, 2, 3), False),       # even kernel sizes, 40 channels
+]
+
+
+@pytest.mark.parametrize("case", STEM_CASES)
+@pytest.mark.parametrize("algo", [capi.ALGO_STEM, capi.ALGO_AUTO])
+def test_conv_stem(ctx, case, algo):
+    n, ic, ih, iw, oc, kh, kw, stride, pads, relu = case
+    rng = np.random.default_rng(ic * 131 + oc + kh * 7 + kw)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, (1, 1), (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=algo, stride=stride, pads=pads, do_relu=relu)
+    assert name == "stem"
+    assert np.array_equal(got, want), "%d mismatches" % (got != want).sum()
+    assert len(np.unique(want)) > 8
+
+
+def test_conv_stem_general_requant_fused_table_and_limits(ctx):
+    """parameters outside the overflow-free form, a table fused behind the requantisation, and the
+    shapes the stem path refuses"""
+    rng = np.random.default_rng(991)
+    x = rnd_i8(rng, (2, 3, 33, 35))
+    w = rnd_w(rng, (32, 3, 3, 3), sigma=60)
+    bias = rng.integers(-(1 << 23), 1 << 23, 32).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, 32) * 128).astype(np.float32)
+    rsh = rng.integers(0, 9, 32).astype(np.float32)
+    rsh[:4] = 0
+    want = oracle_conv(x, w, bias, rsh, mult, 1, (1, 1), (1, 1, 1, 1), (1, 1), (0, 0), False)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=capi.ALGO_STEM, pads=(1, 1, 1, 1))
+    assert name == "stem" and np.array_equal(got, want)
+    table = rng.integers(-128, 128, 256).astype(np.int8)
+    table[0] = 77
+    d = conv_desc(x.shape, w.shape, pads=(1, 1, 1, 1), algo=capi.ALGO_STEM)
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    xt, yt, tt = ctx.from_nchw(x), ctx.tensor(want.shape), ctx.tensor(want.shape)
+    ctx.conv_post(wh, xt, yt, table, tt)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert np.array_equal(ctx.to_nchw(tt), O.lut_i8(want, table))
+    ctx.conv_weights_destroy(wh)
+    for shape, wshape, kw_ in [((1, 8, 9, 9), (16, 8, 3, 3), {}), ((1, 3, 9, 9), (80, 3, 3, 3), {}),
+                               ((1, 3, 9, 9), (16, 3, 3, 3), dict(dil=(2, 2))),
+                               ((1, 3, 30, 30), (16, 3, 3, 3), dict(stride=(1, 3)))]:
+        dd = conv_desc(shape, wshape, algo=capi.ALGO_STEM, **kw_)
+        ww = np.zeros(wshape, np.int8)
+        z = np.zeros(wshape[0], np.int32)
+        with pytest.raises(capi.TpuHipError, match="stem path needs"):
+            ctx.conv_prepack(dd, ww, z, z + (1 << 30), z + 1)
+
+
 TILE_CASES = [
     (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),
     (2, 96, 17, 13, 200, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),   # ragged pixel / channel tails

@@ -49,7 +49,7 @@ class PoolDesc(C.Structure):
         "x_cs", "y_cs")]
 
 
-ALGO_AUTO, ALGO_DIRECT, ALGO_MFMA, ALGO_DEPTHWISE, ALGO_DEPTHWISE_DOT = 0, 1, 2, 3, 4
+ALGO_AUTO, ALGO_DIRECT, ALGO_MFMA, ALGO_DEPTHWISE, ALGO_DEPTHWISE_DOT, ALGO_STEM = 0, 1, 2, 3, 4, 5
 
 # name -> (restype, argtypes); every symbol include/tpuhip.h declares
 PROTOTYPES = {

@@ -23,7 +23,8 @@ using namespace tpuhip;
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3, ALGO_DEPTHWISE_DOT = 4 };
+enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3, ALGO_DEPTHWISE_DOT = 4,
+                ALGO_STEM = 5 };
 
 // per-channel requantisation record
 struct __attribute__((aligned(16))) QParam {
@@ -72,6 +73,8 @@ struct ConvArgs {
   // advance between two tiles of one workgroup, split into (n, oh, ow) parts
   int wgs_per_xcd, pstep_pix, pstep_n, pstep_oh, pstep_ow;
   int npix;
+  int stem_pw;            // stem kernel: input columns one row tile needs, (128 - 1) * sw + 8
+  uint32_t magic_pw;      // floor(2^20 / stem_pw) + 1
   int lo;          // lower clamp bound: 0 with ReLU after saturation, else -128
   int relu_first;  // ReLU on the sum before requantisation (FC)
   // optional fused eltwise add on the conv result (same shape and channel stride as y):
@@ -878,6 +881,155 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// The network stem: at most 4 input channels, so one pixel is one dword and the kw taps of
+// a filter row are kw consecutive dwords of an input row.  A workgroup computes every
+// output channel (at most 64) of 128 consecutive pixels of ONE output row.  The kh input
+// rows that tile needs are fetched once with coalesced loads (lane = pixel), their first
+// dword kept, and laid down in LDS as a compact patch [kh][column]; the MFMA B operand of
+// filter row kh for output pixel p is then the 8 dwords from column p * sw of patch row kh
+// (lane half h takes dwords 4h .. 4h+3): K = 32 bytes per filter row, taps kw .. 7 meeting
+// zero weights.  No im2col gather from global memory, no address arithmetic per tap.  The
+// filter (A operand, 16 bytes per lane per row and 32-channel block) stays in registers;
+// the patch of the next tile is in flight while this one is multiplied and requantised.
+// KH: filter rows held (kh <= KH); TM: 32-channel blocks (oc <= 32 * TM).  sw <= 2, kw <= 8.
+// ---------------------------------------------------------------------------
+constexpr int kStemPW = 264;   // patch row in dwords: 127 * 2 + 8, rounded up
+// A wave takes all (at most two) 32-channel blocks of 32 pixels -- or, when the filter is
+// too large to keep two blocks of it in registers at three waves per SIMD (7 rows, 64
+// channels: 56 registers), one channel block of 64 pixels.
+constexpr bool stem_split(int kh, int tm) { return kh * tm > 7; }
+template <int KH, int TM, bool FAST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void
+conv_stem_kernel(ConvArgs a) {
+  constexpr int NLD = (KH * kStemPW + 255) / 256;
+  constexpr bool SPLIT = stem_split(KH, TM);
+  constexpr int NI = SPLIT ? 1 : TM;   // channel blocks per wave
+  constexpr int NP = SPLIT ? 2 : 1;    // 32-pixel blocks per wave
+  __shared__ uint32_t patch[2][KH * kStemPW];
+  __shared__ uint32_t lutw[64];
+  __shared__ int32_t qlds[4][TM * 32];   // bias, multiplier, rshift, 2^(rshift-1)
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frow = lane & 31, fk = lane >> 5;
+  const int ib = SPLIT ? (wave & 1) : 0;                  // first channel block of this wave
+  const int pbase = SPLIT ? (wave >> 1) * 64 : wave * 32; // first pixel of this wave in the tile
+  for (int e = tid; e < 4 * TM * 32; e += 256) {
+    const int k = e / (TM * 32), c = e - k * (TM * 32);
+    const int32_t *src = k == 0 ? a.bias : k == 1 ? a.qmult : k == 2 ? a.qshift : a.qhpot;
+    qlds[k][c] = src[c];
+  }
+  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+
+  v4i areg[NI][KH];
+  {
+    const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + lane;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int r = 0; r < KH; ++r) areg[i][r] = afrag[((ib + i) * KH + r) * 64];
+  }
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const int nseg = (a.ow + 127) >> 7;
+  const int n_tiles = a.n * a.oh * nseg;
+  const int used = a.kh * a.stem_pw;   // dwords of a patch that are read
+
+  int tile = blockIdx.x;
+  if (tile >= n_tiles) return;         // whole workgroup, before any barrier
+  int n, oh, ow0;
+  auto locate = [&](int t) {
+    const int seg = t % nseg, r = t / nseg;
+    oh = r % a.oh;
+    n = r / a.oh;
+    ow0 = seg << 7;
+  };
+  uint32_t stage[NLD];
+  auto fetch = [&]() {
+    const int ihb = oh * a.sh - a.pt, iwb = ow0 * a.sw - a.pl;
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      const int e = tid + q * 256;
+      const int r = (int)(((uint32_t)e * a.magic_pw) >> 20);
+      const int c = e - r * a.stem_pw;
+      const int ih = ihb + r, iw = iwb + c;
+      const bool ok = (e < used) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+      stage[q] = __builtin_amdgcn_raw_buffer_load_b32(
+          xrsrc, ok ? (uint32_t)(((n * a.ih + ih) * a.iw + iw) * a.x_cs) : kOobOffset, 0, 0);
+    }
+  };
+  auto deposit = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < NLD; ++q) {
+      const int e = tid + q * 256;
+      const int r = (int)(((uint32_t)e * a.magic_pw) >> 20);
+      const int c = e - r * a.stem_pw;
+      if (e < used) patch[buf][r * kStemPW + c] = stage[q];
+    }
+  };
+
+  locate(tile);
+  fetch();
+  deposit(0);
+  __syncthreads();
+  int buf = 0;
+  for (;;) {
+    const int n_cur = n, oh_cur = oh, ow_cur = ow0;
+    const int next = tile + (int)gridDim.x;
+    const bool more = next < n_tiles;
+    if (more) {
+      locate(next);
+      fetch();
+    }
+    v16i acc[NI][NP];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int32_t *pb = &qlds[0][(ib + i) * 32 + fk * 16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i b = *reinterpret_cast<const v4i *>(pb + q * 4);
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+          acc[i][j][q * 4 + 0] = b[0]; acc[i][j][q * 4 + 1] = b[1];
+          acc[i][j][q * 4 + 2] = b[2]; acc[i][j][q * 4 + 3] = b[3];
+        }
+      }
+    }
+    const uint32_t *prow = &patch[buf][(pbase + frow) * a.sw + fk * 4];
+    const int pstep = 32 * a.sw;
+#pragma unroll
+    for (int r = 0; r < KH; ++r) {
+#pragma unroll
+      for (int j = 0; j < NP; ++j) {
+        const uint32_t *src = prow + r * kStemPW + j * pstep;
+        v4i b;
+        b[0] = (int)src[0]; b[1] = (int)src[1]; b[2] = (int)src[2]; b[3] = (int)src[3];
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[i][r], b, acc[i][j], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+      const int ow = ow_cur + pbase + j * 32 + frow;
+      const int pix = ow < a.ow ? (n_cur * a.oh + oh_cur) * a.ow + ow : a.npix;   // npix: nothing stored
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int oc = (ib + i) * 32 + fk * 16;
+        if (oc < a.ocw) {
+          const v16i one[1] = {acc[i][j]};
+          epilogue_rows<1, FAST>(one, a, oc, &qlds[1][oc], &qlds[2][oc], &qlds[3][oc], pix, 32, lut);
+        }
+      }
+    }
+    if (!more) break;
+    deposit(buf ^ 1);
+    __syncthreads();   // the next patch is complete; everyone is done reading this one
+    buf ^= 1;
+    tile = next;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // MFMA kernel without LDS: every wave owns a tile of TM*32 output channels x
 // TN*32 pixels and loads its MFMA operands straight from global memory in the
 // fragment layout (lane l: row l & 31, bytes 16*(l >> 5) .. +15 of a 32-byte K
@@ -1481,6 +1633,8 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.store_y = 1;
   a.magic_kw = (1u << 20) / (uint32_t)d.kw + 1;
   a.x_bytes = (uint32_t)((int64_t)d.n * d.ih * d.iw * d.x_cs);
+  a.stem_pw = 127 * d.sw + 8;
+  a.magic_pw = (1u << 20) / (uint32_t)a.stem_pw + 1;
   if (w->algo == ALGO_MFMA) {
     const TileCfg &t = kTiles[w->tile];
     a.magic_c16 = (1u << 20) / (uint32_t)w->c16 + 1;
@@ -1576,10 +1730,12 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     fill_args(ctx, w, x, y, &a);
     apply_fusion(&a, y, post);
     for (int i = 0; i < 2; ++i) launch_conv_mfma(ctx, w, a);
-    hipEventRecord(e0, ctx->stream);
+    hipError_t er = hipEventRecord(e0, ctx->stream);
     for (int i = 0; i < 5; ++i) launch_conv_mfma(ctx, w, a);
-    hipEventRecord(e1, ctx->stream);
-    const hipError_t es = hipEventSynchronize(e1), el = hipGetLastError();
+    if (er == hipSuccess) er = hipEventRecord(e1, ctx->stream);
+    hipError_t es = hipEventSynchronize(e1);
+    const hipError_t el = hipGetLastError();
+    if (es == hipSuccess) es = er;
     if (es != hipSuccess || el != hipSuccess) {
       // a variant that cannot be launched is skipped; the layer fails only if none can
       set_error(TPUHIP_ERR_HIP, "conv autotune: tile %s failed: %s", kTiles[t].name,
@@ -1588,14 +1744,14 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
       continue;
     }
     float ms = 0;
-    hipEventElapsedTime(&ms, e0, e1);
+    if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) continue;
     if (ms < best_ms) {
       best_ms = ms;
       best = t;
     }
   }
-  hipEventDestroy(e0);
-  hipEventDestroy(e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
   if (rc) return rc;
   if (best < 0) return TPUHIP_ERR_HIP;   // the last launch error is still the message
   if (best != w->tile) rc = pack_mfma_weights(ctx, w, best);
@@ -1630,8 +1786,15 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
     algo = ALGO_MFMA;
     TPUHIP_REQUIRE(forced_tile < kNumTiles, "conv: unknown MFMA tile %d", forced_tile);
   }
-  if (algo == ALGO_AUTO) algo = dense ? ALGO_MFMA : depthwise ? ALGO_DEPTHWISE : ALGO_DIRECT;
-  TPUHIP_REQUIRE(algo >= ALGO_DIRECT && algo <= ALGO_DEPTHWISE_DOT, "conv: unknown algo %d", d.algo);
+  // the stem kernel: one dword per pixel, the taps of a filter row side by side
+  const bool stem_ok = dense && d.ic <= 4 && d.dh == 1 && d.dw == 1 && d.kw <= 8 && d.kh <= 7 &&
+                       d.sw <= 2 && d.oc <= 64;
+  if (algo == ALGO_AUTO)
+    algo = stem_ok ? ALGO_STEM : dense ? ALGO_MFMA : depthwise ? ALGO_DEPTHWISE : ALGO_DIRECT;
+  TPUHIP_REQUIRE(algo >= ALGO_DIRECT && algo <= ALGO_STEM, "conv: unknown algo %d", d.algo);
+  TPUHIP_REQUIRE(algo != ALGO_STEM || stem_ok,
+                 "conv: the stem path needs g == 1, ic <= 4, oc <= 64, kh <= 7, kw <= 8, stride_w <= 2, "
+                 "no dilation, no inserted zeros");
   // the MFMA kernel locates a K group with multiply-shift divisions that are exact
   // for at most 4094 groups of at most 256 16-channel groups each
   const bool mfma_ok = dense && round_up(d.ic, 16) / 16 <= 256 &&
@@ -1677,6 +1840,25 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
           const int j = ch_in_block - 16 * (lane >> 5);
           if (ch < d.oc && j >= 0 && j < 16)
             packed[((size_t)(cb * taps + t) * 64 + lane) * 16 + j] = filter[(size_t)ch * taps + t];
+        }
+  } else if (algo == ALGO_STEM) {
+    // A fragments [32-channel block][filter row][lane][16 bytes]: lane l holds MFMA row l & 31
+    // (channel mfma_row_to_oc(row) of the block) and K bytes 16*(l >> 5) .. +15 of the
+    // 32-byte filter row, K byte = 4 * kw + channel
+    cw->ocp = round_up(d.oc, 16);
+    const int tm = d.oc <= 32 ? 1 : 2, khp = d.kh <= 3 ? 3 : 7;
+    packed.assign((size_t)tm * khp * 1024, 0);
+    for (int i = 0; i < tm; ++i)
+      for (int r = 0; r < d.kh; ++r)
+        for (int lane = 0; lane < 64; ++lane) {
+          const int oc = i * 32 + mfma_row_to_oc(lane & 31, 1);
+          if (oc >= d.oc) continue;
+          for (int j = 0; j < 16; ++j) {
+            const int kw = (lane >> 5) * 4 + j / 4, c = j % 4;
+            if (kw < d.kw && c < d.ic)
+              packed[((size_t)(i * khp + r) * 64 + lane) * 16 + j] =
+                  filter[(((size_t)oc * d.ic + c) * d.kh + r) * d.kw + kw];
+          }
         }
   } else if (algo == ALGO_DEPTHWISE_DOT) {
     // [tap group][channel][4 taps]: one dword per channel and group of four taps
@@ -1732,7 +1914,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   if (!rc) rc = tpuhip_malloc(ctx, qp.size() * sizeof(QParam), (void **)&cw->qp);
   if (!rc) rc = tpuhip_upload(ctx, cw->bias, b32.data(), b32.size() * sizeof(int32_t));
   if (!rc) rc = tpuhip_upload(ctx, cw->qp, qp.data(), qp.size() * sizeof(QParam));
-  if (!rc && (algo == ALGO_MFMA || algo == ALGO_DEPTHWISE || algo == ALGO_DEPTHWISE_DOT)) {
+  if (!rc && algo != ALGO_DIRECT) {
     std::vector<int32_t> planes(3 * nparam);
     for (size_t i = 0; i < nparam; ++i) {
       planes[i] = qp[i].mult;
@@ -1772,6 +1954,7 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
     case ALGO_DIRECT: return "direct";
     case ALGO_DEPTHWISE: return "depthwise";
     case ALGO_DEPTHWISE_DOT: return "depthwise_dot";
+    case ALGO_STEM: return "stem";
     case ALGO_MFMA: return kTiles[w->tile].name;
   }
   return "?";
@@ -1795,6 +1978,7 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     if (rc) return rc;
   }
   TPUHIP_REQUIRE(!post.lut || w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT ||
+                     w->algo == ALGO_STEM ||
                      (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
                  "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
   ConvArgs a;
@@ -1818,6 +2002,22 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
       if (regw) launch(ctx, (conv_depthwise_mfma_kernel<false, true>), grid, block, a);
       else launch(ctx, (conv_depthwise_mfma_kernel<false, false>), grid, block, a);
     }
+  } else if (w->algo == ALGO_STEM) {
+    // one workgroup per resident slot (3 per CU), each walking (image, output row, 128-pixel
+    // segment) tiles
+    const int64_t tiles = (int64_t)a.n * a.oh * ((a.ow + 127) / 128);
+    const bool k3 = a.kh <= 3, one = a.oc <= 32;
+    const dim3 grid((unsigned)std::min<int64_t>(tiles, (int64_t)ctx->num_cu * 3)), block(256);
+#define STEM(KH, TM)                                                                   \
+  do {                                                                                 \
+    if (w->fast) launch(ctx, (conv_stem_kernel<KH, TM, true>), grid, block, a);        \
+    else launch(ctx, (conv_stem_kernel<KH, TM, false>), grid, block, a);               \
+  } while (0)
+    if (k3 && one) STEM(3, 1);
+    else if (k3) STEM(3, 2);
+    else if (one) STEM(7, 1);
+    else STEM(7, 2);
+#undef STEM
   } else if (w->algo == ALGO_DEPTHWISE_DOT) {
     // as many workgroups as are resident at once (3 per CU at this register count): every
     // lane then walks pixels and its filter / parameter loads are paid once (measured best)
@@ -1874,8 +2074,9 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
   TPUHIP_REQUIRE(ctx && w && x && post, "tpuhip_conv2d_post_i8: NULL argument");
   PostOps p;
   if (post->lut) {
-    TPUHIP_REQUIRE(w->algo == ALGO_MFMA || w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT,
-                   "conv2d_post: only dense convs on the MFMA path and depthwise convs can fuse a table");
+    TPUHIP_REQUIRE(w->algo == ALGO_MFMA || w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT ||
+                       w->algo == ALGO_STEM,
+                   "conv2d_post: only dense convs on the MFMA or stem path and depthwise convs can fuse a table");
     p.lut = post->lut;
     p.lut_out = post->lut_out;
   }

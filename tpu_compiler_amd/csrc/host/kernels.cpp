@@ -423,7 +423,8 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
 
 bool Conv2DOpKernel::can_fuse_lut() const {
   const std::string algo = tpuhip_conv2d_algo_name(packed);
-  return (algo.rfind("mfma", 0) == 0 || algo == "depthwise") && !lut_dst && !fused.enable;
+  return (algo.rfind("mfma", 0) == 0 || algo.rfind("depthwise", 0) == 0 || algo == "stem") && !lut_dst &&
+         !fused.enable;
 }
 
 void Conv2DOpKernel::fuse_lut(const int8_t *table, SyncedData dst) {
