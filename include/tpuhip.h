@@ -421,6 +421,45 @@ int tpuhip_npz_add_f32(tpuhip_npz *f, const char *name, const float *data, const
 int tpuhip_npz_delete(tpuhip_npz *f, const char *name);
 int tpuhip_npz_keep(tpuhip_npz *f);
 
+/* ---- INT8 quantisation arithmetic (host only, no GPU) ---------------------- */
+
+/* Replace the helpers the reference's --tpu-quant pass uses to turn fp32 weights and two
+ * calibration thresholds into the float-stored integer operands of the INT8 kernels
+ * (lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp; drivers in QuantizeInt8.cpp).
+ * threshold_x / threshold_y: calibration thresholds of the op's input / output. */
+
+/* QuantizeMultiplier (:182-220): multiplier = quantized * 2^(shift - 31), quantized in [2^30, 2^31) or 0 */
+int tpuhip_quantize_multiplier(double multiplier, int32_t *quantized, int *shift);
+/* findRShiftAndMultiplierFromQScale (:237-289); qdm != 0: the 32-bit form conv and FC use;
+ * else the 8-bit form with max_multiplier (127 in the reference's callers) */
+int tpuhip_find_rshift_and_multiplier(double qscale, int qdm, uint32_t max_multiplier, int *rshift,
+                                      uint32_t *multiplier);
+/* quantizeWeightInt8Multiplier (:741-818) as quantizeInt8ConvOps calls it (QuantizeInt8.cpp:56-166):
+ * filter oc x isz, bias oc or NULL, filter_threshold oc or NULL; outputs float-stored integers:
+ * new_filter (int8), new_bias (int32), rshift and multiplier per output channel */
+int tpuhip_quantize_conv_weights(const float *filter, const float *bias, int64_t oc, int64_t isz,
+                                 float threshold_y, float threshold_x, const float *filter_threshold,
+                                 float *new_filter, float *new_bias, float *rshift, float *multiplier);
+/* quantizeWeightInt8ForFC (:630-690): filter batch x n x k, bias batch x n or NULL, one rshift and
+ * multiplier per batch */
+int tpuhip_quantize_fc_weights(const float *filter, const float *bias, int64_t batch, int64_t n, int64_t k,
+                               float threshold_y, float threshold_x, float *new_filter, float *new_bias,
+                               float *rshift, float *multiplier);
+/* quantizeInt8RescaleNoWeightOps (QuantizeInt8.cpp:669-854): one rshift and one int8 multiplier per
+ * input for eltwise add / max / min and average pooling.  coeff: NULL or one factor per input;
+ * divisor: kh * kw of an average pool, else 1 */
+int tpuhip_quantize_rescale(const float *threshold_x, int n_inputs, float threshold_y, const float *coeff,
+                            int divisor, float *rshift, float *multiplier);
+/* quantizeInt8LeakyReluOps (QuantizeInt8.cpp:349-429): out4 = rshift_pos, multiplier_pos, rshift_neg,
+ * multiplier_neg */
+int tpuhip_quantize_leaky_relu(float negative_slope, float threshold_x, float threshold_y, float *out4);
+/* quantizeInt8LutOps (QuantizeInt8.cpp:531-621): the 256-entry table, indexed by the two's-complement
+ * byte of the input.  kind: 0 sigmoid, 1 tanh, 2 exp, 3 elu, 4 swish, 5 softplus, 6 log, 7 pow;
+ * scale / bias: the op attributes of sigmoid, exp, softplus (1, 0 if none); coeff: pow's exponent.
+ * Entries the reference leaves as NaN (log of a negative input) are NaN here too. */
+int tpuhip_quantize_lut_table(int kind, float threshold_x, float threshold_y, float scale, float bias,
+                              float coeff, float *table256);
+
 #ifdef __cplusplus
 }
 #endif

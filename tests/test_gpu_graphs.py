@@ -524,3 +524,78 @@ def test_graph_with_fp32_edges_quantizes_and_dequantizes_like_the_oracle(tmp_pat
     g2.add(graphs.Op("tpu.relu", "r", ["input"], (1, 16, 4, 4)))
     with pytest.raises(capi.TpuHipError, match="QuantOp in front"):
         module().load(g2)
+
+
+def test_fp32_network_quantized_with_the_host_helpers_tracks_the_fp32_result(tmp_path):
+    """an fp32 network (torch) + max-abs calibration thresholds -> INT8 operands from the
+    quantisation helpers -> the GPU graph.  Bit-exact against the oracle as always, and close to
+    the fp32 network layer by layer, which is what those helpers are for."""
+    import torch
+    import torch.nn.functional as F
+    from tpu_compiler_amd import quantize as Q
+    torch.manual_seed(3)
+    rng = np.random.default_rng(3)
+    n, hw = 4, 20
+    x = torch.tensor(rng.normal(0, 1, (n, 3, hw, hw)).astype(np.float32)).clamp(-3, 3)
+    w1, b1 = torch.randn(16, 3, 3, 3) * 0.3, torch.randn(16) * 0.2
+    w2, b2 = torch.randn(16, 16, 3, 3) * 0.1, torch.randn(16) * 0.2
+    w3, b3 = torch.randn(24, 16, 1, 1) * 0.3, torch.randn(24) * 0.1
+    wf, bf = torch.randn(10, 24) * 0.4, torch.randn(10) * 0.1
+    a1 = F.relu(F.conv2d(x, w1, b1, padding=1))
+    a2 = F.conv2d(a1, w2, b2, padding=1)
+    a3 = F.relu(a1 + a2)
+    a4 = F.conv2d(a3, w3, b3)
+    a5 = F.leaky_relu(a4, 0.1)
+    a6 = a5.mean(dim=(2, 3), keepdim=True)
+    a7 = F.linear(a6.flatten(1), wf, bf)
+    acts = dict(input=x, c1=a1, c2=a2, add=a3, c3=a4, leaky=a5, gap=a6, fc=a7)
+    thr = {k: float(v.abs().max()) for k, v in acts.items()}
+
+    g = graphs.Graph("quantized", 0)
+    xin = g.add(graphs.Op("tpu.input", "input", [], (n, 3, hw, hw)))
+    xin.data = np.clip(np.floor(x.numpy() * (127.0 / thr["input"]) + 0.5), -128, 127).astype(np.int8)
+
+    def conv(name, src, w, b, tx, ty, k, pad, relu):
+        wq, bq, rs, mu = Q.quantize_conv(w.numpy(), b.numpy(), tx, ty)
+        oc = w.shape[0]
+        g.add(graphs.Op("tpu.conv_2d", name, [src], (n, oc, hw, hw),
+                        dict(kernel_h=k, kernel_w=k, stride_h=1, stride_w=1, dilation_h=1, dilation_w=1,
+                             padding_t=pad, padding_b=pad, padding_l=pad, padding_r=pad, group=1, do_relu=int(relu),
+                             with_bias=1),
+                        dict(filter=wq, bias=bq, rshift=rs, multiplier=mu), "RSHIFT_AND_M_I32"))
+
+    conv("c1", "input", w1, b1, thr["input"], thr["c1"], 3, 1, True)
+    conv("c2", "c1", w2, b2, thr["c1"], thr["c2"], 3, 1, False)
+    rs, mu = Q.quantize_rescale([thr["c1"], thr["c2"]], thr["add"])
+    g.add(graphs.Op("tpu.eltwise_add", "add", ["c1", "c2"], (n, 16, hw, hw), dict(do_relu=1),
+                    dict(rshift=rs, multiplier=mu), "RSHIFT_AND_M_I8"))
+    conv("c3", "add", w3, b3, thr["add"], thr["c3"], 1, 0, False)
+    g.add(graphs.Op("tpu.leaky_relu", "leaky", ["c3"], (n, 24, hw, hw), dict(negative_slope=0.1),
+                    Q.quantize_leaky_relu(0.1, thr["c3"], thr["leaky"]), "RSHIFT_AND_M_I8"))
+    rs, mu = Q.quantize_rescale([thr["leaky"]], thr["gap"], divisor=hw * hw)
+    g.add(graphs.Op("tpu.pool_avg_2d", "gap", ["leaky"], (n, 24, 1, 1),
+                    dict(kernel_h=hw, kernel_w=hw, stride_h=1, stride_w=1, padding_t=0, padding_b=0, padding_l=0,
+                         padding_r=0, do_relu=0, count_include_pad=1, pad_value=0),
+                    dict(rshift=rs, multiplier=mu), "RSHIFT_AND_M_I8"))
+    g.add(graphs.Op("tpu.reshape", "flat", ["gap"], (n, 24)))
+    wq, bq, rs, mu = Q.quantize_fc(wf.numpy(), bf.numpy(), thr["gap"], thr["fc"])
+    g.add(graphs.Op("tpu.fully_connected", "fc", ["flat"], (n, 10), dict(do_relu=0),
+                    dict(filter=wq, bias=bq, rshift=rs, multiplier=mu), "RSHIFT_AND_M_I32"))
+    g.outputs = ["fc"]
+
+    want = oracle_graph.run(g)
+    m = module()
+    m.load(g)
+    m.set_tensor("input", xin.data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        got = m.get_tensor_i8(op.name)
+        assert np.array_equal(got, want[op.name].reshape(op.shape)), op.name
+        if op.name in acts and op.name != "input":
+            ref = acts[op.name].numpy().reshape(op.shape)
+            deq = got.astype(np.float64) * thr[op.name] / 127.0
+            cos = (deq * ref).sum() / np.sqrt((deq * deq).sum() * (ref * ref).sum())
+            assert cos > 0.995, (op.name, cos)
+            assert np.abs(deq - ref).max() < 0.06 * thr[op.name], (op.name, np.abs(deq - ref).max() / thr[op.name])
+    m.close()
+    check_through_files(g, xin.data, want, tmp_path)

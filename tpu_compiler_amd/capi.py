@@ -172,6 +172,20 @@ PROTOTYPES.update({
     "tpuhip_npz_add_f32": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int]),
     "tpuhip_npz_delete": (C.c_int, [C.c_void_p, C.c_char_p]),
     "tpuhip_npz_keep": (C.c_int, [C.c_void_p]),
+    "tpuhip_quantize_multiplier": (C.c_int, [C.c_double, C.POINTER(C.c_int32), C.POINTER(C.c_int)]),
+    "tpuhip_find_rshift_and_multiplier": (C.c_int, [C.c_double, C.c_int, C.c_uint32, C.POINTER(C.c_int),
+                                                    C.POINTER(C.c_uint32)]),
+    "tpuhip_quantize_conv_weights": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_float,
+                                               C.c_float, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                               C.c_void_p]),
+    "tpuhip_quantize_fc_weights": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64,
+                                             C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.c_void_p]),
+    "tpuhip_quantize_rescale": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_void_p,
+                                          C.c_void_p]),
+    "tpuhip_quantize_leaky_relu": (C.c_int, [C.c_float, C.c_float, C.c_float, C.c_void_p]),
+    "tpuhip_quantize_lut_table": (C.c_int, [C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
+                                            C.c_void_p]),
 })
 
 
