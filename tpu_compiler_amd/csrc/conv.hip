@@ -934,8 +934,12 @@ conv_stem_kernel(ConvArgs a) {
   const int n_tiles = a.n * a.oh * nseg;
   const int used = a.kh * a.stem_pw;   // dwords of a patch that are read
 
-  int tile = blockIdx.x;
-  if (tile >= n_tiles) return;         // whole workgroup, before any barrier
+  // workgroups are dealt to the 8 XCDs round-robin; each XCD takes a contiguous run of tiles
+  // (consecutive output rows), so the input rows neighbouring tiles share meet in its L2
+  const int per_xcd = (n_tiles + 7) >> 3, wg_stride = (int)(gridDim.x >> 3);
+  const int tile_end = min(n_tiles, ((int)(blockIdx.x & 7) + 1) * per_xcd);
+  int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+  if (tile >= tile_end) return;        // whole workgroup, before any barrier
   int n, oh, ow0;
   auto locate = [&](int t) {
     const int seg = t % nseg, r = t / nseg;
@@ -974,8 +978,8 @@ conv_stem_kernel(ConvArgs a) {
   int buf = 0;
   for (;;) {
     const int n_cur = n, oh_cur = oh, ow_cur = ow0;
-    const int next = tile + (int)gridDim.x;
-    const bool more = next < n_tiles;
+    const int next = tile + wg_stride;
+    const bool more = next < tile_end;
     if (more) {
       locate(next);
       fetch();
@@ -2007,7 +2011,8 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     // segment) tiles
     const int64_t tiles = (int64_t)a.n * a.oh * ((a.ow + 127) / 128);
     const bool k3 = a.kh <= 3, one = a.oc <= 32;
-    const dim3 grid((unsigned)std::min<int64_t>(tiles, (int64_t)ctx->num_cu * 3)), block(256);
+    const int64_t per_xcd = (tiles + 7) / 8;
+    const dim3 grid((unsigned)(8 * std::min<int64_t>(per_xcd, std::max(1, ctx->num_cu * 3 / 8)))), block(256);
 #define STEM(KH, TM)                                                                   \
   do {                                                                                 \
     if (w->fast) launch(ctx, (conv_stem_kernel<KH, TM, true>), grid, block, a);        \
