@@ -198,3 +198,43 @@ def test_emitted_text_reads_back_as_the_same_graph(tmp_path):
                 key = "%s_%s" % (op.name, role)
                 if key in z.files:
                     assert z[key].dtype == np.float32 and np.array_equal(z[key], arr.astype(np.float32))
+
+
+def test_damaged_files_raise_errors_and_never_crash(tmp_path):
+    """truncated and bit-flipped archives / texts either load or are refused with an error"""
+    rng = np.random.default_rng(11)
+    good = tmp_path / "good.npz"
+    np.savez(good, a=np.arange(40, dtype=np.float32).reshape(5, 8), b=np.ones((3, 3), np.float32))
+    blob = good.read_bytes()
+    outcomes = {"ok": 0, "refused": 0}
+    for trial in range(300):
+        data = bytearray(blob)
+        if trial % 3 == 0:
+            data = data[:int(rng.integers(0, len(data)))]
+        else:
+            for _ in range(int(rng.integers(1, 4))):
+                data[int(rng.integers(0, len(data)))] = int(rng.integers(0, 256))
+        p = tmp_path / "damaged.npz"
+        p.write_bytes(bytes(data))
+        try:
+            f = capi.TensorFile(p)
+            for name in f.names():
+                try:
+                    f.read(name)
+                except capi.TpuHipError:
+                    pass
+            f.close()
+            outcomes["ok"] += 1
+        except capi.TpuHipError:
+            outcomes["refused"] += 1
+    assert outcomes["refused"] > 50 and outcomes["ok"] > 10
+    text = HAND_WRITTEN
+    refused = 0
+    for trial in range(200):
+        cut = int(rng.integers(0, len(text)))
+        t = text[:cut] if trial % 2 == 0 else text[:cut] + "@#}{" + text[cut + 3:]
+        try:
+            _describe(tmp_path, t, "damaged.mlir")
+        except capi.TpuHipError:
+            refused += 1
+    assert refused > 150

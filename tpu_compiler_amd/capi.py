@@ -206,7 +206,7 @@ def bind(lib=None, prototypes=None):
 
 def check(lib, status):
     if status != 0:
-        raise TpuHipError(status, lib.tpuhip_last_error().decode())
+        raise TpuHipError(status, lib.tpuhip_last_error().decode("utf-8", "replace"))
 
 
 def mlir_describe(path, lib=None):
@@ -236,27 +236,29 @@ class TensorFile:
             self.h = None
 
     def names(self):
-        return [self.lib.tpuhip_npz_name(self.h, i).decode() for i in range(self.lib.tpuhip_npz_count(self.h))]
+        # member names are bytes in the archive: anything that is not UTF-8 survives the round trip
+        return [self.lib.tpuhip_npz_name(self.h, i).decode("utf-8", "surrogateescape")
+                for i in range(self.lib.tpuhip_npz_count(self.h))]
 
     def info(self, name):
         dims, nd, kind, ws = (C.c_int64 * 8)(), C.c_int(0), C.c_char(b"?"), C.c_int(0)
-        check(self.lib, self.lib.tpuhip_npz_info(self.h, name.encode(), dims, C.byref(nd), C.byref(kind),
+        check(self.lib, self.lib.tpuhip_npz_info(self.h, name.encode("utf-8", "surrogateescape"), dims, C.byref(nd), C.byref(kind),
                                                  C.byref(ws)))
         return tuple(dims[i] for i in range(nd.value)), kind.value.decode(), ws.value
 
     def read(self, name):
         shape, _, _ = self.info(name)
         out = np.empty(shape, np.float32)
-        check(self.lib, self.lib.tpuhip_npz_read_f32(self.h, name.encode(), out.ctypes.data, out.size))
+        check(self.lib, self.lib.tpuhip_npz_read_f32(self.h, name.encode("utf-8", "surrogateescape"), out.ctypes.data, out.size))
         return out
 
     def add(self, name, array):
         a = np.asarray(array, dtype=np.float32, order="C")    # keeps a 0-d array 0-d
         dims = (C.c_int64 * max(a.ndim, 1))(*a.shape)
-        check(self.lib, self.lib.tpuhip_npz_add_f32(self.h, name.encode(), a.ctypes.data, dims, a.ndim))
+        check(self.lib, self.lib.tpuhip_npz_add_f32(self.h, name.encode("utf-8", "surrogateescape"), a.ctypes.data, dims, a.ndim))
 
     def delete(self, name):
-        check(self.lib, self.lib.tpuhip_npz_delete(self.h, name.encode()))
+        check(self.lib, self.lib.tpuhip_npz_delete(self.h, name.encode("utf-8", "surrogateescape")))
 
     def keep(self):
         check(self.lib, self.lib.tpuhip_npz_keep(self.h))
