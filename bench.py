@@ -72,7 +72,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (--gpus %d refused); the path shards "
-                 "by batch with no exchange step, see DESIGN.md" % args.gpus)
+                 "by batch with no exchange step between GPUs" % args.gpus)
 
     import numpy as np
     from tpu_compiler_amd import graphs, module
@@ -140,15 +140,18 @@ def main():
     # per-kernel times, HIP events on the stream the kernels run on
     rows = m.time_kernels(iters=max(5, min(args.steps, 20)))
     by_algo = {}
+    algo_of = {name: algo for name, algo, _ in rows}
     for name, algo, ms in rows:
         op = g.by_name[name]
         if op.type in ("tpu.conv_2d", "tpu.fully_connected"):
-            key = algo if algo != "fc" else "fc"
+            # a conv that runs inside the launch of another ("with <name>") counts towards that launch
+            rides = algo.startswith("with ")
+            key = algo_of[algo[5:]] if rides else algo
             d = by_algo.setdefault(key, {"ms": 0.0, "ops": 0.0, "bytes": 0.0, "launches": 0})
             d["ms"] += ms
             d["ops"] += 2.0 * op.macs
-            d["bytes"] += conv_bytes(op, g)
-            d["launches"] += 1
+            d["bytes"] += conv_bytes(op, g) - (int(np.prod(g.by_name[op.inputs[0]].shape)) if rides else 0)
+            d["launches"] += 0 if rides else 1
     mfma = {k: v for k, v in by_algo.items() if k.startswith("mfma")}
     conv_ms = sum(v["ms"] for v in mfma.values())
     conv_ops = sum(v["ops"] for v in mfma.values())

@@ -164,6 +164,18 @@ typedef struct tpuhip_conv_post {
 } tpuhip_conv_post;
 int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                           const tpuhip_conv_post *post);
+/* Two Conv2DOpKernel::invoke calls as one launch: two dense convs that read the same input
+ * through the same window geometry (kernel, stride, padding, dilation), e.g. the projection
+ * shortcut and the first 1x1 conv of a residual block.  Their filters are stacked along the
+ * output channels; every output tile goes to the result it belongs to, with that conv's own
+ * channel stride and ReLU.  The first conv needs a multiple of 16 output channels.  Results are
+ * those of two tpuhip_conv2d_i8 calls.  No counterpart in the reference (one kernel per op). */
+int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b,
+                               const int8_t *filter_a, const int32_t *bias_a, const int32_t *multiplier_a,
+                               const int32_t *rshift_a, const int8_t *filter_b, const int32_t *bias_b,
+                               const int32_t *multiplier_b, const int32_t *rshift_b,
+                               tpuhip_conv_weights **out);
+int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y_a, void *y_b);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */
@@ -346,7 +358,8 @@ int tpuhip_module_set_returns(tpuhip_module *m, const char *const *names, int n)
 /* Options read at the next tpuhip_module_load: "fuse_eltwise" (default 1: an EltwiseAdd of a conv
  * result runs in that conv's epilogue), "keep_all_tensors" (default 1: every tensor can be read back
  * after an invoke, as with the reference's get_all_tensor; 0: the result of a conv whose only reader
- * is the add fused into it is never written, and reading it back is an error). */
+ * is the add fused into it is never written, and reading it back is an error), "pair_convs"
+ * (default 1: two convs over the same input with the same window geometry run as one launch). */
 int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value);
 int tpuhip_module_load(tpuhip_module *m, const char *target_op);
 /* setTensor / getTensor (:407-430) */

@@ -193,6 +193,19 @@ public:
   // interpreter when nothing else reads it and the caller asked for outputs only)
   void set_store_result(bool store);
   SyncedData result() const { return output_data; }
+  SyncedData input() const { return input_data; }
+  // Two convs that read the same tensor through the same window geometry can run as one launch
+  // with their filters stacked along the output channels (the input is read once, one launch
+  // less).  pair_with packs that and makes `second` a no-op; results are unchanged.  Only the
+  // module interpreter arranges this.
+  bool can_pair_with(const Conv2DOpKernel &second) const;
+  void pair_with(Conv2DOpKernel &second);
+  bool is_paired_first() const { return pair_packed != nullptr; }
+  bool is_paired_second() const { return paired_into != nullptr; }
+  const Conv2DOpKernel *paired_first() const { return paired_into; }
+  // host copies of the integer operands are kept until the interpreter has decided about
+  // pairing; release_host_weights drops them
+  void release_host_weights();
 
 protected:
   // transposed: the attributes describe a DeConv2D; it runs as a stride-1 conv over the
@@ -208,6 +221,13 @@ private:
   SyncedData lut_dst;
   int8_t lut_table[256];
   bool store_lut = true;
+  bool plain = false;                      // an ordinary dense conv (not transposed)
+  std::vector<int8_t> host_w;
+  std::vector<int32_t> host_b, host_m, host_r;
+  tpuhip_conv_weights *pair_packed = nullptr;
+  Conv2DOpKernel *pair_second = nullptr;   // runs inside this kernel's launch
+  Conv2DOpKernel *paired_into = nullptr;   // this kernel's work is done by that one
+  std::string algo_text;
 };
 
 // core/deconv.cpp:7-73, same operands and epilogue as Conv2D
@@ -500,6 +520,9 @@ public:
   tpuhip_ctx *context() const { return ctx_; }
   // conv + eltwise-add fusion (on by default; TPUHIP_FUSE=0 disables); applies at the next loadModule
   bool fuse_eltwise = true;
+  // convs over the same input with the same geometry run as one launch (on by default;
+  // TPUHIP_PAIR=0 disables); applies at the next loadModule
+  bool pair_convs = true;
   // true (default): every tensor of the graph can be read back after an invoke, like the
   // reference.  false: the result of a conv whose only reader is the add fused into it is
   // never written (reading it back is an error); applies at the next loadModule
@@ -515,6 +538,7 @@ private:
   void updateKernelList(ModuleDesc &module, std::string &target_op);
   bool isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op);
   void fuseKernels();
+  void pairConvs();
   tpuhip_ctx *ctx_ = nullptr;
   kernel_map_t kernel_map_;
   kernel_list_t kernel_list_;

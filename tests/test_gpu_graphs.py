@@ -188,6 +188,39 @@ def test_fusion_on_and_off_give_the_same_tensors(monkeypatch):
         m.close()
 
 
+def test_sibling_convs_run_as_one_launch_with_unchanged_results():
+    """the projection shortcut and the first 1x1 conv of a downsampling block read the same tensor
+    through the same window: one launch serves both.  On, off, reloaded and stopped half way, every
+    tensor equals the oracle's."""
+    g = graphs.cfg3_resnet50(batch=2, hw=96)
+    want = oracle_graph.run(g)
+    pairs = [("res%da_branch1" % s, "res%da_branch2a" % s) for s in (2, 3, 4, 5)]
+    for on in (1, 0):
+        m = module()
+        m.set_option("pair_convs", on)
+        m.load(g)
+        algo = dict(m.kernels())
+        for first, second in pairs:
+            assert algo[first].startswith("mfma")
+            assert algo[second] == ("with " + first if on else algo[second]) and (on or algo[second].startswith("mfma"))
+        times = {name: ms for name, _, ms in m.time_kernels(iters=2)}
+        if on:
+            assert all(times[second] == 0 and times[first] > 0 for first, second in pairs)
+        m.set_tensor("input", g.input_op().data.astype(np.float32))
+        m.invoke()
+        for op in g.ops:
+            assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), (on, op.name)
+        if on:
+            # a reload keeps the pairing; stopping at the second conv of a pair still produces it
+            m.load(g)
+            assert dict(m.kernels())["res3a_branch2a"] == "with res3a_branch1"
+            m.set_tensor("input", g.input_op().data.astype(np.float32))
+            m.invoke_to("res3a_branch2a")
+            assert np.array_equal(m.get_tensor_i8("res3a_branch2a"),
+                                  want["res3a_branch2a"].reshape(g.by_name["res3a_branch2a"].shape))
+        m.close()
+
+
 @pytest.mark.parametrize("builder,kw", [(graphs.cfg5_yolo_v3, dict(batch=1, hw=96)),
                                         (graphs.cfg4_mobilenet_v2, dict(batch=2, hw=64)),
                                         (graphs.cfg2_mobilenet_block, dict(batch=1))])

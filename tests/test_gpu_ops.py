@@ -140,6 +140,70 @@ def test_conv_stem_general_requant_fused_table_and_limits(ctx):
             ctx.conv_prepack(dd, ww, z, z + (1 << 30), z + 1)
 
 
+# n, ic, ih, iw, oc_a, oc_b, k, stride, pads, relu_a, relu_b, bias_b
+PAIR_CASES = [
+    (2, 64, 14, 14, 256, 64, 1, (1, 1), (0, 0, 0, 0), False, True, True),     # shortcut + first 1x1 of a block
+    (3, 256, 15, 13, 512, 128, 1, (2, 2), (0, 0, 0, 0), False, True, True),   # the strided pair
+    (1, 40, 9, 11, 48, 24, 3, (1, 1), (1, 1, 1, 1), True, False, False),      # ragged second half, 3x3
+    (16, 32, 28, 28, 64, 40, 1, (1, 1), (0, 0, 0, 0), True, True, True),      # enough pixels to walk tiles
+]
+
+
+@pytest.mark.parametrize("case", PAIR_CASES)
+def test_conv_pair_equals_two_convs(ctx, case):
+    n, ic, ih, iw, oca, ocb, k, stride, pads, relu_a, relu_b, bias_b = case
+    rng = np.random.default_rng(oca * 7 + ocb + ic)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    wa, wb = rnd_w(rng, (oca, ic, k, k)), rnd_w(rng, (ocb, ic, k, k))
+    ba, ra, ma = rnd_params(rng, oca)
+    bb, rb, mb = rnd_params(rng, ocb, 6, 14)
+    want_a = oracle_conv(x, wa, ba, ra, ma, 1, stride, pads, (1, 1), (0, 0), relu_a)
+    want_b = oracle_conv(x, wb, bb if bias_b else np.zeros_like(bb), rb, mb, 1, stride, pads, (1, 1), (0, 0), relu_b)
+    da = conv_desc(x.shape, wa.shape, stride=stride, pads=pads, do_relu=relu_a)
+    db = conv_desc(x.shape, wb.shape, stride=stride, pads=pads, do_relu=relu_b, with_bias=bias_b)
+    wh = ctx.conv_prepack_pair(da, db, (wa, f2i32(ba), f2i32(ma), f2i32(ra)),
+                               (wb, f2i32(bb) if bias_b else None, f2i32(mb), f2i32(rb)))
+    xt, ya, yb = ctx.from_nchw(x), ctx.tensor(want_a.shape), ctx.tensor(want_b.shape)
+    for t in (ya, yb):
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, t.ptr, 0x55, t.nbytes))      # poison: pads must be rewritten
+    ctx.conv_pair(wh, xt, ya, yb)
+    assert ctx.conv_algo_name(wh).startswith("mfma")
+    assert np.array_equal(ctx.to_nchw(ya), want_a), "%d mismatches in a" % (ctx.to_nchw(ya) != want_a).sum()
+    assert np.array_equal(ctx.to_nchw(yb), want_b), "%d mismatches in b" % (ctx.to_nchw(yb) != want_b).sum()
+    assert not ctx.raw(yb)[..., ocb:].any() and not ctx.raw(ya)[..., oca:].any()
+    assert len(np.unique(want_a)) > 8 and len(np.unique(want_b)) > 8
+    # every tile variant splits its output the same way
+    for tile in range(NUM_TILES):
+        da.algo = db.algo = 16 + tile
+        wt = ctx.conv_prepack_pair(da, db, (wa, f2i32(ba), f2i32(ma), f2i32(ra)),
+                                   (wb, f2i32(bb) if bias_b else None, f2i32(mb), f2i32(rb)))
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, ya.ptr, 0x55, ya.nbytes))
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yb.ptr, 0x55, yb.nbytes))
+        ctx.conv_pair(wt, xt, ya, yb)
+        name = ctx.conv_algo_name(wt)
+        assert np.array_equal(ctx.to_nchw(ya), want_a) and np.array_equal(ctx.to_nchw(yb), want_b), name
+        ctx.conv_weights_destroy(wt)
+    # a pair handle does not run as a single conv, nor a single conv as a pair
+    with pytest.raises(capi.TpuHipError, match="pair"):
+        ctx.conv(wh, xt, ya)
+    ctx.conv_weights_destroy(wh)
+
+
+def test_conv_pair_refuses_mismatched_convs(ctx):
+    x_shape = (1, 32, 8, 8)
+    z = lambda oc: (np.zeros((oc, 32, 1, 1), np.int8), None, np.full(oc, 1 << 30, np.int32), np.ones(oc, np.int32))
+    da = conv_desc(x_shape, (64, 32, 1, 1))
+    with pytest.raises(capi.TpuHipError, match="same window geometry"):
+        ctx.conv_prepack_pair(da, conv_desc(x_shape, (16, 32, 1, 1), stride=(2, 2)), z(64), z(16))
+    with pytest.raises(capi.TpuHipError, match="multiple of 16"):
+        ctx.conv_prepack_pair(conv_desc(x_shape, (24, 32, 1, 1)), conv_desc(x_shape, (16, 32, 1, 1)), z(24), z(16))
+    w = ctx.conv_prepack(da, *[z(64)[i] for i in (0, 1, 2, 3)])
+    xt, ya = ctx.tensor(x_shape), ctx.tensor((1, 64, 8, 8))
+    with pytest.raises(capi.TpuHipError, match="not packed as a pair"):
+        ctx.conv_pair(w, xt, ya, ya)
+    ctx.conv_weights_destroy(w)
+
+
 TILE_CASES = [
     (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True),
     (2, 96, 17, 13, 200, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), False),   # ragged pixel / channel tails

@@ -50,7 +50,7 @@ def structured_i32():
     return sorted(vals)
 
 
-def test_srdhm_survey_examples():
+def test_srdhm_worked_examples():
     # ties go toward +inf: -1 * 2^30 / 2^31 = -0.5 -> 0 ; -3 -> -1.5 -> -1 ; 1 -> 0.5 -> 1
     assert O.lib.orc_srdhm(-1, 1 << 30) == 0
     assert O.lib.orc_srdhm(-3, 1 << 30) == -1
@@ -81,7 +81,7 @@ def test_srdhm_identity_multiplier_2_30_is_half_round_up():
         assert O.lib.orc_srdhm(v, 1 << 30) == (v + 1) // 2
 
 
-def test_rdbp_survey_examples():
+def test_rdbp_worked_examples():
     assert O.lib.orc_rdbp(-1, 1) == -1
     assert O.lib.orc_rdbp(1, 1) == 1
     assert O.lib.orc_rdbp(-3, 1) == -2

@@ -154,6 +154,10 @@ PROTOTYPES.update({
                                              C.c_int]),
     "tpuhip_module_ctx": (C.c_void_p, [C.c_void_p]),
     "tpuhip_module_set_option": (C.c_int, [C.c_void_p, C.c_char_p, C.c_int]),
+    "tpuhip_conv2d_prepack_pair": (C.c_int, [C.c_void_p, C.POINTER(ConvDesc), C.POINTER(ConvDesc), C.c_void_p,
+                                             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                             C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "tpuhip_conv2d_pair_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
     "tpuhip_module_weight_file": (C.c_char_p, [C.c_void_p]),
     "tpuhip_module_num_ops": (C.c_int, [C.c_void_p]),
@@ -387,6 +391,24 @@ class Context:
             self.h, C.byref(desc), filt.ctypes.data, None if b is None else b.ctypes.data,
             mult.ctypes.data, rshift.ctypes.data, C.byref(w)))
         return w.value
+
+    def conv_prepack_pair(self, desc_a, desc_b, a, b):
+        """a, b: (filter int8, bias int32 or None, multiplier int32, rshift int32) of two convs over
+        the same input with the same window geometry -> one handle for conv_pair"""
+        keep, ptrs = [], []
+        for filt, bias, mult, rshift in (a, b):
+            arrs = [np.ascontiguousarray(filt, dtype=np.int8),
+                    None if bias is None else np.ascontiguousarray(bias, dtype=np.int32),
+                    np.ascontiguousarray(mult, dtype=np.int32), np.ascontiguousarray(rshift, dtype=np.int32)]
+            keep += arrs
+            ptrs += [None if x is None else x.ctypes.data for x in arrs]
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_conv2d_prepack_pair(self.h, C.byref(desc_a), C.byref(desc_b), *ptrs,
+                                                     C.byref(w)))
+        return w.value
+
+    def conv_pair(self, w, x, y_a, y_b):
+        self._ck(self.lib.tpuhip_conv2d_pair_i8(self.h, w, x.ptr, y_a.ptr, y_b.ptr))
 
     def fc_prepack(self, m, k, n, x_cs, y_cs, do_relu, filt, bias, mult, rshift):
         filt = np.ascontiguousarray(filt, dtype=np.int8)

@@ -41,6 +41,9 @@ struct tpuhip_conv_weights {
   int fast = 0;          // the overflow-free requant form is provably exact for this layer
   bool smallc = false;   // ic <= 4: K packs 4 taps x 4 channels per 16-byte group (LDS kernels only)
   bool tuned = true;     // false: the tile is chosen by timing the candidates on first use
+  // a pair of convs over one input packed as one: first channel, channel stride and ReLU of
+  // the second result (split_oc == 0: an ordinary conv)
+  int split_oc = 0, y2_cs = 0, relu2 = 0;
   std::vector<int8_t> host_filter;  // OIHW copy, kept while the layer can still be repacked
   int8_t *w = nullptr;   // packed filter
   int32_t *bias = nullptr;
@@ -83,6 +86,11 @@ struct ConvArgs {
   int8_t *add_dst;
   int add_m_src, add_m_conv, add_rshift, add_relu;
   int store_y;     // 0: the conv result itself is not written (only what is fused behind it)
+  // two convolutions over one input run as one (their filters stacked along oc): channels
+  // from split_oc on (a multiple of 16, 0 = no second conv) belong to the second one and
+  // go to y2 with its own channel stride and ReLU
+  int split_oc, y2_cs, lo2;
+  int8_t *y2;
   // optional fused 256-entry table on the conv result, applied before the fused add:
   // lut_dst (may be null) receives table[y]; the add then takes table[y]
   int has_lut;
@@ -205,13 +213,22 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
                                               const int32_t *phpot, int pix_first,
                                               int pix_stride, const uint8_t *lut = nullptr) {
   uint32_t outw[TN][4];
+  // where this lane's 16 channels go: the conv's own result, or the second result of a pair
+  int8_t *ydst = a.y;
+  int ycs = a.y_cs, lo = a.lo, ocl = oc;
+  if (a.split_oc > 0 && oc >= a.split_oc) {
+    ydst = a.y2;
+    ycs = a.y2_cs;
+    lo = a.lo2;
+    ocl = oc - a.split_oc;
+  }
   // the other operand of a fused add is fetched now and used after the requantisation
   v4i sv[TN];
   if (a.add_dst) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int pix = min(pix_first + j * pix_stride, a.npix - 1);
-      sv[j] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)pix * a.y_cs + oc);
+      sv[j] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)pix * ycs + ocl);
     }
   }
 #pragma unroll
@@ -229,7 +246,7 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
       outw[j][qd] = pack_sat4(requant_core<FAST>(v0, m4[0], r4[0], h4[0]),
                               requant_core<FAST>(v1, m4[1], r4[1], h4[1]),
                               requant_core<FAST>(v2, m4[2], r4[2], h4[2]),
-                              requant_core<FAST>(v3, m4[3], r4[3], h4[3]), a.lo);
+                              requant_core<FAST>(v3, m4[3], r4[3], h4[3]), lo);
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -237,9 +254,9 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
   for (int j = 0; j < TN; ++j) {
     const int pix = pix_first + j * pix_stride;
     if (pix < a.npix) {
-      const int64_t off = (int64_t)pix * a.y_cs + oc;
+      const int64_t off = (int64_t)pix * ycs + ocl;
       v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
-      if (a.store_y) *reinterpret_cast<v4i *>(a.y + off) = o;
+      if (a.store_y) *reinterpret_cast<v4i *>(ydst + off) = o;
       if (lut) {
         // table lookup per byte (index = the two's-complement byte); the 256-byte table
         // covers each LDS bank once, so any 64 indices are conflict-free.  Pad channels
@@ -1637,6 +1654,9 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.store_y = 1;
   a.magic_kw = (1u << 20) / (uint32_t)d.kw + 1;
   a.x_bytes = (uint32_t)((int64_t)d.n * d.ih * d.iw * d.x_cs);
+  a.split_oc = w->split_oc;
+  a.y2_cs = w->y2_cs;
+  a.lo2 = w->relu2 ? 0 : -128;
   a.stem_pw = 127 * d.sw + 8;
   a.magic_pw = (1u << 20) / (uint32_t)a.stem_pw + 1;
   if (w->algo == ALGO_MFMA) {
@@ -1694,6 +1714,7 @@ struct PostOps {
   const tpuhip_fused_add *f = nullptr;
   const void *add_src = nullptr;
   void *add_out = nullptr;
+  void *y2 = nullptr;            // second result of a packed pair
   bool has_add() const { return f && f->enable; }
 };
 
@@ -1712,6 +1733,7 @@ void apply_fusion(ConvArgs *a, const void *y, const PostOps &p) {
     a->add_relu = p.f->do_relu ? 1 : 0;
   }
   a->store_y = y != nullptr;
+  a->y2 = (int8_t *)p.y2;
 }
 
 // The fused add (if any) is part of what is timed: it shifts the balance between
@@ -1985,6 +2007,8 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
                      w->algo == ALGO_STEM ||
                      (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
                  "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
+  TPUHIP_REQUIRE((w->split_oc != 0) == (post.y2 != nullptr),
+                 "conv: weights packed as a pair run through tpuhip_conv2d_pair_i8 (and only they do)");
   ConvArgs a;
   fill_args(ctx, w, x, y, &a);
   apply_fusion(&a, y, post);
@@ -2093,6 +2117,66 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
   }
   TPUHIP_REQUIRE(y || p.lut_out || p.add_out, "conv2d_post: nothing would be written");
   return run_conv(ctx, w, x, y, p);
+}
+
+int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, const tpuhip_conv_desc *db,
+                               const int8_t *filter_a, const int32_t *bias_a, const int32_t *mult_a,
+                               const int32_t *rshift_a, const int8_t *filter_b, const int32_t *bias_b,
+                               const int32_t *mult_b, const int32_t *rshift_b, tpuhip_conv_weights **out) {
+  TPUHIP_REQUIRE(ctx && da && db && filter_a && filter_b && mult_a && mult_b && rshift_a && rshift_b && out,
+                 "tpuhip_conv2d_prepack_pair: NULL argument");
+  const tpuhip_conv_desc &a = *da, &b = *db;
+  if (int rc = check_desc(a)) return rc;
+  if (int rc = check_desc(b)) return rc;
+  TPUHIP_REQUIRE(a.n == b.n && a.ic == b.ic && a.ih == b.ih && a.iw == b.iw && a.x_cs == b.x_cs &&
+                     a.oh == b.oh && a.ow == b.ow && a.kh == b.kh && a.kw == b.kw && a.sh == b.sh &&
+                     a.sw == b.sw && a.pt == b.pt && a.pb == b.pb && a.pl == b.pl && a.pr == b.pr &&
+                     a.dh == b.dh && a.dw == b.dw,
+                 "conv pair: the two convs must read the same input through the same window geometry");
+  TPUHIP_REQUIRE(a.g == 1 && b.g == 1 && !a.ins_h && !a.ins_w && !b.ins_h && !b.ins_w && !a.relu_first &&
+                     !b.relu_first,
+                 "conv pair: dense convs only");
+  TPUHIP_REQUIRE(a.oc % 16 == 0, "conv pair: the first conv needs a multiple of 16 output channels (%d)", a.oc);
+  TPUHIP_REQUIRE(a.algo == b.algo && (a.algo == ALGO_AUTO || a.algo == ALGO_MFMA || a.algo >= 16),
+                 "conv pair: only the MFMA path (algo 0, 2 or 16 + tile, the same for both)");
+  // one conv with the filters stacked along the output channels
+  tpuhip_conv_desc m = a;
+  m.oc = a.oc + b.oc;
+  m.y_cs = round_up(m.oc, 16);   // only for the checks: each half keeps its own stride
+  m.with_bias = (a.with_bias && bias_a) || (b.with_bias && bias_b) ? 1 : 0;
+  m.algo = a.algo == ALGO_AUTO ? ALGO_MFMA : a.algo;   // the only path whose epilogue can split its output
+  const size_t per_oc = (size_t)a.ic * a.kh * a.kw;
+  std::vector<int8_t> filter((size_t)m.oc * per_oc);
+  memcpy(filter.data(), filter_a, (size_t)a.oc * per_oc);
+  memcpy(filter.data() + (size_t)a.oc * per_oc, filter_b, (size_t)b.oc * per_oc);
+  std::vector<int32_t> bias((size_t)m.oc, 0), mult((size_t)m.oc), rshift((size_t)m.oc);
+  for (int i = 0; i < a.oc; ++i) {
+    if (a.with_bias && bias_a) bias[i] = bias_a[i];
+    mult[i] = mult_a[i];
+    rshift[i] = rshift_a[i];
+  }
+  for (int i = 0; i < b.oc; ++i) {
+    if (b.with_bias && bias_b) bias[a.oc + i] = bias_b[i];
+    mult[a.oc + i] = mult_b[i];
+    rshift[a.oc + i] = rshift_b[i];
+  }
+  tpuhip_conv_weights *cw = nullptr;
+  if (int rc = tpuhip_conv2d_prepack(ctx, &m, filter.data(), bias.data(), mult.data(), rshift.data(), &cw))
+    return rc;
+  cw->d.y_cs = a.y_cs;
+  cw->split_oc = a.oc;
+  cw->y2_cs = b.y_cs;
+  cw->relu2 = b.do_relu ? 1 : 0;
+  *out = cw;
+  return TPUHIP_OK;
+}
+
+int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y_a, void *y_b) {
+  TPUHIP_REQUIRE(ctx && w && x && y_a && y_b, "tpuhip_conv2d_pair_i8: NULL argument");
+  TPUHIP_REQUIRE(w->split_oc > 0, "tpuhip_conv2d_pair_i8: weights were not packed as a pair");
+  PostOps p;
+  p.y2 = y_b;
+  return run_conv(ctx, w, x, y_a, p);
 }
 
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,

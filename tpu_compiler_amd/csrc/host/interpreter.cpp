@@ -51,6 +51,7 @@ void ModuleInterpreter::updateWeightMap(const std::string &name, const float *da
 void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
   updateKernelList(module, target_op);
   fuseKernels();
+  pairConvs();
 }
 
 // Work that rides in a dense conv's epilogue instead of running as a kernel of its own
@@ -143,6 +144,33 @@ void ModuleInterpreter::fuseKernels() {
         conv->has_fused_add() && droppable(conv->final_result().get()))
       conv->set_store_lut(false);
   }
+}
+
+// Convs that read the same tensor through the same window geometry (the projection shortcut
+// and the first 1x1 of a residual block, for one) become one launch: the second one's work
+// moves to the position of the first, which is legal because its only activation operand
+// is available there and nothing reads its result before its own position.  Runs after the
+// add / table fusions, which take precedence.
+void ModuleInterpreter::pairConvs() {
+  std::vector<Conv2DOpKernel *> convs;
+  for (auto &k : kernel_list_)
+    if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) convs.push_back(c);
+  const char *env = getenv("TPUHIP_PAIR");
+  if (pair_convs && !(env && atoi(env) == 0)) {
+    for (size_t i = 0; i < convs.size(); ++i)
+      for (size_t j = i + 1; j < convs.size(); ++j)
+        if (convs[i]->can_pair_with(*convs[j])) {
+          try {
+            convs[i]->pair_with(*convs[j]);
+          } catch (const std::exception &) {
+            // shapes the packed form does not cover stay two launches
+          }
+          break;
+        }
+  }
+  // paired kernels keep their host operands so that a reload can pair them again
+  for (auto *c : convs)
+    if (!c->is_paired_first() && !c->is_paired_second()) c->release_host_weights();
 }
 
 // MlirModuleInterpreter.cpp:85-116
@@ -366,7 +394,8 @@ std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_
     for (auto &krnl : kernel_list_) {
       auto *el = dynamic_cast<EltwiseAddOpKernel *>(krnl.get());
       auto *lu = dynamic_cast<LutOpKernel *>(krnl.get());
-      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) ||
+      auto *cv = dynamic_cast<Conv2DOpKernel *>(krnl.get());
+      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) || (cv && cv->is_paired_second()) ||
                           (el && el->fused_into_producer) || (lu && lu->fused_into_producer));
       if (runs) ck(tpuhip_ctx_set_kernel_events(ctx_, e0[i], e1[i]), "timeKernels");
       krnl->invoke();

@@ -376,13 +376,59 @@ Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
   ck(tpuhip_conv2d_prepack(ctx, &d, w8.data(), d.with_bias ? b32.data() : nullptr, m32.data(),
                            r32.data(), &packed),
      ("Conv2D '" + name + "'").c_str());
+  plain = !transposed && d.g == 1 && !d.ins_h && !d.ins_w && (d.algo == 0 || d.algo == 2 || d.algo >= 16);
+  if (plain) {
+    host_w = std::move(w8);
+    host_b = std::move(b32);
+    host_m = std::move(m32);
+    host_r = std::move(r32);
+  }
 }
 
 Conv2DOpKernel::~Conv2DOpKernel() {
+  if (pair_packed) tpuhip_conv2d_weights_destroy(ctx, pair_packed);
   if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
 }
 
+void Conv2DOpKernel::release_host_weights() {
+  std::vector<int8_t>().swap(host_w);
+  std::vector<int32_t>().swap(host_b);
+  std::vector<int32_t>().swap(host_m);
+  std::vector<int32_t>().swap(host_r);
+}
+
+bool Conv2DOpKernel::can_pair_with(const Conv2DOpKernel &o) const {
+  if (this == &o || !plain || !o.plain || host_w.empty() || o.host_w.empty()) return false;
+  if (pair_packed || paired_into || o.pair_packed || o.paired_into) return false;
+  if (fused.enable || lut_dst || o.fused.enable || o.lut_dst) return false;
+  if (input_data.get() != o.input_data.get() || desc.oc % 16 != 0) return false;
+  const tpuhip_conv_desc &a = desc, &b = o.desc;
+  return a.kh == b.kh && a.kw == b.kw && a.sh == b.sh && a.sw == b.sw && a.pt == b.pt && a.pb == b.pb &&
+         a.pl == b.pl && a.pr == b.pr && a.dh == b.dh && a.dw == b.dw && a.oh == b.oh && a.ow == b.ow;
+}
+
+void Conv2DOpKernel::pair_with(Conv2DOpKernel &second) {
+  if (!can_pair_with(second)) fail("Conv2D '" + name + "': cannot run together with '" + second.name + "'");
+  // the pair runs on the kernel variant asked for the first conv (0: timed on first use)
+  tpuhip_conv_desc da = desc, db = second.desc;
+  db.algo = da.algo;
+  ck(tpuhip_conv2d_prepack_pair(ctx, &da, &db, host_w.data(),
+                                desc.with_bias ? host_b.data() : nullptr, host_m.data(), host_r.data(),
+                                second.host_w.data(), second.desc.with_bias ? second.host_b.data() : nullptr,
+                                second.host_m.data(), second.host_r.data(), &pair_packed),
+     ("Conv2D '" + name + "' + '" + second.name + "'").c_str());
+  pair_second = &second;
+  second.paired_into = this;
+}
+
 void Conv2DOpKernel::invoke() {
+  if (paired_into) return;   // computed by the launch of the conv it is paired with
+  if (pair_packed) {
+    ck(tpuhip_conv2d_pair_i8(ctx, pair_packed, input_data->data(), output_data->data(),
+                             pair_second->output_data->data()),
+       name.c_str());
+    return;
+  }
   if (!fused.enable && !lut_dst) {
     ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
     return;
@@ -403,7 +449,7 @@ void Conv2DOpKernel::invoke() {
 }
 
 bool Conv2DOpKernel::can_fuse_add() const {
-  return std::string(tpuhip_conv2d_algo_name(packed)).rfind("mfma", 0) == 0;
+  return !pair_packed && !paired_into && std::string(tpuhip_conv2d_algo_name(packed)).rfind("mfma", 0) == 0;
 }
 
 void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift,
@@ -424,7 +470,7 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
 bool Conv2DOpKernel::can_fuse_lut() const {
   const std::string algo = tpuhip_conv2d_algo_name(packed);
   return (algo.rfind("mfma", 0) == 0 || algo.rfind("depthwise", 0) == 0 || algo == "stem") && !lut_dst &&
-         !fused.enable;
+         !fused.enable && !pair_packed && !paired_into;
 }
 
 void Conv2DOpKernel::fuse_lut(const int8_t *table, SyncedData dst) {
@@ -450,6 +496,12 @@ void Conv2DOpKernel::set_store_result(bool store) {
 }
 
 void Conv2DOpKernel::clear_fusion() {
+  if (pair_packed) {
+    tpuhip_conv2d_weights_destroy(ctx, pair_packed);
+    pair_packed = nullptr;
+    if (pair_second) pair_second->paired_into = nullptr;
+    pair_second = nullptr;
+  }
   store_result = true;
   output_data->materialized = true;
   if (lut_dst) lut_dst->materialized = true;
@@ -460,7 +512,14 @@ void Conv2DOpKernel::clear_fusion() {
   add_dst.reset();
 }
 
-const char *Conv2DOpKernel::algo_name() const { return tpuhip_conv2d_algo_name(packed); }
+const char *Conv2DOpKernel::algo_name() const {
+  auto *self = const_cast<Conv2DOpKernel *>(this);
+  if (paired_into) {
+    self->algo_text = "with " + paired_into->name;
+    return algo_text.c_str();
+  }
+  return tpuhip_conv2d_algo_name(pair_packed ? pair_packed : packed);
+}
 
 // ---------------------------------------------------------------------------
 // FullyConnected (core/fullyconnected.cpp:7-91)

@@ -96,6 +96,8 @@ int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value) {
       m->interp->fuse_eltwise = value != 0;
     else if (k == "keep_all_tensors")
       m->interp->keep_all_tensors = value != 0;
+    else if (k == "pair_convs")
+      m->interp->pair_convs = value != 0;
     else
       throw std::runtime_error("tpuhip_module_set_option: unknown option '" + k + "'");
   })
