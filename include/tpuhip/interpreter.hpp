@@ -227,7 +227,7 @@ private:
   tpuhip_conv_weights *pair_packed = nullptr;
   Conv2DOpKernel *pair_second = nullptr;   // runs inside this kernel's launch
   Conv2DOpKernel *paired_into = nullptr;   // this kernel's work is done by that one
-  std::string algo_text;
+  mutable std::string algo_text;           // storage behind algo_name() of a paired kernel
 };
 
 // core/deconv.cpp:7-73, same operands and epilogue as Conv2D

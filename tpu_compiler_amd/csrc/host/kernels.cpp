@@ -513,9 +513,8 @@ void Conv2DOpKernel::clear_fusion() {
 }
 
 const char *Conv2DOpKernel::algo_name() const {
-  auto *self = const_cast<Conv2DOpKernel *>(this);
   if (paired_into) {
-    self->algo_text = "with " + paired_into->name;
+    algo_text = "with " + paired_into->name;
     return algo_text.c_str();
   }
   return tpuhip_conv2d_algo_name(pair_packed ? pair_packed : packed);
