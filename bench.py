@@ -217,7 +217,7 @@ def main():
             "frac": round(hbm_bytes / (hbm_ms / 1e3) / 1e9 / PEAK_HBM_GBS, 4), "ms": round(hbm_ms, 4)},
     }
     if not args.no_cpu_baseline:
-        sample = {"cfg1": 8, "cfg2": 8, "cfg3": 8, "cfg4": 16, "cfg5": 1}[args.config]
+        sample = {"cfg1": 64, "cfg2": 16, "cfg3": 32, "cfg4": 64, "cfg5": 2}[args.config]
         out["cpu_baseline"] = cpu_baseline(graph_fn, sample)
     m.close()
     print(json.dumps(out))
