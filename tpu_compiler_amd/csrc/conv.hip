@@ -798,9 +798,14 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
   const int wave = threadIdx.x >> 6;
   const int frow = lane & 31, fk = lane >> 5;
   const int n_cb = (a.ocw + 31) >> 5;
-  const int n_pb = (a.npix + 31) >> 5;
-  const int gw = (int)blockIdx.x * 4 + wave;
-  const int nslots = (int)(gridDim.x * 4) / n_cb;     // pixel blocks in flight (>= 1)
+  // workgroups are dealt to the 8 XCDs round-robin; each XCD takes a contiguous run of pixel
+  // blocks, so the input rows that vertically neighbouring blocks share meet in one L2
+  const int n_pb_all = (a.npix + 31) >> 5;
+  const int pb_per_xcd = (n_pb_all + 7) >> 3;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int n_pb = min(n_pb_all, (xcd + 1) * pb_per_xcd);   // end of this XCD's run
+  const int gw = (int)(blockIdx.x >> 3) * 4 + wave;          // wave index within the XCD
+  const int nslots = (int)(gridDim.x >> 3) * 4 / n_cb;       // pixel blocks in flight per XCD (>= 1)
   const int cb = gw % n_cb;
   int pb = gw / n_cb;
   // a wave's parameters never change: they live in LDS, whose reads do not queue behind
@@ -814,6 +819,8 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
   if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
   __syncthreads();
   if (pb >= nslots) return;                           // no barrier below
+  pb += xcd * pb_per_xcd;
+  if (pb >= n_pb) return;
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
   const int oc = cb * 32 + fk * 16;                   // this lane's 16 channels
   const bool ch_ok = oc < a.ocw;
@@ -2019,8 +2026,9 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     // wave walking pixel blocks of its channel block
     const int n_cb = (a.ocw + 31) / 32, n_pb = (a.npix + 31) / 32;
     const int64_t waves = (int64_t)n_cb * n_pb;
-    const unsigned blocks = (unsigned)std::max<int64_t>(
-        (n_cb + 3) / 4, std::min<int64_t>(ceil_div64(waves, 4), (int64_t)ctx->num_cu * 3));
+    // a multiple of 8 workgroups, every XCD's share holding at least one wave per channel block
+    const unsigned blocks = 8 * (unsigned)std::max<int64_t>(
+        (n_cb + 3) / 4, std::min<int64_t>(ceil_div64(waves, 32), std::max(1, ctx->num_cu * 3 / 8)));
     const dim3 grid(blocks), block(256);
     const bool regw = a.kh * a.kw <= 9;
     if (w->fast) {

@@ -23,11 +23,18 @@ __device__ __forceinline__ int32_t sb(int32_t word, int i) {
   return (int32_t)(int8_t)(word >> (8 * i));
 }
 
+// Workgroups are dealt to the 8 XCDs round-robin.  With a grid that is a multiple of 8 this
+// renumbering gives every XCD a contiguous run of logical blocks, i.e. of output rows, so the
+// input rows that neighbouring windows share are fetched into one L2 instead of several.
+__device__ __forceinline__ unsigned xcd_block() {
+  return (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+}
+
 // PoolingOpKernel INT8 max (core/pooling.cpp:155-157): MKL-DNN pooling_max skips
 // padded positions.
 __global__ __launch_bounds__(256) void pool_max_kernel(PoolArgs a) {
   const int64_t total = (int64_t)a.n * a.oh * a.ow * a.c16;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+  for (int64_t i = (int64_t)xcd_block() * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int cg = (int)(i % a.c16);
     int64_t p = i / a.c16;
@@ -70,7 +77,7 @@ __global__ __launch_bounds__(256) void pool_max_kernel(PoolArgs a) {
 // quotient by a power of two, floor(f + 0.5), clamp.
 __global__ __launch_bounds__(256) void pool_avg_kernel(PoolArgs a) {
   const int64_t total = (int64_t)a.n * a.oh * a.ow * a.c16;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+  for (int64_t i = (int64_t)xcd_block() * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
     const int cg = (int)(i % a.c16);
     int64_t p = i / a.c16;
@@ -188,7 +195,8 @@ int fill_args(const tpuhip_pool_desc *d, const void *x, void *y, PoolArgs *a) {
 
 unsigned blocks_for(const PoolArgs &a) {
   const int64_t total = (int64_t)a.n * a.oh * a.ow * a.c16;
-  return (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 255) / 256, 1 << 16));
+  // a multiple of 8 (see xcd_block)
+  return 8u * (unsigned)std::max<int64_t>(1, std::min<int64_t>((total + 2047) / 2048, 1 << 13));
 }
 
 }  // namespace
