@@ -46,6 +46,7 @@ private:
   const std::string &s;
   size_t i = 0;
   int line = 1;
+  int nesting = 0;   // of attribute values (bounded: the reader recurses)
 
   [[noreturn]] void fail(const std::string &what) const {
     throw std::runtime_error("mlir:" + std::to_string(line) + ": " + what);
@@ -244,7 +245,16 @@ private:
     return d;
   }
 
+  struct Nest {
+    Reader &r;
+    explicit Nest(Reader &reader) : r(reader) {
+      if (++r.nesting > 64) r.fail("attribute values nested more than 64 deep");
+    }
+    ~Nest() { --r.nesting; }
+  };
+
   MlirAttr value() {
+    Nest nest(*this);
     ws();
     MlirAttr a;
     const char c = peek();
