@@ -168,7 +168,7 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
  * through the same window geometry (kernel, stride, padding, dilation), e.g. the projection
  * shortcut and the first 1x1 conv of a residual block.  Their filters are stacked along the
  * output channels; every output tile goes to the result it belongs to, with that conv's own
- * channel stride and ReLU.  The first conv needs a multiple of 16 output channels.  Results are
+ * channel stride and ReLU.  The first conv needs a multiple of 128 output channels.  Results are
  * those of two tpuhip_conv2d_i8 calls.  No counterpart in the reference (one kernel per op). */
 int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b,
                                const int8_t *filter_a, const int32_t *bias_a, const int32_t *multiplier_a,

@@ -144,8 +144,8 @@ def test_conv_stem_general_requant_fused_table_and_limits(ctx):
 PAIR_CASES = [
     (2, 64, 14, 14, 256, 64, 1, (1, 1), (0, 0, 0, 0), False, True, True),     # shortcut + first 1x1 of a block
     (3, 256, 15, 13, 512, 128, 1, (2, 2), (0, 0, 0, 0), False, True, True),   # the strided pair
-    (1, 40, 9, 11, 48, 24, 3, (1, 1), (1, 1, 1, 1), True, False, False),      # ragged second half, 3x3
-    (16, 32, 28, 28, 64, 40, 1, (1, 1), (0, 0, 0, 0), True, True, True),      # enough pixels to walk tiles
+    (1, 40, 9, 11, 128, 24, 3, (1, 1), (1, 1, 1, 1), True, False, False),     # ragged second half, 3x3
+    (16, 32, 28, 28, 128, 40, 1, (1, 1), (0, 0, 0, 0), True, True, True),     # enough pixels to walk tiles
 ]
 
 
@@ -192,13 +192,13 @@ def test_conv_pair_equals_two_convs(ctx, case):
 def test_conv_pair_refuses_mismatched_convs(ctx):
     x_shape = (1, 32, 8, 8)
     z = lambda oc: (np.zeros((oc, 32, 1, 1), np.int8), None, np.full(oc, 1 << 30, np.int32), np.ones(oc, np.int32))
-    da = conv_desc(x_shape, (64, 32, 1, 1))
+    da = conv_desc(x_shape, (128, 32, 1, 1))
     with pytest.raises(capi.TpuHipError, match="same window geometry"):
-        ctx.conv_prepack_pair(da, conv_desc(x_shape, (16, 32, 1, 1), stride=(2, 2)), z(64), z(16))
-    with pytest.raises(capi.TpuHipError, match="multiple of 16"):
-        ctx.conv_prepack_pair(conv_desc(x_shape, (24, 32, 1, 1)), conv_desc(x_shape, (16, 32, 1, 1)), z(24), z(16))
-    w = ctx.conv_prepack(da, *[z(64)[i] for i in (0, 1, 2, 3)])
-    xt, ya = ctx.tensor(x_shape), ctx.tensor((1, 64, 8, 8))
+        ctx.conv_prepack_pair(da, conv_desc(x_shape, (16, 32, 1, 1), stride=(2, 2)), z(128), z(16))
+    with pytest.raises(capi.TpuHipError, match="multiple of 128"):
+        ctx.conv_prepack_pair(conv_desc(x_shape, (64, 32, 1, 1)), conv_desc(x_shape, (16, 32, 1, 1)), z(64), z(16))
+    w = ctx.conv_prepack(da, *[z(128)[i] for i in (0, 1, 2, 3)])
+    xt, ya = ctx.tensor(x_shape), ctx.tensor((1, 128, 8, 8))
     with pytest.raises(capi.TpuHipError, match="not packed as a pair"):
         ctx.conv_pair(w, xt, ya, ya)
     ctx.conv_weights_destroy(w)

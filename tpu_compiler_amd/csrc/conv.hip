@@ -87,7 +87,7 @@ struct ConvArgs {
   int add_m_src, add_m_conv, add_rshift, add_relu;
   int store_y;     // 0: the conv result itself is not written (only what is fused behind it)
   // two convolutions over one input run as one (their filters stacked along oc): channels
-  // from split_oc on (a multiple of 16, 0 = no second conv) belong to the second one and
+  // from split_oc on (a multiple of 128, 0 = no second conv) belong to the second one and
   // go to y2 with its own channel stride and ReLU
   int split_oc, y2_cs, lo2;
   int8_t *y2;
@@ -207,21 +207,30 @@ __device__ __forceinline__ int32_t requant_core(int32_t v, int32_t mult, int32_t
 // Epilogue of one wave tile row block: the lane's 16 consecutive channels
 // (starting at oc) of TN pixels.  Requantise, saturate (+ReLU) and store 16 bytes
 // per pixel.  Parameters are read four channels at a time to keep few registers live.
+// Where an output-channel tile is written.  A pair of convs packed as one: a workgroup (or
+// wave) whose tile lies in the second conv's channels writes that conv's result, with its
+// channel stride and ReLU; split_oc is a multiple of 128, so no tile straddles it.  Chosen
+// once per workgroup, before any tile is computed, from a uniform tile base.
+struct OutRoute {
+  int8_t *y;
+  int y_cs, lo, shift;   // shift: first channel of the tensor written
+};
+__device__ __forceinline__ OutRoute route_out(const ConvArgs &a, int oc_tile_base) {
+  const bool second = a.split_oc > 0 && oc_tile_base >= a.split_oc;
+  return OutRoute{second ? a.y2 : a.y, second ? a.y2_cs : a.y_cs, second ? a.lo2 : a.lo,
+                  second ? a.split_oc : 0};
+}
+
 template <int TN, bool FAST>
 __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
                                               const int32_t *pmult, const int32_t *pshift,
                                               const int32_t *phpot, int pix_first,
-                                              int pix_stride, const uint8_t *lut = nullptr) {
+                                              int pix_stride, const uint8_t *lut, const OutRoute &out) {
   uint32_t outw[TN][4];
-  // where this lane's 16 channels go: the conv's own result, or the second result of a pair
-  int8_t *ydst = a.y;
-  int ycs = a.y_cs, lo = a.lo, ocl = oc;
-  if (a.split_oc > 0 && oc >= a.split_oc) {
-    ydst = a.y2;
-    ycs = a.y2_cs;
-    lo = a.lo2;
-    ocl = oc - a.split_oc;
-  }
+  // channel index within the tensor written (a pair's second result starts at split_oc)
+  int8_t *const ydst = out.y;
+  const int ycs = out.y_cs, lo = out.lo;
+  const int ocl = oc - out.shift;
   // the other operand of a fused add is fetched now and used after the requantisation
   v4i sv[TN];
   if (a.add_dst) {
@@ -498,6 +507,7 @@ conv_mfma_kernel(ConvArgs a) {
   if (logical >= a.n_tiles) return;
   const int pix_tile = logical / a.n_oc_tiles;
   const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;   // the same for every tile of a walk
+  const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
   int pix0 = pix_tile * BN;
 
   const __amdgpu_buffer_rsrc_t xrsrc =
@@ -767,10 +777,10 @@ conv_mfma_kernel(ConvArgs a) {
       if (oc < a.ocw) {
         if (PERSIST)
           epilogue_rows<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc,
-                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32, lut);
+                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32, lut, out);
         else
           epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
-                                  pix_done + wn * TN * 32 + frow, 32, lut);
+                                  pix_done + wn * TN * 32 + frow, 32, lut, out);
       }
     }
     if (!PERSIST || !more) break;
@@ -822,6 +832,7 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
   pb += xcd * pb_per_xcd;
   if (pb >= n_pb) return;
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
   const int oc = cb * 32 + fk * 16;                   // this lane's 16 channels
   const bool ch_ok = oc < a.ocw;
   const int taps = a.kh * a.kw;
@@ -889,7 +900,7 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
 #pragma unroll
         for (int t = 0; t < 9; ++t) bt[t] = tap_load(t);
       }
-      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix_done, 32, lut);
+      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix_done, 32, lut, out);
       if (!more) break;
     }
   } else {
@@ -898,7 +909,7 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
       bias_acc(acc[0]);
       for (int t = 0; t < taps; ++t)
         acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[t * 64], tap_load(t), acc[0], 0, 0, 0);
-      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix, 32, lut);
+      if (ch_ok) epilogue_rows<1, FAST>(acc, a, oc, pmult, pshift, phpot, pix, 32, lut, out);
       advance();
     }
   }
@@ -943,6 +954,7 @@ conv_stem_kernel(ConvArgs a) {
   }
   if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
 
   v4i areg[NI][KH];
   {
@@ -1045,7 +1057,7 @@ conv_stem_kernel(ConvArgs a) {
         const int oc = (ib + i) * 32 + fk * 16;
         if (oc < a.ocw) {
           const v16i one[1] = {acc[i][j]};
-          epilogue_rows<1, FAST>(one, a, oc, &qlds[1][oc], &qlds[2][oc], &qlds[3][oc], pix, 32, lut);
+          epilogue_rows<1, FAST>(one, a, oc, &qlds[1][oc], &qlds[2][oc], &qlds[3][oc], pix, 32, lut, out);
         }
       }
     }
@@ -1078,6 +1090,7 @@ conv_mfma_reg_kernel(ConvArgs a) {
   const int pix_tile = wt / a.n_oc_tiles;
   const int oc_tile = wt - pix_tile * a.n_oc_tiles;
   const int oc0 = oc_tile * (TM * 32);
+  const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
   const int pix0 = pix_tile * (TN * 32);
 
   const __amdgpu_buffer_rsrc_t xrsrc =
@@ -1217,7 +1230,8 @@ conv_mfma_reg_kernel(ConvArgs a) {
   for (int i = 0; i < TM; ++i) {
     const int oc = ocw0 + i * 16;
     if (oc < a.ocw)
-      epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pix0 + frow, 32);
+      epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pix0 + frow, 32,
+                              nullptr, out);
   }
 }
 
@@ -1238,6 +1252,7 @@ conv_mfma_splitk_kernel(ConvArgs a) {
   const int pix_tile = wt / a.n_oc_tiles;
   const int oc_tile = wt - pix_tile * a.n_oc_tiles;
   const int oc0 = oc_tile * (TM * 32);
+  const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
   const int pix0 = pix_tile * (TN * 32);
 
   const __amdgpu_buffer_rsrc_t xrsrc =
@@ -1410,7 +1425,7 @@ conv_mfma_splitk_kernel(ConvArgs a) {
     const int oc = ocw0 + i * 16;
     if (oc < a.ocw)
       epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
-                             pix0 + j * 32 + frow, 32);
+                             pix0 + j * 32 + frow, 32, nullptr, out);
   }
 }
 
@@ -2144,7 +2159,7 @@ int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, cons
   TPUHIP_REQUIRE(a.g == 1 && b.g == 1 && !a.ins_h && !a.ins_w && !b.ins_h && !b.ins_w && !a.relu_first &&
                      !b.relu_first,
                  "conv pair: dense convs only");
-  TPUHIP_REQUIRE(a.oc % 16 == 0, "conv pair: the first conv needs a multiple of 16 output channels (%d)", a.oc);
+  TPUHIP_REQUIRE(a.oc % 128 == 0, "conv pair: the first conv needs a multiple of 128 output channels (%d)", a.oc);
   TPUHIP_REQUIRE(a.algo == b.algo && (a.algo == ALGO_AUTO || a.algo == ALGO_MFMA || a.algo >= 16),
                  "conv pair: only the MFMA path (algo 0, 2 or 16 + tile, the same for both)");
   // one conv with the filters stacked along the output channels

@@ -401,7 +401,7 @@ bool Conv2DOpKernel::can_pair_with(const Conv2DOpKernel &o) const {
   if (this == &o || !plain || !o.plain || host_w.empty() || o.host_w.empty()) return false;
   if (pair_packed || paired_into || o.pair_packed || o.paired_into) return false;
   if (fused.enable || lut_dst || o.fused.enable || o.lut_dst) return false;
-  if (input_data.get() != o.input_data.get() || desc.oc % 16 != 0) return false;
+  if (input_data.get() != o.input_data.get() || desc.oc % 128 != 0) return false;
   const tpuhip_conv_desc &a = desc, &b = o.desc;
   return a.kh == b.kh && a.kw == b.kw && a.sh == b.sh && a.sw == b.sw && a.pt == b.pt && a.pb == b.pb &&
          a.pl == b.pl && a.pr == b.pr && a.dh == b.dh && a.dw == b.dw && a.oh == b.oh && a.ow == b.ow;
