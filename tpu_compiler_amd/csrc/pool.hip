@@ -139,16 +139,28 @@ __global__ __launch_bounds__(256) void pool_avg_split_kernel(PoolArgs a) {
 #pragma unroll
   for (int k = 0; k < 16; ++k) sum[k] = 0;
   const int taps = a.kh * a.kw;
-  for (int t = sub; t < taps; t += LANES) {
-    const int kh = t / a.kw, kw = t - kh * a.kw;
-    const int ih = oh * a.sh - a.pt + kh, iw = ow * a.sw - a.pl + kw;
-    if (ih < 0 || ih >= a.ih || iw < 0 || iw >= a.iw) continue;
-    const v4i v = *reinterpret_cast<const v4i *>(
-        a.x + ((int64_t)(b * a.ih + ih) * a.iw + iw) * a.x_cs + cg * 16);
+  // up to MAXT window positions of this lane are requested before any is added, so their
+  // latencies overlap instead of lining up one behind the other
+  constexpr int MAXT = 8;
+  const uint32_t magic_kw = (1u << 20) / (uint32_t)a.kw + 1;   // t / kw == (t * magic) >> 20 for t < 4095
+  for (int t0 = sub; t0 < taps; t0 += LANES * MAXT) {
+    v4i v[MAXT];
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int u = 0; u < MAXT; ++u) {
+      const int t = t0 + u * LANES;
+      const int kh = (int)(((uint32_t)t * magic_kw) >> 20), kw = t - kh * a.kw;
+      const int ih = oh * a.sh - a.pt + kh, iw = ow * a.sw - a.pl + kw;
+      const bool ok = (t < taps) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+      v[u] = v4i{0, 0, 0, 0};
+      if (ok)
+        v[u] = *reinterpret_cast<const v4i *>(a.x + ((int64_t)(b * a.ih + ih) * a.iw + iw) * a.x_cs + cg * 16);
+    }
 #pragma unroll
-      for (int k = 0; k < 4; ++k) sum[q * 4 + k] += sb(v[q], k);
+    for (int u = 0; u < MAXT; ++u)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) sum[q * 4 + k] += sb(v[u][q], k);
   }
 #pragma unroll
   for (int k = 0; k < 16; ++k)
