@@ -122,7 +122,8 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
         elif t == "tpu.clip":
             y = O.clip_i8(ins[0], op.attrs["min"], op.attrs["max"], op.weights["rshift"][0],
                           op.weights["multiplier"][0])
-        elif t == "tpu.lut":
+        elif t == "tpu.lut" or (op.param_type == "LUT_INT8" and "table" in op.weights):
+            # sigmoid, tanh, exp, ... in INT8 are all one 256-entry table lookup
             y = O.lut_i8(ins[0], op.weights["table"])
         elif t == "tpu.relu":
             y = O.relu_i8(ins[0])
