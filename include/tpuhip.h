@@ -467,11 +467,27 @@ int tpuhip_quantize_rescale(const float *threshold_x, int n_inputs, float thresh
  * multiplier_neg */
 int tpuhip_quantize_leaky_relu(float negative_slope, float threshold_x, float threshold_y, float *out4);
 /* quantizeInt8LutOps (QuantizeInt8.cpp:531-621): the 256-entry table, indexed by the two's-complement
- * byte of the input.  kind: 0 sigmoid, 1 tanh, 2 exp, 3 elu, 4 swish, 5 softplus, 6 log, 7 pow;
+ * byte of the input.  kind: 0 sigmoid, 1 tanh, 2 exp, 3 elu, 4 swish, 5 softplus, 6 log, 7 pow, 8 mish;
  * scale / bias: the op attributes of sigmoid, exp, softplus (1, 0 if none); coeff: pow's exponent.
  * Entries the reference leaves as NaN (log of a negative input) are NaN here too. */
 int tpuhip_quantize_lut_table(int kind, float threshold_x, float threshold_y, float scale, float bias,
                               float coeff, float *table256);
+
+/* tpuc-opt --import-calibration-table --calibration-table T --tpu-quant in.mlir -o out.mlir
+ * (lib/Dialect/TPU/Quantization/ImportCalibrationTable.cpp:250-415, Quantization.cpp:657-787,
+ * QuantizeInt8.cpp): reads an fp32 TPU-dialect function and the weight .npz it names, takes the
+ * thresholds of the calibration table (`name threshold [min max]` per line), and writes the INT8
+ * function (weights quantised, rescaling operands added, tpu.quant ops at the fp32 edges) with a new
+ * weight file -- out_weights, or out.mlir's stem + "_weights.npz" when NULL.  What it writes is
+ * what tpuhip_module_load_mlir loads.  Host code only, no GPU.  Op kinds: conv_2d, deconv_2d,
+ * fully_connected, eltwise add / max / min / mul, broadcast add / sub / mul, pool_avg_2d,
+ * pool_max_2d, relu, leaky_relu, prelu, clip, concat, the table activations (sigmoid, tanh, exp, elu,
+ * swish, softplus, log, pow, mish), upsample, pad, crop, permute, reorg, pixelshuffle, tile,
+ * reverse, shuffle_channel, reshape; anything else is refused by name.  `missing` (may be NULL)
+ * receives, one per line, the ops the table had no threshold for (the reference warns and goes
+ * on); *needed = its length + 1. */
+int tpuhip_quantize_mlir_files(const char *in_mlir, const char *calibration_table, const char *out_mlir,
+                               const char *out_weights, char *missing, size_t capacity, size_t *needed);
 
 #ifdef __cplusplus
 }

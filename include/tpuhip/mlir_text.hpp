@@ -26,6 +26,7 @@ struct MlirAttr {
   enum Kind { Int, Float, Bool, String, Array, Dict, Unit, Other };
   Kind kind = Unit;
   double num = 0;                 // Int / Float / Bool
+  std::string ty;                 // Int / Float: the type written after ':' ("i32", "f32", ...), "" if none
   std::string str;                // String: the unescaped text; Other: the raw text
   std::vector<MlirAttr> items;    // Array
   std::vector<std::pair<std::string, MlirAttr>> fields;   // Dict, in file order
@@ -58,6 +59,14 @@ struct MlirFunc {
 
 // Parses the first func of the text.  Throws std::runtime_error("mlir:<line>: ...").
 MlirFunc parseMlirText(const std::string &text);
+
+// The function back as text in the same generic syntax (what parseMlirText reads and what the
+// reference's tools read): numbers keep the type they were written with (i32 / f32 when they
+// had none), floats print as %e where that reads back to the same float and as their bit
+// pattern otherwise, attribute values the reader did not understand are written back verbatim.
+std::string printMlir(const MlirFunc &func);
+// the type of a tensor of `shape` and element type `elem` ("f32", "si8", ...)
+MlirType tensorType(const std::vector<int64_t> &shape, const std::string &elem);
 
 struct MlirWeight {
   std::string name;               // key in the weight file

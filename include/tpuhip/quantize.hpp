@@ -60,7 +60,7 @@ void quantizeLeakyRelu(float negative_slope, float threshold_x, float threshold_
 // 256-entry tables of the table-lookup activations (quantizeInt8LutOps, QuantizeInt8.cpp:531-621),
 // index = the two's-complement byte of the int8 input.  scale / bias: the op attributes of
 // sigmoid, exp and softplus (1 and 0 when the op has none); coeff: the exponent of pow.
-enum class LutKind { Sigmoid, TanH, Exp, Elu, Swish, SoftPlus, Log, Pow };
+enum class LutKind { Sigmoid, TanH, Exp, Elu, Swish, SoftPlus, Log, Pow, Mish };
 void quantizeLutTable(LutKind kind, float threshold_x, float threshold_y, float scale, float bias,
                       float coeff, float table256[256]);
 

@@ -13,6 +13,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -1540,9 +1541,12 @@ int conv_mode(const tpuhip_conv_weights *w) {
 }
 
 int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
-  static int cache[kMaxTiles][2][3];   // 0 = not asked yet
+  // 0 = not asked yet.  Contexts on several host threads may ask at once: every writer
+  // stores the same value, so relaxed atomics are all that is needed.
+  static std::atomic<int> cache[kMaxTiles][2][3];
   const int mode = conv_mode(w);
-  int &c = cache[w->tile][w->fast ? 1 : 0][mode];
+  std::atomic<int> &slot = cache[w->tile][w->fast ? 1 : 0][mode];
+  int c = slot.load(std::memory_order_relaxed);
   if (c == 0) {
     if (w->fast)
       c = mode == kModeSmallC ? persist_occupancy<true, kModeSmallC>(w->tile)
@@ -1552,6 +1556,7 @@ int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
       c = mode == kModeSmallC ? persist_occupancy<false, kModeSmallC>(w->tile)
           : mode == kModeUniform ? persist_occupancy<false, kModeUniform>(w->tile)
                                  : persist_occupancy<false, kModeGeneral>(w->tile);
+    slot.store(c, std::memory_order_relaxed);
   }
   return c;
 }

@@ -4,6 +4,7 @@
 
 #include <cctype>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -301,12 +302,14 @@ private:
         // a float written as its bit pattern
         const unsigned long long bits = std::strtoull(tok.c_str(), nullptr, 16);
         a.kind = MlirAttr::Float;
+        a.ty = ty;
         if (ty == "f64") { double d; std::memcpy(&d, &bits, 8); a.num = d; }
         else if (ty == "f32") { uint32_t w = (uint32_t)bits; float f; std::memcpy(&f, &w, 4); a.num = f; }
         else if (ty == "bf16") { uint32_t w = (uint32_t)bits << 16; float f; std::memcpy(&f, &w, 4); a.num = f; }
         else fail("f16 bit patterns are not supported");
         return a;
       }
+      a.ty = ty;
       if (real || (!ty.empty() && ty[0] == 'f') || ty == "bf16") {
         a.kind = MlirAttr::Float;
         a.num = std::strtod(tok.c_str(), nullptr);
@@ -493,6 +496,154 @@ std::string quant_of_elem(const std::string &elem) {
 MlirFunc parseMlirText(const std::string &text) {
   Reader r(text);
   return r.module();
+}
+
+namespace {
+
+std::string quote(const std::string &v) {
+  std::string out = "\"";
+  for (unsigned char c : v) {
+    if (c == '"' || c == '\\') { out += '\\'; out += (char)c; }
+    else if (c == '\n') out += "\\n";
+    else if (c == '\t') out += "\\t";
+    else if (c < 0x20 || c == 0x7f) {
+      static const char hex[] = "0123456789ABCDEF";
+      out += '\\'; out += hex[c >> 4]; out += hex[c & 15];
+    } else out += (char)c;
+  }
+  return out + "\"";
+}
+
+std::string print_float(double num, const std::string &ty) {
+  char buf[64];
+  if (ty == "f64") {
+    std::snprintf(buf, sizeof buf, "%.17e", num);
+    return std::string(buf) + " : f64";
+  }
+  const float f = (float)num;
+  std::snprintf(buf, sizeof buf, "%.6e", (double)f);
+  if (!std::isfinite(f) || (float)std::strtod(buf, nullptr) != f) {
+    uint32_t w;
+    std::memcpy(&w, &f, 4);
+    std::snprintf(buf, sizeof buf, "0x%08X", w);
+  }
+  return std::string(buf) + " : " + (ty.empty() || ty == "bf16" || ty == "f16" ? "f32" : ty);
+}
+
+void print_attr(const MlirAttr &a, std::string &out);
+
+void print_dict(const MlirAttr &d, std::string &out) {
+  out += '{';
+  bool first = true;
+  for (auto &f : d.fields) {
+    if (!first) out += ", ";
+    first = false;
+    bool plain = !f.first.empty() && !std::isdigit((unsigned char)f.first[0]);
+    for (char c : f.first) plain = plain && (std::isalnum((unsigned char)c) || c == '_' || c == '.' || c == '$');
+    out += plain ? f.first : quote(f.first);
+    if (f.second.kind != MlirAttr::Unit) {
+      out += " = ";
+      print_attr(f.second, out);
+    }
+  }
+  out += '}';
+}
+
+void print_attr(const MlirAttr &a, std::string &out) {
+  switch (a.kind) {
+    case MlirAttr::Int: {
+      char buf[48];
+      std::snprintf(buf, sizeof buf, "%lld", (long long)a.num);
+      out += buf;
+      out += " : " + (a.ty.empty() ? std::string("i32") : a.ty);
+      break;
+    }
+    case MlirAttr::Float: out += print_float(a.num, a.ty); break;
+    case MlirAttr::Bool: out += a.num != 0 ? "true" : "false"; break;
+    case MlirAttr::String: out += quote(a.str); break;
+    case MlirAttr::Array: {
+      out += '[';
+      for (size_t k = 0; k < a.items.size(); ++k) {
+        if (k) out += ", ";
+        print_attr(a.items[k], out);
+      }
+      out += ']';
+      break;
+    }
+    case MlirAttr::Dict: print_dict(a, out); break;
+    case MlirAttr::Unit: out += "unit"; break;
+    case MlirAttr::Other: out += a.str; break;
+  }
+}
+
+std::string type_list(const std::vector<MlirType> &t) {
+  std::string out;
+  for (size_t k = 0; k < t.size(); ++k) out += (k ? ", " : "") + t[k].text;
+  return out;
+}
+
+// "5#1" -> "%5#1"
+std::string use(const std::string &id) { return "%" + id; }
+
+}  // namespace
+
+MlirType tensorType(const std::vector<int64_t> &shape, const std::string &elem) {
+  MlirType t;
+  t.shaped = true;
+  t.shape = shape;
+  t.elem = elem;
+  t.text = "tensor<";
+  for (auto d : shape) t.text += (d < 0 ? std::string("?") : std::to_string(d)) + "x";
+  t.text += elem + ">";
+  return t;
+}
+
+std::string printMlir(const MlirFunc &f) {
+  std::string out = "module {\n  func @" + f.name + "(";
+  for (size_t k = 0; k < f.args.size(); ++k)
+    out += (k ? ", " : "") + use(f.args[k].first) + ": " + f.args[k].second.text;
+  out += ")";
+  if (f.results.size() == 1) out += " -> " + f.results[0].text;
+  else if (f.results.size() > 1) out += " -> (" + type_list(f.results) + ")";
+  if (!f.attrs.fields.empty()) {
+    out += " attributes ";
+    print_dict(f.attrs, out);
+  }
+  out += " {\n";
+  for (auto &o : f.ops) {
+    out += "    ";
+    if (o.opname == "std.return") {
+      out += "return";
+      if (!o.operands.empty()) {
+        out += ' ';
+        for (size_t k = 0; k < o.operands.size(); ++k) out += (k ? ", " : "") + use(o.operands[k]);
+        out += " : " + type_list(o.operand_types);
+      }
+      out += '\n';
+      continue;
+    }
+    if (!o.results.empty()) {
+      // "5#0", "5#1" were written as %5:2
+      const size_t hash = o.results[0].find('#');
+      if (hash != std::string::npos)
+        out += use(o.results[0].substr(0, hash)) + ":" + std::to_string(o.results.size());
+      else
+        for (size_t k = 0; k < o.results.size(); ++k) out += (k ? ", " : "") + use(o.results[k]);
+      out += " = ";
+    }
+    out += quote(o.opname) + "(";
+    for (size_t k = 0; k < o.operands.size(); ++k) out += (k ? ", " : "") + use(o.operands[k]);
+    out += ")";
+    if (!o.attrs.fields.empty()) {
+      out += ' ';
+      print_dict(o.attrs, out);
+    }
+    out += " : (" + type_list(o.operand_types) + ") -> ";
+    out += o.result_types.size() == 1 ? o.result_types[0].text : "(" + type_list(o.result_types) + ")";
+    out += '\n';
+  }
+  out += "  }\n}\n";
+  return out;
 }
 
 MlirModule moduleFromMlir(const MlirFunc &func) {

@@ -250,6 +250,15 @@ void quantizeLutTable(LutKind kind, float threshold_x, float threshold_y, float 
       index = in * threshold_x / 127.0;
       out = (scale * logf(expf(index) + 1) + bias) * 127.0 / threshold_y;
       break;
+    case LutKind::Mish: {
+      // my_mish_activate (lib/Dialect/TPU/Interpreter/NativeCpuImplementation.cpp:527-537):
+      // x * tanh(softplus(x)), all in float, tanh as 2 / (1 + exp(-2 s)) - 1
+      index = in * threshold_x / 127.0;
+      const float xv = (float)index;
+      const float sp = logf(expf(xv) + 1);
+      out = xv * (2 / (1 + expf(-2 * sp)) - 1) * 127.0 / threshold_y;
+      break;
+    }
     }
     // INT8(): floor(x + 0.5) clamped (QuantizeInt8.cpp:48-51); a NaN (log of a negative
     // input) passes through both std::min and std::max as their first argument does

@@ -1,8 +1,11 @@
 // C ABI over the host-side quantisation arithmetic: exceptions become status codes.
+#include <cstring>
 #include <stdexcept>
+#include <string>
 
 #include "tpuhip.h"
 #include "tpuhip/quantize.hpp"
+#include "tpuhip/quantize_pass.hpp"
 
 namespace tpuhip {
 int set_error(int status, const char *fmt, ...);
@@ -83,8 +86,24 @@ int tpuhip_quantize_lut_table(int kind, float threshold_x, float threshold_y, fl
                               float coeff, float *table256) {
   QGUARD({
     if (!table256) throw std::runtime_error("quantize_lut_table: NULL argument");
-    if (kind < 0 || kind > (int)LutKind::Pow) throw std::runtime_error("quantize_lut_table: unknown kind");
+    if (kind < 0 || kind > (int)LutKind::Mish) throw std::runtime_error("quantize_lut_table: unknown kind");
     quantizeLutTable((LutKind)kind, threshold_x, threshold_y, scale, bias, coeff, table256);
+  })
+}
+
+int tpuhip_quantize_mlir_files(const char *in_mlir, const char *calibration_table, const char *out_mlir,
+                               const char *out_weights, char *missing, size_t capacity, size_t *needed) {
+  QGUARD({
+    if (!in_mlir || !calibration_table || !out_mlir) throw std::runtime_error("quantize_mlir_files: NULL path");
+    std::string text;
+    for (auto &name : quantizeFiles(in_mlir, calibration_table, out_mlir, out_weights ? out_weights : ""))
+      text += name + "\n";
+    if (needed) *needed = text.size() + 1;
+    if (missing && capacity) {
+      const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+      std::memcpy(missing, text.data(), n);
+      missing[n] = '\0';
+    }
   })
 }
 

@@ -23,6 +23,9 @@ _POOL_PARAM = ["kernel_h", "kernel_w", "padding_t", "padding_b", "padding_l", "p
 _BOOLS = {"do_relu", "is_dw", "with_bias", "count_include_pad", "input_transpose", "output_transpose",
           "fused_relu", "do_early_stride"}
 _FLOATS = {"scale", "min", "max", "negative_slope", "const_val", "threshold"}
+# the activations that become a table lookup in INT8: input, table, mantissa table
+_LUT_OPS = {"tpu.sigmoid", "tpu.tanh", "tpu.exp", "tpu.elu", "tpu.swish", "tpu.softplus", "tpu.log", "tpu.pow",
+            "tpu.mish", "tpu.sqrt"}
 # numbered scalars of an op description <-> array attributes of the dialect
 _ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4}
 # flag scalars <-> string attributes
@@ -118,7 +121,7 @@ def write_mlir(graph, mlir_path, weight_file=None, func_name="tpu_func"):
             continue
         roles = _WEIGHT_OPERANDS.get(op.type)
         if roles is None:
-            roles = _WEIGHT_OPERANDS["tpu.lut"] if "table" in op.weights else []
+            roles = _WEIGHT_OPERANDS["tpu.lut"] if "table" in op.weights or op.type in _LUT_OPS else []
         opd, opd_t = [ids[s] for s in op.inputs], [types[s] for s in op.inputs]
         for role in roles:
             if role is None or role not in op.weights:

@@ -7,7 +7,7 @@ import numpy as np
 
 from . import capi
 
-LUT_KINDS = {"sigmoid": 0, "tanh": 1, "exp": 2, "elu": 3, "swish": 4, "softplus": 5, "log": 6, "pow": 7}
+LUT_KINDS = {"sigmoid": 0, "tanh": 1, "exp": 2, "elu": 3, "swish": 4, "softplus": 5, "log": 6, "pow": 7, "mish": 8}
 
 
 def _f32(a):
@@ -90,3 +90,17 @@ def quantize_lut_table(kind, threshold_x, threshold_y, scale=1.0, bias=0.0, coef
     capi.check(lib, lib.tpuhip_quantize_lut_table(LUT_KINDS[kind], threshold_x, threshold_y, scale, bias, coeff,
                                                   out.ctypes.data))
     return out
+
+
+def quantize_files(in_mlir, calibration_table, out_mlir, out_weights=None, lib=None):
+    """``tpuc-opt --import-calibration-table --calibration-table T --tpu-quant in.mlir -o out.mlir``:
+    an fp32 TPU-dialect file + its weight .npz + a calibration table -> the INT8 file ``module.load``
+    runs, with its own weight file.  Returns the names of the ops the table had no threshold for."""
+    import ctypes as C
+    lib = lib or capi.bind()
+    args = [str(in_mlir).encode(), str(calibration_table).encode(), str(out_mlir).encode(),
+            None if out_weights is None else str(out_weights).encode()]
+    buf = C.create_string_buffer(1 << 16)
+    need = C.c_size_t(0)
+    capi.check(lib, lib.tpuhip_quantize_mlir_files(*args, buf, len(buf), C.byref(need)))
+    return [n for n in buf.value.decode().split("\n") if n]
