@@ -190,13 +190,13 @@ def _index(i, thx):
     return v, Decimal(float(np.float32(v) * np.float32(thx))) / Decimal(127)
 
 
-@pytest.mark.parametrize("kind", ["sigmoid", "tanh", "exp", "elu", "swish", "softplus", "log"])
+@pytest.mark.parametrize("kind", ["sigmoid", "tanh", "exp", "elu", "swish", "softplus", "log", "mish"])
 def test_activation_tables_against_40_digit_arithmetic(kind):
     thx, thy, scale, bias = 5.3, (1.0 if kind in ("sigmoid", "tanh") else 6.1), 1.0, 0.0
     if kind == "exp":
         thx, thy = 2.0, 7.5
     table = Q.quantize_lut_table(kind, thx, thy, scale, bias)
-    margin = Decimal("1e-2") if kind == "softplus" else Decimal("1e-9")    # softplus runs in float32
+    margin = Decimal("1e-2") if kind in ("softplus", "mish") else Decimal("1e-9")    # these run in float32
     decided = 0
     for i in range(256):
         v, x = _index(i, thx)
@@ -216,6 +216,9 @@ def test_activation_tables_against_40_digit_arithmetic(kind):
             y = x / (1 + (-x).exp())
         elif kind == "softplus":
             y = (x.exp() + 1).ln()
+        elif kind == "mish":
+            e = (2 * (x.exp() + 1).ln()).exp()          # x * tanh(softplus(x))
+            y = x * (e - 1) / (e + 1)
         else:
             y = x.ln()
         t = y * Decimal(127) / Decimal(float(np.float32(thy)))
@@ -225,7 +228,7 @@ def test_activation_tables_against_40_digit_arithmetic(kind):
             continue                            # too close to a rounding tie to call
         decided += 1
         assert table[i] == want, (kind, i, v, float(t))
-    assert decided >= (120 if kind == "log" else 250)
+    assert decided >= (120 if kind == "log" else 240 if kind == "mish" else 250)
     assert len(np.unique(table[~np.isnan(table)])) > 20
 
 
