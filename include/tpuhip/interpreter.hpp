@@ -245,8 +245,11 @@ public:
   ~FullyConnectedOpKernel() override;
   void invoke() override;
   int m = 0, k = 0, n = 0;
+  // "fc/<conv tile variant it runs as>" (the variant is timed on first use)
+  const char *algo_name() const;
 
 private:
+  mutable std::string algo_text;
   tpuhip_conv_weights *packed = nullptr;
   SyncedData input_data, output_data;
 };

@@ -570,6 +570,11 @@ FullyConnectedOpKernel::~FullyConnectedOpKernel() {
   if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
 }
 
+const char *FullyConnectedOpKernel::algo_name() const {
+  algo_text = std::string("fc/") + tpuhip_conv2d_algo_name(packed);
+  return algo_text.c_str();
+}
+
 void FullyConnectedOpKernel::invoke() {
   ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
 }

@@ -207,7 +207,7 @@ const char *tpuhip_module_kernel_algo(tpuhip_module *m, int i) {
   auto *k = kernel_at(m, i);
   if (!k) return nullptr;
   if (auto *c = dynamic_cast<Conv2DOpKernel *>(k)) return c->algo_name();
-  if (dynamic_cast<FullyConnectedOpKernel *>(k)) return "fc";
+  if (auto *f = dynamic_cast<FullyConnectedOpKernel *>(k)) return f->algo_name();
   return "";
 }
 

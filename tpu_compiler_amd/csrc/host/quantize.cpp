@@ -74,12 +74,23 @@ int8_t findRShiftAndMultiplierFromQScale(double qscale, uint32_t *multiplier, bo
   return 0;
 }
 
+namespace {
+// qscale * 2^rshift as the uint32 the reference's `(uint32_t)(qscale * (1 << rshift))` yields.
+// That expression is undefined from rshift 31 on (and for products outside uint32), which only
+// a degenerate threshold reaches; here those cases give the exact product, clamped.
+uint32_t scaled_u32(double qscale, int rshift) {
+  const double v = rshift < 31 ? qscale * (1 << rshift) : std::ldexp(qscale, rshift);
+  if (!(v > 0)) return 0;
+  return v >= 4294967295.0 ? 4294967295u : (uint32_t)v;
+}
+}  // namespace
+
 uint32_t findMultiplierU32FromQScaleAndRShift(double qscale, int8_t rshift) {
-  return (uint32_t)(qscale * (1 << rshift));
+  return scaled_u32(qscale, rshift);
 }
 
 int8_t findMultiplierI8FromQScaleAndRShift(double qscale, int8_t rshift) {
-  return (int8_t)(uint32_t)(qscale * (1 << rshift));
+  return (int8_t)scaled_u32(qscale, rshift);
 }
 
 double findQScaleForFilter(float max_filter, float threshold_y, float threshold_x, int quant_bitwidth) {
