@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--batch", type=int, default=0,
+                    help="images per step instead of the configuration's own batch (a different workload: "
+                         "named as such in config.workload, recorded tiles not applied)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-layer", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--save-tiles", default="", help="write the conv tile chosen for every layer")
@@ -80,9 +83,9 @@ def main():
     from tpu_compiler_amd import graphs, module
 
     graph_fn = graphs.CONFIGS[args.config]
-    g = graph_fn()
+    g = graph_fn(batch=args.batch) if args.batch > 0 else graph_fn()
     batch = g.input_op().shape[0]
-    if not args.tiles and not args.autotune and not args.save_tiles:
+    if not args.tiles and not args.autotune and not args.save_tiles and args.batch <= 0:
         recorded = os.path.join(ROOT, RECORDED_TILES.get(args.config, ""))
         if os.path.isfile(recorded):
             args.tiles = recorded
