@@ -21,6 +21,12 @@ def check_through_files(g, x, want, tmp_path):
     m = module()
     m.load(str(path))
     assert m.get_weight_file_path() == os.path.basename(wfile)
+    import contextlib
+    import io
+    err = io.StringIO()
+    with contextlib.redirect_stderr(err):
+        m.dump()
+    assert err.getvalue() == open(path).read()
     assert [(i["name"], i["type"], i["quant"]) for i in m.op_info] == [(o.name, o.type, o.quant) for o in g.ops]
     assert list(m.get_output_details()) == list(g.outputs)
     m.set_tensor(g.input_op().name, np.asarray(x, np.float32))
@@ -136,6 +142,14 @@ def test_module_api_semantics():
     assert m.get_output_details() == ["fc1000"]
     assert m.tensor_dtype("conv1") == "INT8"
     assert m.tensor_shape("pool5_flat") == (1, 2048)
+    import contextlib
+    import io
+    err = io.StringIO()
+    with contextlib.redirect_stderr(err):
+        m.dump()
+    assert "tpu.conv_2d conv1 INT8" in err.getvalue() and err.getvalue().count("\n") == len(g.ops)
+    with pytest.raises(NotImplementedError):
+        m.set_plugin("plugin.so")
     x0 = g.input_op().data
     x1 = np.ascontiguousarray(x0[:, :, ::-1, :])
     want0 = oracle_graph.run(g)

@@ -56,6 +56,7 @@ class module:
         self.h = h
         self.op_info = []
         self.graph = None
+        self._mlir_path = None
 
     def close(self):
         if self.h:
@@ -77,6 +78,7 @@ class module:
         name, like pymlir, or for a graph object built in Python."""
         if isinstance(graph, (str, os.PathLike)):
             self.graph = None
+            self._mlir_path = os.fspath(graph)
             self._ck(self.lib.tpuhip_module_load_mlir(self.h, os.fspath(graph).encode(),
                                                       target_op.encode() if target_op else None))
             self.op_info = []
@@ -87,6 +89,7 @@ class module:
                                      "quant": q.value.decode()})
             return
         self.graph = graph
+        self._mlir_path = None
         self._ck(self.lib.tpuhip_module_clear_ops(self.h))
         self.op_info = []
         for op in graph.ops:
@@ -118,6 +121,21 @@ class module:
         ra = (C.c_char_p * max(len(rets), 1))(*rets)
         self._ck(self.lib.tpuhip_module_set_returns(self.h, ra, len(rets)))
         self._ck(self.lib.tpuhip_module_load(self.h, target_op.encode() if target_op else None))
+
+    def dump(self):
+        """pymlir's module.dump(): the loaded module as text on stderr -- the file's own text when it
+        was loaded from a file, else one line per op of the Python-built graph"""
+        import sys
+        if self._mlir_path:
+            sys.stderr.write(open(self._mlir_path).read())
+        elif self.graph is not None:
+            for op in self.graph.ops:
+                sys.stderr.write("%s %s %s %s %s <- %s\n" % (op.type, op.name, op.quant, op.param_type,
+                                                              list(op.shape), ", ".join(op.inputs)))
+
+    def set_plugin(self, path):
+        """pymlir's module.set_plugin(): custom-op plugins are not part of this build"""
+        raise NotImplementedError("custom op plugins are not supported")
 
     def get_weight_file_path(self):
         return (self.lib.tpuhip_module_weight_file(self.h) or b"").decode()
