@@ -296,11 +296,13 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
  *   TILE                  p[0] axis, p[1] tiles
  *   REVERSE               p[0] axis
  *   SHUFFLE_CHANNEL       p[0] group
- *   DEPTH_TO_SPACE        p[0] upscale factor, p[1] 1 = "DCR" mode, 0 = CRD */
+ *   DEPTH_TO_SPACE        p[0] upscale factor, p[1] 1 = "DCR" mode, 0 = CRD
+ *   SWAP_CHANNEL          p[0..ic-1] channel_order (output channel k is input channel p[k];
+ *                         at most 8 channels; core/swap_channel.cpp:21-34) */
 enum {
   TPUHIP_MOVE_PAD_CONST = 0, TPUHIP_MOVE_PAD_EDGE = 1, TPUHIP_MOVE_CROP = 2, TPUHIP_MOVE_PERMUTE = 3,
   TPUHIP_MOVE_REORG = 4, TPUHIP_MOVE_TILE = 5, TPUHIP_MOVE_REVERSE = 6,
-  TPUHIP_MOVE_SHUFFLE_CHANNEL = 7, TPUHIP_MOVE_DEPTH_TO_SPACE = 8
+  TPUHIP_MOVE_SHUFFLE_CHANNEL = 7, TPUHIP_MOVE_DEPTH_TO_SPACE = 8, TPUHIP_MOVE_SWAP_CHANNEL = 9
 };
 typedef struct tpuhip_move_desc {
   int kind;
@@ -483,7 +485,7 @@ int tpuhip_quantize_lut_table(int kind, float threshold_x, float threshold_y, fl
  * fully_connected, eltwise add / max / min / mul, broadcast add / sub / mul, pool_avg_2d,
  * pool_max_2d, relu, leaky_relu, prelu, clip, concat, the table activations (sigmoid, tanh, exp, elu,
  * swish, softplus, log, pow, mish), upsample, pad, crop, permute, reorg, pixelshuffle, tile,
- * reverse, shuffle_channel, reshape; anything else is refused by name.  `missing` (may be NULL)
+ * reverse, shuffle_channel, swap_channel, mul_const, reshape; anything else is refused by name.  `missing` (may be NULL)
  * receives, one per line, the ops the table had no threshold for (the reference warns and goes
  * on); *needed = its length + 1. */
 int tpuhip_quantize_mlir_files(const char *in_mlir, const char *calibration_table, const char *out_mlir,

@@ -349,6 +349,22 @@ public:
   ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
 };
 
+// INT8 ZeroMask (core/zero_mask.cpp:8-35): 127 where the input is non-zero (positive) or zero
+// (not positive), else 0.  A function of one byte, so it runs as a table.
+class ZeroMaskOpKernel : public LutOpKernel {
+public:
+  static constexpr const char *OpName = "CPUZeroMaskOp";
+  ZeroMaskOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+};
+
+// INT8 MulConst (core/eltwise.cpp:360-401): F32ToInt8(x * const_val, nearest even), optional
+// ReLU; const_val is 1, -1 or 0 after the quantisation pass.  Also a table.
+class MulConstOpKernel : public LutOpKernel {
+public:
+  static constexpr const char *OpName = "CPUMulConstOp";
+  MulConstOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+};
+
 // operands: [0]input [1]slope (c values) [2..5]unused [6]rshift_pos [7]multiplier_pos
 // [8]rshift_neg (core/activation.cpp:165-183).  Realised as one 256-entry table per channel.
 class PReluOpKernel : public CPUOpKernel {
@@ -455,6 +471,7 @@ TPUHIP_MOVE_KERNEL(TileOpKernel, "CPUTileOp")                        // core/til
 TPUHIP_MOVE_KERNEL(ReverseOpKernel, "CPUReverseOp")                  // core/reverse.cpp:7-42
 TPUHIP_MOVE_KERNEL(ShuffleChannelOpKernel, "CPUShuffleChannelOp")    // core/shuffle_channel.cpp:7-48
 TPUHIP_MOVE_KERNEL(DepthToSpaceOpKernel, "CPUPixelShuffleOp")        // core/depthtospace.cpp:60-80
+TPUHIP_MOVE_KERNEL(SwapChannelOpKernel, "CPUSwapChannelOp")          // core/swap_channel.cpp:8-35
 #undef TPUHIP_MOVE_KERNEL
 
 // tpu.reshape whose source and result are not the same bytes in channels-last

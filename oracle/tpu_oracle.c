@@ -661,6 +661,42 @@ void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *is, int r,
         }
 }
 
+/* SwapChannelOpKernel::invoke (core/swap_channel.cpp:21-34): output channel j is input channel
+ * order[j], whole frames copied */
+void orc_swap_channel_i8(const int8_t *x, int8_t *y, const int64_t *s, const int *order) {
+  const int64_t frame = s[2] * s[3], batch = frame * s[1];
+  for (int64_t i = 0; i < s[0]; ++i)
+    for (int64_t j = 0; j < s[1]; ++j)
+      memcpy(y + i * batch + frame * j, x + i * batch + frame * order[j], (size_t)frame);
+}
+
+/* ZeroMaskOpKernel::invoke (core/zero_mask.cpp:19-33), INT8: the mask value is 127 */
+void orc_zero_mask_i8(const int8_t *x, int8_t *y, int64_t n, int positive) {
+  for (int64_t i = 0; i < n; ++i)
+    y[i] = x[i] == 0 ? (positive ? 0 : 127) : (positive ? 127 : 0);
+}
+
+/* F32ToInt(v, 0) + F32ToInt8 (QuantizationArithmetic.cpp:917-947): nearest, ties to even, on
+ * |v|; then saturated */
+static int8_t f32_to_int8_nearest_even(float v) {
+  float integer;
+  const float fraction = modff(fabsf(v), &integer);
+  int32_t q = (int32_t)integer;
+  if (fraction > 0.5f) q += 1;
+  else if (fraction == 0.5f && (q & 1)) q += 1;
+  if (v < 0) q = -q;
+  return (int8_t)(q > 127 ? 127 : q < -128 ? -128 : q);
+}
+
+/* MulConstOpKernel::invoke (core/eltwise.cpp:386-401), INT8: F32ToInt8(x * const_val, 0), then
+ * the optional ReLU */
+void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, int do_relu) {
+  for (int64_t i = 0; i < n; ++i) {
+    int8_t v = f32_to_int8_nearest_even((float)x[i] * const_val);
+    y[i] = do_relu && v < 0 ? 0 : v;
+  }
+}
+
 /* ------------------------------------------------------------------------- */
 /* transposed convolution                                                     */
 /* ------------------------------------------------------------------------- */

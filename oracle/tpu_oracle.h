@@ -179,6 +179,10 @@ void orc_reverse_i8(const int8_t *x, int8_t *y, const int64_t *shape, int axis);
 /* core/shuffle_channel.cpp:21-48 */
 void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, int group);
 /* core/depthtospace.cpp:8-58 (pixelshuffle), dcr_mode as in :60 */
+/* core/swap_channel.cpp:21-34, core/zero_mask.cpp:19-33, core/eltwise.cpp:386-401 (INT8 branches) */
+void orc_swap_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, const int *order);
+void orc_zero_mask_i8(const int8_t *x, int8_t *y, int64_t n, int positive);
+void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, int do_relu);
 void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int upscale,
                            int dcr_mode);
 

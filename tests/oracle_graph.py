@@ -26,6 +26,7 @@ _BINARY = {"tpu.eltwise_max": O.BIN_MAX, "tpu.eltwise_min": O.BIN_MIN, "tpu.eltw
 
 
 _MOVES = {"tpu.pad": ("pad_const", ["pads*"]), "tpu.crop": ("crop", ["crop_offset*", "steps*"]),
+          "tpu.swap_channel": ("swap_channel", ["channel_order*"]),
           "tpu.permute": ("permute", ["order*"]), "tpu.reorg": ("reorg", ["stride"]),
           "tpu.tile": ("tile", ["axis", "tiles"]), "tpu.reverse": ("reverse", ["axis"]),
           "tpu.shuffle_channel": ("shuffle_channel", ["group"]),
@@ -103,7 +104,8 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             params = []
             for k in keys:
                 if k.endswith("*"):
-                    base, cnt, dflt = k[:-1], (8 if k.startswith("pads") else 4), (1 if k.startswith("steps") else 0)
+                    base, dflt = k[:-1], (1 if k.startswith("steps") else 0)
+                    cnt = 8 if k.startswith("pads") else ins[0].shape[1] if k.startswith("channel_order") else 4
                     params += [int(a.get(base + str(i), dflt)) for i in range(cnt)]
                 else:
                     params.append(int(a.get(k, 0)))
@@ -127,6 +129,10 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             y = O.lut_i8(ins[0], op.weights["table"])
         elif t == "tpu.relu":
             y = O.relu_i8(ins[0])
+        elif t == "tpu.zero_mask":
+            y = O.zero_mask_i8(ins[0], op.attrs.get("positive", 0))
+        elif t == "tpu.mul_const":
+            y = O.mul_const_i8(ins[0], op.attrs["const_val"], op.attrs.get("do_relu", 0))
         elif t == "tpu.upsample":
             y = O.upsample_i8(ins[0], int(op.attrs["scale_h"]), int(op.attrs["scale_w"]))
         elif t == "tpu.concat":

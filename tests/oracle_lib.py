@@ -86,6 +86,9 @@ def _load():
     lib.orc_reverse_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_shuffle_channel_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_depth_to_space_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
+    lib.orc_swap_channel_i8.argtypes = [i8p, i8p, i64p, C.POINTER(C.c_int)]
+    lib.orc_zero_mask_i8.argtypes = [i8p, i8p, C.c_int64, C.c_int]
+    lib.orc_mul_const_i8.argtypes = [i8p, i8p, C.c_int64, C.c_float, C.c_int]
     lib.orc_pool_max_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc)]
     lib.orc_pool_avg_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc), C.c_float, C.c_float]
     lib.orc_leaky_relu_i8.argtypes = [i8p, i8p, C.c_size_t] + [C.c_float] * 4
@@ -269,7 +272,7 @@ def move_i8(kind, x, params, out_shape=None):
         out = (s[0], s[1] * p[0] * p[0], s[2] // p[0], s[3] // p[0])
     elif kind == "tile":
         out = tuple(s[k] * (p[1] if k == p[0] else 1) for k in range(4))
-    elif kind in ("reverse", "shuffle_channel"):
+    elif kind in ("reverse", "shuffle_channel", "swap_channel"):
         out = s
     else:
         out = (s[0], s[1] // (p[0] * p[0]), s[2] * p[0], s[3] * p[0])
@@ -289,13 +292,29 @@ def move_i8(kind, x, params, out_shape=None):
         lib.orc_reverse_i8(xp, yp, _shape64(s), p[0])
     elif kind == "shuffle_channel":
         lib.orc_shuffle_channel_i8(xp, yp, _shape64(s), p[0])
+    elif kind == "swap_channel":
+        lib.orc_swap_channel_i8(xp, yp, _shape64(s), _ints(p[:s[1]]))
     else:
         lib.orc_depth_to_space_i8(xp, yp, _shape64(s), p[0], p[1])
     return y
 
 
 MOVE_KINDS = ["pad_const", "pad_edge", "crop", "permute", "reorg", "tile", "reverse",
-              "shuffle_channel", "depth_to_space"]
+              "shuffle_channel", "depth_to_space", "swap_channel"]
+
+
+def zero_mask_i8(x, positive):
+    x = _i8(x)
+    y = np.empty(x.shape, np.int8)
+    lib.orc_zero_mask_i8(_p(x, C.c_int8), _p(y, C.c_int8), x.size, int(bool(positive)))
+    return y
+
+
+def mul_const_i8(x, const_val, do_relu=False):
+    x = _i8(x)
+    y = np.empty(x.shape, np.int8)
+    lib.orc_mul_const_i8(_p(x, C.c_int8), _p(y, C.c_int8), x.size, float(const_val), int(bool(do_relu)))
+    return y
 
 
 def prelu_i8(x, slope, rshift_pos, multiplier_pos, rshift_neg):

@@ -437,6 +437,45 @@ def test_graph_with_data_movement_ops_matches_the_oracle(tmp_path):
     check_through_files(g, g.input_op().data, want, tmp_path)
 
 
+@pytest.mark.parametrize("fuse", [1, 0])
+def test_graph_with_swap_channel_mul_const_and_zero_mask(tmp_path, fuse):
+    """BGR<->RGB swap in front of a stem conv, then the two byte-wise ops that run as tables
+    (fused into the conv in front of them when fusion is on)"""
+    b = graphs.Builder("byte_ops", graphs.BASE_SEED + 81, 2, (6, 12))
+    x = b.input("input", 3, 18, 14)
+    g = b.g
+    g.add(graphs.Op("tpu.swap_channel", "bgr", [x], g.by_name[x].shape,
+                    dict(channel_order0=2, channel_order1=1, channel_order2=0)))
+    b.cal["bgr"] = b.cal[x][:, [2, 1, 0]]
+    c1 = b.conv("c1", "bgr", 24, 3, relu=False)
+    c2 = b.conv("c2", "bgr", 24, 3, relu=False)
+    shp = g.by_name[c1].shape
+    g.add(graphs.Op("tpu.mul_const", "neg", [c1], shp, dict(const_val=-1.0, do_relu=1)))
+    g.add(graphs.Op("tpu.zero_mask", "mask", [c2], shp, dict(positive=1)))
+    g.add(graphs.Op("tpu.zero_mask", "hole", ["neg"], shp, dict(positive=0)))
+    g.add(graphs.Op("tpu.eltwise_min", "both", ["mask", "hole"], shp, dict(do_relu=0),
+                    dict(rshift=np.array([0], np.float32), multiplier=np.array([1, 1], np.float32)),
+                    "RSHIFT_AND_M_I8"))
+    g.outputs = ["both", "neg"]
+    want = oracle_graph.run(g)
+    assert np.array_equal(want["bgr"], g.input_op().data[:, [2, 1, 0]])
+    assert np.array_equal(want["neg"], np.clip(-want["c1"].astype(np.int64), 0, 127))
+    assert set(np.unique(want["mask"])) == {0, 127} and set(np.unique(want["hole"])) == {0, 127}
+    m = module()
+    m.set_option("keep_all_tensors", 1)
+    m.set_option("fuse_eltwise", fuse)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()
+    check_through_files(g, g.input_op().data, want, tmp_path)
+    g.ops[1].attrs["channel_order1"] = 3
+    with pytest.raises(capi.TpuHipError, match="channel_order"):
+        module().load(g)
+
+
 def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle(tmp_path):
     """uint8 image -> ScaleLut (per-channel 256-entry tables) -> conv"""
     rng = np.random.default_rng(6)

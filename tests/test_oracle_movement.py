@@ -65,6 +65,28 @@ def test_shuffle_channel_is_group_transpose():
     assert np.array_equal(O.move_i8("shuffle_channel", x, [g]), want)
 
 
+def test_swap_channel_is_fancy_indexing_of_the_channel_axis():
+    rng = np.random.default_rng(3)
+    x = rng.integers(-128, 128, (2, 3, 5, 4)).astype(np.int8)
+    for order in ([2, 1, 0], [0, 1, 2], [1, 1, 2]):          # a repeat is legal: frames are copied
+        assert np.array_equal(O.move_i8("swap_channel", x, order), x[:, order])
+
+
+def test_zero_mask_and_mul_const_on_every_byte():
+    x = np.arange(-128, 128).astype(np.int8).reshape(1, 256, 1, 1)
+    xi = x.astype(np.int64)
+    assert np.array_equal(O.zero_mask_i8(x, True), np.where(xi != 0, 127, 0))
+    assert np.array_equal(O.zero_mask_i8(x, False), np.where(xi == 0, 127, 0))
+    # the three constants the quantisation pass leaves, and fractions for the rounding rule:
+    # nearest, ties to even on the magnitude (numpy's rint), saturated; -(-128) saturates to 127
+    for c in (1.0, -1.0, 0.0, 0.5, -0.5, 1.5, 0.3):
+        want = np.clip(np.rint(xi.astype(np.float32) * np.float32(c)), -128, 127)
+        assert np.array_equal(O.mul_const_i8(x, c), want), c
+        assert np.array_equal(O.mul_const_i8(x, c, True), np.maximum(want, 0)), c
+    assert O.mul_const_i8(x, -1.0).ravel()[0] == 127
+    assert O.mul_const_i8(x, 0.5).ravel()[128 + 1] == 0 and O.mul_const_i8(x, 0.5).ravel()[128 + 3] == 2
+
+
 def test_depth_to_space_both_modes():
     x = rnd((2, 12, 3, 4), 7)
     r = 2

@@ -317,6 +317,32 @@ def test_pass_refuses_what_it_cannot_quantise(tmp_path):
         Q.quantize_files(tmp_path / "nope.mlir", tmp_path / "t", tmp_path / "o.mlir")
 
 
+def test_mul_const_and_swap_channel_through_the_pass(tmp_path):
+    g = graphs.Graph("mc", 0)
+    xin = graphs.Op("tpu.input", "input", [], (1, 3, 4, 4))
+    xin.quant = "NONE"
+    xin.data = np.zeros((1, 3, 4, 4), np.float32)
+    g.add(xin)
+    fp32_op(g, "tpu.swap_channel", "bgr", ["input"], (1, 3, 4, 4), dict(channel_order0=2, channel_order1=1, channel_order2=0))
+    fp32_op(g, "tpu.mul_const", "scaled", ["bgr"], (1, 3, 4, 4), dict(const_val=-2.5, do_relu=0))
+    g.outputs = ["scaled"]
+    path = tmp_path / "mc.mlir"
+    mlir_text.write_mlir(g, path)
+    open(tmp_path / "t", "w").write("input 2.0\nbgr 1.5\nscaled 3.0\n")
+    assert Q.quantize_files(path, tmp_path / "t", tmp_path / "o.mlir") == []
+    out = tmp_path / "o.mlir"
+    # the rules run in the reference's order: mul_const takes |const| times its input's threshold
+    # as the table gave it (1.5), and only afterwards does the pass-through swap_channel take its
+    # own input's (2.0); only the sign of the constant is left
+    assert f32_attr(out, "bgr", "threshold") == np.float32(2.0)
+    assert f32_attr(out, "scaled", "threshold") == np.float32(3.75)
+    assert f32_attr(out, "scaled", "const_val") == np.float32(-1.0)
+    assert f32_attr(out, "scaled_dequant", "scale") == np.float32(3.75) / np.float32(128)
+    ops, _, _ = describe(out)
+    assert ops["bgr"]["quant"] == ops["scaled"]["quant"] == "INT8"
+    assert "channel_order0=2" in ops["bgr"]["line"] and "channel_order2=0" in ops["bgr"]["line"]
+
+
 REF_GRAPHS = ["conv", "conv_1_oc", "deconv", "fc", "eltwise_add", "avg_pool", "max_pool", "relu", "concat",
               "broadcast_mul", "permute", "pixel_shuffle", "reorg", "reverse", "tile", "crop"]
 

@@ -273,6 +273,12 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {
       krnl = std::make_shared<ClipOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.zero_mask") {
+      krnl = std::make_shared<ZeroMaskOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.mul_const") {
+      krnl = std::make_shared<MulConstOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.swap_channel") {
+      krnl = std::make_shared<SwapChannelOpKernel>(*op, valueMapping, weightMapping);
     } else if (is_lut_op(t)) {
       krnl = std::make_shared<LutOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.relu") {

@@ -722,6 +722,16 @@ ShuffleChannelOpKernel::ShuffleChannelOpKernel(OpDesc &op, value_map_t &v, weigh
   desc.kind = TPUHIP_MOVE_SHUFFLE_CHANNEL;
   desc.p[0] = (int)op.attr("group");
 }
+SwapChannelOpKernel::SwapChannelOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "SwapChannel") {
+  desc.kind = TPUHIP_MOVE_SWAP_CHANNEL;
+  if (desc.ic > 8) fail("SwapChannel '" + name + "': at most 8 channels");
+  for (int k = 0; k < desc.ic; ++k) {
+    desc.p[k] = (int)op.attr("channel_order" + std::to_string(k));
+    if (desc.p[k] < 0 || desc.p[k] >= desc.ic)
+      fail("SwapChannel '" + name + "': channel_order[" + std::to_string(k) + "] = " + std::to_string(desc.p[k]));
+  }
+}
 DepthToSpaceOpKernel::DepthToSpaceOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
     : MoveOpKernel(op, v, w, "DepthToSpace") {
   desc.kind = TPUHIP_MOVE_DEPTH_TO_SPACE;
@@ -783,7 +793,8 @@ LutOpKernel::LutOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &we
   if (!input_data) fail(op.type + " '" + name + "': input missing");
   if (input_data->size() != output_data->size()) fail(op.type + " '" + name + "': shape mismatch");
   memset(table, 0, sizeof(table));
-  if (op.type != "tpu.leaky_relu" && op.type != "tpu.clip") {
+  if (op.type != "tpu.leaky_relu" && op.type != "tpu.clip" && op.type != "tpu.zero_mask" &&
+      op.type != "tpu.mul_const") {
     // y0_table_op = opdTensors[1] (core/activation.cpp:34-37): 256 float-stored int8 entries,
     // indexed by the two's-complement byte of the input
     auto y0 = opdTensors.size() > 1 ? opdTensors[1].weight : nullptr;
@@ -914,6 +925,33 @@ ClipOpKernel::ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &
                        f2u32(opdTensors[3].weight->at(0)), f2u32(opdTensors[4].weight->at(0)),
                        table),
      name.c_str());
+}
+
+ZeroMaskOpKernel::ZeroMaskOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : LutOpKernel(op, valueMapping, weightMapping) {
+  const bool positive = op.attr("positive", 0) != 0;
+  for (int i = 0; i < 256; ++i) {
+    const bool zero = (int8_t)i == 0;
+    table[i] = (int8_t)(zero ? (positive ? 0 : 127) : (positive ? 127 : 0));
+  }
+}
+
+MulConstOpKernel::MulConstOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : LutOpKernel(op, valueMapping, weightMapping) {
+  const float const_val = (float)op.attr("const_val");
+  const bool do_relu = op.attr("do_relu", 0) != 0;
+  for (int i = 0; i < 256; ++i) {
+    // F32ToInt(v, 0) on |v|: nearest, ties to even (QuantizationArithmetic.cpp:917-938), saturated
+    const float v = (float)(int8_t)i * const_val;
+    float integer;
+    const float fraction = std::modf(std::fabs(v), &integer);
+    int q = (int)integer;
+    if (fraction > 0.5f) q += 1;
+    else if (fraction == 0.5f && (q & 1)) q += 1;
+    if (v < 0) q = -q;
+    q = std::max(-128, std::min(127, q));
+    table[i] = (int8_t)(do_relu && q < 0 ? 0 : q);
+  }
 }
 
 ReluOpKernel::ReluOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)

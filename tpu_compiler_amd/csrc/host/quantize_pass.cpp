@@ -133,7 +133,7 @@ const std::set<std::string> kForward = {
 // quantizeInt8BypassOps users within the INT8 interpreter's op set (QuantizeInt8.cpp:1606-1640)
 const std::set<std::string> kBypass = {
     "tpu.crop", "tpu.pad", "tpu.permute", "tpu.pixelshuffle", "tpu.pool_max_2d", "tpu.relu", "tpu.reorg",
-    "tpu.reverse", "tpu.shuffle_channel", "tpu.tile", "tpu.upsample"};
+    "tpu.reverse", "tpu.shuffle_channel", "tpu.swap_channel", "tpu.tile", "tpu.upsample"};
 const std::map<std::string, LutKind> kLut = {
     {"tpu.sigmoid", LutKind::Sigmoid}, {"tpu.tanh", LutKind::TanH}, {"tpu.exp", LutKind::Exp},
     {"tpu.elu", LutKind::Elu}, {"tpu.swish", LutKind::Swish}, {"tpu.softplus", LutKind::SoftPlus},
@@ -246,6 +246,17 @@ std::vector<std::string> importCalibrationTable(MlirFunc &func, const Calibratio
     const float ty = g.threshold(&o), tx = g.threshold(p);
     if (tx == ty || g.uses[o.operands[0]] != 1) return false;
     g.set_threshold(p, ty);
+    return true;
+  });
+  // mul_const: the result's threshold follows the input's (:133-150)
+  until_stable([&](MlirOp &o) {
+    if (o.opname != "tpu.mul_const" || !g.has_quant(&o) || o.operands.empty()) return false;
+    MlirOp *p = g.producer(o.operands[0]);
+    if (!p || !g.has_quant(p)) return false;
+    const float c = (float)num_attr(o.attrs, "const_val", 0.0);
+    const float tx = g.threshold(p), ty = g.threshold(&o);
+    if (c == 0 || tx * std::abs(c) == ty) return false;
+    g.set_threshold(&o, tx * std::abs(c));
     return true;
   });
   // forward (:184-208)
@@ -593,7 +604,10 @@ struct Quantizer {
     else if (t == "tpu.concat") concat(o);
     else if (t == "tpu.leaky_relu") leaky_relu(o);
     else if (t == "tpu.prelu") prelu(o);
-    else if (kLut.count(t)) lut(o, kLut.at(t));
+    else if (t == "tpu.mul_const") {   // quantizeInt8MulConstOps (:1178-1197): only the sign is left
+      const float c = (float)num_attr(o.attrs, "const_val", 0.0);
+      field(o.attrs, "const_val") = f32_attr(c > 0.0f ? 1.0f : c < 0.0f ? -1.0f : 0.0f);
+    } else if (kLut.count(t)) lut(o, kLut.at(t));
     else if (kBypass.count(t)) bypass(o);
     else fail("op '" + name_of(o) + "': no INT8 quantisation for " + t);
     set_result_elem(o, "si8");

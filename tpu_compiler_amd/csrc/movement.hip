@@ -1,6 +1,6 @@
 // Pure data movement on int8 channels-last tensors: Pad, Crop, Permute, Reorg, Tile,
-// Reverse, ShuffleChannel, DepthToSpace (core/pad.cpp, crop.cpp, permute.cpp, reorg.cpp,
-// tile.cpp, reverse.cpp, shuffle_channel.cpp, depthtospace.cpp).  Each is an index map from
+// Reverse, ShuffleChannel, DepthToSpace, SwapChannel (core/pad.cpp, crop.cpp, permute.cpp,
+// reorg.cpp, tile.cpp, reverse.cpp, shuffle_channel.cpp, depthtospace.cpp, swap_channel.cpp).  Each is an index map from
 // the logical (n, c, h, w) of an output element to that of its source; one kernel
 // evaluates the map per element and moves the byte.  A lane produces four consecutive
 // output channels of a pixel (one dword store); pad channels are written as zero.
@@ -85,6 +85,15 @@ __device__ __forceinline__ bool source_of(const MoveArgs &a, const int (&o)[4], 
       s[3] = o[3];
       return true;
     }
+    case TPUHIP_MOVE_SWAP_CHANNEL:
+      s[0] = o[0];
+      s[1] = o[1];
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (o[1] == k) s[1] = a.p[k];
+      s[2] = o[2];
+      s[3] = o[3];
+      return true;
     default: {   // TPUHIP_MOVE_DEPTH_TO_SPACE: p[0] = upscale factor, p[1] = DCR mode
       const int r = a.p[0];
       const int dh = o[2] % r, dw = o[3] % r;
@@ -204,7 +213,7 @@ extern "C" int tpuhip_dequant_i8_to_f32(tpuhip_ctx *ctx, const void *x, void *y_
 
 extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");
-  TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_DEPTH_TO_SPACE,
+  TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_SWAP_CHANNEL,
                  "move: unknown kind %d", d->kind);
   TPUHIP_REQUIRE(d->in > 0 && d->ic > 0 && d->ih > 0 && d->iw > 0 && d->on > 0 && d->oc > 0 &&
                      d->oh > 0 && d->ow > 0,
@@ -284,6 +293,14 @@ extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const 
                      is[1], p[0]);
       for (int k = 0; k < 4; ++k) TPUHIP_REQUIRE(os[k] == is[k], "shuffle_channel: shapes differ");
       a.p[0] = p[0];
+      break;
+    case TPUHIP_MOVE_SWAP_CHANNEL:
+      TPUHIP_REQUIRE(is[1] <= 8, "swap_channel: at most 8 channels (%d)", is[1]);
+      for (int k = 0; k < 4; ++k) TPUHIP_REQUIRE(os[k] == is[k], "swap_channel: shapes differ");
+      for (int k = 0; k < is[1]; ++k) {
+        TPUHIP_REQUIRE(p[k] >= 0 && p[k] < is[1], "swap_channel: channel_order[%d] = %d", k, p[k]);
+        a.p[k] = p[k];
+      }
       break;
     default:
       TPUHIP_REQUIRE(p[0] >= 1 && is[1] % (p[0] * p[0]) == 0, "depth_to_space: bad upscale factor %d", p[0]);

@@ -21,13 +21,13 @@ _CONV_PARAM = ["kernel_h", "kernel_w", "stride_h", "stride_w", "dilation_h", "di
 _POOL_PARAM = ["kernel_h", "kernel_w", "padding_t", "padding_b", "padding_l", "padding_r", "pad_value",
                "stride_h", "stride_w", "count_include_pad"]
 _BOOLS = {"do_relu", "is_dw", "with_bias", "count_include_pad", "input_transpose", "output_transpose",
-          "fused_relu", "do_early_stride"}
+          "fused_relu", "do_early_stride", "positive"}
 _FLOATS = {"scale", "min", "max", "negative_slope", "const_val", "threshold"}
 # the activations that become a table lookup in INT8: input, table, mantissa table
 _LUT_OPS = {"tpu.sigmoid", "tpu.tanh", "tpu.exp", "tpu.elu", "tpu.swish", "tpu.softplus", "tpu.log", "tpu.pow",
             "tpu.mish", "tpu.sqrt"}
 # numbered scalars of an op description <-> array attributes of the dialect
-_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4}
+_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4, "channel_order": 8}
 # flag scalars <-> string attributes
 _FLAGS = {"mode_edge": ("mode", "edge"), "mode_dcr": ("mode", "DCR")}
 

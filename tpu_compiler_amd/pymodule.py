@@ -38,7 +38,8 @@ _WEIGHT_OPERANDS = {
     "tpu.relu": [],
     "tpu.quant": [],
     "tpu.pad": [], "tpu.crop": [], "tpu.permute": [], "tpu.reorg": [], "tpu.tile": [],
-    "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [],
+    "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [], "tpu.swap_channel": [],
+    "tpu.zero_mask": [], "tpu.mul_const": [None, None, None, None],
     "tpu.upsample": [],
     "tpu.concat": [None, None, "rshift", "multiplier"],
     "tpu.reshape": [],
