@@ -1,0 +1,66 @@
+"""The benchmark's command-line contract: what can be checked without a GPU (the refusal of
+more than one GPU, the recorded tile file, the CPU baseline leg) and, on the GPU, the one JSON
+line with its required keys."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_recorded_tiles_name_layers_and_variants_that_exist():
+    sys.path.insert(0, ROOT)
+    import bench
+    from tpu_compiler_amd import capi, graphs
+    lib = capi.bind()
+    names = []
+    while lib.tpuhip_conv2d_tile_name(len(names)):
+        names.append(lib.tpuhip_conv2d_tile_name(len(names)).decode())
+    for cfg, rel in bench.RECORDED_TILES.items():
+        tiles = json.load(open(os.path.join(ROOT, rel)))
+        g = graphs.CONFIGS[cfg]()
+        convs = {o.name for o in g.ops if o.type == "tpu.conv_2d"}
+        assert set(tiles) <= convs, sorted(set(tiles) - convs)
+        assert set(tiles.values()) <= set(names), sorted(set(tiles.values()) - set(names))
+        assert len(tiles) >= 40
+
+
+def test_cpu_baseline_leg_reports_what_it_ran():
+    sys.path.insert(0, ROOT)
+    import bench
+    from tpu_compiler_amd import graphs
+    out = bench.cpu_baseline(graphs.CONFIGS["cfg1"], 2, seconds=0.2)
+    assert out["kind"] == "port" and out["unit"] == "images/s" and out["value"] > 0
+    assert out["cores"] >= 1 and "cfg1" in out["sample"] and "2 images" in out["sample"]
+
+
+@pytest.mark.gpu
+def test_bench_prints_one_json_line_with_the_contract_keys():
+    r = subprocess.run([sys.executable, BENCH, "--config", "cfg2", "--steps", "5", "--warmup", "2"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better",
+                "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 5 and d["warmup"] == 2 and d["vs_baseline"] is None
+    assert d["metric"] == "images_per_sec" and d["unit"] == "images/s" and d["higher_is_better"] is True
+    assert "workload" in d["config"] and "model" not in d["config"]
+    assert np.isclose(d["value"], d["config"]["global_batch"] / (d["ms_per_step"] / 1e3), rtol=1e-2)
+    r_ = d["roofline"]
+    assert r_["bound"] in ("hbm", "mfma") and np.isclose(r_["frac"], r_["achieved"] / r_["peak"], atol=1e-3)
+    c = d["cpu_baseline"]
+    assert c["kind"] in ("port", "reference") and c["value"] > 0 and c["cores"] >= 1 and c["sample"]
