@@ -28,22 +28,44 @@ def sources():
     return srcs
 
 
-def build(verbose=True):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + HIPCC_FLAGS
-    for s in sources():
-        # .cpp host files are compiled as HIP too so they can include the runtime headers
-        cmd += ["-x", "hip", s]
-    cmd += ["-lz", "-o", LIB]
-    if verbose:
-        print(" ".join(cmd), flush=True)
+def _compile(args):
+    hipcc, src, obj = args
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    # .cpp host files are compiled as HIP too so they can include the runtime headers
+    cmd = [hipcc] + flags + ["-x", "hip", "-c", src, "-o", obj]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines()
-                    if "packed-fp32-ops" not in l and "warning generated" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+    return src, res.returncode, res.stdout
+
+
+def build(verbose=True, jobs=None):
+    """Compiles every source to an object of its own (in parallel: one file holds most of the
+    kernels and takes most of the time) and links them; objects go to a temporary directory."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = sources()
+    jobs = jobs or max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 1)), 16))
+    with tempfile.TemporaryDirectory(prefix="tpuhip_build_") as tmp:
+        work = [(hipcc, s, os.path.join(tmp, "%02d_%s.o" % (i, os.path.basename(s)))) for i, s in enumerate(srcs)]
+        if verbose:
+            print("%s %s -c <%d sources>  (%d at a time)" % (hipcc, " ".join(HIPCC_FLAGS), len(srcs), jobs),
+                  flush=True)
+        with ThreadPoolExecutor(jobs) as pool:
+            results = list(pool.map(_compile, work))
+        log = []
+        for src, rc, out in results:
+            text = "\n".join(l for l in out.splitlines()
+                             if "packed-fp32-ops" not in l and "warning generated" not in l)
+            if rc != 0:
+                raise RuntimeError("hipcc failed on %s:\n%s" % (src, text))
+            if text.strip():
+                log.append(text)
+        link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + [w[2] for w in work] + ["-lz", "-o", LIB]
+        res = subprocess.run(link, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("link failed:\n" + res.stdout)
+    if verbose and log:
+        print("\n".join(log))
     return LIB
 
 
