@@ -260,6 +260,14 @@ int tpuhip_clip_table(float min, float max, uint32_t rshift, uint32_t multiplier
 /* Replaces ReluOpKernel::invoke (core/activation.cpp:155-164). */
 int tpuhip_relu_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t bytes);
 
+/* INT8 LRN across channels; replaces lrn_int8 / LrnOpKernel::invoke (core/lrn.cpp:104-166, :212-215).
+ * sqr_lut256 / power_lut256: the two 256-entry tables quantizeInt8LrnOps writes (values 0..255, the
+ * first indexed by the input byte); sum_rshift, lrn_rshift, quant0, quant1: the op's attributes
+ * sum_rshift, lrn_rshift, quant_data0, quant_data1.  Refused where the reference's float arithmetic
+ * would stop being exact (255 * quant0 * local_size or 255 * 128 * quant1 reaching 2^24). */
+int tpuhip_lrn_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t pixels, int c, int cs, int local_size,
+                  const uint8_t *sqr_lut256, const uint8_t *power_lut256, int sum_rshift, int lrn_rshift,
+                  int quant0, int quant1);
 /* One table per channel: y[.., c] = tables[c * 256 + (uint8_t)x[.., c]]; tables is DEVICE memory
  * (c * 256 bytes).  With tpuhip_prelu_tables (host) it replaces PReluOpKernel::invoke, INT8 branch
  * (core/activation.cpp:185-224): slope holds the c float-stored int8 slopes. */

@@ -349,6 +349,19 @@ public:
   ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
 };
 
+// INT8 LRN (core/lrn.cpp:168-235).  operands: [0]input [1]sqr_lut [2]power_lut [3]scale (unused)
+class LrnOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPULrnOp";
+  LrnOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+  uint8_t sqr_lut[256], power_lut[256];
+  int local_size = 0, sum_rshift = 0, lrn_rshift = 0, quant_data0 = 0, quant_data1 = 0;
+};
+
 // INT8 ZeroMask (core/zero_mask.cpp:8-35): 127 where the input is non-zero (positive) or zero
 // (not positive), else 0.  A function of one byte, so it runs as a table.
 class ZeroMaskOpKernel : public LutOpKernel {

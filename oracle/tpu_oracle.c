@@ -697,6 +697,43 @@ void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, in
   }
 }
 
+/* lrn_int8 (core/lrn.cpp:104-166): squares from a table indexed by the input byte, a sliding
+ * sum over local_size channels kept as a running float (add the head, subtract the tail),
+ * rescaled to a table index, the power table entry times the input. */
+void orc_lrn_i8(const int8_t *x, int8_t *y, int n, int c, int h, int w, int local_size,
+                const float *sqr_lut, const float *power_lut, int sq_right_shift, int lrn_right_shift,
+                int quant0, int quant1) {
+  const int pre_pad = (local_size - 1) / 2, padded_c = c + local_size - 1;
+  const int64_t frame = (int64_t)h * w, batch = frame * c;
+  float *padded = (float *)calloc((size_t)(padded_c * frame), sizeof(float));
+  float *scale = (float *)calloc((size_t)(n * batch), sizeof(float));
+  float *square = padded + pre_pad * frame;
+  for (int in = 0; in < n; ++in) {
+    const int8_t *xn = x + in * batch;
+    float *sn = scale + in * batch;
+    for (int64_t i = 0; i < batch; ++i) square[i] = sqr_lut[(uint8_t)xn[i]];
+    for (int ic = 0; ic < local_size; ++ic)
+      for (int64_t i = 0; i < frame; ++i) sn[i] += (float)quant0 * padded[ic * frame + i];
+    for (int ic = 1; ic < c; ++ic) {
+      memcpy(sn + ic * frame, sn + (ic - 1) * frame, (size_t)frame * sizeof(float));
+      for (int64_t i = 0; i < frame; ++i) sn[ic * frame + i] += (float)quant0 * padded[(ic + local_size - 1) * frame + i];
+      for (int64_t i = 0; i < frame; ++i) sn[ic * frame + i] += (float)-quant0 * padded[(ic - 1) * frame + i];
+    }
+  }
+  const float sq_scale = 1.0f / (1 << sq_right_shift), lrn_scale = 1.0f / (1 << lrn_right_shift);
+  for (int64_t i = 0; i < n * batch; ++i) {
+    float t = floorf(scale[i] * sq_scale + 0.5f);
+    if (t < 0.0f) t = 0.0f;
+    else if (t > 255.0f) t = 255.0f;
+    float o = power_lut[(uint8_t)t];
+    o *= (float)x[i] * quant1 * lrn_scale;
+    o = floorf(o + 0.5f);
+    y[i] = (int8_t)(o < -128.0f ? -128.0f : o > 127.0f ? 127.0f : o);
+  }
+  free(padded);
+  free(scale);
+}
+
 /* ------------------------------------------------------------------------- */
 /* transposed convolution                                                     */
 /* ------------------------------------------------------------------------- */

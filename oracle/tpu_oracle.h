@@ -183,6 +183,10 @@ void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, in
 void orc_swap_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, const int *order);
 void orc_zero_mask_i8(const int8_t *x, int8_t *y, int64_t n, int positive);
 void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, int do_relu);
+/* core/lrn.cpp:104-166, INT8 */
+void orc_lrn_i8(const int8_t *x, int8_t *y, int n, int c, int h, int w, int local_size,
+                const float *sqr_lut, const float *power_lut, int sq_right_shift, int lrn_right_shift,
+                int quant0, int quant1);
 void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int upscale,
                            int dcr_mode);
 

@@ -129,6 +129,10 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             y = O.lut_i8(ins[0], op.weights["table"])
         elif t == "tpu.relu":
             y = O.relu_i8(ins[0])
+        elif t == "tpu.lrn":
+            a = op.attrs
+            y = O.lrn_i8(ins[0], a["local_size"], op.weights["sqr_lut"], op.weights["power_lut"], a["sum_rshift"],
+                         a["lrn_rshift"], a["quant_data0"], a["quant_data1"])
         elif t == "tpu.zero_mask":
             y = O.zero_mask_i8(ins[0], op.attrs.get("positive", 0))
         elif t == "tpu.mul_const":

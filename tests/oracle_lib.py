@@ -87,6 +87,7 @@ def _load():
     lib.orc_shuffle_channel_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_depth_to_space_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_swap_channel_i8.argtypes = [i8p, i8p, i64p, C.POINTER(C.c_int)]
+    lib.orc_lrn_i8.argtypes = [i8p, i8p] + [C.c_int] * 5 + [C.POINTER(C.c_float)] * 2 + [C.c_int] * 4
     lib.orc_zero_mask_i8.argtypes = [i8p, i8p, C.c_int64, C.c_int]
     lib.orc_mul_const_i8.argtypes = [i8p, i8p, C.c_int64, C.c_float, C.c_int]
     lib.orc_pool_max_i8.argtypes = [i8p, i8p, C.POINTER(PoolDesc)]
@@ -301,6 +302,16 @@ def move_i8(kind, x, params, out_shape=None):
 
 MOVE_KINDS = ["pad_const", "pad_edge", "crop", "permute", "reorg", "tile", "reverse",
               "shuffle_channel", "depth_to_space", "swap_channel"]
+
+
+def lrn_i8(x, local_size, sqr_lut, power_lut, sum_rshift, lrn_rshift, quant0, quant1):
+    x = _i8(x)
+    y = np.empty(x.shape, np.int8)
+    sq, pw = _f32(sqr_lut), _f32(power_lut)
+    n, c, h, w = x.shape
+    lib.orc_lrn_i8(_p(x, C.c_int8), _p(y, C.c_int8), n, c, h, w, int(local_size), _p(sq, C.c_float),
+                   _p(pw, C.c_float), int(sum_rshift), int(lrn_rshift), int(quant0), int(quant1))
+    return y
 
 
 def zero_mask_i8(x, positive):

@@ -476,6 +476,39 @@ def test_graph_with_swap_channel_mul_const_and_zero_mask(tmp_path, fuse):
         module().load(g)
 
 
+def test_graph_with_lrn_matches_the_oracle(tmp_path):
+    """conv + ReLU -> LRN across channels -> max pool (the opening of GoogLeNet / AlexNet-style nets)"""
+    rng = np.random.default_rng(8)
+    b = graphs.Builder("lrn_net", graphs.BASE_SEED + 82, 2, (6, 12))
+    x = b.input("input", 3, 20, 20)
+    c1 = b.conv("c1", x, 48, 3, stride=2, relu=True)
+    g = b.g
+    shp = g.by_name[c1].shape
+    idx = np.arange(256)
+    sq = np.minimum(np.floor((idx / 16.0) ** 2 + 0.5), 255).astype(np.float32)
+    pw = np.minimum(np.floor(255.0 * (1 + idx / 64.0) ** -0.75 + 0.5), 255).astype(np.float32)
+    g.add(graphs.Op("tpu.lrn", "norm", [c1], shp,
+                    dict(local_size=5, sum_rshift=4, lrn_rshift=8, quant_data0=13, quant_data1=2),
+                    dict(sqr_lut=np.tile(sq, 32).reshape(1, 32, 16, 16), power_lut=np.tile(pw, 32).reshape(1, 32, 16, 16))))
+    b.cal["norm"] = oracle_graph.run(g, upto="norm")["norm"][:1].astype(np.int64)
+    p = b.pool_max("pool", "norm", 3, 2, (0, 1, 0, 1))
+    g.outputs = [p]
+    want = oracle_graph.run(g)
+    assert len(np.unique(want["norm"])) > 8 and (want["norm"] != want["c1"]).mean() > 0.3
+    m = module()
+    m.set_option("keep_all_tensors", 1)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()
+    check_through_files(g, g.input_op().data, want, tmp_path)
+    g.by_name["norm"].weights["sqr_lut"] = g.by_name["norm"].weights["sqr_lut"] + 0.5
+    with pytest.raises(capi.TpuHipError, match="not an integer"):
+        module().load(g)
+
+
 def test_graph_with_uint8_input_and_scale_lut_matches_the_oracle(tmp_path):
     """uint8 image -> ScaleLut (per-channel 256-entry tables) -> conv"""
     rng = np.random.default_rng(6)

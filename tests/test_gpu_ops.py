@@ -727,3 +727,33 @@ def test_data_movement_rejects_bad_arguments(ctx):
         ctx.move(capi.MOVE_SHUFFLE_CHANNEL, x, y, [5])
     with pytest.raises(capi.TpuHipError, match="expected"):
         ctx.move(capi.MOVE_PAD_CONST, x, y, [0, 0, 1, 0, 0, 0, 0, 0])
+
+
+@pytest.mark.parametrize("shape,local_size,sum_rshift,lrn_rshift,q0,q1", [
+    ((2, 64, 9, 7), 5, 8, 9, 120, 93),
+    ((1, 21, 5, 5), 3, 0, 3, 1, 2),          # channels not a multiple of 4 or 16
+    ((3, 192, 4, 6), 5, 11, 12, 200, 255),
+    ((1, 4, 3, 3), 7, 6, 9, 64, 2),          # window wider than the tensor
+])
+def test_lrn_matches_the_oracle(ctx, shape, local_size, sum_rshift, lrn_rshift, q0, q1):
+    rng = np.random.default_rng(shape[1] + local_size)
+    x = rnd_i8(rng, shape)
+    sq, pw = rng.integers(0, 256, 256), rng.integers(0, 256, 256)
+    want = O.lrn_i8(x, local_size, sq, pw, sum_rshift, lrn_rshift, q0, q1)
+    xt, yt = ctx.from_nchw(x), ctx.tensor(shape)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.lrn(xt, yt, local_size, sq, pw, sum_rshift, lrn_rshift, q0, q1)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., shape[1]:].any()          # pad channels rewritten as zero
+    assert len(np.unique(want)) > 8
+
+
+def test_lrn_refuses_parameters_whose_float_form_is_inexact(ctx):
+    xt, yt = ctx.tensor((1, 16, 2, 2)), ctx.tensor((1, 16, 2, 2))
+    t = np.zeros(256, np.uint8)
+    with pytest.raises(capi.TpuHipError, match="quant_data0"):
+        ctx.lrn(xt, yt, 5, t, t, 8, 8, 20000, 10)
+    with pytest.raises(capi.TpuHipError, match="quant_data1"):
+        ctx.lrn(xt, yt, 5, t, t, 8, 8, 100, 600)
+    with pytest.raises(capi.TpuHipError, match="local_size"):
+        ctx.lrn(xt, yt, 0, t, t, 8, 8, 100, 100)

@@ -301,3 +301,59 @@ def test_concat_vs_numpy_and_requant():
     bq = np.clip((b.astype(np.int64) * 5 + 4) >> 3, -128, 127)
     want = np.maximum(np.concatenate([a.astype(np.int64), bq], 1), 0)
     assert np.array_equal(y.astype(np.int64), want)
+
+
+def lrn_by_definition(x, local_size, sq, pw, sum_rshift, lrn_rshift, q0, q1):
+    """the INT8 LRN as exact integer arithmetic written from the definition: window sum of the
+    squares table over the channels, one rounding shift to the index, one to the result"""
+    n, c, h, w = x.shape
+    sqv = np.asarray(sq, np.int64)[x.astype(np.uint8)]
+    pre = (local_size - 1) // 2
+    pad = np.zeros((n, c + local_size - 1, h, w), np.int64)
+    pad[:, pre:pre + c] = sqv
+    s = sum(pad[:, k:k + c] for k in range(local_size)) * q0
+    t = np.clip((s + ((1 << sum_rshift) >> 1)) >> sum_rshift, 0, 255)
+    m = np.asarray(pw, np.int64)[t] * x.astype(np.int64) * q1
+    return np.clip((m + ((1 << lrn_rshift) >> 1)) >> lrn_rshift, -128, 127).astype(np.int8)
+
+
+@pytest.mark.parametrize("local_size,sum_rshift,lrn_rshift,q0,q1", [(5, 8, 9, 120, 93), (3, 0, 0, 1, 1),
+                                                                     (1, 4, 12, 255, 255), (4, 10, 7, 77, 40)])
+def test_lrn_float_restatement_equals_the_integer_definition(local_size, sum_rshift, lrn_rshift, q0, q1):
+    """the oracle keeps the reference's float running sums; under the exactness bounds the result
+    must equal plain integer arithmetic, negative inputs (which index the upper table half) included"""
+    rng = np.random.default_rng(local_size * 7 + q0)
+    x = rng.integers(-128, 128, (2, 11, 4, 3)).astype(np.int8)
+    x[0, :, 0, 0] = 127
+    x[1, :, 0, 0] = -128
+    sq = rng.integers(0, 256, 256)
+    pw = rng.integers(0, 256, 256)
+    if lrn_rshift == 0:
+        pw = pw % 3
+    got = O.lrn_i8(x, local_size, sq, pw, sum_rshift, lrn_rshift, q0, q1)
+    want = lrn_by_definition(x, local_size, sq, pw, sum_rshift, lrn_rshift, q0, q1)
+    assert np.array_equal(got, want)
+    assert len(np.unique(got)) > 3
+
+
+def test_lrn_with_realistic_tables_tracks_the_float_formula():
+    """tables as the quantiser builds them (QuantizeInt8.cpp:299-329) for a ReLU-ed input: the INT8
+    result must follow x / (k + alpha/n * sum x^2)^beta"""
+    rng = np.random.default_rng(2)
+    thx, thy, alpha, beta, k, n_ = 4.0, 4.2, 1e-2, 0.75, 1.0, 5
+    xf = np.abs(rng.normal(0, 1.2, (1, 16, 6, 6))).clip(0, thx)
+    x = np.clip(np.floor(xf * 128 / thx + 0.5), -128, 127).astype(np.int8)
+    sq_thy, sumsq_thy = alpha / n_ * thx * thx, alpha * thx * thx * 1.0
+    scale_thy = k ** -beta
+    idx = np.arange(256)
+    sq = np.minimum(np.floor((thx / 128.0 * idx) ** 2 * 256.0 / sq_thy * alpha / n_ + 0.5), 255)
+    pw = np.minimum(np.floor((idx / (256.0 / sumsq_thy) + k) ** -beta * (256.0 / scale_thy) + 0.5), 255)
+    # sum of squares tables -> index: sq_thy / sumsq_thy as quant0 / 2^shift; result: thx*scale_thy/(thy*256)
+    q0, r0 = int(round(sq_thy / sumsq_thy * 2 ** 12)), 12
+    q1, r1 = int(round(thx * scale_thy / (thy * 256.0) * 2 ** 14)), 14
+    got = O.lrn_i8(x, n_, sq, pw, r0, r1, q0, q1).astype(np.float64) * thy / 128
+    xr = x.astype(np.float64) * thx / 128
+    pad = np.zeros((1, 16 + n_ - 1, 6, 6))
+    pad[:, 2:18] = xr ** 2
+    ref = xr / (k + alpha / n_ * sum(pad[:, j:j + 16] for j in range(n_))) ** beta
+    assert np.abs(got - ref).max() < 0.05 * thy

@@ -188,6 +188,8 @@ PROTOTYPES.update({
     "tpuhip_quantize_rescale": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_void_p,
                                           C.c_void_p]),
     "tpuhip_quantize_leaky_relu": (C.c_int, [C.c_float, C.c_float, C.c_float, C.c_void_p]),
+    "tpuhip_lrn_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int,
+                                C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "tpuhip_quantize_mlir_files": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p,
                                              C.c_size_t, C.POINTER(C.c_size_t)]),
     "tpuhip_quantize_lut_table": (C.c_int, [C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
@@ -393,6 +395,15 @@ class Context:
             self.h, C.byref(desc), filt.ctypes.data, None if b is None else b.ctypes.data,
             mult.ctypes.data, rshift.ctypes.data, C.byref(w)))
         return w.value
+
+    def lrn(self, x, y, local_size, sqr_lut, power_lut, sum_rshift, lrn_rshift, quant0, quant1):
+        sq = np.ascontiguousarray(sqr_lut, dtype=np.uint8)
+        pw = np.ascontiguousarray(power_lut, dtype=np.uint8)
+        assert sq.size == 256 and pw.size == 256
+        n, c, h, w = x.shape
+        self._ck(self.lib.tpuhip_lrn_i8(self.h, x.ptr, y.ptr, n * h * w, c, x.cs, int(local_size),
+                                        sq.ctypes.data, pw.ctypes.data, int(sum_rshift), int(lrn_rshift),
+                                        int(quant0), int(quant1)))
 
     def conv_prepack_pair(self, desc_a, desc_b, a, b):
         """a, b: (filter int8, bias int32 or None, multiplier int32, rshift int32) of two convs over

@@ -4,6 +4,8 @@
 // bytes per lane per access where the layout allows it; none uses MFMA.
 #include "common.hpp"
 
+#include <cstring>
+
 #include <algorithm>
 #include <cmath>
 
@@ -341,6 +343,52 @@ int launch_lut(tpuhip_ctx *ctx, const void *x, void *y, const int8_t *table, int
   return TPUHIP_OK;
 }
 
+// INT8 LRN across channels (core/lrn.cpp:104-166).  A lane produces four consecutive channels
+// of a pixel; the window of local_size channels around each is summed from the squares table
+// (indexed by the input byte), rescaled to an index into the power table, and that entry
+// scales the input.  All integers: the reference's float arithmetic is exact for them.
+struct LrnArgs {
+  const int8_t *x;
+  int8_t *y;
+  int64_t total;   // pixels * (cs / 4)
+  int c, cs, local_size, sum_rshift, lrn_rshift, quant0, quant1;
+  Table256 sqr, power;
+};
+
+__global__ __launch_bounds__(kThreads) void lrn_kernel(LrnArgs a) {
+  __shared__ uint32_t tsq[64], tpw[64];
+  if (threadIdx.x < 64) {
+    tsq[threadIdx.x] = a.sqr.w[threadIdx.x];
+    tpw[threadIdx.x] = a.power.w[threadIdx.x];
+  }
+  __syncthreads();
+  const uint8_t *sq = reinterpret_cast<const uint8_t *>(tsq);
+  const uint8_t *pw = reinterpret_cast<const uint8_t *>(tpw);
+  const int c4 = a.cs >> 2, pre_pad = (a.local_size - 1) / 2;
+  const int rnd_s = a.sum_rshift > 0 ? 1 << (a.sum_rshift - 1) : 0;
+  const int rnd_l = a.lrn_rshift > 0 ? 1 << (a.lrn_rshift - 1) : 0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int cq = (int)(i % c4);
+    const int64_t pix = i / c4;
+    const int8_t *row = a.x + pix * a.cs;
+    uint32_t word = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int ch = cq * 4 + b;
+      if (ch >= a.c) continue;   // pad channels stay zero
+      int s = 0;
+      const int lo = max(ch - pre_pad, 0), hi = min(ch - pre_pad + a.local_size, a.c);
+      for (int k = lo; k < hi; ++k) s += sq[(uint8_t)row[k]];
+      const int t = min(max((s * a.quant0 + rnd_s) >> a.sum_rshift, 0), 255);
+      const int m = (int)pw[t] * (int)row[ch] * a.quant1;
+      const int o = min(max((m + rnd_l) >> a.lrn_rshift, -128), 127);
+      word |= (uint32_t)(uint8_t)(int8_t)o << (8 * b);
+    }
+    *reinterpret_cast<uint32_t *>(a.y + pix * a.cs + cq * 4) = word;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -402,6 +450,37 @@ int tpuhip_lut_i8(tpuhip_ctx *ctx, const void *x, void *y, const int8_t *table25
   TPUHIP_REQUIRE(c > 0 && cs >= c && cs % 16 == 0, "lut: bad channels %d / stride %d", c, cs);
   if (pixels == 0) return TPUHIP_OK;
   return launch_lut(ctx, x, y, table256, (int64_t)pixels, c, cs, cs, 0);
+}
+
+int tpuhip_lrn_i8(tpuhip_ctx *ctx, const void *x, void *y, size_t pixels, int c, int cs, int local_size,
+                  const uint8_t *sqr_lut256, const uint8_t *power_lut256, int sum_rshift, int lrn_rshift,
+                  int quant0, int quant1) {
+  TPUHIP_REQUIRE(ctx && x && y && sqr_lut256 && power_lut256, "lrn: NULL argument");
+  TPUHIP_REQUIRE(c > 0 && cs >= c && cs % 16 == 0, "lrn: bad channels %d / stride %d", c, cs);
+  TPUHIP_REQUIRE(local_size >= 1 && local_size <= 64, "lrn: local_size %d outside [1,64]", local_size);
+  TPUHIP_REQUIRE(sum_rshift >= 0 && sum_rshift <= 23 && lrn_rshift >= 0 && lrn_rshift <= 23,
+                 "lrn: shifts %d / %d outside [0,23]", sum_rshift, lrn_rshift);
+  // the reference computes in float; these bounds keep every intermediate an exact integer
+  // multiple of a power of two below 2^24, so the integer form used here gives the same bytes
+  // (the running sum holds one more term than the window while the head is added before the
+  // tail is subtracted; the rounding term is half a unit of the shifted result)
+  TPUHIP_REQUIRE(quant0 >= 0 && (int64_t)255 * quant0 * (local_size + 1) + (1ll << sum_rshift) < (1 << 24),
+                 "lrn: quant_data0 %d too large for exact float sums", quant0);
+  TPUHIP_REQUIRE(quant1 >= 0 && (int64_t)255 * 128 * quant1 + (1ll << lrn_rshift) < (1 << 24),
+                 "lrn: quant_data1 %d too large for exact float products", quant1);
+  if (pixels == 0) return TPUHIP_OK;
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  LrnArgs a{};
+  a.x = (const int8_t *)x;
+  a.y = (int8_t *)y;
+  a.total = (int64_t)pixels * (cs / 4);
+  a.c = c; a.cs = cs; a.local_size = local_size;
+  a.sum_rshift = sum_rshift; a.lrn_rshift = lrn_rshift; a.quant0 = quant0; a.quant1 = quant1;
+  memcpy(a.sqr.w, sqr_lut256, 256);
+  memcpy(a.power.w, power_lut256, 256);
+  launch(ctx, lrn_kernel, dim3(grid_for(a.total, kThreads * 2)), dim3(kThreads), a);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
 }
 
 int tpuhip_lut_per_channel_i8(tpuhip_ctx *ctx, const void *x, void *y, const void *tables,

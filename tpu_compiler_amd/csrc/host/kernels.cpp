@@ -927,6 +927,36 @@ ClipOpKernel::ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &
      name.c_str());
 }
 
+LrnOpKernel::LrnOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Lrn");
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data || input_data->slot_bytes() != output_data->slot_bytes()) fail("Lrn '" + name + "': shape mismatch");
+  if (opdTensors.size() < 3 || !opdTensors[1].weight || !opdTensors[2].weight ||
+      opdTensors[1].weight->size() < 256 || opdTensors[2].weight->size() < 256)
+    fail("Lrn '" + name + "': the sqr / power table operands are missing");
+  for (int i = 0; i < 256; ++i) {
+    const float s = opdTensors[1].weight->at(i), p = opdTensors[2].weight->at(i);
+    if (!(s >= 0 && s <= 255 && s == std::floor(s) && p >= 0 && p <= 255 && p == std::floor(p)))
+      fail("Lrn '" + name + "': table entry " + std::to_string(i) + " is not an integer in [0,255]");
+    sqr_lut[i] = (uint8_t)s;
+    power_lut[i] = (uint8_t)p;
+  }
+  local_size = (int)op.attr("local_size");
+  sum_rshift = (int)op.attr("sum_rshift");
+  lrn_rshift = (int)op.attr("lrn_rshift");
+  quant_data0 = (int)op.attr("quant_data0");
+  quant_data1 = (int)op.attr("quant_data1");
+}
+
+void LrnOpKernel::invoke() {
+  ck(tpuhip_lrn_i8(ctx, input_data->data(), output_data->data(),
+                   (size_t)input_data->n * input_data->h * input_data->w, input_data->c, input_data->cs,
+                   local_size, sqr_lut, power_lut, sum_rshift, lrn_rshift, quant_data0, quant_data1),
+     name.c_str());
+}
+
 ZeroMaskOpKernel::ZeroMaskOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
     : LutOpKernel(op, valueMapping, weightMapping) {
   const bool positive = op.attr("positive", 0) != 0;

@@ -40,6 +40,7 @@ _WEIGHT_OPERANDS = {
     "tpu.pad": [], "tpu.crop": [], "tpu.permute": [], "tpu.reorg": [], "tpu.tile": [],
     "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [], "tpu.swap_channel": [],
     "tpu.zero_mask": [], "tpu.mul_const": [None, None, None, None],
+    "tpu.lrn": ["sqr_lut", "power_lut", None],
     "tpu.upsample": [],
     "tpu.concat": [None, None, "rshift", "multiplier"],
     "tpu.reshape": [],
