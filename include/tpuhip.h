@@ -321,6 +321,17 @@ typedef struct tpuhip_move_desc {
 } tpuhip_move_desc;
 int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y);
 
+/* ---- Reduce over consecutive axes ------------------------------------------
+ * Replaces ReduceOpKernel::invoke (core/reduce.cpp:54-117) for INT8 tensors.  kind: 0 mean, 1 sum,
+ * 2 max, 3 min, over the logical NCHW axes first_axis..last_axis of the input; the result holds
+ * the remaining elements in order, shaped out_nchw (with or without the reduced axes kept as 1).
+ * In INT8 a mean is a sum whose 1/count lives in the multiplier.  rshift / multiplier: the op's
+ * quant operands; (0, 1) means none, which a sum over more than one element refuses because the
+ * reference then leaves a raw sum that is no int8 value. */
+int tpuhip_reduce_i8(tpuhip_ctx *ctx, int kind, const void *x, void *y, const int *in_nchw, int x_cs,
+                     const int *out_nchw, int y_cs, int first_axis, int last_axis, int rshift,
+                     uint32_t multiplier);
+
 /* ---- QuantOp at the graph edges -------------------------------------------
  * Replaces QuantOpKernel::invoke (core/quant.cpp:133-166) for the two conversions an INT8 graph
  * has: fp32 -> int8 right after an input (round(src * scale), half away from zero, clamped,

@@ -349,6 +349,20 @@ public:
   ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
 };
 
+// ReduceMean / ReduceSum / ReduceMax / ReduceMin (core/reduce.cpp:7-117), INT8.
+// operands: [0]input [1]lut [2]mantissa_lut (unused) [3]rshift [4]multiplier; attribute axes
+class ReduceOpKernel : public CPUOpKernel {
+public:
+  static constexpr const char *OpName = "CPUReduceOp";
+  ReduceOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  void invoke() override;
+
+private:
+  SyncedData input_data, output_data;
+  int kind = 0, first_axis = 0, last_axis = 0, rshift = 0;
+  uint32_t multiplier = 1;
+};
+
 // INT8 LRN (core/lrn.cpp:168-235).  operands: [0]input [1]sqr_lut [2]power_lut [3]scale (unused)
 class LrnOpKernel : public CPUOpKernel {
 public:

@@ -734,6 +734,33 @@ void orc_lrn_i8(const int8_t *x, int8_t *y, int n, int c, int h, int w, int loca
   free(scale);
 }
 
+/* ReduceOpKernel::invoke (core/reduce.cpp:54-117), INT8, kinds 0 mean / 1 sum / 2 max / 3 min over
+ * the axes between outer and inner.  In INT8 the mean is a sum too (its 1/axis is folded into the
+ * multiplier); the float result is requantised when rshift != 0 or multiplier != 1 and stored
+ * as it is otherwise. */
+void orc_reduce_i8(int kind, const int8_t *x, int8_t *y, int64_t outer, int64_t axis, int64_t inner,
+                   float rshift, float multiplier) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t i = 0; i < inner; ++i) {
+      float v;
+      if (kind <= 1) {
+        v = 0.0f;
+        for (int64_t a = 0; a < axis; ++a) v += (float)x[o * axis * inner + a * inner + i];
+      } else {
+        v = (float)x[o * axis * inner + i];
+        for (int64_t a = 1; a < axis; ++a) {
+          const float t = (float)x[o * axis * inner + a * inner + i];
+          if (kind == 2 && t > v) v = t;
+          else if (kind == 3 && t < v) v = t;
+        }
+      }
+      if (rshift != 0 || multiplier != 1)
+        y[o * inner + i] = orc_apply_mult_rshift_sat8_f(v, (uint32_t)rshift, (uint32_t)multiplier, 0);
+      else
+        y[o * inner + i] = (int8_t)v;   /* callers only ask for this when v is an int8 value */
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 /* transposed convolution                                                     */
 /* ------------------------------------------------------------------------- */

@@ -187,6 +187,9 @@ void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, in
 void orc_lrn_i8(const int8_t *x, int8_t *y, int n, int c, int h, int w, int local_size,
                 const float *sqr_lut, const float *power_lut, int sq_right_shift, int lrn_right_shift,
                 int quant0, int quant1);
+/* core/reduce.cpp:54-117, INT8; kind 0 mean, 1 sum, 2 max, 3 min */
+void orc_reduce_i8(int kind, const int8_t *x, int8_t *y, int64_t outer, int64_t axis, int64_t inner,
+                   float rshift, float multiplier);
 void orc_depth_to_space_i8(const int8_t *x, int8_t *y, const int64_t *ishape, int upscale,
                            int dcr_mode);
 

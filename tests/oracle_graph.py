@@ -129,6 +129,12 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             y = O.lut_i8(ins[0], op.weights["table"])
         elif t == "tpu.relu":
             y = O.relu_i8(ins[0])
+        elif t in ("tpu.reduce_mean", "tpu.reduce_sum", "tpu.reduce_max", "tpu.reduce_min"):
+            axes = [int(op.attrs["axes%d" % k]) for k in range(4) if "axes%d" % k in op.attrs]
+            full = (ins[0].shape[0],) + tuple(op.shape[1:])
+            y = O.reduce_i8(t[len("tpu.reduce_"):], ins[0], axes, full,
+                            op.weights["rshift"][0] if "rshift" in op.weights else 0,
+                            op.weights["multiplier"][0] if "multiplier" in op.weights else 1)
         elif t == "tpu.lrn":
             a = op.attrs
             y = O.lrn_i8(ins[0], a["local_size"], op.weights["sqr_lut"], op.weights["power_lut"], a["sum_rshift"],

@@ -87,6 +87,7 @@ def _load():
     lib.orc_shuffle_channel_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_depth_to_space_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_swap_channel_i8.argtypes = [i8p, i8p, i64p, C.POINTER(C.c_int)]
+    lib.orc_reduce_i8.argtypes = [C.c_int, i8p, i8p, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_float]
     lib.orc_lrn_i8.argtypes = [i8p, i8p] + [C.c_int] * 5 + [C.POINTER(C.c_float)] * 2 + [C.c_int] * 4
     lib.orc_zero_mask_i8.argtypes = [i8p, i8p, C.c_int64, C.c_int]
     lib.orc_mul_const_i8.argtypes = [i8p, i8p, C.c_int64, C.c_float, C.c_int]
@@ -311,6 +312,24 @@ def lrn_i8(x, local_size, sqr_lut, power_lut, sum_rshift, lrn_rshift, quant0, qu
     n, c, h, w = x.shape
     lib.orc_lrn_i8(_p(x, C.c_int8), _p(y, C.c_int8), n, c, h, w, int(local_size), _p(sq, C.c_float),
                    _p(pw, C.c_float), int(sum_rshift), int(lrn_rshift), int(quant0), int(quant1))
+    return y
+
+
+REDUCE_KINDS = {"mean": 0, "sum": 1, "max": 2, "min": 3}
+
+
+def reduce_i8(kind, x, axes, out_shape, rshift=0, multiplier=1):
+    """reduce over consecutive axes of an NCHW tensor; out_shape as the op declares it"""
+    x = _i8(x)
+    axes = [int(a) for a in axes]
+    assert axes == list(range(axes[0], axes[-1] + 1))
+    outer = int(np.prod(x.shape[:axes[0]], dtype=np.int64))
+    axis = int(np.prod(x.shape[axes[0]:axes[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(x.shape[axes[-1] + 1:], dtype=np.int64))
+    y = np.empty(tuple(out_shape), np.int8)
+    assert y.size == outer * inner
+    lib.orc_reduce_i8(REDUCE_KINDS[kind], _p(x, C.c_int8), _p(y, C.c_int8), outer, axis, inner,
+                      float(rshift), float(multiplier))
     return y
 
 

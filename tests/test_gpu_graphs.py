@@ -476,6 +476,46 @@ def test_graph_with_swap_channel_mul_const_and_zero_mask(tmp_path, fuse):
         module().load(g)
 
 
+def test_graph_with_reduce_ops_matches_the_oracle(tmp_path):
+    """mean / max over the image, sum / min over the channels, with and without the reduced axes kept"""
+    b = graphs.Builder("reduce_net", graphs.BASE_SEED + 83, 2, (6, 12))
+    x = b.input("input", 8, 9, 7)
+    c1 = b.conv("c1", x, 40, 3, relu=False)
+    g = b.g
+    f32 = lambda *v: np.array(v, np.float32)
+
+    def red(t, name, shape, axes, rshift=None, mult=None):
+        w = {} if rshift is None else dict(rshift=f32(rshift), multiplier=f32(mult))
+        g.add(graphs.Op("tpu.reduce_" + t, name, [c1], shape, {"axes%d" % k: a for k, a in enumerate(axes)}, w,
+                        "RSHIFT_AND_M_I8" if w else "NONE"))
+        return name
+
+    outs = [red("mean", "gmean", (2, 40, 1, 1), [2, 3], 9, 41), red("max", "gmax", (2, 40, 1, 1), [2, 3]),
+            red("sum", "csum", (2, 1, 9, 7), [1], 6, 19), red("min", "cmin", (2, 9, 7), [1], 1, 3),
+            red("max", "wmax", (2, 40, 9), [3], 0, 1), red("mean", "all", (2, 1), [1, 2, 3], 14, 90)]
+    g.outputs = outs
+    want = oracle_graph.run(g)
+    for name in outs:
+        assert len(np.unique(want[name])) > (3 if name == "all" else 8) or want[name].size < 4, name
+    m = module()
+    m.set_option("keep_all_tensors", 1)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()
+    check_through_files(g, g.input_op().data, want, tmp_path)
+    # a sum without rescaling is no int8 tensor
+    g.by_name["csum"].weights = {}
+    m = module()
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    with pytest.raises(capi.TpuHipError, match="no int8 value"):
+        m.invoke()
+    m.close()
+
+
 def test_graph_with_lrn_matches_the_oracle(tmp_path):
     """conv + ReLU -> LRN across channels -> max pool (the opening of GoogLeNet / AlexNet-style nets)"""
     rng = np.random.default_rng(8)

@@ -357,3 +357,24 @@ def test_lrn_with_realistic_tables_tracks_the_float_formula():
     pad[:, 2:18] = xr ** 2
     ref = xr / (k + alpha / n_ * sum(pad[:, j:j + 16] for j in range(n_))) ** beta
     assert np.abs(got - ref).max() < 0.05 * thy
+
+
+@pytest.mark.parametrize("kind", ["mean", "sum", "max", "min"])
+@pytest.mark.parametrize("axes", [[2, 3], [1], [1, 2, 3], [3]])
+def test_reduce_is_numpy_reduction_then_the_float_requant(kind, axes):
+    rng = np.random.default_rng(len(axes) * 11 + len(kind))
+    x = rng.integers(-128, 128, (2, 7, 5, 6)).astype(np.int8)
+    fn = {"mean": np.sum, "sum": np.sum, "max": np.max, "min": np.min}[kind]     # an INT8 mean is a sum
+    red = fn(x.astype(np.int64), axis=tuple(axes), keepdims=True)
+    for rshift, mult in [(7, 55), (0, 3), (12, 200)] + ([(0, 1)] if kind in ("max", "min") else []):
+        got = O.reduce_i8(kind, x, axes, red.shape, rshift, mult)
+        if (rshift, mult) == (0, 1):
+            want = red
+        else:
+            # float product, float quotient, floor(f + 0.5), clamp: all exact here (|sum * mult| < 2^24)
+            want = np.clip(np.floor(red.astype(np.float64) * mult / (1 << rshift) + 0.5), -128, 127)
+        assert np.array_equal(got, want), (rshift, mult)
+    # without the reduced axes in the shape the bytes are the same
+    squeezed = tuple(d for k, d in enumerate(red.shape) if k not in axes)
+    assert np.array_equal(O.reduce_i8(kind, x, axes, squeezed, 7, 55).ravel(),
+                          O.reduce_i8(kind, x, axes, red.shape, 7, 55).ravel())

@@ -188,6 +188,8 @@ PROTOTYPES.update({
     "tpuhip_quantize_rescale": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_void_p,
                                           C.c_void_p]),
     "tpuhip_quantize_leaky_relu": (C.c_int, [C.c_float, C.c_float, C.c_float, C.c_void_p]),
+    "tpuhip_reduce_i8": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_int), C.c_int,
+                                   C.POINTER(C.c_int), C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint32]),
     "tpuhip_lrn_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int,
                                 C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]),
     "tpuhip_quantize_mlir_files": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p, C.c_char_p,

@@ -273,6 +273,8 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<PReluOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.clip") {
       krnl = std::make_shared<ClipOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.reduce_mean" || t == "tpu.reduce_sum" || t == "tpu.reduce_max" || t == "tpu.reduce_min") {
+      krnl = std::make_shared<ReduceOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.lrn") {
       krnl = std::make_shared<LrnOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.zero_mask") {

@@ -927,6 +927,35 @@ ClipOpKernel::ClipOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &
      name.c_str());
 }
 
+ReduceOpKernel::ReduceOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
+    : CPUOpKernel(op, valueMapping, weightMapping) {
+  require_int8("Reduce");
+  input_data = opdTensors.at(0).act;
+  output_data = resTensor;
+  if (!input_data) fail("Reduce '" + name + "': input missing");
+  kind = op.type == "tpu.reduce_mean" ? 0 : op.type == "tpu.reduce_sum" ? 1 : op.type == "tpu.reduce_max" ? 2 : 3;
+  // consecutive axes, as the reference asserts (reduce.cpp:33-37)
+  int count = 0;
+  while (op.attrs.count("axes" + std::to_string(count))) ++count;
+  if (count == 0) fail("Reduce '" + name + "': no axes");
+  first_axis = (int)op.attr("axes0");
+  last_axis = (int)op.attr("axes" + std::to_string(count - 1));
+  for (int i = 1; i < count; ++i)
+    if ((int)op.attr("axes" + std::to_string(i)) != first_axis + i) fail("Reduce '" + name + "': axes must be consecutive");
+  if (first_axis < 0 || last_axis > 3) fail("Reduce '" + name + "': axes outside a 4-D tensor");
+  // quant_rshift = opdTensors[3], quant_multiplier = opdTensors[4]; absent: 0 and 1 (reduce.cpp:14-20)
+  if (opdTensors.size() > 3 && opdTensors[3].weight) rshift = (int)f2u32(opdTensors[3].weight->at(0));
+  if (opdTensors.size() > 4 && opdTensors[4].weight) multiplier = f2u32(opdTensors[4].weight->at(0));
+}
+
+void ReduceOpKernel::invoke() {
+  const int in[4] = {input_data->n, input_data->c, input_data->h, input_data->w};
+  const int out[4] = {output_data->n, output_data->c, output_data->h, output_data->w};
+  ck(tpuhip_reduce_i8(ctx, kind, input_data->data(), output_data->data(), in, input_data->cs, out,
+                      output_data->cs, first_axis, last_axis, rshift, multiplier),
+     name.c_str());
+}
+
 LrnOpKernel::LrnOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping)
     : CPUOpKernel(op, valueMapping, weightMapping) {
   require_int8("Lrn");

@@ -211,6 +211,109 @@ extern "C" int tpuhip_dequant_i8_to_f32(tpuhip_ctx *ctx, const void *x, void *y_
   return TPUHIP_OK;
 }
 
+namespace {
+
+// Reduce over consecutive logical (NCHW) axes: kind 0 mean / 1 sum / 2 max / 3 min
+// (core/reduce.cpp:54-117, INT8).  A lane produces four consecutive channels of an output
+// pixel; each walks its `axis` sources through the logical index map.
+struct ReduceArgs {
+  const int8_t *x;
+  int8_t *y;
+  int kind, requant;
+  int ic, ih, iw, ics;
+  int oc, oh, ow, ocs;
+  int axis, inner;
+  float mult, inv_pot;
+  int64_t total;   // output pixels * (ocs / 4)
+};
+
+__global__ __launch_bounds__(kThreads) void reduce_kernel(ReduceArgs a) {
+  const int c4 = a.ocs >> 2;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int cq = (int)(i % c4);
+    const int pix = (int)(i / c4);
+    const int w = pix % a.ow;
+    const int h = (pix / a.ow) % a.oh;
+    const int n = pix / (a.ow * a.oh);
+    uint32_t word = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int c = cq * 4 + b;
+      if (c >= a.oc) continue;
+      // logical flat index of the output element, split at the reduced axes
+      const int64_t e = (((int64_t)n * a.oc + c) * a.oh + h) * a.ow + w;
+      const int64_t o = e / a.inner, in = e - o * a.inner;
+      int acc = a.kind == 2 ? -128 : a.kind == 3 ? 127 : 0;
+      for (int k = 0; k < a.axis; ++k) {
+        const int64_t l = (o * a.axis + k) * a.inner + in;
+        const int sw = (int)(l % a.iw);
+        const int64_t t1 = l / a.iw;
+        const int sh = (int)(t1 % a.ih);
+        const int64_t t2 = t1 / a.ih;
+        const int sc = (int)(t2 % a.ic);
+        const int64_t sn = t2 / a.ic;
+        const int v = a.x[((sn * a.ih + sh) * a.iw + sw) * a.ics + sc];
+        acc = a.kind <= 1 ? acc + v : a.kind == 2 ? max(acc, v) : min(acc, v);
+      }
+      int r = acc;
+      if (a.requant) {
+        // the float overload of applyMultiplierAndRShiftAndSaturateInt8 without qdm
+        const float prod = __fmul_rn((float)acc, a.mult);
+        r = saturate_int8_f(__fmul_rn(prod, a.inv_pot));   // power-of-two scaling: exact
+      }
+      word |= (uint32_t)(uint8_t)(int8_t)r << (8 * b);
+    }
+    *reinterpret_cast<uint32_t *>(a.y + (int64_t)pix * a.ocs + cq * 4) = word;
+  }
+}
+
+}  // namespace
+
+extern "C" int tpuhip_reduce_i8(tpuhip_ctx *ctx, int kind, const void *x, void *y, const int *in_nchw,
+                                int x_cs, const int *out_nchw, int y_cs, int first_axis, int last_axis,
+                                int rshift, uint32_t multiplier) {
+  TPUHIP_REQUIRE(ctx && x && y && in_nchw && out_nchw, "reduce: NULL argument");
+  TPUHIP_REQUIRE(kind >= 0 && kind <= 3, "reduce: unknown kind %d", kind);
+  TPUHIP_REQUIRE(first_axis >= 0 && first_axis <= last_axis && last_axis < 4, "reduce: axes %d..%d", first_axis,
+                 last_axis);
+  int64_t outer = 1, axis = 1, inner = 1, out_count = 1;
+  for (int k = 0; k < 4; ++k) {
+    TPUHIP_REQUIRE(in_nchw[k] > 0 && out_nchw[k] > 0, "reduce: non-positive dimension");
+    (k < first_axis ? outer : k <= last_axis ? axis : inner) *= in_nchw[k];
+    out_count *= out_nchw[k];
+  }
+  TPUHIP_REQUIRE(out_count == outer * inner, "reduce: the result holds %lld elements, expected %lld",
+                 (long long)out_count, (long long)(outer * inner));
+  TPUHIP_REQUIRE(x_cs >= in_nchw[1] && x_cs % 16 == 0 && y_cs >= out_nchw[1] && y_cs % 16 == 0,
+                 "reduce: channel strides must be multiples of 16 covering the channels");
+  TPUHIP_REQUIRE(outer * axis * inner < (1ll << 31) && axis * 128 < (1ll << 24),
+                 "reduce: tensor too large (the reference's float sum must stay exact)");
+  TPUHIP_REQUIRE(rshift >= 0 && rshift <= 30, "reduce: rshift %d outside [0,30]", rshift);
+  const bool requant = rshift != 0 || multiplier != 1;
+  TPUHIP_REQUIRE(requant || kind >= 2 || axis == 1,
+                 "reduce: a sum with rshift 0 and multiplier 1 has no int8 value (the reference leaves "
+                 "the raw sum in its float tensor)");
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  ReduceArgs a{};
+  a.x = (const int8_t *)x;
+  a.y = (int8_t *)y;
+  a.kind = kind;
+  a.requant = requant ? 1 : 0;
+  a.ic = in_nchw[1]; a.ih = in_nchw[2]; a.iw = in_nchw[3]; a.ics = x_cs;
+  a.oc = out_nchw[1]; a.oh = out_nchw[2]; a.ow = out_nchw[3]; a.ocs = y_cs;
+  a.axis = (int)axis;
+  a.inner = (int)inner;
+  a.mult = (float)multiplier;
+  a.inv_pot = 1.0f / (float)(1u << rshift);
+  a.total = (int64_t)out_nchw[0] * out_nchw[2] * out_nchw[3] * (y_cs / 4);
+  const unsigned blocks = (unsigned)std::max<int64_t>(
+      1, std::min<int64_t>(ceil_div64(a.total, kThreads), (int64_t)ctx->num_cu * 32));
+  launch(ctx, reduce_kernel, dim3(blocks), dim3(kThreads), a);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
 extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");
   TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_SWAP_CHANNEL,

@@ -27,7 +27,7 @@ _FLOATS = {"scale", "min", "max", "negative_slope", "const_val", "threshold"}
 _LUT_OPS = {"tpu.sigmoid", "tpu.tanh", "tpu.exp", "tpu.elu", "tpu.swish", "tpu.softplus", "tpu.log", "tpu.pow",
             "tpu.mish", "tpu.sqrt"}
 # numbered scalars of an op description <-> array attributes of the dialect
-_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4, "channel_order": 8}
+_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4, "channel_order": 8, "axes": 4}
 # flag scalars <-> string attributes
 _FLAGS = {"mode_edge": ("mode", "edge"), "mode_dcr": ("mode", "DCR")}
 

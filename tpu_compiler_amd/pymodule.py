@@ -41,6 +41,8 @@ _WEIGHT_OPERANDS = {
     "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [], "tpu.swap_channel": [],
     "tpu.zero_mask": [], "tpu.mul_const": [None, None, None, None],
     "tpu.lrn": ["sqr_lut", "power_lut", None],
+    "tpu.reduce_mean": [None, None, "rshift", "multiplier"], "tpu.reduce_sum": [None, None, "rshift", "multiplier"],
+    "tpu.reduce_max": [None, None, "rshift", "multiplier"], "tpu.reduce_min": [None, None, "rshift", "multiplier"],
     "tpu.upsample": [],
     "tpu.concat": [None, None, "rshift", "multiplier"],
     "tpu.reshape": [],
