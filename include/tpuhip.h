@@ -504,7 +504,8 @@ int tpuhip_quantize_lut_table(int kind, float threshold_x, float threshold_y, fl
  * fully_connected, eltwise add / max / min / mul, broadcast add / sub / mul, pool_avg_2d,
  * pool_max_2d, relu, leaky_relu, prelu, clip, concat, the table activations (sigmoid, tanh, exp, elu,
  * swish, softplus, log, pow, mish), upsample, pad, crop, permute, reorg, pixelshuffle, tile,
- * reverse, shuffle_channel, swap_channel, mul_const, reshape; anything else is refused by name.  `missing` (may be NULL)
+ * reverse, shuffle_channel, swap_channel, mul_const, lrn (with its threshold_parts), reshape;
+ * anything else is refused by name.  `missing` (may be NULL)
  * receives, one per line, the ops the table had no threshold for (the reference warns and goes
  * on); *needed = its length + 1. */
 int tpuhip_quantize_mlir_files(const char *in_mlir, const char *calibration_table, const char *out_mlir,

@@ -424,6 +424,89 @@ def test_quantized_files_run_bit_exact_and_track_the_fp32_network(tmp_path):
     m.close()
 
 
+def lrn_network():
+    """conv + ReLU -> LRN: -> (fp32 graph, input, torch activations, the three inner thresholds)"""
+    import torch
+    import torch.nn.functional as F
+    torch.manual_seed(5)
+    rng = np.random.default_rng(5)
+    n, hw, size, alpha, beta, k = 2, 10, 5, 2e-2, 0.75, 1.0
+    x = torch.tensor(rng.normal(0, 1, (n, 4, hw, hw)).astype(np.float32))
+    w, b = torch.randn(24, 4, 3, 3) * 0.5, torch.randn(24) * 0.3
+    a1 = F.relu(F.conv2d(x, w, b, padding=1))
+    one = alpha / size * a1 * a1
+    pad = F.pad(one, (0, 0, 0, 0, (size - 1) // 2, size - 1 - (size - 1) // 2))
+    two = sum(pad[:, j:j + 24] for j in range(size))
+    three = (two + k) ** -beta
+    y = F.local_response_norm(a1, size, alpha, beta, k)
+    assert torch.allclose(y, a1 * three, atol=1e-5)
+    g = graphs.Graph("lrn32", 0)
+    xin = graphs.Op("tpu.input", "input", [], tuple(x.shape))
+    xin.quant = "NONE"
+    xin.data = x.numpy()
+    g.add(xin)
+    fp32_op(g, "tpu.conv_2d", "c1", ["input"], tuple(a1.shape), conv_attrs(3, 1, True),
+            dict(filter=w.numpy(), bias=b.numpy()))
+    parts = [float(one.max()), float(two.max()), float(three.max())]
+    fp32_op(g, "tpu.lrn", "norm", ["c1"], tuple(a1.shape),
+            dict(local_size=size, alpha=alpha, beta=beta, k=k, sum_rshift=0, lrn_rshift=0, quant_data0=0, quant_data1=0,
+                 threshold_parts0=parts[0], threshold_parts1=parts[1], threshold_parts2=parts[2]))
+    g.outputs = ["norm"]
+    return g, x.numpy(), dict(input=x, c1=a1, norm=y), parts
+
+
+def test_lrn_tables_and_fractions_from_the_pass(tmp_path):
+    g, x, acts, parts = lrn_network()
+    path = tmp_path / "lrn.mlir"
+    mlir_text.write_mlir(g, path)
+    thr = measured_thresholds(acts)
+    open(tmp_path / "t", "w").write("".join("%s %.7g\n" % kv for kv in thr.items()))
+    out = tmp_path / "lrn_int8.mlir"
+    assert Q.quantize_files(path, tmp_path / "t", out) == []
+    ops, weights, _ = describe(out)
+    line = ops["norm"]["line"]
+    attr = lambda key: int(re.search(r"\b%s=(-?\d+)" % key, line).group(1))
+    # x / y ~ quant / 2^shift, shift as large as keeps the quantised numerator within 8 bits + 1
+    r0, q0, r1, q1 = attr("sum_rshift"), attr("quant_data0"), attr("lrn_rshift"), attr("quant_data1")
+    f32 = np.float32
+    assert 0 < q0 <= 256 and abs(q0 / 2.0 ** r0 - f32(parts[0]) / f32(parts[1])) <= 0.5 / 2.0 ** r0 + 1e-7
+    want1 = f32(thr["c1"]) * f32(parts[2]) / (f32(thr["norm"]) * 256.0)
+    assert 0 < q1 <= 256 and abs(q1 / 2.0 ** r1 - want1) <= 0.5 / 2.0 ** r1 + 1e-7
+    assert r0 == 15 or 2.0 ** (r0 + 1) >= 256.0 * parts[1] / parts[0]
+    with np.load(tmp_path / "lrn_int8_weights.npz") as z:
+        sq, pw = z["norm_sq_gen_weight"], z["norm_power_gen_weight"]
+    assert sq.shape == pw.shape == (1, 32, 16, 16)
+    sq, pw = sq.reshape(32, 256), pw.reshape(32, 256)
+    assert (sq == sq[0]).all() and (pw == pw[0]).all()
+    idx = np.arange(256)
+    # squares of thx/128 * idx scaled to 256 per sq threshold; (sum + k)^-beta scaled to 256 per its threshold
+    sq_real = np.minimum((thr["c1"] / 128.0 * idx) ** 2 * 2e-2 / 5 * 256.0 / parts[0], 255)
+    pw_real = np.minimum((idx / (256.0 / parts[1]) + 1.0) ** -0.75 * 256.0 / parts[2], 255)
+    assert np.abs(sq[0] - sq_real).max() <= 0.5 + 1e-3 and np.abs(pw[0] - pw_real).max() <= 0.5 + 1e-3
+    assert sq[0][0] == 0 and np.all(np.diff(sq[0]) >= 0) and np.all(np.diff(pw[0]) <= 0)
+
+
+@pytest.mark.gpu
+def test_lrn_graph_quantised_and_run_tracks_torch(tmp_path):
+    g, x, acts, parts = lrn_network()
+    path = tmp_path / "lrn.mlir"
+    mlir_text.write_mlir(g, path)
+    thr = measured_thresholds(acts)
+    open(tmp_path / "t", "w").write("".join("%s %.7g\n" % kv for kv in thr.items()))
+    out = tmp_path / "lrn_int8.mlir"
+    assert Q.quantize_files(path, tmp_path / "t", out) == []
+    m = module()
+    m.load(str(out))
+    m.set_tensor("input", x)
+    m.invoke()
+    got = m.get_tensor("norm_dequant").astype(np.float64).ravel()
+    ref = acts["norm"].numpy().astype(np.float64).ravel()
+    cos = (got * ref).sum() / np.sqrt((got * got).sum() * (ref * ref).sum())
+    assert cos > 0.995, cos
+    assert np.abs(got - ref).max() < 0.06 * thr["norm"]
+    m.close()
+
+
 def single_op_graph(kind, rng):
     """-> (fp32 graph, {input name: array}, torch result): the op graphs of the reference's backend
     tests (conv.mlir, deconv.mlir, fc.mlir, eltwise_add.mlir, avg_pool.mlir) rebuilt at small sizes"""

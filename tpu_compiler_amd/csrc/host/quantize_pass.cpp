@@ -579,6 +579,65 @@ struct Quantizer {
     create_weight(o, 1, "y0_table", std::move(table), {1, lanes, 16, 16}, "INT8");
   }
 
+  // quantize_fraction (:251-262): x / y as an integer over 2^rshift, the largest shift (up to
+  // 15) whose power of two stays below 256 * y / x
+  static void quantize_fraction(float x, float y, int &rshift_width, int &x_quantized) {
+    const float y_ceiling = 256.0 / x * y;
+    rshift_width = 0;
+    float y_quantized = 1.0;
+    while ((y_quantized * 2) < y_ceiling && rshift_width < 15) {
+      rshift_width += 1;
+      y_quantized = (float)(1 << rshift_width);
+    }
+    x_quantized = (int)std::floor((x / y) * y_quantized + 0.5);
+  }
+
+  void lrn(MlirOp &o) {   // quantizeInt8LrnOps (:264-347)
+    if (o.operands.size() < 3) fail("lrn '" + name_of(o) + "' needs the two table operands");
+    const uint32_t local_size = (uint32_t)num_attr(o.attrs, "local_size", 0);
+    const float alpha = (float)num_attr(o.attrs, "alpha", 0), beta = (float)num_attr(o.attrs, "beta", 0),
+                k = (float)num_attr(o.attrs, "k", 0);
+    auto *parts = o.attrs.get("threshold_parts");
+    if (local_size == 0 || !parts || parts->kind != MlirAttr::Array || parts->items.size() < 3)
+      fail("lrn '" + name_of(o) + "': local_size and the three threshold_parts (squares, their sum, the scale) are needed");
+    const float sq_thy = (float)parts->items[0].num, sumsq_thy = (float)parts->items[1].num,
+                scale_thy = (float)parts->items[2].num;
+    const float threshold_x = g.previous_threshold(o), threshold_y = g.threshold(&o);
+    int quant_x0 = 0, sum_rshift = 0, quant_x1 = 0, lrn_rshift = 0;
+    quantize_fraction(sq_thy, sumsq_thy, sum_rshift, quant_x0);
+    quantize_fraction(threshold_x * scale_thy, threshold_y * 256.0, lrn_rshift, quant_x1);
+    auto i32 = [](int v) {
+      MlirAttr a;
+      a.kind = MlirAttr::Int;
+      a.num = v;
+      a.ty = "i32";
+      return a;
+    };
+    field(o.attrs, "sum_rshift") = i32(sum_rshift);
+    field(o.attrs, "quant_data0") = i32(quant_x0);
+    field(o.attrs, "lrn_rshift") = i32(lrn_rshift);
+    field(o.attrs, "quant_data1") = i32(quant_x1);
+    const int lanes = 32;
+    std::vector<float> sq_table((size_t)lanes * 256), power_table((size_t)lanes * 256);
+    for (int idx = 0; idx < 256; ++idx) {
+      // the mix of float and double below is the reference's
+      float lut_input = threshold_x / 128.0 * idx;
+      float lut_output = std::pow(lut_input, 2) * 256.0 / sq_thy;
+      lut_output = lut_output * alpha / local_size;
+      lut_output = std::floor(lut_output + 0.5);
+      if (lut_output > 255.0) lut_output = 255.0;
+      for (int n = 0; n < lanes; ++n) sq_table[(size_t)n * 256 + idx] = lut_output;
+      lut_input = (float)idx / (256.0 / sumsq_thy);
+      lut_output = std::pow(lut_input + k, -beta);
+      lut_output = lut_output * (256.0 / scale_thy);
+      lut_output = std::floor(lut_output + 0.5);
+      if (lut_output > 255.0) lut_output = 255.0;
+      for (int n = 0; n < lanes; ++n) power_table[(size_t)n * 256 + idx] = lut_output;
+    }
+    create_weight(o, 1, "sq_gen_weight", std::move(sq_table), {1, lanes, 16, 16}, "UINT8");
+    create_weight(o, 2, "power_gen_weight", std::move(power_table), {1, lanes, 16, 16}, "UINT8");
+  }
+
   void bypass(MlirOp &o) {   // quantizeInt8BypassOps (:1206-1248)
     g.set_param_type(&o, "NONE");
     const float tx = g.previous_threshold(o), ty = g.threshold(&o);
@@ -604,6 +663,7 @@ struct Quantizer {
     else if (t == "tpu.concat") concat(o);
     else if (t == "tpu.leaky_relu") leaky_relu(o);
     else if (t == "tpu.prelu") prelu(o);
+    else if (t == "tpu.lrn") lrn(o);
     else if (t == "tpu.mul_const") {   // quantizeInt8MulConstOps (:1178-1197): only the sign is left
       const float c = (float)num_attr(o.attrs, "const_val", 0.0);
       field(o.attrs, "const_val") = f32_attr(c > 0.0f ? 1.0f : c < 0.0f ? -1.0f : 0.0f);

@@ -22,7 +22,9 @@ _POOL_PARAM = ["kernel_h", "kernel_w", "padding_t", "padding_b", "padding_l", "p
                "stride_h", "stride_w", "count_include_pad"]
 _BOOLS = {"do_relu", "is_dw", "with_bias", "count_include_pad", "input_transpose", "output_transpose",
           "fused_relu", "do_early_stride", "positive"}
-_FLOATS = {"scale", "min", "max", "negative_slope", "const_val", "threshold"}
+_FLOATS = {"scale", "min", "max", "negative_slope", "const_val", "threshold", "alpha", "beta", "k"}
+# numbered float scalars <-> float array attributes
+_FLOAT_ARRAYS = {"threshold_parts": 3}
 # the activations that become a table lookup in INT8: input, table, mantissa table
 _LUT_OPS = {"tpu.sigmoid", "tpu.tanh", "tpu.exp", "tpu.elu", "tpu.swish", "tpu.softplus", "tpu.log", "tpu.pow",
             "tpu.mish", "tpu.sqrt"}
@@ -82,6 +84,10 @@ def _attr_dict(op):
         vals = [a.pop(base + str(i)) for i in range(n) if base + str(i) in a]
         if vals:
             fields.append("%s = [%s]" % (base, ", ".join("%d : i32" % int(v) for v in vals)))
+    for base, n in _FLOAT_ARRAYS.items():
+        vals = [a.pop(base + str(i)) for i in range(n) if base + str(i) in a]
+        if vals:
+            fields.append("%s = [%s]" % (base, ", ".join(_f32(v) for v in vals)))
     for flag, (key, text) in _FLAGS.items():
         if a.pop(flag, 0):
             fields.append('%s = "%s"' % (key, text))
