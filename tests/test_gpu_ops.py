@@ -16,6 +16,9 @@ def capi_tile_name(t):
 
 
 NUM_TILES = next(t for t in range(1024) if capi_tile_name(t) is None)
+# the patch variants take 3x3 / stride 1 / pad 1 layers only; the others take any dense conv
+PATCH_TILES = [t for t in range(NUM_TILES) if "patch" in capi_tile_name(t)]
+GENERAL_TILES = [t for t in range(NUM_TILES) if t not in PATCH_TILES]
 
 
 @pytest.fixture(scope="module")
@@ -173,7 +176,7 @@ def test_conv_pair_equals_two_convs(ctx, case):
     assert not ctx.raw(yb)[..., ocb:].any() and not ctx.raw(ya)[..., oca:].any()
     assert len(np.unique(want_a)) > 8 and len(np.unique(want_b)) > 8
     # every tile variant splits its output the same way
-    for tile in range(NUM_TILES):
+    for tile in GENERAL_TILES:
         da.algo = db.algo = 16 + tile
         wt = ctx.conv_prepack_pair(da, db, (wa, f2i32(ba), f2i32(ma), f2i32(ra)),
                                    (wb, f2i32(bb) if bias_b else None, f2i32(mb), f2i32(rb)))
@@ -245,8 +248,80 @@ def test_conv_persistent_tiles_walk(ctx, case, tile):
     assert np.array_equal(got, want), "%s (general requant): %d mismatches" % (name, (got != want).sum())
 
 
+# n, c, h, w, oc, relu, fused add: 3x3 / stride 1 / pad 1 layers for the kernels that keep the input
+# rows of a tile in LDS
+PATCH_CASES = [
+    (2, 64, 56, 56, 64, True, False),      # ResNet-50 stage 2
+    (3, 128, 28, 28, 128, True, True),     # stage 3, with the add fused behind it
+    (2, 256, 14, 14, 256, False, False),   # stage 4: the image splits into two tiles of 7 rows
+    (1, 512, 7, 7, 72, True, False),       # whole image in one tile, ragged output channels
+    (2, 64, 9, 7, 40, False, True),        # tiny map, 63 of 128 pixel slots idle
+    (1, 128, 5, 20, 64, True, False),
+    (1, 64, 37, 30, 200, True, False),     # rows do not divide into equal tiles; four channel tiles
+    (5, 64, 3, 100, 16, False, False),     # wide and short
+]
+
+
+@pytest.mark.parametrize("case", PATCH_CASES)
+@pytest.mark.parametrize("tile", PATCH_TILES)
+def test_conv_patch_tile_variants(ctx, case, tile):
+    n, c, h, w_, oc, relu, add = case
+    bk = 256 if "k256" in capi_tile_name(tile) else 128 if "k128" in capi_tile_name(tile) else 64
+    if c % bk:
+        pytest.skip("%d-byte K steps need a multiple of %d channels" % (bk, bk))
+    rng = np.random.default_rng(c + h * 3 + oc + tile)
+    x = rnd_i8(rng, (n, c, h, w_))
+    w = rnd_w(rng, (oc, c, 3, 3), sigma=14)
+    bias, rsh, mult = rnd_params(rng, oc)
+    for general in (False, True):
+        r = rsh.copy()
+        if general:
+            r[::3] = 0      # an rshift of 0 forces the general requant form
+        want = oracle_conv(x, w, bias, r, mult, 1, (1, 1), (1, 1, 1, 1), (1, 1), (0, 0), relu)
+        d = conv_desc(x.shape, w.shape, pads=(1, 1, 1, 1), do_relu=relu, algo=16 + tile)
+        xt, yt = ctx.from_nchw(x), ctx.tensor(want.shape)
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+        wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(r))
+        assert "patch" in ctx.conv_algo_name(wh)
+        if add:
+            other = rnd_i8(rng, want.shape)
+            z_ref = O.eltwise_add_i8([other, want], [61, 47], [6], True)
+            ot, zt = ctx.from_nchw(other), ctx.tensor(want.shape)
+            ctx.conv_add(wh, xt, yt, ot, zt, 61, 47, 6, True)
+            assert np.array_equal(ctx.to_nchw(zt), z_ref)
+        else:
+            ctx.conv(wh, xt, yt)
+        got = ctx.to_nchw(yt)
+        assert np.array_equal(got, want), "%s: %d mismatches" % (ctx.conv_algo_name(wh), (got != want).sum())
+        assert not ctx.raw(yt)[..., oc:].any()
+        ctx.conv_weights_destroy(wh)
+    assert len(np.unique(want)) > 8
+
+
+@pytest.mark.parametrize("tile", PATCH_TILES)
+def test_conv_patch_tiles_refuse_other_layers(ctx, tile):
+    z = lambda oc, ic, k: (np.zeros((oc, ic, k, k), np.int8), None, np.full(oc, 1 << 30, np.int32), np.ones(oc, np.int32))
+    for shape, wshape, kw in [((1, 64, 8, 8), (64, 64, 3, 3), dict(stride=(2, 2), pads=(1, 1, 1, 1))),
+                              ((1, 96, 8, 8), (64, 96, 3, 3), dict(pads=(1, 1, 1, 1))),
+                              ((1, 64, 8, 8), (64, 64, 1, 1), dict()),
+                              ((1, 64, 8, 300), (64, 64, 3, 3), dict(pads=(1, 1, 1, 1)))]:
+        d = conv_desc(shape, wshape, algo=16 + tile, **kw)
+        wh = ctx.conv_prepack(d, *z(wshape[0], wshape[1], wshape[2]))
+        xt, yt = ctx.tensor(shape), ctx.tensor((d.n, d.oc, d.oh, d.ow))
+        with pytest.raises(capi.TpuHipError, match="3x3 / stride 1 / pad 1"):
+            ctx.conv(wh, xt, yt)
+        ctx.conv_weights_destroy(wh)
+    # nor do they run a pair
+    da, db = conv_desc((1, 64, 8, 8), (128, 64, 3, 3), pads=(1, 1, 1, 1), algo=16 + tile), \
+        conv_desc((1, 64, 8, 8), (16, 64, 3, 3), pads=(1, 1, 1, 1), algo=16 + tile)
+    wp = ctx.conv_prepack_pair(da, db, z(128, 64, 3), z(16, 64, 3))
+    with pytest.raises(capi.TpuHipError, match="single 3x3"):
+        ctx.conv_pair(wp, ctx.tensor((1, 64, 8, 8)), ctx.tensor((1, 128, 8, 8)), ctx.tensor((1, 16, 8, 8)))
+    ctx.conv_weights_destroy(wp)
+
+
 @pytest.mark.parametrize("case", TILE_CASES)
-@pytest.mark.parametrize("tile", range(NUM_TILES))
+@pytest.mark.parametrize("tile", GENERAL_TILES)
 def test_conv_every_mfma_tile_variant(ctx, case, tile):
     n, ic, ih, iw, oc, kh, kw, stride, pads, dil, relu = case
     rng = np.random.default_rng(ic * 7 + oc + tile)

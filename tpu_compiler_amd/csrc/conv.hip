@@ -222,11 +222,13 @@ __device__ __forceinline__ OutRoute route_out(const ConvArgs &a, int oc_tile_bas
                   second ? a.split_oc : 0};
 }
 
+// pix_limit: pixels from this index on are not written (a.npix, or the end of a tile that
+// stops short of its 32-pixel blocks)
 template <int TN, bool FAST>
-__device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
-                                              const int32_t *pmult, const int32_t *pshift,
-                                              const int32_t *phpot, int pix_first,
-                                              int pix_stride, const uint8_t *lut, const OutRoute &out) {
+__device__ __forceinline__ void epilogue_rows_lim(const v16i (&acc)[TN], const ConvArgs &a, int oc,
+                                                  const int32_t *pmult, const int32_t *pshift,
+                                                  const int32_t *phpot, int pix_first, int pix_stride,
+                                                  const uint8_t *lut, const OutRoute &out, int pix_limit) {
   uint32_t outw[TN][4];
   // channel index within the tensor written (a pair's second result starts at split_oc)
   int8_t *const ydst = out.y;
@@ -263,7 +265,7 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int pix = pix_first + j * pix_stride;
-    if (pix < a.npix) {
+    if (pix < pix_limit) {
       const int64_t off = (int64_t)pix * ycs + ocl;
       v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
       if (a.store_y) *reinterpret_cast<v4i *>(ydst + off) = o;
@@ -310,6 +312,14 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
       }
     }
   }
+}
+
+template <int TN, bool FAST>
+__device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvArgs &a, int oc,
+                                              const int32_t *pmult, const int32_t *pshift,
+                                              const int32_t *phpot, int pix_first,
+                                              int pix_stride, const uint8_t *lut, const OutRoute &out) {
+  epilogue_rows_lim<TN, FAST>(acc, a, oc, pmult, pshift, phpot, pix_first, pix_stride, lut, out, a.npix);
 }
 
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
@@ -785,6 +795,238 @@ conv_mfma_kernel(ConvArgs a) {
       }
     }
     if (!PERSIST || !more) break;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 3x3 / stride 1 / pad 1 convolutions on feature maps narrow enough that a few whole
+// rows fit a tile: the input patch of the tile ((TH + 2) rows x (W + 2) columns x C
+// channels, borders zero) is fetched ONCE into LDS and the nine taps are formed from it,
+// where the implicit-GEMM kernel above fetches every activation byte nine times.  Only
+// the filter streams through the K loop (registers -> LDS, as above).  A workgroup
+// computes BM output channels x TH rows of one image; pixels of the tile are its rows
+// flattened, so they are consecutive in the output tensor too.
+//   a.stem_pw = W + 2, a.magic_pw = floor(2^20 / (W + 2)) + 1, a.pstep_pix = TH,
+//   a.pstep_n = tiles per image, a.pstep_oh = log2(C / 16), a.pstep_ow = swizzle shift
+// C is 64, 128, 256 or 512 and a multiple of BK; the patch holds at most kPatchBytes (static
+// LDS; with 256-byte K steps it is dynamic LDS of the layer's exact size, at most
+// kPatchBytesDyn: a static array costs about half a microsecond less per launch).
+// ---------------------------------------------------------------------------
+constexpr int kPatchBytes = 45056;       // static patch (K steps up to 128 bytes)
+constexpr int kPatchBytesDyn = 65536;    // dynamic patch (256-byte K steps: the filter tiles take 32 KB)
+
+template <int BM, int BN, int BK, int DEPTH, int OCC, bool FAST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+conv_patch_kernel(ConvArgs a) {
+  constexpr int WM = 2, WN = 2, NT = 256;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  constexpr int CH = BK / 16;
+  constexpr int SW = CH == 4 ? 2 : CH == 8 ? 1 : 0;
+  constexpr int RP = NT / CH;
+  constexpr int NW = (BM + RP - 1) / RP;
+  constexpr bool DYN = BK == 256;
+  constexpr int NPL = (DYN ? kPatchBytesDyn : kPatchBytes) / 16 / NT;   // patch chunks per thread at most
+  static_assert(TM >= 1 && TN >= 1, "bad tile");
+  static_assert(DEPTH % 2 == 0 && DEPTH >= 2, "register ring depth");
+
+  __shared__ v4i lds[2][BM * CH];
+  __shared__ __attribute__((aligned(16))) int32_t qlds[4 * BM];
+  __shared__ v4i patch_static[DYN ? 1 : kPatchBytes / 16];
+  extern __shared__ __attribute__((aligned(16))) v4i patch_dynamic[];   // sized by the launch
+  v4i *const patch = DYN ? patch_dynamic : patch_static;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  if (logical >= a.n_tiles) return;
+  const int pt = logical / a.n_oc_tiles;
+  const int oc0 = (logical - pt * a.n_oc_tiles) * BM;
+  const int img = pt / a.pstep_n;
+  const int r0 = (pt - img * a.pstep_n) * a.pstep_pix;
+  const int rows = min(a.pstep_pix, a.oh - r0);
+  const int pix_base = (img * a.oh + r0) * a.ow;
+  const int pix_limit = pix_base + rows * a.ow;
+  const int pw = a.stem_pw;
+  const int lg = a.pstep_oh, cht = 1 << lg, swp = a.pstep_ow;
+
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  // ---- the patch: chunk q = position * (C / 16) + 16-channel group
+  const int n_chunks = (a.pstep_pix + 2) * pw << lg;
+  v4i preg[NPL];
+#pragma unroll
+  for (int u = 0; u < NPL; ++u) {
+    const int q = tid + u * NT;
+    const int pos = q >> lg, cc = q & (cht - 1);
+    const int pr = (int)(((uint32_t)pos * a.magic_pw) >> 20);
+    const int pc = pos - pr * pw;
+    const int row = r0 - 1 + pr, col = pc - 1;
+    const bool ok = q < n_chunks && (unsigned)row < (unsigned)a.ih && (unsigned)col < (unsigned)a.iw;
+    preg[u] = buffer_load16(xrsrc, ok ? (uint32_t)(((img * a.ih + row) * a.iw + col) * a.x_cs + cc * 16)
+                                      : kOobOffset);
+  }
+
+  int32_t qv[4] = {0, 0, 0, 0};
+  static_assert(BM <= NT, "one parameter row per thread");
+  if (tid < BM) {
+    qv[0] = a.bias[oc0 + tid];
+    qv[1] = a.qmult[oc0 + tid];
+    qv[2] = a.qshift[oc0 + tid];
+    qv[3] = a.qhpot[oc0 + tid];
+  }
+
+  // ---- the filter: as in conv_mfma_kernel
+  const int kc = tid % CH;
+  const int lrow = tid / CH;
+  uint32_t woff[NW];
+#pragma unroll
+  for (int s = 0; s < NW; ++s) {
+    const int r = lrow + RP * s;
+    woff[s] = r < BM ? (uint32_t)((oc0 + r) * a.kp + kc * 16) : kOobOffset;
+    asm volatile("" : "+v"(woff[s]));
+  }
+  v4i wreg[DEPTH][NW];
+  const int nsteps = a.kp / BK;
+  auto load_tile = [&](int slot, int step) {
+    const bool in_k = step < nsteps;
+#pragma unroll
+    for (int s = 0; s < NW; ++s)
+      wreg[slot][s] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+          wrsrc, in_k ? woff[s] : kOobOffset, step * BK, 0);
+  };
+  auto store_tile = [&](int slot, int buf) {
+    v4i *base = lds[buf];
+#pragma unroll
+    for (int s = 0; s < NW; ++s) {
+      const int r = lrow + RP * s;
+      if (BM % RP == 0 || r < BM) base[r * CH + (kc ^ ((r >> SW) & (CH - 1)))] = wreg[slot][s];
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  const int lch0 = wm * TM * 32 + fk * 16 * TM;
+  const int ocw0 = oc0 + lch0;
+
+  // top-left patch position of this lane's pixels (idle slots past the tile read position 0)
+  int pos0[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int p = (wn * TN + j) * 32 + frow;
+    const uint32_t pr = a.ow == 1 ? (uint32_t)p : __umulhi((uint32_t)p, a.magic_ow);
+    const int pc = p - (int)pr * a.ow;
+    pos0[j] = p < rows * a.ow ? (int)pr * pw + pc : 0;
+  }
+
+  // park the patch and the parameters
+#pragma unroll
+  for (int u = 0; u < NPL; ++u) {
+    const int q = tid + u * NT;
+    const int pos = q >> lg, cc = q & (cht - 1);
+    if (q < n_chunks) patch[(pos << lg) + (cc ^ ((pos >> swp) & (cht - 1)))] = preg[u];
+  }
+  if (tid < BM) {
+    qlds[tid] = qv[0];
+    qlds[BM + tid] = qv[1];
+    qlds[2 * BM + tid] = qv[2];
+    qlds[3 * BM + tid] = qv[3];
+  }
+
+  v16i acc[TM][TN];
+  constexpr int KK = BK / 32;
+  v4i fa[2][TM], fb[2][TN];
+  // fragments of 32-byte K slice kk of K step `step`: the filter from its LDS tile, the
+  // activations from the patch at the step's tap
+  auto read_frag = [&](int buf, int step, int kk, int fs) {
+    const v4i *wl = lds[buf];
+    const int chunk = kk * 2 + fk;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int r = (wm * TM + i) * 32 + frow;
+      fa[fs][i] = wl[r * CH + (chunk ^ ((r >> SW) & (CH - 1)))];
+    }
+    const int kg0 = step * CH;
+    const int tap = kg0 >> lg, cg = (kg0 & (cht - 1)) + chunk;
+    const int tkh = (int)(((uint32_t)tap * a.magic_kw) >> 20);
+    const int tap_off = tkh * pw + (tap - tkh * 3);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int pos = pos0[j] + tap_off;
+      fb[fs][j] = patch[(pos << lg) + (cg ^ ((pos >> swp) & (cht - 1)))];
+    }
+  };
+  auto mfma_frag = [&](int fs) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[fs][i], fb[fs][j], acc[i][j], 0, 0, 0);
+  };
+  int ks = 0;   // K step being multiplied
+  auto step_body = [&](int d) {
+    const int buf = d & 1;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + 1 < KK) read_frag(buf, ks, kk + 1, (kk + 1) & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_frag(kk & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk == 0) store_tile((d + 1) % DEPTH, buf ^ 1);
+    }
+    __syncthreads();
+    ++ks;
+    read_frag(buf ^ 1, min(ks, nsteps - 1), 0, 0);
+  };
+
+  __syncthreads();   // publishes qlds and the patch
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const v4i *bp = reinterpret_cast<const v4i *>(qlds + lch0 + i * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const v4i bq = bp[q];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        acc[i][j][q * 4 + 0] = bq[0];
+        acc[i][j][q * 4 + 1] = bq[1];
+        acc[i][j][q * 4 + 2] = bq[2];
+        acc[i][j][q * 4 + 3] = bq[3];
+      }
+    }
+  }
+  store_tile(0, 0);
+  __syncthreads();
+  read_frag(0, 0, 0, 0);
+
+  const int full = nsteps / DEPTH;
+#pragma nounroll
+  for (int g = 0; g < full; ++g) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      load_tile(d, (g + 1) * DEPTH + d);
+      step_body(d);
+    }
+  }
+  const int rem = nsteps - full * DEPTH;
+#pragma unroll
+  for (int d = 0; d < DEPTH - 1; ++d)
+    if (d < rem) step_body(d);
+
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int oc = ocw0 + i * 16;
+    const int lc = lch0 + i * 16;
+    if (oc < a.ocw)
+      epilogue_rows_lim<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
+                                  pix_base + wn * TN * 32 + frow, 32, nullptr, out, pix_limit);
   }
 }
 
@@ -1440,7 +1682,8 @@ struct TileCfg {
   int bm, bn, wm, wn;
   const char *name;
   int reg;   // 0: LDS kernel, one tile per workgroup; 1: the LDS-free kernel, bm x bn is the
-             // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups
+             // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups;
+             // 4: patch kernel (bn = pixel slots of a tile of whole rows)
   int bk;    // K bytes per step
 };
 
@@ -1468,6 +1711,14 @@ struct TileCfg {
   Y(16, "mfma_splitk_64x64", true, 2, 2, 4, 2)     \
   Y(17, "mfma_splitk_32x64", true, 1, 2, 4, 3)
 
+// patch kernels (3x3 / stride 1 / pad 1, input rows held in LDS): Z(index, name, BM, BN, BK, ring depth, waves per SIMD)
+#define TPUHIP_PATCH_TILES(Z)                          \
+  Z(18, "mfma_patch_64x128", 64, 128, 64, 2, 3)        \
+  Z(19, "mfma_patch_64x256", 64, 256, 64, 2, 2)        \
+  Z(20, "mfma_patch_64x128_k128", 64, 128, 128, 2, 2)  \
+  Z(21, "mfma_patch_64x128_k256", 64, 128, 256, 2, 2)  \
+  Z(22, "mfma_patch_64x64_k256", 64, 64, 256, 2, 2)
+
 struct TileTable {
   TileCfg t[64];
   int n = 0;
@@ -1482,6 +1733,11 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_REG_TILES(Y)
 #undef Y
+#define Z(i, name, BM, BN, BK, D, O) \
+  t[i] = TileCfg{BM, BN, 2, 2, name, 4, BK}; \
+  n = n > i ? n : i + 1;
+    TPUHIP_PATCH_TILES(Z)
+#undef Z
   }
 };
 const TileTable kTileTable;
@@ -1496,6 +1752,21 @@ void launch_reg(tpuhip_ctx *ctx, dim3 grid, const ConvArgs &a) {
     launch(ctx, (conv_mfma_splitk_kernel<TM, TN, D, O, FAST, UNI>), grid, dim3(256), a);
   else
     launch(ctx, (conv_mfma_reg_kernel<TM, TN, D, O, FAST, UNI>), grid, dim3(256), a);
+}
+
+// the patch kernel's LDS patch is dynamic: (rows + 2) x (W + 2) x C bytes of this layer
+template <typename F>
+void launch_patch(tpuhip_ctx *ctx, F kernel, dim3 grid, const ConvArgs &a, bool dynamic) {
+  static bool raised = false;   // per kernel instantiation; the same value from any thread
+  if (dynamic && !raised) {
+    (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kPatchBytesDyn);
+    raised = true;
+  }
+  const unsigned smem = dynamic ? (unsigned)((a.pstep_pix + 2) * a.stem_pw * (a.c16 * 16)) : 0u;
+  if (ctx->prof_start)
+    hipExtLaunchKernelGGL(kernel, grid, dim3(256), smem, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a);
+  else
+    hipLaunchKernelGGL(kernel, grid, dim3(256), smem, ctx->stream, a);
 }
 
 template <bool FAST, int MODE>
@@ -1513,6 +1784,10 @@ void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
   case i: launch_reg<SPLIT, TM, TN, D, O, FAST, UNI>(ctx, grid, a); break;
     TPUHIP_REG_TILES(Y)
 #undef Y
+#define Z(i, name, BM, BN, BK, D, O) \
+  case i: launch_patch(ctx, (conv_patch_kernel<BM, BN, BK, D, O, FAST>), grid, a, BK == 256); break;
+    TPUHIP_PATCH_TILES(Z)
+#undef Z
   }
 }
 
@@ -1624,7 +1899,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
     for (int c = 0; c < d.ic; ++c)
       for (int k = 0; k < d.kh * d.kw; ++k)
         rowbuf[(size_t)k * kstride + c] = src[(size_t)c * d.kh * d.kw + k];
-    if (t.reg == 0 || t.reg == 3) {
+    if (t.reg == 0 || t.reg == 3 || t.reg == 4) {
       memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
     } else {
       // fragment order: [row / 32][K step][kk][lane = (row & 31) + 32 * half][16 bytes]
@@ -1651,8 +1926,24 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 // the fused table lives in the LDS of the LDS kernels
 bool tile_has_lds_epilogue(int t) { return kTiles[t].reg == 0 || kTiles[t].reg == 3; }
 
+// rows of one image a patch tile holds; 0: the layer does not fit the patch kernel
+int patch_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
+  const bool shape_ok = d.g == 1 && d.kh == 3 && d.kw == 3 && d.sh == 1 && d.sw == 1 && d.dh == 1 && d.dw == 1 &&
+                        d.pt == 1 && d.pb == 1 && d.pl == 1 && d.pr == 1 && !d.ins_h && !d.ins_w &&
+                        d.oh == d.ih && d.ow == d.iw && d.x_cs == d.ic &&
+                        (d.ic == 64 || d.ic == 128 || d.ic == 256 || d.ic == 512) && d.ic % c.bk == 0;
+  if (!shape_ok || d.ow > c.bn) return 0;
+  // as many rows as the pixel slots and the patch buffer allow, then evened out over the image
+  const int fit = (int)((c.bk == 256 ? kPatchBytesDyn : kPatchBytes) / ((int64_t)(d.ow + 2) * d.ic)) - 2;
+  const int th_max = std::min(std::min(c.bn / d.ow, d.oh), fit);
+  if (th_max < 1) return 0;
+  const int tiles = (d.oh + th_max - 1) / th_max;
+  return (d.oh + tiles - 1) / tiles;
+}
+
 bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
+  if (c.reg == 4 && patch_rows(d, c) == 0) return false;
   if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
@@ -1698,6 +1989,20 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
     const int n_wgs = t.reg == 1 ? (a.n_tiles + 3) / 4 : a.n_tiles;
     a.tiles_per_xcd = (n_wgs + 7) / 8;
     a.wgs_per_xcd = a.tiles_per_xcd;
+    if (t.reg == 4) {
+      const int th = patch_rows(d, t);
+      const int tiles_per_img = (d.oh + th - 1) / th;
+      const int n_pix_tiles = d.n * tiles_per_img;
+      a.n_tiles = n_pix_tiles * a.n_oc_tiles;
+      a.tiles_per_xcd = (n_pix_tiles + 7) / 8 * a.n_oc_tiles;
+      a.wgs_per_xcd = a.tiles_per_xcd;
+      a.stem_pw = d.ow + 2;
+      a.magic_pw = (1u << 20) / (uint32_t)a.stem_pw + 1;
+      a.pstep_pix = th;
+      a.pstep_n = tiles_per_img;
+      a.pstep_oh = w->c16 == 4 ? 2 : w->c16 == 8 ? 3 : w->c16 == 16 ? 4 : 5;     // log2(C / 16)
+      a.pstep_ow = w->c16 == 4 ? 2 : w->c16 == 8 ? 1 : 0;                        // swizzle shift
+    }
     if (t.reg == 3) {
       // every XCD owns a run of whole pixel tiles; a workgroup keeps its channel tile
       const int n_pix_tiles = a.n_tiles / a.n_oc_tiles;
@@ -1777,6 +2082,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
   for (int t = 0; t < kNumTiles && !rc; ++t) {
     if (!tile_is_candidate(w->d, t)) continue;
     if (post.lut && !tile_has_lds_epilogue(t)) continue;
+    if (w->split_oc && kTiles[t].reg == 4) continue;   // the patch kernel writes one result
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
@@ -2034,6 +2340,9 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
                      w->algo == ALGO_STEM ||
                      (w->algo == ALGO_MFMA && tile_has_lds_epilogue(w->tile)),
                  "conv: kernel variant %s cannot fuse a table", tpuhip_conv2d_algo_name(w));
+  TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 4) || (!w->split_oc && patch_rows(w->d, kTiles[w->tile]) > 0),
+                 "conv: tile variant %s needs a single 3x3 / stride 1 / pad 1 conv with 64, 128, 256 or 512 input "
+                 "channels on a map narrow enough for its row patch", kTiles[w->tile].name);
   TPUHIP_REQUIRE((w->split_oc != 0) == (post.y2 != nullptr),
                  "conv: weights packed as a pair run through tpuhip_conv2d_pair_i8 (and only they do)");
   ConvArgs a;
