@@ -292,7 +292,8 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
 
 /* ---- pure data movement, 4-d shapes -----------------------------------------
  * Replaces PadOpKernel, CropOpKernel, PermuteOpKernel, ReorgOpKernel, TileOpKernel,
- * ReverseOpKernel, ShuffleChannelOpKernel, DepthToSpaceOpKernel (core/pad.cpp:114-141,
+ * ReverseOpKernel, ShuffleChannelOpKernel, DepthToSpaceOpKernel, SwapChannelOpKernel,
+ * DilateOpKernel, ReflectionPadOpKernel (core/pad.cpp:114-141,
  * crop.cpp:44-92, permute.cpp:8-44, reorg.cpp:20-42, tile.cpp:24-42, reverse.cpp:19-42,
  * shuffle_channel.cpp:21-48, depthtospace.cpp:8-80).  p[]:
  *   PAD_CONST / PAD_EDGE  p[0..3] pads at the beginning of n,c,h,w, p[4..7] at the end (constant
@@ -306,11 +307,17 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
  *   SHUFFLE_CHANNEL       p[0] group
  *   DEPTH_TO_SPACE        p[0] upscale factor, p[1] 1 = "DCR" mode, 0 = CRD
  *   SWAP_CHANNEL          p[0..ic-1] channel_order (output channel k is input channel p[k];
- *                         at most 8 channels; core/swap_channel.cpp:21-34) */
+ *                         at most 8 channels; core/swap_channel.cpp:21-34)
+ *   DILATE                p[0] ins_w, p[1] ins_h (fill values between columns / rows), p[2]
+ *                         fill_constant, an int8 value (DilateOpKernel, core/dilate.cpp:11-59)
+ *   REFLECTION_PAD        p[0] / p[1] columns added left / right of w, mirrored about the first /
+ *                         last column, each less than w (ReflectionPadOpKernel,
+ *                         core/reflectionpad.cpp:21-46) */
 enum {
   TPUHIP_MOVE_PAD_CONST = 0, TPUHIP_MOVE_PAD_EDGE = 1, TPUHIP_MOVE_CROP = 2, TPUHIP_MOVE_PERMUTE = 3,
   TPUHIP_MOVE_REORG = 4, TPUHIP_MOVE_TILE = 5, TPUHIP_MOVE_REVERSE = 6,
-  TPUHIP_MOVE_SHUFFLE_CHANNEL = 7, TPUHIP_MOVE_DEPTH_TO_SPACE = 8, TPUHIP_MOVE_SWAP_CHANNEL = 9
+  TPUHIP_MOVE_SHUFFLE_CHANNEL = 7, TPUHIP_MOVE_DEPTH_TO_SPACE = 8, TPUHIP_MOVE_SWAP_CHANNEL = 9,
+  TPUHIP_MOVE_DILATE = 10, TPUHIP_MOVE_REFLECTION_PAD = 11
 };
 typedef struct tpuhip_move_desc {
   int kind;

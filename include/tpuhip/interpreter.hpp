@@ -498,6 +498,8 @@ TPUHIP_MOVE_KERNEL(TileOpKernel, "CPUTileOp")                        // core/til
 TPUHIP_MOVE_KERNEL(ReverseOpKernel, "CPUReverseOp")                  // core/reverse.cpp:7-42
 TPUHIP_MOVE_KERNEL(ShuffleChannelOpKernel, "CPUShuffleChannelOp")    // core/shuffle_channel.cpp:7-48
 TPUHIP_MOVE_KERNEL(DepthToSpaceOpKernel, "CPUPixelShuffleOp")        // core/depthtospace.cpp:60-80
+TPUHIP_MOVE_KERNEL(DilateOpKernel, "CPUDilateOp")                    // core/dilate.cpp:34-59
+TPUHIP_MOVE_KERNEL(ReflectionPadOpKernel, "CPUReflectionPadOp")      // core/reflectionpad.cpp:7-46
 TPUHIP_MOVE_KERNEL(SwapChannelOpKernel, "CPUSwapChannelOp")          // core/swap_channel.cpp:8-35
 #undef TPUHIP_MOVE_KERNEL
 

@@ -628,6 +628,36 @@ void orc_reverse_i8(const int8_t *x, int8_t *y, const int64_t *s, int axis) {
         }
 }
 
+/* core/dilate.cpp:11-33 (dilateActivation as DilateOpKernel::invoke calls it: no pads, no
+ * trailing inserts): ins_h / ins_w fill values between the rows / columns. */
+void orc_dilate_i8(const int8_t *x, int8_t *y, const int64_t *s, int ins_h, int ins_w, int fill) {
+  const int n = (int)s[0], c = (int)s[1], h = (int)s[2], w = (int)s[3];
+  const int oh = (h - 1) * (ins_h + 1) + 1, ow = (w - 1) * (ins_w + 1) + 1;
+  for (int in = 0; in < n; in++)
+    for (int ic = 0; ic < c; ic++)
+      for (int _oh = 0; _oh < oh; _oh++)
+        for (int _ow = 0; _ow < ow; _ow++) {
+          const int64_t out_idx = (((int64_t)(in * c + ic) * oh) + _oh) * ow + _ow;
+          const int64_t in_nc = (int64_t)(in * c + ic) * h * w;
+          y[out_idx] = (int8_t)fill;
+          if (_ow % (ins_w + 1) == 0 && _oh % (ins_h + 1) == 0)
+            y[out_idx] = x[in_nc + (_oh / (ins_h + 1)) * w + _ow / (ins_w + 1)];
+        }
+}
+
+/* core/reflectionpad.cpp:21-46: mirror padding of the last dimension, the edge element
+ * itself not repeated. */
+void orc_reflection_pad_i8(const int8_t *x, int8_t *y, const int64_t *s, int pad_l, int pad_r) {
+  const int64_t rows = s[0] * s[1] * s[2];
+  const int K = (int)s[3], OK = K + pad_l + pad_r;
+  for (int64_t n = 0; n < rows; ++n)
+    for (int k = 0; k < K; ++k) y[n * OK + k + pad_l] = x[n * K + k];
+  for (int64_t n = 0; n < rows; ++n) {
+    for (int p = 0; p < pad_l; ++p) y[n * OK + pad_l - p - 1] = x[n * K + p + 1];
+    for (int p = 0; p < pad_r; ++p) y[n * OK + OK - pad_r + p] = x[n * K + K - p - 2];
+  }
+}
+
 void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *s, int group) {
   const int64_t frame = s[2] * s[3], batch = frame * s[1];
   const int col = (int)(s[1] / group);

@@ -181,6 +181,8 @@ void orc_shuffle_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, in
 /* core/depthtospace.cpp:8-58 (pixelshuffle), dcr_mode as in :60 */
 /* core/swap_channel.cpp:21-34, core/zero_mask.cpp:19-33, core/eltwise.cpp:386-401 (INT8 branches) */
 void orc_swap_channel_i8(const int8_t *x, int8_t *y, const int64_t *shape, const int *order);
+void orc_dilate_i8(const int8_t *x, int8_t *y, const int64_t *shape, int ins_h, int ins_w, int fill);
+void orc_reflection_pad_i8(const int8_t *x, int8_t *y, const int64_t *shape, int pad_l, int pad_r);
 void orc_zero_mask_i8(const int8_t *x, int8_t *y, int64_t n, int positive);
 void orc_mul_const_i8(const int8_t *x, int8_t *y, int64_t n, float const_val, int do_relu);
 /* core/lrn.cpp:104-166, INT8 */

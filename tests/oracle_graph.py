@@ -27,6 +27,8 @@ _BINARY = {"tpu.eltwise_max": O.BIN_MAX, "tpu.eltwise_min": O.BIN_MIN, "tpu.eltw
 
 _MOVES = {"tpu.pad": ("pad_const", ["pads*"]), "tpu.crop": ("crop", ["crop_offset*", "steps*"]),
           "tpu.swap_channel": ("swap_channel", ["channel_order*"]),
+          "tpu.dilate": ("dilate", ["ins0", "ins1", "fill_constant"]),
+          "tpu.reflection_pad": ("reflection_pad", ["pads0", "pads1"]),
           "tpu.permute": ("permute", ["order*"]), "tpu.reorg": ("reorg", ["stride"]),
           "tpu.tile": ("tile", ["axis", "tiles"]), "tpu.reverse": ("reverse", ["axis"]),
           "tpu.shuffle_channel": ("shuffle_channel", ["group"]),

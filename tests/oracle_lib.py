@@ -84,6 +84,8 @@ def _load():
     lib.orc_reorg_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_tile_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_reverse_i8.argtypes = [i8p, i8p, i64p, C.c_int]
+    lib.orc_dilate_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int, C.c_int]
+    lib.orc_reflection_pad_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_shuffle_channel_i8.argtypes = [i8p, i8p, i64p, C.c_int]
     lib.orc_depth_to_space_i8.argtypes = [i8p, i8p, i64p, C.c_int, C.c_int]
     lib.orc_swap_channel_i8.argtypes = [i8p, i8p, i64p, C.POINTER(C.c_int)]
@@ -276,6 +278,10 @@ def move_i8(kind, x, params, out_shape=None):
         out = tuple(s[k] * (p[1] if k == p[0] else 1) for k in range(4))
     elif kind in ("reverse", "shuffle_channel", "swap_channel"):
         out = s
+    elif kind == "dilate":      # p = ins_w, ins_h, fill_constant
+        out = (s[0], s[1], (s[2] - 1) * (p[1] + 1) + 1, (s[3] - 1) * (p[0] + 1) + 1)
+    elif kind == "reflection_pad":
+        out = (s[0], s[1], s[2], s[3] + p[0] + p[1])
     else:
         out = (s[0], s[1] // (p[0] * p[0]), s[2] * p[0], s[3] * p[0])
     y = np.empty(out, np.int8)
@@ -296,13 +302,17 @@ def move_i8(kind, x, params, out_shape=None):
         lib.orc_shuffle_channel_i8(xp, yp, _shape64(s), p[0])
     elif kind == "swap_channel":
         lib.orc_swap_channel_i8(xp, yp, _shape64(s), _ints(p[:s[1]]))
+    elif kind == "dilate":
+        lib.orc_dilate_i8(xp, yp, _shape64(s), p[1], p[0], p[2])
+    elif kind == "reflection_pad":
+        lib.orc_reflection_pad_i8(xp, yp, _shape64(s), p[0], p[1])
     else:
         lib.orc_depth_to_space_i8(xp, yp, _shape64(s), p[0], p[1])
     return y
 
 
 MOVE_KINDS = ["pad_const", "pad_edge", "crop", "permute", "reorg", "tile", "reverse",
-              "shuffle_channel", "depth_to_space", "swap_channel"]
+              "shuffle_channel", "depth_to_space", "swap_channel", "dilate", "reflection_pad"]
 
 
 def lrn_i8(x, local_size, sqr_lut, power_lut, sum_rshift, lrn_rshift, quant0, quant1):

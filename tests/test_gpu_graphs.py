@@ -476,6 +476,42 @@ def test_graph_with_swap_channel_mul_const_and_zero_mask(tmp_path, fuse):
         module().load(g)
 
 
+def test_graph_with_dilate_and_reflection_pad(tmp_path):
+    """a conv on a dilated map (what a transposed conv is lowered to) and one on a mirrored border"""
+    b = graphs.Builder("dilate_reflect", graphs.BASE_SEED + 83, 2, (6, 12))
+    x = b.input("input", 16, 9, 7)
+    g = b.g
+    n, c, h, w = g.by_name[x].shape
+    g.add(graphs.Op("tpu.dilate", "holes", [x], (n, c, 2 * h - 1, 3 * w - 2), dict(ins0=2, ins1=1, fill_constant=-3)))
+    cal = np.full((1, c, 2 * h - 1, 3 * w - 2), -3, np.int64)
+    cal[:, :, ::2, ::3] = b.cal[x]
+    b.cal["holes"] = cal
+    g.add(graphs.Op("tpu.reflection_pad", "mirror", [x], (n, c, h, w + 5), dict(pads0=2, pads1=3)))
+    b.cal["mirror"] = np.pad(b.cal[x], ((0, 0), (0, 0), (0, 0), (2, 3)), mode="reflect")
+    c1 = b.conv("c1", "holes", 24, 3)
+    c2 = b.conv("c2", "mirror", 24, 3)
+    g.outputs = [c1, c2]
+    want = oracle_graph.run(g)
+    xin = g.input_op().data
+    assert np.array_equal(want["mirror"], np.pad(xin, ((0, 0), (0, 0), (0, 0), (2, 3)), mode="reflect"))
+    assert np.array_equal(want["holes"][:, :, ::2, ::3], xin) and (want["holes"][:, :, 1::2] == -3).all()
+    m = module()
+    m.set_option("keep_all_tensors", 1)
+    m.load(g)
+    m.set_tensor("input", xin.astype(np.float32))
+    m.invoke()
+    for op in g.ops:
+        assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), op.name
+    m.close()
+    check_through_files(g, xin, want, tmp_path)
+    g.ops[2].attrs["pads1"] = w
+    with pytest.raises(capi.TpuHipError, match="reflection_pad: pads"):
+        mm = module()
+        mm.load(g)
+        mm.set_tensor("input", xin.astype(np.float32))
+        mm.invoke()
+
+
 def test_graph_with_reduce_ops_matches_the_oracle(tmp_path):
     """mean / max over the image, sum / min over the channels, with and without the reduced axes kept"""
     b = graphs.Builder("reduce_net", graphs.BASE_SEED + 83, 2, (6, 12))

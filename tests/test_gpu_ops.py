@@ -777,6 +777,12 @@ MOVES = [
     ("shuffle_channel", (2, 24, 3, 4), [3], None),
     ("depth_to_space", (2, 36, 3, 4), [3, 0], None),
     ("depth_to_space", (2, 64, 3, 4), [2, 1], None),
+    ("dilate", (2, 20, 5, 4), [1, 2, -7], None),       # ins_w, ins_h, fill_constant
+    ("dilate", (1, 3, 6, 7), [3, 0, 0], None),
+    ("dilate", (2, 17, 1, 9), [0, 0, 5], None),        # nothing inserted: a copy
+    ("reflection_pad", (2, 20, 5, 6), [2, 5], None),
+    ("reflection_pad", (1, 3, 4, 9), [0, 8], None),
+    ("reflection_pad", (3, 33, 2, 2), [1, 1], None),
 ]
 
 
@@ -798,6 +804,12 @@ def test_data_movement_rejects_bad_arguments(ctx):
         ctx.move(capi.MOVE_CROP, x, y, [0, 1, 0, 0, 1, 1, 1, 1])
     with pytest.raises(capi.TpuHipError, match="permutation"):
         ctx.move(capi.MOVE_PERMUTE, x, y, [0, 1, 2, 2])
+    with pytest.raises(capi.TpuHipError, match="no int8 value"):
+        ctx.move(O.MOVE_KINDS.index("dilate"), x, ctx.tensor((1, 16, 7, 7)), [1, 1, 200])
+    with pytest.raises(capi.TpuHipError, match="dilate: output shape"):
+        ctx.move(O.MOVE_KINDS.index("dilate"), x, ctx.tensor((1, 16, 8, 8)), [1, 1, 0])
+    with pytest.raises(capi.TpuHipError, match="reflection_pad: pads"):
+        ctx.move(O.MOVE_KINDS.index("reflection_pad"), x, ctx.tensor((1, 16, 4, 9)), [4, 1])
     with pytest.raises(capi.TpuHipError, match="group"):
         ctx.move(capi.MOVE_SHUFFLE_CHANNEL, x, y, [5])
     with pytest.raises(capi.TpuHipError, match="expected"):

@@ -72,6 +72,21 @@ def test_swap_channel_is_fancy_indexing_of_the_channel_axis():
         assert np.array_equal(O.move_i8("swap_channel", x, order), x[:, order])
 
 
+def test_dilate_is_a_strided_scatter_into_the_fill_value():
+    x = rnd((2, 3, 4, 5), 8)
+    for ins_w, ins_h, fill in [(1, 2, -7), (0, 3, 0), (2, 0, 127), (0, 0, 1)]:
+        want = np.full((2, 3, (4 - 1) * (ins_h + 1) + 1, (5 - 1) * (ins_w + 1) + 1), fill, np.int8)
+        want[:, :, ::ins_h + 1, ::ins_w + 1] = x
+        assert np.array_equal(O.move_i8("dilate", x, [ins_w, ins_h, fill]), want), (ins_w, ins_h, fill)
+
+
+def test_reflection_pad_is_numpy_reflect_on_the_last_axis():
+    x = rnd((2, 3, 4, 6), 9)
+    for left, right in [(0, 0), (2, 0), (0, 3), (5, 5), (1, 4)]:
+        want = np.pad(x, ((0, 0), (0, 0), (0, 0), (left, right)), mode="reflect")
+        assert np.array_equal(O.move_i8("reflection_pad", x, [left, right]), want), (left, right)
+
+
 def test_zero_mask_and_mul_const_on_every_byte():
     x = np.arange(-128, 128).astype(np.int8).reshape(1, 256, 1, 1)
     xi = x.astype(np.int64)

@@ -343,6 +343,33 @@ def test_mul_const_and_swap_channel_through_the_pass(tmp_path):
     assert "channel_order0=2" in ops["bgr"]["line"] and "channel_order2=0" in ops["bgr"]["line"]
 
 
+def test_dilate_and_reflection_pad_through_the_pass(tmp_path):
+    g = graphs.Graph("dr", 0)
+    xin = graphs.Op("tpu.input", "input", [], (1, 3, 4, 6))
+    xin.quant = "NONE"
+    xin.data = np.zeros((1, 3, 4, 6), np.float32)
+    g.add(xin)
+    fp32_op(g, "tpu.dilate", "holes", ["input"], (1, 3, 7, 11), dict(ins0=1, ins1=1, fill_constant=0))
+    fp32_op(g, "tpu.reflection_pad", "mirror", ["input"], (1, 3, 4, 11), dict(pads0=2, pads1=3))
+    g.outputs = ["holes", "mirror"]
+    path, out = tmp_path / "dr.mlir", tmp_path / "o.mlir"
+    mlir_text.write_mlir(g, path)
+    open(tmp_path / "t", "w").write("input 2.0\nholes 2.0\nmirror 2.0\n")
+    assert Q.quantize_files(path, tmp_path / "t", out) == []
+    ops, weights, _ = describe(out)
+    assert ops["holes"]["quant"] == ops["mirror"]["quant"] == "INT8"
+    wfile = [f for f in os.listdir(tmp_path) if f.endswith(".npz") and f.startswith("o")]
+    assert len(wfile) == 1, os.listdir(tmp_path)
+    w = np.load(tmp_path / wfile[0])
+    # one anti-diagonal 0/1 matrix per side, the size of that side's pad
+    for i, k in enumerate((2, 3)):
+        assert np.array_equal(w["mirror_select_%d" % i], np.fliplr(np.eye(k, dtype=np.float32)))
+    # a pass-through op whose sides disagree is refused (dilate is one; the mirror op is not checked)
+    open(tmp_path / "t", "w").write("input 2.0\nholes 1.0\nmirror 1.0\n")
+    with pytest.raises(capi.TpuHipError, match="thresholds differ"):
+        Q.quantize_files(path, tmp_path / "t", out)
+
+
 REF_GRAPHS = ["conv", "conv_1_oc", "deconv", "fc", "eltwise_add", "avg_pool", "max_pool", "relu", "concat",
               "broadcast_mul", "permute", "pixel_shuffle", "reorg", "reverse", "tile", "crop"]
 

@@ -40,7 +40,8 @@ class MoveDesc(C.Structure):
 
 
 (MOVE_PAD_CONST, MOVE_PAD_EDGE, MOVE_CROP, MOVE_PERMUTE, MOVE_REORG, MOVE_TILE, MOVE_REVERSE,
- MOVE_SHUFFLE_CHANNEL, MOVE_DEPTH_TO_SPACE) = range(9)
+ MOVE_SHUFFLE_CHANNEL, MOVE_DEPTH_TO_SPACE, MOVE_SWAP_CHANNEL, MOVE_DILATE,
+ MOVE_REFLECTION_PAD) = range(12)
 
 
 class PoolDesc(C.Structure):

@@ -261,6 +261,10 @@ void ModuleInterpreter::updateKernelList(ModuleDesc &module, std::string &target
       krnl = std::make_shared<TileOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.reverse") {
       krnl = std::make_shared<ReverseOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.dilate") {
+      krnl = std::make_shared<DilateOpKernel>(*op, valueMapping, weightMapping);
+    } else if (t == "tpu.reflection_pad") {
+      krnl = std::make_shared<ReflectionPadOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.shuffle_channel") {
       krnl = std::make_shared<ShuffleChannelOpKernel>(*op, valueMapping, weightMapping);
     } else if (t == "tpu.pixelshuffle") {

@@ -732,6 +732,18 @@ SwapChannelOpKernel::SwapChannelOpKernel(OpDesc &op, value_map_t &v, weight_map_
       fail("SwapChannel '" + name + "': channel_order[" + std::to_string(k) + "] = " + std::to_string(desc.p[k]));
   }
 }
+DilateOpKernel::DilateOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Dilate") {
+  desc.kind = TPUHIP_MOVE_DILATE;
+  desc.p[0] = (int)op.attr("ins0", 0);   // ins = [w, h], both optional (core/dilate.cpp:43-47)
+  desc.p[1] = (int)op.attr("ins1", 0);
+  desc.p[2] = (int)op.attr("fill_constant", 0);
+}
+ReflectionPadOpKernel::ReflectionPadOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
+    : MoveOpKernel(op, v, w, "ReflectionPad") {
+  desc.kind = TPUHIP_MOVE_REFLECTION_PAD;
+  desc.p[0] = (int)op.attr("pads0");
+  desc.p[1] = (int)op.attr("pads1");
+}
 DepthToSpaceOpKernel::DepthToSpaceOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
     : MoveOpKernel(op, v, w, "DepthToSpace") {
   desc.kind = TPUHIP_MOVE_DEPTH_TO_SPACE;

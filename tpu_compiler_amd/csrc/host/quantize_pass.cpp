@@ -132,7 +132,7 @@ const std::set<std::string> kForward = {
     "tpu.shuffle_channel", "tpu.swap_channel", "tpu.tile", "tpu.upsample"};
 // quantizeInt8BypassOps users within the INT8 interpreter's op set (QuantizeInt8.cpp:1606-1640)
 const std::set<std::string> kBypass = {
-    "tpu.crop", "tpu.pad", "tpu.permute", "tpu.pixelshuffle", "tpu.pool_max_2d", "tpu.relu", "tpu.reorg",
+    "tpu.crop", "tpu.dilate", "tpu.pad", "tpu.permute", "tpu.pixelshuffle", "tpu.pool_max_2d", "tpu.relu", "tpu.reorg",
     "tpu.reverse", "tpu.shuffle_channel", "tpu.swap_channel", "tpu.tile", "tpu.upsample"};
 const std::map<std::string, LutKind> kLut = {
     {"tpu.sigmoid", LutKind::Sigmoid}, {"tpu.tanh", LutKind::TanH}, {"tpu.exp", LutKind::Exp},
@@ -667,6 +667,20 @@ struct Quantizer {
     else if (t == "tpu.mul_const") {   // quantizeInt8MulConstOps (:1178-1197): only the sign is left
       const float c = (float)num_attr(o.attrs, "const_val", 0.0);
       field(o.attrs, "const_val") = f32_attr(c > 0.0f ? 1.0f : c < 0.0f ? -1.0f : 0.0f);
+    } else if (t == "tpu.reflection_pad") {
+      // ReflectionPadOp::quantizeInt8 (:1389-1414): one K x K anti-diagonal 0/1 matrix per pad
+      // (what the TPU multiplies the edge columns by to mirror them; the interpreter does not
+      // read them), named <op>_select_<i>, in operand slots 1 and 2
+      auto *pads = o.attrs.get("pads");
+      if (!pads || pads->kind != MlirAttr::Array || pads->items.size() != 2)
+        fail("reflection_pad '" + name_of(o) + "': pads must hold two numbers");
+      for (size_t i = 0; i < 2; ++i) {
+        const int64_t K = (int64_t)pads->items[i].num;
+        if (K < 0) fail("reflection_pad '" + name_of(o) + "': negative pad");
+        std::vector<float> select((size_t)(K * K), 0.0f);
+        for (int64_t r = 0; r < K; ++r) select[(size_t)(r * K + (K - r - 1))] = 1.0f;
+        create_weight(o, i + 1, "select_" + std::to_string(i), std::move(select), {K, K}, "INT8");
+      }
     } else if (kLut.count(t)) lut(o, kLut.at(t));
     else if (kBypass.count(t)) bypass(o);
     else fail("op '" + name_of(o) + "': no INT8 quantisation for " + t);

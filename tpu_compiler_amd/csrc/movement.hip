@@ -1,6 +1,7 @@
 // Pure data movement on int8 channels-last tensors: Pad, Crop, Permute, Reorg, Tile,
-// Reverse, ShuffleChannel, DepthToSpace, SwapChannel (core/pad.cpp, crop.cpp, permute.cpp,
-// reorg.cpp, tile.cpp, reverse.cpp, shuffle_channel.cpp, depthtospace.cpp, swap_channel.cpp).  Each is an index map from
+// Reverse, ShuffleChannel, DepthToSpace, SwapChannel, Dilate, ReflectionPad (core/pad.cpp, crop.cpp, permute.cpp,
+// reorg.cpp, tile.cpp, reverse.cpp, shuffle_channel.cpp, depthtospace.cpp, swap_channel.cpp,
+// dilate.cpp, reflectionpad.cpp).  Each is an index map from
 // the logical (n, c, h, w) of an output element to that of its source; one kernel
 // evaluates the map per element and moves the byte.  A lane produces four consecutive
 // output channels of a pixel (one dword store); pad channels are written as zero.
@@ -21,10 +22,11 @@ struct MoveArgs {
   int in, ic, ih, iw, ics;
   int on, oc, oh, ow, ocs;
   int p[12];
+  int fill;        // the byte of an element without a source (0 except for Dilate)
   int64_t total;   // output pixels * (ocs / 4)
 };
 
-// source of output element o = (n, c, h, w); false: the element is padding (zero)
+// source of output element o = (n, c, h, w); false: the element has none and takes a.fill
 __device__ __forceinline__ bool source_of(const MoveArgs &a, const int (&o)[4], int (&s)[4]) {
   switch (a.kind) {
     case TPUHIP_MOVE_PAD_CONST: {
@@ -94,6 +96,24 @@ __device__ __forceinline__ bool source_of(const MoveArgs &a, const int (&o)[4], 
       s[2] = o[2];
       s[3] = o[3];
       return true;
+    case TPUHIP_MOVE_DILATE: {
+      // p[0] = ins_w + 1, p[1] = ins_h + 1: input elements sit on that grid
+      const int qh = o[2] / a.p[1], qw = o[3] / a.p[0];
+      s[0] = o[0];
+      s[1] = o[1];
+      s[2] = qh;
+      s[3] = qw;
+      return qh * a.p[1] == o[2] && qw * a.p[0] == o[3];
+    }
+    case TPUHIP_MOVE_REFLECTION_PAD: {
+      // p[0] = columns added on the left; mirrored about the first / last column
+      const int j = o[3] - a.p[0];
+      s[0] = o[0];
+      s[1] = o[1];
+      s[2] = o[2];
+      s[3] = j < 0 ? -j : j >= a.iw ? 2 * (a.iw - 1) - j : j;
+      return true;
+    }
     default: {   // TPUHIP_MOVE_DEPTH_TO_SPACE: p[0] = upscale factor, p[1] = DCR mode
       const int r = a.p[0];
       const int dh = o[2] % r, dw = o[3] % r;
@@ -122,8 +142,9 @@ __global__ __launch_bounds__(kThreads) void move_kernel(MoveArgs a) {
       if (c >= a.oc) continue;
       const int o[4] = {n, c, h, w};
       int s[4] = {0, 0, 0, 0};
-      if (!source_of(a, o, s)) continue;
-      const int8_t v = a.x[((int64_t)(s[0] * a.ih + s[2]) * a.iw + s[3]) * a.ics + s[1]];
+      const int8_t v = source_of(a, o, s)
+                           ? a.x[((int64_t)(s[0] * a.ih + s[2]) * a.iw + s[3]) * a.ics + s[1]]
+                           : (int8_t)a.fill;
       word |= (uint32_t)(uint8_t)v << (8 * b);
     }
     *reinterpret_cast<uint32_t *>(a.y + (int64_t)pix * a.ocs + cq * 4) = word;
@@ -316,7 +337,7 @@ extern "C" int tpuhip_reduce_i8(tpuhip_ctx *ctx, int kind, const void *x, void *
 
 extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");
-  TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_SWAP_CHANNEL,
+  TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_REFLECTION_PAD,
                  "move: unknown kind %d", d->kind);
   TPUHIP_REQUIRE(d->in > 0 && d->ic > 0 && d->ih > 0 && d->iw > 0 && d->on > 0 && d->oc > 0 &&
                      d->oh > 0 && d->ow > 0,
@@ -404,6 +425,26 @@ extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const 
         TPUHIP_REQUIRE(p[k] >= 0 && p[k] < is[1], "swap_channel: channel_order[%d] = %d", k, p[k]);
         a.p[k] = p[k];
       }
+      break;
+    case TPUHIP_MOVE_DILATE:
+      // p[0] = ins_w, p[1] = ins_h, p[2] = fill_constant
+      TPUHIP_REQUIRE(p[0] >= 0 && p[1] >= 0, "dilate: negative ins (%d, %d)", p[0], p[1]);
+      TPUHIP_REQUIRE(p[2] >= -128 && p[2] <= 127, "dilate: fill_constant %d is no int8 value", p[2]);
+      TPUHIP_REQUIRE(os[0] == is[0] && os[1] == is[1] &&
+                         (int64_t)os[2] == (int64_t)(is[2] - 1) * (p[1] + 1) + 1 &&
+                         (int64_t)os[3] == (int64_t)(is[3] - 1) * (p[0] + 1) + 1,
+                     "dilate: output shape does not match");
+      a.p[0] = p[0] + 1;
+      a.p[1] = p[1] + 1;
+      a.fill = p[2];
+      break;
+    case TPUHIP_MOVE_REFLECTION_PAD:
+      // p[0] / p[1] columns added on the left / right; a mirror image needs a column to mirror
+      TPUHIP_REQUIRE(p[0] >= 0 && p[1] >= 0 && p[0] < is[3] && p[1] < is[3],
+                     "reflection_pad: pads (%d, %d) must be in [0, w = %d)", p[0], p[1], is[3]);
+      TPUHIP_REQUIRE(os[0] == is[0] && os[1] == is[1] && os[2] == is[2] && os[3] == is[3] + p[0] + p[1],
+                     "reflection_pad: output shape does not match");
+      a.p[0] = p[0];
       break;
     default:
       TPUHIP_REQUIRE(p[0] >= 1 && is[1] % (p[0] * p[0]) == 0, "depth_to_space: bad upscale factor %d", p[0]);

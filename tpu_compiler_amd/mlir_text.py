@@ -29,7 +29,7 @@ _FLOAT_ARRAYS = {"threshold_parts": 3}
 _LUT_OPS = {"tpu.sigmoid", "tpu.tanh", "tpu.exp", "tpu.elu", "tpu.swish", "tpu.softplus", "tpu.log", "tpu.pow",
             "tpu.mish", "tpu.sqrt"}
 # numbered scalars of an op description <-> array attributes of the dialect
-_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4, "channel_order": 8, "axes": 4}
+_ARRAYS = {"pads": 8, "crop_offset": 4, "steps": 4, "order": 4, "channel_order": 8, "axes": 4, "ins": 2}
 # flag scalars <-> string attributes
 _FLAGS = {"mode_edge": ("mode", "edge"), "mode_dcr": ("mode", "DCR")}
 

@@ -39,6 +39,7 @@ _WEIGHT_OPERANDS = {
     "tpu.quant": [],
     "tpu.pad": [], "tpu.crop": [], "tpu.permute": [], "tpu.reorg": [], "tpu.tile": [],
     "tpu.reverse": [], "tpu.shuffle_channel": [], "tpu.pixelshuffle": [], "tpu.swap_channel": [],
+    "tpu.dilate": [], "tpu.reflection_pad": [None, None],
     "tpu.zero_mask": [], "tpu.mul_const": [None, None, None, None],
     "tpu.lrn": ["sqr_lut", "power_lut", None],
     "tpu.reduce_mean": [None, None, "rshift", "multiplier"], "tpu.reduce_sum": [None, None, "rshift", "multiplier"],
