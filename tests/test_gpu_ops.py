@@ -298,6 +298,79 @@ def test_conv_patch_tile_variants(ctx, case, tile):
     assert len(np.unique(want)) > 8
 
 
+def _random_conv_case(rng):
+    """a dense conv of one of three families: 3x3 / stride 1 / pad 1 on the channel counts the
+    row-patch kernels take, 1x1 with stride 1 or 2, or anything goes"""
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        ic, kh, kw, stride, pads, dil = int(rng.choice([64, 128, 256, 512])), 3, 3, (1, 1), (1, 1, 1, 1), (1, 1)
+        iw, n, oc = int(rng.integers(1, 130)), int(rng.integers(1, 4)), int(rng.integers(1, 200))
+        ih = min(int(rng.integers(1, 40)), max(1, 400000 // (n * iw * ic)))
+    elif kind == 1:
+        s = int(rng.integers(1, 3))
+        ic, kh, kw, stride, pads, dil = int(rng.integers(1, 300)), 1, 1, (s, s), (0, 0, 0, 0), (1, 1)
+        ih, iw, n, oc = int(rng.integers(1, 30)), int(rng.integers(1, 30)), int(rng.integers(1, 5)), int(rng.integers(1, 400))
+    else:
+        ic, kh, kw = int(rng.integers(1, 100)), int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pads = tuple(int(v) for v in rng.integers(0, 4, 4))
+        ih, iw, n, oc = int(rng.integers(1, 24)), int(rng.integers(1, 24)), int(rng.integers(1, 4)), int(rng.integers(1, 150))
+        if ih + pads[0] + pads[1] < dil[0] * (kh - 1) + 1 or iw + pads[2] + pads[3] < dil[1] * (kw - 1) + 1:
+            return None
+    return n, ic, ih, iw, oc, kh, kw, stride, pads, dil
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_conv_random_shapes_every_tile_variant(ctx, seed):
+    """25 random convs per seed, each through every tile variant that takes it, with and without
+    the fused add and with both requant forms; all must give the oracle's bytes"""
+    ran = set()
+    for it in range(25):
+        rng = np.random.default_rng(7000 + seed * 100 + it)
+        case = _random_conv_case(rng)
+        if case is None:
+            continue
+        n, ic, ih, iw, oc, kh, kw, stride, pads, dil = case
+        relu, add, general = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), rng.integers(0, 4) == 0
+        x = rnd_i8(rng, (n, ic, ih, iw))
+        w = rnd_w(rng, (oc, ic, kh, kw), sigma=max(2.0, min(40.0, 375.0 / (ic * kh * kw) ** 0.5)))
+        bias, rsh, mult = rnd_params(rng, oc, 5, 11)
+        if general:
+            rsh[::3] = 0
+        want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, dil, (0, 0), relu)
+        other = rnd_i8(rng, want.shape)
+        z_ref = O.eltwise_add_i8([other, want], [61, 47], [6], True)
+        xt, ot = ctx.from_nchw(x), ctx.from_nchw(other)
+        yt, zt = ctx.tensor(want.shape), ctx.tensor(want.shape)
+        for tile in GENERAL_TILES + PATCH_TILES:
+            d = conv_desc(x.shape, w.shape, stride=stride, pads=pads, dil=dil, do_relu=relu, algo=16 + tile)
+            try:
+                wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+            except capi.TpuHipError:
+                continue       # this variant does not take the layer
+            ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+            try:
+                if add:
+                    ctx.conv_add(wh, xt, yt, ot, zt, 61, 47, 6, True)
+                else:
+                    ctx.conv(wh, xt, yt)
+            except capi.TpuHipError as e:
+                assert "tile variant" in str(e)
+                ctx.conv_weights_destroy(wh)
+                continue
+            label = (it, capi_tile_name(tile), x.shape, w.shape, stride, pads, dil, relu, add, bool(general))
+            assert np.array_equal(ctx.to_nchw(yt), want), label
+            assert not ctx.raw(yt)[..., oc:].any(), label
+            if add:
+                assert np.array_equal(ctx.to_nchw(zt), z_ref), label
+            ran.add(capi_tile_name(tile))
+            ctx.conv_weights_destroy(wh)
+        for t in (xt, ot, yt, zt):
+            t.free()
+    assert len(ran) >= 15, sorted(ran)
+
+
 @pytest.mark.parametrize("tile", PATCH_TILES)
 def test_conv_patch_tiles_refuse_other_layers(ctx, tile):
     z = lambda oc, ic, k: (np.zeros((oc, ic, k, k), np.int8), None, np.full(oc, 1 << 30, np.int32), np.ones(oc, np.int32))
