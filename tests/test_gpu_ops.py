@@ -917,3 +917,89 @@ def test_lrn_refuses_parameters_whose_float_form_is_inexact(ctx):
         ctx.lrn(xt, yt, 5, t, t, 8, 8, 100, 600)
     with pytest.raises(capi.TpuHipError, match="local_size"):
         ctx.lrn(xt, yt, 0, t, t, 8, 8, 100, 100)
+
+
+def test_random_pool_add_table_upsample_concat_sweep(ctx):
+    """700 random cases over max / average pooling (windows, strides, pads, global), n-input add,
+    byte tables, leaky relu, upsample and concat (with and without rescaling) against the oracle"""
+    seen = {}
+    for it in range(700):
+        rng = np.random.default_rng(888000 + it)
+        kind = ["max", "avg", "add", "lut", "leaky", "up", "concat"][int(rng.integers(0, 7))]
+        n, c, ih, iw = int(rng.integers(1, 4)), int(rng.integers(1, 150)), int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        x = rnd_i8(rng, (n, c, ih, iw))
+        xt = ctx.from_nchw(x)
+        tmp = [xt]
+        try:
+            if kind in ("max", "avg"):
+                if rng.integers(0, 5) == 0:
+                    k, s, pads = (ih, iw), (1, 1), (0, 0, 0, 0)
+                else:
+                    k = (int(rng.integers(1, 5)), int(rng.integers(1, 5)))
+                    s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+                    pads = tuple(int(min(v, kk - 1)) for v, kk in zip(rng.integers(0, 3, 4), (k[0], k[0], k[1], k[1])))
+                if ih + pads[0] + pads[1] < k[0] or iw + pads[2] + pads[3] < k[1]:
+                    continue
+                d0, d = O.make_pool_desc(x.shape, k, s, pads), pool_desc(x.shape, k, s, pads)
+                yt = ctx.tensor((n, c, d0.oh, d0.ow))
+                tmp.append(yt)
+                if kind == "max":
+                    want = O.pool_max_i8(x, d0)
+                    ctx.pool_max(d, xt, yt)
+                else:
+                    mult, rs = int(rng.integers(1, 256)), int(rng.integers(0, 14))
+                    want = O.pool_avg_i8(x, d0, rs, mult)
+                    ctx.pool_avg(d, xt, yt, mult, rs)
+            elif kind == "add":
+                nin = int(rng.integers(2, 5))
+                xs = [x] + [rnd_i8(rng, x.shape) for _ in range(nin - 1)]
+                mult = [int(v) for v in rng.integers(-128, 128, nin)]
+                rs, relu = int(rng.integers(0, 12)), bool(rng.integers(0, 2))
+                want = O.eltwise_add_i8(xs, mult, [rs], relu)
+                xts = [xt] + [ctx.from_nchw(v) for v in xs[1:]]
+                yt = ctx.tensor(x.shape)
+                tmp += xts[1:] + [yt]
+                ctx.eltwise_add(xts, mult, rs, relu, yt)
+            elif kind == "lut":
+                table = rnd_i8(rng, 256)
+                want = table[x.astype(np.uint8)]
+                yt = ctx.tensor(x.shape)
+                tmp.append(yt)
+                ctx.lut(xt, yt, table)
+            elif kind == "leaky":
+                rp, mp, rn, mn = (int(rng.integers(0, 9)), int(rng.integers(1, 128)), int(rng.integers(0, 9)),
+                                  int(rng.integers(1, 128)))
+                want = O.leaky_relu_i8(x, rp, mp, rn, mn)
+                yt = ctx.tensor(x.shape)
+                tmp.append(yt)
+                ctx.leaky_relu(xt, yt, rp, mp, rn, mn)
+            elif kind == "up":
+                sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+                want = O.upsample_i8(x, sh, sw)
+                yt = ctx.tensor(want.shape)
+                tmp.append(yt)
+                ctx.upsample(xt, yt, sh, sw)
+            else:
+                axis, nin, xs = int(rng.integers(0, 4)), int(rng.integers(2, 5)), [x]
+                for _ in range(nin - 1):
+                    shp = list(x.shape)
+                    shp[axis] = int(rng.integers(1, 40))
+                    xs.append(rnd_i8(rng, shp))
+                rs = mult = None
+                relu = False
+                if rng.integers(0, 2):
+                    rs = [int(v) for v in rng.integers(0, 8, nin)]
+                    mult = [int(v) for v in rng.integers(1, 128, nin)]
+                    relu = bool(rng.integers(0, 2))
+                want = O.concat_i8(xs, axis, rs, mult, relu)
+                xts = [xt] + [ctx.from_nchw(v) for v in xs[1:]]
+                yt = ctx.tensor(want.shape)
+                tmp += xts[1:] + [yt]
+                ctx.concat(xts, axis, yt, rs, mult, relu)
+            assert np.array_equal(ctx.to_nchw(yt), want), (it, kind, x.shape, want.shape)
+            assert not ctx.raw(yt)[..., want.shape[1]:].any(), (it, kind)
+            seen[kind] = seen.get(kind, 0) + 1
+        finally:
+            for t in tmp:
+                t.free()
+    assert len(seen) == 7 and min(seen.values()) > 50, seen
