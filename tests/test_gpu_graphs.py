@@ -794,3 +794,81 @@ def test_fp32_network_quantized_with_the_host_helpers_tracks_the_fp32_result(tmp
             assert np.abs(deq - ref).max() < 0.06 * thr[op.name], (op.name, np.abs(deq - ref).max() / thr[op.name])
     m.close()
     check_through_files(g, xin.data, want, tmp_path)
+
+
+def _random_graph(it):
+    """a random DAG of convs (1x1 / 3x3 / depthwise, some strided), adds, leaky relu, clip, max pool,
+    upsample and concat over earlier tensors; None when the builder's guards reject it"""
+    rng = np.random.default_rng(424200 + it)
+    b = graphs.Builder("fz%d" % it, graphs.BASE_SEED + 1000 + it, int(rng.integers(1, 3)), (5, 11))
+    hw = int(rng.integers(5, 15))
+    vals = [b.input("input", int(rng.choice([3, 16, 24, 64])), hw, hw + int(rng.integers(0, 4)))]
+    g = b.g
+    kinds = ["conv1", "conv3", "add", "leaky", "clip", "pool", "concat", "conv1", "conv3", "add", "up", "dw"]
+    try:
+        for k in range(int(rng.integers(3, 14))):
+            kind = kinds[int(rng.integers(0, 12))]
+            src = vals[int(rng.integers(0, len(vals)))] if rng.integers(0, 3) else vals[-1]
+            shp = g.by_name[src].shape
+            name = "%s_%d" % (kind, k)
+            if kind == "conv1":
+                s = 2 if (rng.integers(0, 4) == 0 and shp[2] > 3) else 1
+                vals.append(b.conv(name, src, int(rng.choice([16, 24, 64, 128, 40])), 1, stride=s,
+                                   relu=bool(rng.integers(0, 2))))
+            elif kind == "conv3":
+                vals.append(b.conv(name, src, int(rng.choice([16, 24, 64, 72])), 3, relu=bool(rng.integers(0, 2))))
+            elif kind == "dw":
+                if shp[1] >= 8:
+                    vals.append(b.conv(name, src, shp[1], 3, groups=shp[1], relu=bool(rng.integers(0, 2))))
+            elif kind == "add":
+                same = [v for v in vals if g.by_name[v].shape == shp and v != "input"]
+                if same and src != "input":
+                    other = same[int(rng.integers(0, len(same)))]
+                    vals.append(b.add(name, [src, other] if rng.integers(0, 2) else [other, src],
+                                      bool(rng.integers(0, 2))))
+            elif kind == "leaky":
+                vals.append(b.leaky(name, src))
+            elif kind == "clip":
+                vals.append(b.clip(name, src, -int(rng.integers(0, 100)), int(rng.integers(1, 100))))
+            elif kind == "pool":
+                if shp[2] >= 3 and shp[3] >= 3:
+                    vals.append(b.pool_max(name, src, 2, 2, (0, 0, 0, 0)))
+            elif kind == "up":
+                if shp[2] * shp[3] <= 400:
+                    vals.append(b.upsample(name, src, 2))
+            else:
+                same = [v for v in vals if g.by_name[v].shape[0] == shp[0] and g.by_name[v].shape[2:] == shp[2:]]
+                if len(same) >= 2:
+                    take = rng.choice(len(same), size=min(len(same), int(rng.integers(2, 4))), replace=False)
+                    vals.append(b.concat(name, [same[int(i)] for i in take]))
+    except (AssertionError, ValueError):
+        return None
+    if len(vals) < 2:
+        return None
+    return b.finish(vals[1:][-3:])
+
+
+def test_random_graphs_with_and_without_fusion_and_pairing():
+    """80 random graphs: whatever the interpreter folds into conv epilogues, packs into one launch
+    or leaves unwritten, every tensor it keeps must equal the oracle's"""
+    ran = fused = 0
+    for it in range(80):
+        g = _random_graph(it)
+        if g is None:
+            continue
+        want = oracle_graph.run(g)
+        for fuse, pair, keep in ((1, 1, 1), (1, 1, 0), (0, 0, 1)):
+            m = module()
+            m.set_option("keep_all_tensors", keep)
+            m.set_option("fuse_eltwise", fuse)
+            m.set_option("pair_convs", pair)
+            m.load(g)
+            m.set_tensor("input", g.input_op().data.astype(np.float32))
+            m.invoke()
+            for name in ([op.name for op in g.ops] if keep else g.outputs):
+                assert np.array_equal(m.get_tensor_i8(name), want[name].reshape(g.by_name[name].shape)), \
+                    (it, fuse, pair, keep, name, [(o.type, o.name, o.inputs) for o in g.ops])
+            m.close()
+        ran += 1
+        fused += any(o.type == "tpu.eltwise_add" for o in g.ops)
+    assert ran >= 60 and fused >= 20, (ran, fused)
