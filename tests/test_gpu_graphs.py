@@ -872,3 +872,96 @@ def test_random_graphs_with_and_without_fusion_and_pairing():
         ran += 1
         fused += any(o.type == "tpu.eltwise_add" for o in g.ops)
     assert ran >= 60 and fused >= 20, (ran, fused)
+
+
+def _random_single_op_graph(it):
+    """one transposed conv (dense / grouped / depthwise, strides, dilation, pads, output padding),
+    one reduce (kind, consecutive axes, kept or dropped, rescaled or not) or one FC behind an input"""
+    f32 = lambda *v: np.array(v, np.float32)
+    rng = np.random.default_rng(616100 + it)
+    kind = ["deconv", "reduce", "fc"][int(rng.integers(0, 3))]
+    g = graphs.Graph("fz", 1)
+    n = int(rng.integers(1, 3))
+    if kind == "deconv":
+        grp = int(rng.choice([1, 1, 2, 0]))
+        ic = int(rng.integers(1, 40))
+        oc = int(rng.integers(1, 40))
+        if grp == 0:
+            grp = ic
+            oc = ic
+        elif grp == 2:
+            (ic, oc) = (2 * int(rng.integers(1, 16)), 2 * int(rng.integers(1, 16)))
+        (ih, iw) = (int(rng.integers(1, 10)), int(rng.integers(1, 10)))
+        k = int(rng.integers(1, 5))
+        stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pads = tuple((int(min(v, dil[i // 2] * (k - 1))) for (i, v) in enumerate(rng.integers(0, 3, 4))))
+        oh = (ih - 1) * stride[0] - pads[0] - pads[1] + dil[0] * (k - 1) + 1 + int(rng.integers(0, stride[0]))
+        ow = (iw - 1) * stride[1] - pads[2] - pads[3] + dil[1] * (k - 1) + 1 + int(rng.integers(0, stride[1]))
+        if oh < 1 or ow < 1:
+            return (None, kind)
+        x = rng.integers(-128, 128, (n, ic, ih, iw)).astype(np.int8)
+        g.add(graphs.Op("tpu.input", "input", [], x.shape)).data = x
+        w = np.clip(np.rint(rng.normal(0, 30, (oc, ic // grp, k, k))), -127, 127).astype(np.float32)
+        bias = rng.integers(-2000, 2000, oc).astype(np.float32)
+        mult = (rng.integers(1 << 23, 1 << 24, oc) * 128).astype(np.float32)
+        rsh = rng.integers(3, 11, oc).astype(np.float32)
+        g.add(graphs.Op("tpu.deconv_2d", "y", ["input"], (n, oc, oh, ow),
+                        dict(kernel_h=k, kernel_w=k, stride_h=stride[0], stride_w=stride[1], padding_t=pads[0],
+                             padding_b=pads[1], padding_l=pads[2], padding_r=pads[3], dilation_h=dil[0],
+                             dilation_w=dil[1], group=grp, with_bias=1, do_relu=int(rng.integers(0, 2))),
+                        dict(filter=w.ravel(), bias=bias, rshift=rsh, multiplier=mult), "RSHIFT_AND_M_I32"))
+    elif kind == "reduce":
+        (c, ih, iw) = (int(rng.integers(1, 60)), int(rng.integers(1, 12)), int(rng.integers(1, 12)))
+        x = rng.integers(-128, 128, (n, c, ih, iw)).astype(np.int8)
+        g.add(graphs.Op("tpu.input", "input", [], x.shape)).data = x
+        t = ["mean", "sum", "max", "min"][int(rng.integers(0, 4))]
+        a0 = int(rng.integers(1, 4))
+        a1 = int(rng.integers(a0, 4))
+        axes = list(range(a0, a1 + 1))
+        keep = bool(rng.integers(0, 2))
+        full = [n, c, ih, iw]
+        shape = tuple(1 if i in axes else d for i, d in enumerate(full)) if keep else \
+            tuple(d for i, d in enumerate(full) if i not in axes)
+        cnt = int(np.prod([full[i] for i in axes]))
+        if t in ("mean", "sum") or rng.integers(0, 2):
+            rs = int(rng.integers(0, 15))
+            m_ = int(rng.integers(1, 256))
+            wts = dict(rshift=f32(rs), multiplier=f32(m_))
+            pt = "RSHIFT_AND_M_I8"
+        else:
+            wts = {}
+            pt = "NONE"
+        g.add(graphs.Op("tpu.reduce_" + t, "y", ["input"], shape, {"axes%d" % k: a for k, a in enumerate(axes)},
+                        wts, pt))
+    else:
+        (m_, k, nn) = (n, int(rng.integers(1, 600)), int(rng.integers(1, 300)))
+        x = rng.integers(-128, 128, (m_, k, 1, 1)).astype(np.int8)
+        g.add(graphs.Op("tpu.input", "input", [], x.shape)).data = x
+        sig = min(30.0, 900.0 / k ** 0.5)
+        w = np.clip(np.rint(rng.normal(0, sig, (nn, k))), -127, 127).astype(np.float32)
+        bias = rng.integers(-2000, 2000, nn).astype(np.float32)
+        mult = f32(float(int(rng.integers(1 << 23, 1 << 24)) * 128))
+        g.add(graphs.Op("tpu.fully_connected", "y", ["input"], (m_, nn), dict(do_relu=int(rng.integers(0, 2))),
+                        dict(filter=w, bias=bias, rshift=f32(int(rng.integers(4, 12))), multiplier=mult),
+                        "RSHIFT_AND_M_I32"))
+    g.outputs = ["y"]
+    return (g, kind)
+
+
+def test_random_deconv_reduce_and_fc_graphs():
+    ran = {}
+    for it in range(240):
+        g, kind = _random_single_op_graph(it)
+        if g is None:
+            continue
+        want = oracle_graph.run(g)["y"]
+        m = module()
+        m.load(g)
+        m.set_tensor("input", g.input_op().data.astype(np.float32))
+        m.invoke()
+        got = m.get_tensor_i8("y")
+        assert np.array_equal(got, want.reshape(got.shape)), (it, [(o.type, o.shape, o.attrs) for o in g.ops])
+        m.close()
+        ran[kind] = ran.get(kind, 0) + 1
+    assert len(ran) == 3 and min(ran.values()) > 50, ran
