@@ -628,33 +628,34 @@ void orc_reverse_i8(const int8_t *x, int8_t *y, const int64_t *s, int axis) {
         }
 }
 
-/* core/dilate.cpp:11-33 (dilateActivation as DilateOpKernel::invoke calls it: no pads, no
- * trailing inserts): ins_h / ins_w fill values between the rows / columns. */
+/* Dilate as DilateOpKernel::invoke runs it (core/dilate.cpp:11-33, 51-59: no pads, nothing
+ * inserted after the last row / column): the input lands on every (ins_h+1)-th row and
+ * (ins_w+1)-th column of the result, everything else is the fill value. */
 void orc_dilate_i8(const int8_t *x, int8_t *y, const int64_t *s, int ins_h, int ins_w, int fill) {
-  const int n = (int)s[0], c = (int)s[1], h = (int)s[2], w = (int)s[3];
-  const int oh = (h - 1) * (ins_h + 1) + 1, ow = (w - 1) * (ins_w + 1) + 1;
-  for (int in = 0; in < n; in++)
-    for (int ic = 0; ic < c; ic++)
-      for (int _oh = 0; _oh < oh; _oh++)
-        for (int _ow = 0; _ow < ow; _ow++) {
-          const int64_t out_idx = (((int64_t)(in * c + ic) * oh) + _oh) * ow + _ow;
-          const int64_t in_nc = (int64_t)(in * c + ic) * h * w;
-          y[out_idx] = (int8_t)fill;
-          if (_ow % (ins_w + 1) == 0 && _oh % (ins_h + 1) == 0)
-            y[out_idx] = x[in_nc + (_oh / (ins_h + 1)) * w + _ow / (ins_w + 1)];
-        }
+  const int64_t planes = s[0] * s[1], h = s[2], w = s[3];
+  const int64_t step_h = ins_h + 1, step_w = ins_w + 1;
+  const int64_t oh = (h - 1) * step_h + 1, ow = (w - 1) * step_w + 1;
+  for (int64_t p = 0; p < planes; ++p) {
+    const int8_t *src = x + p * h * w;
+    int8_t *dst = y + p * oh * ow;
+    for (int64_t r = 0; r < oh; ++r)
+      for (int64_t c = 0; c < ow; ++c) {
+        const int on_grid = r % step_h == 0 && c % step_w == 0;
+        dst[r * ow + c] = on_grid ? src[(r / step_h) * w + c / step_w] : (int8_t)fill;
+      }
+  }
 }
 
-/* core/reflectionpad.cpp:21-46: mirror padding of the last dimension, the edge element
- * itself not repeated. */
+/* ReflectionPad (core/reflectionpad.cpp:21-46): the last dimension grows by pad_l + pad_r; the
+ * new columns mirror the row about its first / last element, which is not repeated. */
 void orc_reflection_pad_i8(const int8_t *x, int8_t *y, const int64_t *s, int pad_l, int pad_r) {
-  const int64_t rows = s[0] * s[1] * s[2];
-  const int K = (int)s[3], OK = K + pad_l + pad_r;
-  for (int64_t n = 0; n < rows; ++n)
-    for (int k = 0; k < K; ++k) y[n * OK + k + pad_l] = x[n * K + k];
-  for (int64_t n = 0; n < rows; ++n) {
-    for (int p = 0; p < pad_l; ++p) y[n * OK + pad_l - p - 1] = x[n * K + p + 1];
-    for (int p = 0; p < pad_r; ++p) y[n * OK + OK - pad_r + p] = x[n * K + K - p - 2];
+  const int64_t rows = s[0] * s[1] * s[2], w = s[3], ow = w + pad_l + pad_r;
+  for (int64_t r = 0; r < rows; ++r) {
+    const int8_t *src = x + r * w;
+    int8_t *dst = y + r * ow;
+    memcpy(dst + pad_l, src, (size_t)w);
+    for (int64_t d = 1; d <= pad_l; ++d) dst[pad_l - d] = src[d];             /* left: 1, 2, ... outwards */
+    for (int64_t d = 1; d <= pad_r; ++d) dst[pad_l + w - 1 + d] = src[w - 1 - d];
   }
 }
 
