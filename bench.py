@@ -60,6 +60,9 @@ def main():
                     help="images per step instead of the configuration's own batch (a different workload: "
                          "named as such in config.workload, recorded tiles not applied)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--host-io", action="store_true",
+                    help="also time steps that take the input from and return the outputs to host fp32 "
+                         "buffers (set_tensor + invoke + get_tensor), reported as host_io, never as value")
     ap.add_argument("--per-layer", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--save-tiles", default="", help="write the conv tile chosen for every layer")
     ap.add_argument("--tiles", default="", help="use the conv tiles recorded in this file instead "
@@ -221,6 +224,24 @@ def main():
             "achieved": round(hbm_bytes / (hbm_ms / 1e3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": round(hbm_bytes / (hbm_ms / 1e3) / 1e9 / PEAK_HBM_GBS, 4), "ms": round(hbm_ms, 4)},
     }
+    if args.host_io:
+        # the boundary as pymlir's run(x) uses it: fp32 NCHW in host memory -> device int8 and back
+        x_host = g.input_op().data.astype(np.float32)
+        in_name = g.input_op().name
+        for _ in range(2):
+            m.set_tensor(in_name, x_host)
+            m.invoke()
+            outs = [m.get_tensor(name) for name in g.outputs]
+        m.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            m.set_tensor(in_name, x_host)
+            m.invoke()
+            outs = [m.get_tensor(name) for name in g.outputs]
+        ms_io = (time.perf_counter() - t0) * 1e3 / args.steps
+        out["host_io"] = {"ms_per_step": round(ms_io, 4), "images_per_s": round(batch / (ms_io / 1e3), 1),
+                          "host_bytes_in": int(x_host.nbytes), "host_bytes_out": int(sum(o.nbytes for o in outs)),
+                          "what": "set_tensor(fp32, caller's pageable buffer) + invoke + get_tensor(fp32) per step"}
     if not args.no_cpu_baseline:
         sample = {"cfg1": 64, "cfg2": 16, "cfg3": 32, "cfg4": 64, "cfg5": 2}[args.config]
         out["cpu_baseline"] = cpu_baseline(graph_fn, sample)

@@ -58,6 +58,12 @@ const char *tpuhip_version(void);
 /* Replaces TensorData's std::vector<float> storage (cpukernel.h:15-24). */
 int tpuhip_malloc(tpuhip_ctx *ctx, size_t bytes, void **dptr);
 int tpuhip_free(tpuhip_ctx *ctx, void *dptr);
+/* Page-locked host memory for staging tensors that cross the host boundary (set_tensor /
+ * get_tensor of the module, which hold the reference's std::vector<float> contract,
+ * MlirModuleInterpreter.h:47-52): copies from it run as DMA instead of through the driver's
+ * bounce buffers.  No counterpart in the reference (its tensors never leave host memory). */
+int tpuhip_host_malloc(tpuhip_ctx *ctx, size_t bytes, void **hptr);
+int tpuhip_host_free(tpuhip_ctx *ctx, void *hptr);
 int tpuhip_memset(tpuhip_ctx *ctx, void *dptr, int value, size_t bytes);
 int tpuhip_upload(tpuhip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int tpuhip_download(tpuhip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);

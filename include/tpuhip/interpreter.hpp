@@ -90,6 +90,8 @@ private:
   tpuhip_ctx *ctx_;
   size_t size_;
   void *base_ = nullptr;
+  // staging for assign(): a pinned host copy and its fp32 image on the device, made on first use
+  void *stage_host_ = nullptr, *stage_dev_ = nullptr;
   void *ptr_ = nullptr;
   int32_t cur_ = 0;
 };
@@ -550,6 +552,8 @@ public:
   void invokeTo(std::string name, int32_t bidx);
   void invoke(int32_t bidx) { invokeTo("", bidx); }
   void setTensor(std::string &name, const std::vector<float> &data, int32_t bidx);
+  // the same from a plain buffer (what a C caller holds): no intermediate vector
+  void setTensor(std::string &name, const float *data, size_t count, int32_t bidx);
   std::shared_ptr<std::vector<float>> getTensor(std::string &name, int32_t bidx);
   void getTensorI8(const std::string &name, int8_t *dst, size_t num, int32_t bidx);
   std::vector<int64_t> getTensorShape(std::string &name);

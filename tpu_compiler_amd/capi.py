@@ -63,6 +63,8 @@ PROTOTYPES = {
     "tpuhip_version": (C.c_char_p, []),
     "tpuhip_malloc": (C.c_int, [C.c_void_p, C.c_size_t, c_void_pp]),
     "tpuhip_free": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_host_malloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "tpuhip_host_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_memset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t]),
     "tpuhip_upload": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "tpuhip_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),

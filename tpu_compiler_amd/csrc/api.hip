@@ -103,6 +103,21 @@ int tpuhip_free(tpuhip_ctx *ctx, void *dptr) {
   return TPUHIP_OK;
 }
 
+int tpuhip_host_malloc(tpuhip_ctx *ctx, size_t bytes, void **hptr) {
+  TPUHIP_REQUIRE(ctx && hptr, "tpuhip_host_malloc: NULL argument");
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  TPUHIP_CHECK_HIP(hipHostMalloc(hptr, bytes ? bytes : 1, hipHostMallocDefault));
+  return TPUHIP_OK;
+}
+
+int tpuhip_host_free(tpuhip_ctx *ctx, void *hptr) {
+  TPUHIP_REQUIRE(ctx, "tpuhip_host_free: NULL context");
+  if (!hptr) return TPUHIP_OK;
+  TPUHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+  TPUHIP_CHECK_HIP(hipHostFree(hptr));
+  return TPUHIP_OK;
+}
+
 __global__ void fill_bytes_kernel(uint8_t *p, uint8_t v, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;

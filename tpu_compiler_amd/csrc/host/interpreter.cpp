@@ -345,9 +345,13 @@ void ModuleInterpreter::fastInvokeAllBatch(std::string name, int32_t batch) {
 }
 
 void ModuleInterpreter::setTensor(std::string &name, const std::vector<float> &data, int32_t bidx) {
+  setTensor(name, data.data(), data.size(), bidx);
+}
+
+void ModuleInterpreter::setTensor(std::string &name, const float *data, size_t count, int32_t bidx) {
   auto it = activationMapping.find(name);
   if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");
-  it->second->assign(data.data(), data.size(), bidx);
+  it->second->assign(data, count, bidx);
 }
 
 std::shared_ptr<std::vector<float>> ModuleInterpreter::getTensor(std::string &name, int32_t bidx) {

@@ -95,6 +95,8 @@ TensorData::TensorData(tpuhip_ctx *ctx, int32_t batch_, const SyncedDataShape &s
 }
 
 TensorData::~TensorData() {
+  if (stage_dev_) tpuhip_free(ctx_, stage_dev_);
+  if (stage_host_) tpuhip_host_free(ctx_, stage_host_);
   if (base_) tpuhip_free(ctx_, base_);
 }
 
@@ -113,25 +115,30 @@ void TensorData::assign(const float *first, size_t num, int32_t bidx) {
     return;
   }
   const float lo = is_unsigned ? 0.0f : -128.0f, hi = is_unsigned ? 255.0f : 127.0f;
-  for (size_t i = 0; i < num; ++i)
-    if (!(first[i] >= lo && first[i] <= hi) || first[i] != std::nearbyint(first[i]))
-      fail("TensorData::assign: element " + std::to_string(i) + " = " + std::to_string(first[i]) +
-           (is_unsigned ? " is not a uint8 value" : " is not an int8 value"));
-  std::vector<float> wrapped;   // 128..255 travel as the int8 value with the same byte
-  if (is_unsigned) {
-    wrapped.assign(first, first + num);
-    for (auto &v : wrapped)
-      if (v >= 128.0f) v -= 256.0f;
-    first = wrapped.data();
+  if (!stage_host_) ck(tpuhip_host_malloc(ctx_, num * sizeof(float), &stage_host_), "TensorData::assign");
+  if (!stage_dev_) ck(tpuhip_malloc(ctx_, num * sizeof(float), &stage_dev_), "TensorData::assign");
+  // One pass: copy into the pinned buffer, check that every element is an integer of the
+  // tensor's byte range, and let 128..255 travel as the int8 value with the same byte.  No
+  // early exit and no library call in the loop, so it vectorises; adding and subtracting
+  // 1.5 * 2^23 rounds a float of magnitude below 2^22 to an integer.
+  float *stage = static_cast<float *>(stage_host_);
+  const float magic = 12582912.0f, wrap_from = is_unsigned ? 128.0f : 1e9f;
+  unsigned bad = 0;
+  for (size_t i = 0; i < num; ++i) {
+    const float v = first[i];
+    const float r = (v + magic) - magic;
+    bad |= (unsigned)!(v >= lo && v <= hi) | (unsigned)(r != v);
+    stage[i] = v >= wrap_from ? v - 256.0f : v;
   }
-  void *tmp = nullptr;
-  ck(tpuhip_malloc(ctx_, num * sizeof(float), &tmp), "TensorData::assign");
-  int rc = tpuhip_upload(ctx_, tmp, first, num * sizeof(float));
-  if (!rc)
-    rc = tpuhip_nchw_f32_to_nhwc_i8(ctx_, tmp, (char *)base_ + slot_bytes() * (size_t)bidx, n, c, h,
-                                    w, cs);
-  tpuhip_free(ctx_, tmp);  // synchronises the stream first
-  ck(rc, "TensorData::assign");
+  if (bad)
+    for (size_t i = 0; i < num; ++i)
+      if (!(first[i] >= lo && first[i] <= hi) || first[i] != std::nearbyint(first[i]))
+        fail("TensorData::assign: element " + std::to_string(i) + " = " + std::to_string(first[i]) +
+             (is_unsigned ? " is not a uint8 value" : " is not an int8 value"));
+  ck(tpuhip_upload(ctx_, stage_dev_, stage, num * sizeof(float)), "TensorData::assign");
+  ck(tpuhip_nchw_f32_to_nhwc_i8(ctx_, stage_dev_, (char *)base_ + slot_bytes() * (size_t)bidx, n, c, h, w,
+                                cs),
+     "TensorData::assign");
 }
 
 std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {

@@ -115,8 +115,7 @@ int tpuhip_module_set_tensor(tpuhip_module *m, const char *name, const float *da
   GUARD(m, {
     if (!name || !data) throw std::runtime_error("set_tensor: NULL argument");
     std::string n(name);
-    std::vector<float> v(data, data + count);
-    m->interp->setTensor(n, v, bidx);
+    m->interp->setTensor(n, data, count, bidx);
   })
 }
 
