@@ -47,7 +47,7 @@ def test_cpu_baseline_leg_reports_what_it_ran():
 
 @pytest.mark.gpu
 def test_bench_prints_one_json_line_with_the_contract_keys():
-    r = subprocess.run([sys.executable, BENCH, "--config", "cfg2", "--steps", "5", "--warmup", "2"],
+    r = subprocess.run([sys.executable, BENCH, "--config", "cfg2", "--steps", "5", "--warmup", "2", "--host-io"],
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if l.strip()]
@@ -62,5 +62,7 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     assert np.isclose(d["value"], d["config"]["global_batch"] / (d["ms_per_step"] / 1e3), rtol=1e-2)
     r_ = d["roofline"]
     assert r_["bound"] in ("hbm", "mfma") and np.isclose(r_["frac"], r_["achieved"] / r_["peak"], atol=1e-3)
+    # the leg with host buffers in and out every step is reported beside the value, and is slower
+    assert d["host_io"]["ms_per_step"] > d["ms_per_step"] and d["host_io"]["host_bytes_in"] > 0
     c = d["cpu_baseline"]
     assert c["kind"] in ("port", "reference") and c["value"] > 0 and c["cores"] >= 1 and c["sample"]
