@@ -208,6 +208,8 @@ public:
   // host copies of the integer operands are kept until the interpreter has decided about
   // pairing; release_host_weights drops them
   void release_host_weights();
+  // dissolves the pair this kernel belongs to (as first or second), leaving no link behind
+  void unpair();
 
 protected:
   // transposed: the attributes describe a DeConv2D; it runs as a stride-1 conv over the

@@ -205,9 +205,6 @@ __device__ __forceinline__ int32_t requant_core(int32_t v, int32_t mult, int32_t
   return rdbp(x, rshift, mask, mask >> 1);
 }
 
-// Epilogue of one wave tile row block: the lane's 16 consecutive channels
-// (starting at oc) of TN pixels.  Requantise, saturate (+ReLU) and store 16 bytes
-// per pixel.  Parameters are read four channels at a time to keep few registers live.
 // Where an output-channel tile is written.  A pair of convs packed as one: a workgroup (or
 // wave) whose tile lies in the second conv's channels writes that conv's result, with its
 // channel stride and ReLU; split_oc is a multiple of 128, so no tile straddles it.  Chosen
@@ -222,6 +219,84 @@ __device__ __forceinline__ OutRoute route_out(const ConvArgs &a, int oc_tile_bas
                   second ? a.split_oc : 0};
 }
 
+// Requantises the lane's 16 consecutive channels of TN pixels (one row block of a wave tile):
+// saturated (+ReLU) bytes, 16 per pixel.  Parameters are read four channels at a time to keep
+// few registers live.
+template <int TN, bool FAST>
+__device__ __forceinline__ void requant_rows(const v16i (&acc)[TN], int relu_first, int lo,
+                                             const int32_t *pmult, const int32_t *pshift,
+                                             const int32_t *phpot, uint32_t (&outw)[TN][4]) {
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
+    const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
+    const v4i h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int32_t v0 = acc[j][qd * 4 + 0], v1 = acc[j][qd * 4 + 1], v2 = acc[j][qd * 4 + 2],
+              v3 = acc[j][qd * 4 + 3];
+      if (relu_first) {
+        v0 = max(v0, 0); v1 = max(v1, 0); v2 = max(v2, 0); v3 = max(v3, 0);
+      }
+      outw[j][qd] = pack_sat4(requant_core<FAST>(v0, m4[0], r4[0], h4[0]),
+                              requant_core<FAST>(v1, m4[1], r4[1], h4[1]),
+                              requant_core<FAST>(v2, m4[2], r4[2], h4[2]),
+                              requant_core<FAST>(v3, m4[3], r4[3], h4[3]), lo);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// What happens to 16 requantised channels (first channel oc of the launch, byte offset off in
+// the tensor written): the store, the fused table, the fused add with its operand sv.
+__device__ __forceinline__ void finish_chunk(v4i o, const v4i &sv, int64_t off, int oc, const ConvArgs &a,
+                                             int8_t *ydst, const uint8_t *lut) {
+  if (a.store_y) *reinterpret_cast<v4i *>(ydst + off) = o;
+  if (lut) {
+    // table lookup per byte (index = the two's-complement byte); the 256-byte table
+    // covers each LDS bank once, so any 64 indices are conflict-free.  Pad channels
+    // stay zero whatever table[0] is.
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t wd = (uint32_t)o[q];
+      const uint32_t r = (uint32_t)lut[wd & 255u] | ((uint32_t)lut[(wd >> 8) & 255u] << 8) |
+                         ((uint32_t)lut[(wd >> 16) & 255u] << 16) | ((uint32_t)lut[wd >> 24] << 24);
+      const int valid = a.oc - (oc + q * 4);   // channels of this dword that exist
+      const uint32_t mask = valid >= 4 ? 0xffffffffu : valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
+      o[q] = (int)(r & mask);
+    }
+    if (a.lut_dst) *reinterpret_cast<v4i *>(a.lut_dst + off) = o;
+  }
+  if (a.add_dst) {
+    // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
+    // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
+    // unused byte lanes are zero), with the rounding term as its addend: adding
+    // 2^(r-1) before the ReLU gives the same quotient as after it.
+    int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
+    int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
+    int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
+    // one scalar and one vector copy of the uniform operands, made once
+    asm volatile("" : "+s"(rnd), "+v"(mpair), "+s"(floor_));
+    v4i z;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      int32_t t[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[q],
+                                                    0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
+        int32_t sum;   // the three-operand form: no copy of the addend into the result first
+        asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(sum) : "v"(pair), "v"(mpair), "s"(rnd));
+        t[b] = max(sum, floor_) >> a.add_rshift;
+      }
+      z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
+    }
+    *reinterpret_cast<v4i *>(a.add_dst + off) = z;
+  }
+}
+
+// Epilogue of one wave tile row block, written straight from the MFMA result layout: every
+// lane stores the 16 bytes of its own pixel.
 // pix_limit: pixels from this index on are not written (a.npix, or the end of a tile that
 // stops short of its 32-pixel blocks)
 template <int TN, bool FAST>
@@ -231,8 +306,7 @@ __device__ __forceinline__ void epilogue_rows_lim(const v16i (&acc)[TN], const C
                                                   const uint8_t *lut, const OutRoute &out, int pix_limit) {
   uint32_t outw[TN][4];
   // channel index within the tensor written (a pair's second result starts at split_oc)
-  int8_t *const ydst = out.y;
-  const int ycs = out.y_cs, lo = out.lo;
+  const int ycs = out.y_cs;
   const int ocl = oc - out.shift;
   // the other operand of a fused add is fetched now and used after the requantisation
   v4i sv[TN];
@@ -243,73 +317,78 @@ __device__ __forceinline__ void epilogue_rows_lim(const v16i (&acc)[TN], const C
       sv[j] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)pix * ycs + ocl);
     }
   }
-#pragma unroll
-  for (int qd = 0; qd < 4; ++qd) {
-    const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
-    const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
-    const v4i h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      int32_t v0 = acc[j][qd * 4 + 0], v1 = acc[j][qd * 4 + 1], v2 = acc[j][qd * 4 + 2],
-              v3 = acc[j][qd * 4 + 3];
-      if (a.relu_first) {
-        v0 = max(v0, 0); v1 = max(v1, 0); v2 = max(v2, 0); v3 = max(v3, 0);
-      }
-      outw[j][qd] = pack_sat4(requant_core<FAST>(v0, m4[0], r4[0], h4[0]),
-                              requant_core<FAST>(v1, m4[1], r4[1], h4[1]),
-                              requant_core<FAST>(v2, m4[2], r4[2], h4[2]),
-                              requant_core<FAST>(v3, m4[3], r4[3], h4[3]), lo);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
+  requant_rows<TN, FAST>(acc, a.relu_first, out.lo, pmult, pshift, phpot, outw);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int pix = pix_first + j * pix_stride;
     if (pix < pix_limit) {
-      const int64_t off = (int64_t)pix * ycs + ocl;
-      v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
-      if (a.store_y) *reinterpret_cast<v4i *>(ydst + off) = o;
-      if (lut) {
-        // table lookup per byte (index = the two's-complement byte); the 256-byte table
-        // covers each LDS bank once, so any 64 indices are conflict-free.  Pad channels
-        // stay zero whatever table[0] is.
+      const v4i o = {(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+      finish_chunk(o, sv[j], (int64_t)pix * ycs + ocl, oc, a, out.y, lut);
+    }
+  }
+}
+
+// The same epilogue through LDS, so that global memory sees whole rows: a workgroup's tile of
+// BM channels x BN pixels is requantised into a staging area (stage_rows: rows of BM bytes +
+// 16 bytes of padding, which spreads the 16-byte writes of 8 neighbouring pixels over all
+// banks), and after a barrier the threads walk it in memory order -- BM / 16 neighbouring
+// lanes cover one pixel's BM contiguous bytes -- doing the fused table / add and the stores
+// there.  A lane-per-pixel store touches 64 different lines per instruction; written this way
+// a 256-byte-row tensor takes a third of the time.
+template <int BM>
+constexpr int stage_row_bytes() { return BM + 16; }
+
+template <int TM, int TN, int BM, bool FAST>
+__device__ __forceinline__ void stage_rows(const v16i (&acc)[TM][TN], int relu_first, int lo, int8_t *stage,
+                                           int row0, int col0, const int32_t *pmult, const int32_t *pshift,
+                                           const int32_t *phpot) {
+  // row0: the lane's first pixel row in the tile (rows j * 32 further on follow), col0: its
+  // first channel byte; the parameter pointers are those of col0
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const uint32_t wd = (uint32_t)o[q];
-          const uint32_t r = (uint32_t)lut[wd & 255u] | ((uint32_t)lut[(wd >> 8) & 255u] << 8) |
-                             ((uint32_t)lut[(wd >> 16) & 255u] << 16) | ((uint32_t)lut[wd >> 24] << 24);
-          const int valid = a.oc - (oc + q * 4);   // channels of this dword that exist
-          const uint32_t mask = valid >= 4 ? 0xffffffffu : valid <= 0 ? 0u : (1u << (8 * valid)) - 1u;
-          o[q] = (int)(r & mask);
-        }
-        if (a.lut_dst) *reinterpret_cast<v4i *>(a.lut_dst + off) = o;
-      }
-      if (a.add_dst) {
-        // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
-        // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
-        // unused byte lanes are zero), with the rounding term as its addend: adding
-        // 2^(r-1) before the ReLU gives the same quotient as after it.
-        int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
-        int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
-        int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
-        // one scalar and one vector copy of the uniform operands, made once
-        asm volatile("" : "+s"(rnd), "+v"(mpair), "+s"(floor_));
-        v4i z;
+  for (int i = 0; i < TM; ++i) {
+    uint32_t outw[TN][4];
+    requant_rows<TN, FAST>(acc[i], relu_first, lo, pmult + i * 16, pshift + i * 16, phpot + i * 16, outw);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          int32_t t[4];
+    for (int j = 0; j < TN; ++j)
+      *reinterpret_cast<v4i *>(stage + (row0 + j * 32) * stage_row_bytes<BM>() + col0 + i * 16) =
+          v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+  }
+}
+
+// chunks of 16 bytes of a BM x BN tile handled per thread
+template <int BM, int BN, int NT>
+constexpr int flush_chunks() { return (BN * (BM / 16) + NT - 1) / NT; }
+
+// requests the fused add's other operand for this thread's chunks (before the requantisation,
+// whose arithmetic then hides the latency)
+template <int BM, int BN, int NT>
+__device__ __forceinline__ void flush_prefetch(const ConvArgs &a, int tid, int pix0, int pix_limit, int oc0,
+                                               const OutRoute &out, v4i (&sv)[flush_chunks<BM, BN, NT>()]) {
+  constexpr int CPR = BM / 16, NU = flush_chunks<BM, BN, NT>();
+  if (!a.add_dst) return;
 #pragma unroll
-          for (int b = 0; b < 4; ++b) {
-            const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[j][q],
-                                                        0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
-            int32_t sum;   // the three-operand form: no copy of the addend into the result first
-            asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(sum) : "v"(pair), "v"(mpair), "s"(rnd));
-            t[b] = max(sum, floor_) >> a.add_rshift;
-          }
-          z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
-        }
-        *reinterpret_cast<v4i *>(a.add_dst + off) = z;
-      }
+  for (int u = 0; u < NU; ++u) {
+    const int q = tid + u * NT;
+    const int row = q / CPR, cc = q - row * CPR;
+    const int pix = pix0 + row, oc = oc0 + cc * 16;
+    if (q < BN * CPR && pix < pix_limit && oc < a.ocw)
+      sv[u] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)pix * out.y_cs + (oc - out.shift));
+  }
+}
+
+template <int BM, int BN, int NT>
+__device__ __forceinline__ void flush_tile(const ConvArgs &a, const int8_t *stage, int tid, int pix0,
+                                           int pix_limit, int oc0, const OutRoute &out, const uint8_t *lut,
+                                           const v4i (&sv)[flush_chunks<BM, BN, NT>()]) {
+  constexpr int CPR = BM / 16, NU = flush_chunks<BM, BN, NT>();
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int q = tid + u * NT;
+    const int row = q / CPR, cc = q - row * CPR;
+    const int pix = pix0 + row, oc = oc0 + cc * 16;
+    if (q < BN * CPR && pix < pix_limit && oc < a.ocw) {
+      const v4i o = *reinterpret_cast<const v4i *>(stage + row * stage_row_bytes<BM>() + cc * 16);
+      finish_chunk(o, sv[u], (int64_t)pix * out.y_cs + (oc - out.shift), oc, a, out.y, lut);
     }
   }
 }
@@ -781,20 +860,22 @@ conv_mfma_kernel(ConvArgs a) {
       }
     }
 
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int oc = ocw0 + i * 16;
-      const int lc = lch0 + i * 16;
-      if (oc < a.ocw) {
-        if (PERSIST)
-          epilogue_rows<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc,
-                                  qlds + 3 * BM + lc, pix_done + wn * TN * 32 + frow, 32, lut, out);
-        else
-          epilogue_rows<TN, FAST>(acc[i], a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc,
-                                  pix_done + wn * TN * 32 + frow, 32, lut, out);
-      }
-    }
+    // the requantised tile goes through LDS (the K tiles' space: after the last barrier of the
+    // K loop no wave needs them) and leaves in memory order
+    int8_t *const stage = reinterpret_cast<int8_t *>(&lds[0][0]);
+    static_assert(BN * stage_row_bytes<BM>() <= (int)sizeof(lds), "the staged tile must fit the K tiles");
+    v4i sv[flush_chunks<BM, BN, NT>()];
+    flush_prefetch<BM, BN, NT>(a, tid, pix_done, a.npix, oc0, out, sv);
+    if (PERSIST)
+      stage_rows<TM, TN, BM, FAST>(acc, a.relu_first, out.lo, stage, wn * TN * 32 + frow, lch0,
+                                   qlds + BM + lch0, qlds + 2 * BM + lch0, qlds + 3 * BM + lch0);
+    else
+      stage_rows<TM, TN, BM, FAST>(acc, a.relu_first, out.lo, stage, wn * TN * 32 + frow, lch0,
+                                   a.qmult + ocw0, a.qshift + ocw0, a.qhpot + ocw0);
+    __syncthreads();
+    flush_tile<BM, BN, NT>(a, stage, tid, pix_done, a.npix, oc0, out, lut, sv);
     if (!PERSIST || !more) break;
+    __syncthreads();   // the next tile's first K tile lands where the staged bytes are still read
   }
 }
 
@@ -1019,15 +1100,18 @@ conv_patch_kernel(ConvArgs a) {
   for (int d = 0; d < DEPTH - 1; ++d)
     if (d < rem) step_body(d);
 
+  // the requantised tile goes through LDS (the patch's space: after the last barrier of the K
+  // loop no wave needs it; the launch sizes a dynamic patch for the staged tile as well) and
+  // leaves in memory order
   const OutRoute out{a.y, a.y_cs, a.lo, 0};
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int oc = ocw0 + i * 16;
-    const int lc = lch0 + i * 16;
-    if (oc < a.ocw)
-      epilogue_rows_lim<TN, FAST>(acc[i], a, oc, qlds + BM + lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
-                                  pix_base + wn * TN * 32 + frow, 32, nullptr, out, pix_limit);
-  }
+  int8_t *const stage = reinterpret_cast<int8_t *>(patch);
+  static_assert(BN * stage_row_bytes<BM>() <= (DYN ? kPatchBytesDyn : kPatchBytes), "the staged tile must fit the patch");
+  v4i sv[flush_chunks<BM, BN, NT>()];
+  flush_prefetch<BM, BN, NT>(a, tid, pix_base, pix_limit, oc0, out, sv);
+  stage_rows<TM, TN, BM, FAST>(acc, a.relu_first, out.lo, stage, wn * TN * 32 + frow, lch0, qlds + BM + lch0,
+                               qlds + 2 * BM + lch0, qlds + 3 * BM + lch0);
+  __syncthreads();
+  flush_tile<BM, BN, NT>(a, stage, tid, pix_base, pix_limit, oc0, out, nullptr, sv);
 }
 
 // ---------------------------------------------------------------------------
@@ -1756,13 +1840,14 @@ void launch_reg(tpuhip_ctx *ctx, dim3 grid, const ConvArgs &a) {
 
 // the patch kernel's LDS patch is dynamic: (rows + 2) x (W + 2) x C bytes of this layer
 template <typename F>
-void launch_patch(tpuhip_ctx *ctx, F kernel, dim3 grid, const ConvArgs &a, bool dynamic) {
+void launch_patch(tpuhip_ctx *ctx, F kernel, dim3 grid, const ConvArgs &a, bool dynamic, unsigned stage_bytes) {
   static bool raised = false;   // per kernel instantiation; the same value from any thread
   if (dynamic && !raised) {
     (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kPatchBytesDyn);
     raised = true;
   }
-  const unsigned smem = dynamic ? (unsigned)((a.pstep_pix + 2) * a.stem_pw * (a.c16 * 16)) : 0u;
+  // the patch, or the staged output tile that takes its place in the epilogue if that is larger
+  const unsigned smem = dynamic ? std::max((unsigned)((a.pstep_pix + 2) * a.stem_pw * (a.c16 * 16)), stage_bytes) : 0u;
   if (ctx->prof_start)
     hipExtLaunchKernelGGL(kernel, grid, dim3(256), smem, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a);
   else
@@ -1785,7 +1870,7 @@ void launch_mfma(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
     TPUHIP_REG_TILES(Y)
 #undef Y
 #define Z(i, name, BM, BN, BK, D, O) \
-  case i: launch_patch(ctx, (conv_patch_kernel<BM, BN, BK, D, O, FAST>), grid, a, BK == 256); break;
+  case i: launch_patch(ctx, (conv_patch_kernel<BM, BN, BK, D, O, FAST>), grid, a, BK == 256, BN * stage_row_bytes<BM>()); break;
     TPUHIP_PATCH_TILES(Z)
 #undef Z
   }

@@ -393,8 +393,27 @@ Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
 }
 
 Conv2DOpKernel::~Conv2DOpKernel() {
-  if (pair_packed) tpuhip_conv2d_weights_destroy(ctx, pair_packed);
+  unpair();
   if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
+}
+
+// Dissolves the pair this kernel is part of, from either side, so that neither partner keeps
+// a pointer to the other (a partial reload may destroy one of them and keep the other).
+void Conv2DOpKernel::unpair() {
+  if (pair_packed) {
+    tpuhip_conv2d_weights_destroy(ctx, pair_packed);
+    pair_packed = nullptr;
+  }
+  if (pair_second) {
+    pair_second->paired_into = nullptr;
+    pair_second = nullptr;
+  }
+  if (paired_into) {
+    Conv2DOpKernel *first = paired_into;
+    paired_into = nullptr;
+    first->pair_second = nullptr;
+    first->unpair();   // drops the packed pair, which would still write this kernel's result
+  }
 }
 
 void Conv2DOpKernel::release_host_weights() {
@@ -475,9 +494,9 @@ void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_c
 }
 
 bool Conv2DOpKernel::can_fuse_lut() const {
-  const std::string algo = tpuhip_conv2d_algo_name(packed);
-  return (algo.rfind("mfma", 0) == 0 || algo.rfind("depthwise", 0) == 0 || algo == "stem") && !lut_dst &&
-         !fused.enable && !pair_packed && !paired_into;
+  // the packed conv answers for its kernel variant: a tile variant fixed by the caller, or
+  // chosen by timing before a table was asked for, may have no table stage in its epilogue
+  return tpuhip_conv2d_can_fuse_table(packed) != 0 && !lut_dst && !fused.enable && !pair_packed && !paired_into;
 }
 
 void Conv2DOpKernel::fuse_lut(const int8_t *table, SyncedData dst) {
@@ -503,12 +522,7 @@ void Conv2DOpKernel::set_store_result(bool store) {
 }
 
 void Conv2DOpKernel::clear_fusion() {
-  if (pair_packed) {
-    tpuhip_conv2d_weights_destroy(ctx, pair_packed);
-    pair_packed = nullptr;
-    if (pair_second) pair_second->paired_into = nullptr;
-    pair_second = nullptr;
-  }
+  unpair();
   store_result = true;
   output_data->materialized = true;
   if (lut_dst) lut_dst->materialized = true;
