@@ -186,6 +186,12 @@ int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */
 const char *tpuhip_conv2d_tile_name(int tile);
+/* 1 when tpuhip_conv2d_post_i8 can apply a 256-entry table in this packed conv's epilogue: depthwise
+ * and stem kernels always, a dense conv unless its tile variant is fixed (asked for by the caller, or
+ * already chosen by timing) to one without a table stage.  The interpreter asks before it folds a
+ * table op into its producer (the decision MlirModuleInterpreter.cpp:165-344 never has to make: the
+ * reference runs every op as its own kernel). */
+int tpuhip_conv2d_can_fuse_table(const tpuhip_conv_weights *w);
 
 /* ---- FullyConnected ----------------------------------------------------- */
 

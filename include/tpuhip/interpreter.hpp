@@ -594,6 +594,10 @@ private:
   bool isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op);
   void fuseKernels();
   void pairConvs();
+  void spreadDirtiness();
+  // kernels that run as one launch (a conv with the table op / add folded into it, the two
+  // convs of a pair): rebuilt by every loadModule
+  std::vector<std::vector<CPUOpKernel *>> launch_groups_;
   tpuhip_ctx *ctx_ = nullptr;
   kernel_map_t kernel_map_;
   kernel_list_t kernel_list_;

@@ -228,6 +228,31 @@ def test_damaged_files_raise_errors_and_never_crash(tmp_path):
         except capi.TpuHipError:
             outcomes["refused"] += 1
     assert outcomes["refused"] > 50 and outcomes["ok"] > 10
+    # crafted zip64 records whose 64-bit offsets sit just under 2^64: offset + record size wraps, so
+    # only a check against the bytes that are left refuses them
+    import struct
+    eocd = blob.rfind(b"PK\x05\x06")
+    cd_off = struct.unpack_from("<I", blob, eocd + 16)[0]
+    for e64_off, cd64, lho64 in ((2**64 - 8, cd_off, None), (None, 2**64 - 40, None), (None, cd_off, 2**64 - 29)):
+        body = bytearray(blob[:eocd])
+        if lho64 is not None:
+            # first central entry: local header offset escapes to a zip64 extra field
+            struct.pack_into("<I", body, cd_off + 42, 0xffffffff)
+            nlen, xlen = struct.unpack_from("<HH", body, cd_off + 28)
+            extra = struct.pack("<HHQ", 1, 8, lho64)
+            struct.pack_into("<H", body, cd_off + 30, xlen + len(extra))
+            at = cd_off + 46 + nlen + xlen
+            body[at:at] = extra
+        rec64_at = len(body)
+        rec64 = struct.pack("<IQHHIIQQQQ", 0x06064b50, 44, 45, 45, 0, 0, 2, 2, len(body) - cd_off, cd64)
+        loc64 = struct.pack("<IIQI", 0x07064b50, 0, rec64_at if e64_off is None else e64_off, 1)
+        tail = bytearray(blob[eocd:eocd + 22])
+        struct.pack_into("<HH", tail, 8, 0xffff, 0xffff)
+        struct.pack_into("<I", tail, 16, 0xffffffff)
+        p = tmp_path / "zip64.npz"
+        p.write_bytes(bytes(body) + rec64 + loc64 + bytes(tail))
+        with pytest.raises(capi.TpuHipError):
+            capi.TensorFile(p)
     text = HAND_WRITTEN
     refused = 0
     for trial in range(200):

@@ -187,6 +187,33 @@ def test_module_api_semantics():
     m.close()
 
 
+def test_partial_reload_of_fused_and_paired_kernels_after_fast_invoke():
+    """fastInvokeAllBatch clears the dirty flags; a reload that rebuilds only the add fused into a
+    retained conv, the second conv of a pair, or its first, must run the launch that writes the
+    rebuilt kernel's fresh result tensor (MlirModuleInterpreter.cpp:85-116, 383-405)."""
+    g = graphs.cfg3_resnet50(batch=1, hw=64)
+    x = g.input_op().data.astype(np.float32)
+    m = module(max_batch=1)
+    m.load(g)
+    m.set_tensor("input", x, 0)
+    m.fast_invoke_all_batch("", 1)
+    kern = dict(m.kernels())
+    assert kern["res3a_branch2a"] == "with res3a_branch1", kern["res3a_branch2a"]
+    want = oracle_graph.run(g)
+    assert np.array_equal(m.get_tensor_i8("fc1000", 0), want["fc1000"])
+    for name, attr in (("res2b", "do_relu"),               # the add folded into res2b_branch2c
+                       ("res3a_branch2a", "do_relu"),      # second conv of a pair
+                       ("res4a_branch1", "do_relu"),       # first conv of a pair
+                       ("res5c", "do_relu")):
+        g.by_name[name].attrs[attr] = 0 if g.by_name[name].attrs.get(attr, 0) else 1
+        m.load(g)
+        m.fast_invoke_all_batch("", 1)
+        want = oracle_graph.run(g)
+        for op in g.ops:
+            assert np.array_equal(m.get_tensor_i8(op.name, 0), want[op.name].reshape(op.shape)), (name, op.name)
+    m.close()
+
+
 def test_fusion_on_and_off_give_the_same_tensors(monkeypatch):
     g = graphs.cfg3_resnet50(batch=2, hw=96)
     want = oracle_graph.run(g)

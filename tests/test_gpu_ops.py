@@ -18,7 +18,15 @@ def capi_tile_name(t):
 NUM_TILES = next(t for t in range(1024) if capi_tile_name(t) is None)
 # the patch variants take 3x3 / stride 1 / pad 1 layers only; the others take any dense conv
 PATCH_TILES = [t for t in range(NUM_TILES) if "patch" in capi_tile_name(t)]
-GENERAL_TILES = [t for t in range(NUM_TILES) if t not in PATCH_TILES]
+# the pointwise variants take unpadded 1x1 layers with at most the K in their name
+PW_TILES = [t for t in range(NUM_TILES) if "_pw_" in capi_tile_name(t)]
+GENERAL_TILES = [t for t in range(NUM_TILES) if t not in PATCH_TILES and t not in PW_TILES]
+
+
+def tile_k(tile):
+    """K bytes a patch variant consumes per step / a pointwise variant holds"""
+    name = capi_tile_name(tile)
+    return 256 if "k256" in name else 128 if "k128" in name else 64
 
 
 @pytest.fixture(scope="module")
@@ -175,17 +183,30 @@ def test_conv_pair_equals_two_convs(ctx, case):
     assert np.array_equal(ctx.to_nchw(yb), want_b), "%d mismatches in b" % (ctx.to_nchw(yb) != want_b).sum()
     assert not ctx.raw(yb)[..., ocb:].any() and not ctx.raw(ya)[..., oca:].any()
     assert len(np.unique(want_a)) > 8 and len(np.unique(want_b)) > 8
-    # every tile variant splits its output the same way
-    for tile in GENERAL_TILES:
+    # every tile variant splits its output the same way (a pointwise variant takes the pair if it takes
+    # the layer and the first conv ends at one of its tile boundaries)
+    ran_pw = 0
+    for tile in GENERAL_TILES + PW_TILES:
         da.algo = db.algo = 16 + tile
-        wt = ctx.conv_prepack_pair(da, db, (wa, f2i32(ba), f2i32(ma), f2i32(ra)),
-                                   (wb, f2i32(bb) if bias_b else None, f2i32(mb), f2i32(rb)))
+        try:
+            wt = ctx.conv_prepack_pair(da, db, (wa, f2i32(ba), f2i32(ma), f2i32(ra)),
+                                       (wb, f2i32(bb) if bias_b else None, f2i32(mb), f2i32(rb)))
+        except capi.TpuHipError as e:
+            assert tile in PW_TILES and "tile" in str(e), str(e)
+            continue
         ctx._ck(ctx.lib.tpuhip_memset(ctx.h, ya.ptr, 0x55, ya.nbytes))
         ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yb.ptr, 0x55, yb.nbytes))
-        ctx.conv_pair(wt, xt, ya, yb)
+        try:
+            ctx.conv_pair(wt, xt, ya, yb)
+        except capi.TpuHipError as e:
+            assert tile in PW_TILES and "tile variant" in str(e), str(e)
+            ctx.conv_weights_destroy(wt)
+            continue
+        ran_pw += tile in PW_TILES
         name = ctx.conv_algo_name(wt)
         assert np.array_equal(ctx.to_nchw(ya), want_a) and np.array_equal(ctx.to_nchw(yb), want_b), name
         ctx.conv_weights_destroy(wt)
+    assert ran_pw >= (1 if k == 1 else 0)
     # a pair handle does not run as a single conv, nor a single conv as a pair
     with pytest.raises(capi.TpuHipError, match="pair"):
         ctx.conv(wh, xt, ya)
@@ -262,13 +283,10 @@ PATCH_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", PATCH_CASES)
-@pytest.mark.parametrize("tile", PATCH_TILES)
+# a variant with K steps of 128 or 256 bytes takes layers whose channel count is a multiple of that
+@pytest.mark.parametrize("tile,case", [(t, c) for t in PATCH_TILES for c in PATCH_CASES if c[1] % tile_k(t) == 0])
 def test_conv_patch_tile_variants(ctx, case, tile):
     n, c, h, w_, oc, relu, add = case
-    bk = 256 if "k256" in capi_tile_name(tile) else 128 if "k128" in capi_tile_name(tile) else 64
-    if c % bk:
-        pytest.skip("%d-byte K steps need a multiple of %d channels" % (bk, bk))
     rng = np.random.default_rng(c + h * 3 + oc + tile)
     x = rnd_i8(rng, (n, c, h, w_))
     w = rnd_w(rng, (oc, c, 3, 3), sigma=14)
@@ -296,6 +314,92 @@ def test_conv_patch_tile_variants(ctx, case, tile):
         assert not ctx.raw(yt)[..., oc:].any()
         ctx.conv_weights_destroy(wh)
     assert len(np.unique(want)) > 8
+
+
+# n, ic, ih, iw, oc, stride, relu: unpadded 1x1 layers for the kernels that keep their filter slice in LDS
+PW_CASES = [
+    (2, 64, 56, 56, 256, 1, False),     # ResNet-50 stage 2 expansion: whole 256-byte rows per tile
+    (2, 256, 56, 56, 64, 1, True),      # its reduction
+    (3, 128, 28, 28, 512, 1, False),
+    (2, 256, 29, 27, 128, 2, True),     # strided, ragged pixel tail
+    (1, 40, 9, 11, 72, 1, True),        # K padded from 48 to 64, ragged channels
+    (1, 200, 5, 7, 300, 1, False),      # K padded from 208 to 256
+    (6, 96, 31, 17, 100, 1, False),     # K 96 -> 128
+    (40, 64, 30, 30, 64, 1, True),      # enough pixels that every workgroup walks several tiles
+    (1, 16, 1, 1, 16, 1, False),        # one pixel
+]
+
+
+@pytest.mark.parametrize("tile,case", [(t, c) for t in PW_TILES for c in PW_CASES
+                                       if (c[1] + 15) // 16 * 16 <= tile_k(t) and
+                                       (tile_k(t) == 64 or (c[1] + 15) // 16 * 16 > tile_k(t) // 2)])
+@pytest.mark.parametrize("post", ["plain", "add", "add_only", "table_add"])
+def test_conv_pointwise_tile_variants(ctx, case, tile, post):
+    n, ic, ih, iw, oc, stride, relu = case
+    rng = np.random.default_rng(ic * 13 + oc + tile)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, 1, 1))
+    bias, rsh, mult = rnd_params(rng, oc)
+    y_ref = oracle_conv(x, w, bias, rsh, mult, 1, (stride, stride), (0, 0, 0, 0), (1, 1), (0, 0), relu)
+    d = conv_desc(x.shape, w.shape, stride=(stride, stride), do_relu=relu, algo=16 + tile)
+    xt = ctx.from_nchw(x)
+    yt, tt, zt = ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape)
+    for t in (yt, tt, zt):
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, t.ptr, 0x55, t.nbytes))      # poison: pads must be rewritten
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    assert "_pw_" in ctx.conv_algo_name(wh)
+    other = rnd_i8(rng, y_ref.shape)
+    ot = ctx.from_nchw(other)
+    if post == "plain":
+        ctx.conv(wh, xt, yt)
+    elif post in ("add", "add_only"):
+        z_ref = O.eltwise_add_i8([other, y_ref], [-61, 47], [6], post == "add")
+        ctx.conv_add(wh, xt, yt if post == "add" else None, ot, zt, -61, 47, 6, post == "add")
+        assert np.array_equal(ctx.to_nchw(zt), z_ref)
+        assert not ctx.raw(zt)[..., oc:].any()
+    else:
+        table = rnd_i8(rng, 256)
+        table[0] = 77                                  # pad channels must stay 0 all the same
+        t_ref = O.lut_i8(y_ref, table)
+        z_ref = O.eltwise_add_i8([other, t_ref], [37, 51], [5], True)
+        ctx.conv_post(wh, xt, yt, table, tt, (ot, zt, 37, 51, 5, True))
+        assert np.array_equal(ctx.to_nchw(tt), t_ref) and not ctx.raw(tt)[..., oc:].any()
+        assert np.array_equal(ctx.to_nchw(zt), z_ref) and not ctx.raw(zt)[..., oc:].any()
+    if post == "add_only":
+        assert (ctx.raw(yt) == 0x55).all()      # the conv result was not written
+    else:
+        got = ctx.to_nchw(yt)
+        assert np.array_equal(got, y_ref), "%s: %d mismatches" % (ctx.conv_algo_name(wh), (got != y_ref).sum())
+        assert not ctx.raw(yt)[..., oc:].any()
+    assert y_ref.size < 1000 or len(np.unique(y_ref)) > 8
+    ctx.conv_weights_destroy(wh)
+    for t in (xt, ot, yt, tt, zt):
+        t.free()
+
+
+@pytest.mark.parametrize("tile", PW_TILES)
+def test_conv_pointwise_tiles_refuse_other_layers(ctx, tile):
+    """3x3, padded, too many channels, an rshift of 0 (the general requant form): refused by name"""
+    k = tile_k(tile)
+    ok = lambda oc: (None, np.full(oc, 1 << 30, np.int32), np.full(oc, 8, np.int32))
+    xt, yt = ctx.tensor((1, 2 * k, 8, 8)), ctx.tensor((1, 32, 8, 8))
+    for shape, wshape, kw, rs0 in (((1, 64, 8, 8), (32, 64, 3, 3), dict(pads=(1, 1, 1, 1)), False),
+                                   ((1, 2 * k, 8, 8), (32, 2 * k, 1, 1), {}, False),
+                                   ((1, k, 6, 6), (32, k, 1, 1), dict(pads=(1, 1, 1, 1)), False),
+                                   ((1, k, 8, 8), (32, k, 1, 1), {}, True)):
+        d = conv_desc(shape, wshape, algo=16 + tile, **kw)
+        b, m, r = ok(wshape[0])
+        if rs0:
+            r = r.copy()
+            r[5] = 0
+        with pytest.raises(capi.TpuHipError, match="tile"):
+            wh = ctx.conv_prepack(d, np.ones(wshape, np.int8), b, m, r)
+            try:
+                ctx.conv(wh, xt, yt)
+            finally:
+                ctx.conv_weights_destroy(wh)
+    xt.free()
+    yt.free()
 
 
 def _random_conv_case(rng):
@@ -343,7 +447,7 @@ def test_conv_random_shapes_every_tile_variant(ctx, seed):
         z_ref = O.eltwise_add_i8([other, want], [61, 47], [6], True)
         xt, ot = ctx.from_nchw(x), ctx.from_nchw(other)
         yt, zt = ctx.tensor(want.shape), ctx.tensor(want.shape)
-        for tile in GENERAL_TILES + PATCH_TILES:
+        for tile in GENERAL_TILES + PATCH_TILES + PW_TILES:
             d = conv_desc(x.shape, w.shape, stride=stride, pads=pads, dil=dil, do_relu=relu, algo=16 + tile)
             try:
                 wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
@@ -356,7 +460,7 @@ def test_conv_random_shapes_every_tile_variant(ctx, seed):
                 else:
                     ctx.conv(wh, xt, yt)
             except capi.TpuHipError as e:
-                assert "tile variant" in str(e)
+                assert "tile variant" in str(e), str(e)
                 ctx.conv_weights_destroy(wh)
                 continue
             label = (it, capi_tile_name(tile), x.shape, w.shape, stride, pads, dil, relu, add, bool(general))

@@ -86,6 +86,7 @@ PROTOTYPES = {
     "tpuhip_conv2d_i8": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_conv2d_algo_name": (C.c_char_p, [C.c_void_p]),
     "tpuhip_conv2d_tile_name": (C.c_char_p, [C.c_int]),
+    "tpuhip_conv2d_can_fuse_table": (C.c_int, [C.c_void_p]),
     "tpuhip_conv2d_add_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd)]),
     "tpuhip_conv2d_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost)]),
     "tpuhip_lut_per_channel_i8": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t, C.c_int, C.c_int]),

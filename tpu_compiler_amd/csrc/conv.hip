@@ -50,6 +50,7 @@ struct tpuhip_conv_weights {
   int32_t *bias = nullptr;
   QParam *qp = nullptr;
   int32_t *qplanes = nullptr;   // mult | rshift | hpot planes of nparam entries each
+  int32_t *qc64 = nullptr;      // low | high words of bias * mult + 2^30 (the addend of the 64-bit multiply-add)
   int nparam = 0;
   int ocp = 0;           // padded output channels (rows of w / entries of bias, qp)
   int kp = 0;            // padded K in bytes (row stride of w) for the MFMA path
@@ -63,6 +64,7 @@ struct ConvArgs {
   const int32_t *bias;
   const QParam *qp;
   const int32_t *qmult, *qshift, *qhpot;   // the same per-channel data as planes (MFMA epilogue)
+  const int32_t *qclo, *qchi;              // bias * mult + 2^30 per channel, low and high words
   int8_t *y;
   int n, ih, iw, x_cs;
   int oh, ow, y_cs;
@@ -1115,6 +1117,248 @@ conv_patch_kernel(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// Pointwise (1x1, unpadded) convolutions with at most 256 input channels: the
+// weights stay, the pixels stream.
+//
+// Most layers of a residual network are of this kind, and for them the multiply-adds are
+// the small part: at K = 64 a 32x32 block of outputs costs two MFMAs (64 clocks) and about
+// 500 clocks of requantisation on the vector ALU, and every byte of the big operand is
+// used once.  So the kernel is laid out around the epilogue and the memory pipeline:
+//   * a workgroup keeps its whole BM x K slice of the filter in LDS for its lifetime (the
+//     image of that slice, swizzled, is what the packed filter holds: a straight copy) and
+//     walks tiles of BN pixels; nothing of the filter is fetched per tile, no K loop with
+//     barriers exists;
+//   * the pixel rows of a tile are K contiguous bytes each, fetched with whole-row loads
+//     (K / 16 neighbouring lanes per pixel) TWO tiles ahead into registers and parked in a
+//     double-buffered LDS tile one tile ahead;
+//   * the accumulators start at zero (the first MFMA of a block takes a literal 0) and the
+//     bias rides in the 64-bit multiply-add of the requantisation: (acc + b) * m + 2^30 ==
+//     acc * m + (b * m + 2^30), one per-channel 64-bit constant (needs the overflow-free
+//     form of the layer, which the host proves; other layers take the general kernel);
+//   * BM is as wide as the layer allows (up to 256 channels), so a tile's output -- and the
+//     other operand of a fused add -- are whole rows of the tensors: staged through LDS,
+//     read and written in memory order;
+//   * one barrier per tile (the staged tile is double-buffered where LDS allows, SD == 2).
+// K is padded to KP = 64, 128 or 256 with zero weights; the bytes a pixel row lacks are
+// whatever follows it in memory (finite integers times zero; past the end of the tensor the
+// buffer descriptor supplies zeros).
+// ---------------------------------------------------------------------------
+template <int TN>
+__device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, const int32_t *pclo,
+                                                 const int32_t *pchi, const int32_t *pmult,
+                                                 const int32_t *pshift, const int32_t *phpot,
+                                                 uint32_t (&outw)[TN][4]) {
+#pragma unroll
+  for (int qd = 0; qd < 4; ++qd) {
+    const v4i cl = *reinterpret_cast<const v4i *>(pclo + qd * 4);
+    const v4i ch = *reinterpret_cast<const v4i *>(pchi + qd * 4);
+    const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
+    const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
+    const v4i h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      int32_t y[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int64_t c = (int64_t)(((uint64_t)(uint32_t)ch[e] << 32) | (uint32_t)cl[e]);
+        const int64_t p = (int64_t)acc[j][qd * 4 + e] * (int64_t)m4[e] + c;
+        const int32_t x = (int32_t)(p >> 31);
+        y[e] = (x + h4[e] + (x >> 31)) >> r4[e];
+      }
+      outw[j][qd] = pack_sat4(y[0], y[1], y[2], y[3], lo);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <int BM, int BN, int WM, int WN, int KP, int SD, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+conv_pw_kernel(ConvArgs a) {
+  constexpr int NT = 256;
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
+  static_assert(KP == 64 || KP == 128 || KP == 256, "padded K");
+  constexpr int KC = KP / 64;              // 64-byte K chunks
+  constexpr int CPRK = KP / 16;            // 16-byte chunks of a pixel row
+  constexpr int RPP = NT / CPRK;           // pixel rows per pass of the loader
+  constexpr int NXC = BN / RPP;            // activation chunks per thread per tile
+  constexpr int NWC = BM * KP / 16 / NT;   // filter chunks per thread
+  static_assert(BN % RPP == 0 && NXC >= 1 && NWC >= 1, "loader shape");
+  constexpr int SROW = stage_row_bytes<BM>();
+  extern __shared__ __attribute__((aligned(16))) v4i pw_smem[];
+  v4i *const wA = pw_smem;                                       // [KC][BM][4 chunks], swizzled
+  v4i *const xB = wA + KC * BM * 4;                              // [2][KC][BN][4 chunks], swizzled
+  int8_t *const stage0 = reinterpret_cast<int8_t *>(xB + 2 * KC * BN * 4);   // [SD][BN][SROW]
+  int32_t *const qlds = reinterpret_cast<int32_t *>(stage0 + SD * BN * SROW);   // 5 planes of BM
+  uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  // tiles are dealt as in conv_mfma_kernel: every XCD a contiguous run of pixel tiles, a
+  // workgroup keeps its output-channel tile and walks pixel tiles
+  int ltile = (int)(blockIdx.x >> 3);
+  int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + ltile;
+  if (logical >= a.n_tiles) return;
+  const int pix_tile = logical / a.n_oc_tiles;
+  const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;
+  const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
+  int pix0 = pix_tile * BN;
+
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+
+  // ---- loader: this thread fetches chunk c of pixel rows lrow + RPP * u
+  const int c = tid % CPRK, lrow = tid / CPRK;
+  int lpix0 = pix0;                       // first pixel of the tile being fetched
+  int low = pix0 % a.ow;
+  int loh, ln;
+  {
+    const int t = pix0 / a.ow;
+    loh = t % a.oh;
+    ln = t / a.oh;
+  }
+  v4i breg[NXC];
+  auto load_B = [&](bool exists) {
+#pragma unroll
+    for (int u = 0; u < NXC; ++u) {
+      const int row = lrow + RPP * u;
+      const bool pv = exists && lpix0 + row < a.npix;
+      const uint32_t t1 = (uint32_t)(low + row);
+      const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
+      const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
+      const uint32_t t2 = (uint32_t)loh + q1;
+      const uint32_t q2 = a.oh == 1 ? t2 : __umulhi(t2, a.magic_oh);
+      const int oh = (int)(t2 - q2 * (uint32_t)a.oh);
+      const int n = ln + (int)q2;
+      const uint32_t off = (uint32_t)(((n * a.ih + oh * a.sh) * a.iw + ow * a.sw) * a.x_cs + c * 16);
+      breg[u] = buffer_load16(xrsrc, pv ? off : kOobOffset);
+    }
+  };
+  auto advance_load = [&]() {
+    lpix0 += a.pstep_pix;
+    low += a.pstep_ow;
+    if (low >= a.ow) { low -= a.ow; ++loh; }
+    loh += a.pstep_oh;
+    if (loh >= a.oh) { loh -= a.oh; ++ln; }
+    ln += a.pstep_n;
+  };
+  auto store_B = [&](int slot) {
+    v4i *base = xB + slot * (KC * BN * 4) + (c >> 2) * (BN * 4);
+#pragma unroll
+    for (int u = 0; u < NXC; ++u) {
+      const int row = lrow + RPP * u;
+      base[row * 4 + ((c & 3) ^ ((row >> 2) & 3))] = breg[u];
+    }
+  };
+  // does the tile j steps ahead of the current one exist?
+  auto exists_ahead = [&](int j) {
+    return ltile + j * a.wgs_per_xcd < a.tiles_per_xcd && logical + j * a.wgs_per_xcd < a.n_tiles;
+  };
+
+  load_B(true);
+  {
+    // the filter slice: a straight copy of its LDS image
+    const v4i *wsrc = reinterpret_cast<const v4i *>(a.w) + (size_t)(oc0 / BM) * (BM * KP / 16);
+    v4i wreg[NWC];
+#pragma unroll
+    for (int u = 0; u < NWC; ++u) wreg[u] = wsrc[tid + u * NT];
+    if (tid < BM) {
+      qlds[tid] = a.qclo[oc0 + tid];
+      qlds[BM + tid] = a.qchi[oc0 + tid];
+      qlds[2 * BM + tid] = a.qmult[oc0 + tid];
+      qlds[3 * BM + tid] = a.qshift[oc0 + tid];
+      qlds[4 * BM + tid] = a.qhpot[oc0 + tid];
+    }
+    if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+#pragma unroll
+    for (int u = 0; u < NWC; ++u) wA[tid + u * NT] = wreg[u];
+  }
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  store_B(0);
+  advance_load();
+  load_B(exists_ahead(1));
+  __syncthreads();
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  const int lch0 = wm * TM * 32 + fk * 16 * TM;   // first of this lane's 16 * TM channels in the tile
+  // fragment chunk indices (row * 4 + swizzled chunk) of this lane, for kk = 0 and 1
+  int ia[TM][2], ib[TN][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int r = (wm * TM + i) * 32 + frow;
+    ia[i][0] = r * 4 + (fk ^ ((r >> 2) & 3));
+    ia[i][1] = r * 4 + ((2 + fk) ^ ((r >> 2) & 3));
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int r = (wn * TN + j) * 32 + frow;
+    ib[j][0] = r * 4 + (fk ^ ((r >> 2) & 3));
+    ib[j][1] = r * 4 + ((2 + fk) ^ ((r >> 2) & 3));
+  }
+
+  int cur = 0, sd = 0;
+  for (;;) {
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    const v4i *xb = xB + cur * (KC * BN * 4);
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        v4i fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[i] = wA[kc * (BM * 4) + ia[i][kk]];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[j] = xb[kc * (BN * 4) + ib[j][kk]];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+
+    // the next tile's pixels go to the other LDS tile (free since the barrier of the last
+    // epilogue), the one after that is requested
+    const bool more = exists_ahead(1);
+    store_B(cur ^ 1);
+    advance_load();
+    load_B(exists_ahead(2));
+
+    int8_t *const stage = stage0 + sd * (BN * SROW);
+    v4i sv[flush_chunks<BM, BN, NT>()];
+    flush_prefetch<BM, BN, NT>(a, tid, pix0, a.npix, oc0, out, sv);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      uint32_t outw[TN][4];
+      const int lc = lch0 + i * 16;
+      requant_rows_c64<TN>(acc[i], out.lo, qlds + lc, qlds + BM + lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
+                           qlds + 4 * BM + lc, outw);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        *reinterpret_cast<v4i *>(stage + ((wn * TN + j) * 32 + frow) * SROW + lc) =
+            v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+    }
+    __syncthreads();   // publishes the staged tile and the next tile's pixels
+    flush_tile<BM, BN, NT>(a, stage, tid, pix0, a.npix, oc0, out, lut, sv);
+    if (!more) break;
+    ltile += a.wgs_per_xcd;
+    logical += a.wgs_per_xcd;
+    pix0 += a.pstep_pix;
+    cur ^= 1;
+    if (SD == 2) sd ^= 1;
+    else __syncthreads();   // one staging area: everyone has read it before it is written again
+  }
+}
+
+// ---------------------------------------------------------------------------
 // depthwise on the matrix cores.  A depthwise tap is a 32x32 DIAGONAL matrix times
 // the 32 channels x 32 pixels activation block: D[c][pix] += W_t[c][c] * X_t[pix][c],
 // one v_mfma_i32_32x32x32_i8 per tap (K = the 32 channels).  31/32 of the multiplies
@@ -1767,8 +2011,8 @@ struct TileCfg {
   const char *name;
   int reg;   // 0: LDS kernel, one tile per workgroup; 1: the LDS-free kernel, bm x bn is the
              // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups;
-             // 4: patch kernel (bn = pixel slots of a tile of whole rows)
-  int bk;    // K bytes per step
+             // 4: patch kernel (bn = pixel slots of a tile of whole rows); 5: pointwise kernel
+  int bk;    // K bytes per step (pointwise kernel: the padded K it holds)
 };
 
 // The tile variants, in the order of their public index (conv desc algo = 16 + index).
@@ -1803,6 +2047,18 @@ struct TileCfg {
   Z(21, "mfma_patch_64x128_k256", 64, 128, 256, 2, 2)  \
   Z(22, "mfma_patch_64x64_k256", 64, 64, 256, 2, 2)
 
+// pointwise kernels (1x1, unpadded, at most KP input channels, the filter slice resident in LDS):
+// W(index, name, BM, BN, WM, WN, KP, staging buffers, waves per SIMD)
+#define TPUHIP_PW_TILES(W)                                  \
+  W(23, "mfma_pw_64x128_k64", 64, 128, 2, 2, 64, 2, 3)      \
+  W(24, "mfma_pw_64x128_k128", 64, 128, 2, 2, 128, 2, 2)    \
+  W(25, "mfma_pw_64x64_k256", 64, 64, 2, 2, 256, 2, 2)      \
+  W(26, "mfma_pw_128x64_k64", 128, 64, 2, 2, 64, 2, 3)      \
+  W(27, "mfma_pw_128x64_k128", 128, 64, 2, 2, 128, 2, 3)    \
+  W(28, "mfma_pw_128x64_k256", 128, 64, 2, 2, 256, 1, 2)    \
+  W(29, "mfma_pw_256x64_k64", 256, 64, 4, 1, 64, 2, 2)      \
+  W(30, "mfma_pw_256x64_k128", 256, 64, 4, 1, 128, 1, 2)
+
 struct TileTable {
   TileCfg t[64];
   int n = 0;
@@ -1822,6 +2078,11 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_PATCH_TILES(Z)
 #undef Z
+#define W(i, name, BM, BN, WM, WN, KP, SD, O) \
+  t[i] = TileCfg{BM, BN, WM, WN, name, 5, KP}; \
+  n = n > i ? n : i + 1;
+    TPUHIP_PW_TILES(W)
+#undef W
   }
 };
 const TileTable kTileTable;
@@ -1852,6 +2113,60 @@ void launch_patch(tpuhip_ctx *ctx, F kernel, dim3 grid, const ConvArgs &a, bool 
     hipExtLaunchKernelGGL(kernel, grid, dim3(256), smem, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a);
   else
     hipLaunchKernelGGL(kernel, grid, dim3(256), smem, ctx->stream, a);
+}
+
+// dynamic LDS of a pointwise tile variant: filter slice, two pixel tiles, the staged output
+// tile(s), five parameter planes, the fused table
+constexpr unsigned pw_lds_bytes(int bm, int bn, int kp, int sd) {
+  return (unsigned)(bm * kp + 2 * bn * kp + sd * bn * (bm + 16) + 5 * bm * 4 + 256);
+}
+
+// raises the kernel's dynamic LDS limit once; on failure the runtime's last error stays set
+// for the caller to report
+template <typename F>
+bool pw_prepare(F kernel, unsigned lds) {
+  static bool raised = false;   // per kernel instantiation; the same value from any thread
+  if (!raised) {
+    if (hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return false;
+    raised = true;
+  }
+  return true;
+}
+
+void launch_pw(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
+  switch (tile) {
+#define W(i, name, BM, BN, WM, WN, KP, SD, O)                                                           \
+  case i: {                                                                                             \
+    auto kernel = conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>;                                            \
+    constexpr unsigned lds = pw_lds_bytes(BM, BN, KP, SD);                                              \
+    if (!pw_prepare(kernel, lds)) break;                                                                \
+    if (ctx->prof_start)                                                                                \
+      hipExtLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
+    else                                                                                                \
+      hipLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, a);                                 \
+  } break;
+    TPUHIP_PW_TILES(W)
+#undef W
+  }
+}
+
+// workgroups of pointwise tile variant `tile` that fit on one CU at once
+int pw_occupancy(int tile) {
+  int n = 0;
+  hipError_t e = hipErrorInvalidValue;
+  switch (tile) {
+#define W(i, name, BM, BN, WM, WN, KP, SD, O)                                                           \
+  case i:                                                                                               \
+    if (pw_prepare(conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>, pw_lds_bytes(BM, BN, KP, SD)))             \
+      e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>, 256, \
+                                                       pw_lds_bytes(BM, BN, KP, SD));                   \
+    break;
+    TPUHIP_PW_TILES(W)
+#undef W
+  }
+  if (e != hipSuccess) (void)hipGetLastError();
+  return e == hipSuccess && n > 0 ? n : 1;
 }
 
 template <bool FAST, int MODE>
@@ -1904,11 +2219,13 @@ int persist_wgs_per_cu(const tpuhip_conv_weights *w) {
   // 0 = not asked yet.  Contexts on several host threads may ask at once: every writer
   // stores the same value, so relaxed atomics are all that is needed.
   static std::atomic<int> cache[kMaxTiles][2][3];
-  const int mode = conv_mode(w);
+  const int mode = kTiles[w->tile].reg == 5 ? 0 : conv_mode(w);
   std::atomic<int> &slot = cache[w->tile][w->fast ? 1 : 0][mode];
   int c = slot.load(std::memory_order_relaxed);
   if (c == 0) {
-    if (w->fast)
+    if (kTiles[w->tile].reg == 5)
+      c = pw_occupancy(w->tile);
+    else if (w->fast)
       c = mode == kModeSmallC ? persist_occupancy<true, kModeSmallC>(w->tile)
           : mode == kModeUniform ? persist_occupancy<true, kModeUniform>(w->tile)
                                  : persist_occupancy<true, kModeGeneral>(w->tile);
@@ -1970,6 +2287,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
   cw->c16 = icp / 16;
   cw->k16 = cw->smallc ? (d.kh * d.kw * 4 + 15) / 16 : d.kh * d.kw * cw->c16;
   cw->kp = round_up(cw->k16 * 16, tile_bk(t));
+  if (t.reg == 5 && cw->kp != t.bk) return set_error(TPUHIP_ERR_INVALID, "conv: tile %s holds %d input channels", t.name, t.bk);
   std::vector<int8_t> packed((size_t)ocp * cw->kp, 0);
   const int8_t *filter = cw->host_filter.data();
   std::vector<int8_t> rowbuf((size_t)cw->kp);
@@ -1986,6 +2304,15 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
         rowbuf[(size_t)k * kstride + c] = src[(size_t)c * d.kh * d.kw + k];
     if (t.reg == 0 || t.reg == 3 || t.reg == 4) {
       memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
+    } else if (t.reg == 5) {
+      // the LDS image of every output-channel tile: [64-byte K chunk][row][4 x 16 bytes], the
+      // 16-byte position XORed with (row >> 2) & 3
+      const int r = row - tile0;
+      int8_t *img = packed.data() + (size_t)(tile0 / t.bm) * t.bm * cw->kp;
+      for (int kc = 0; kc < cw->kp / 64; ++kc)
+        for (int c4 = 0; c4 < 4; ++c4)
+          memcpy(img + ((size_t)(kc * t.bm + r) * 4 + (c4 ^ ((r >> 2) & 3))) * 16,
+                 rowbuf.data() + (size_t)kc * 64 + c4 * 16, 16);
     } else {
       // fragment order: [row / 32][K step][kk][lane = (row & 31) + 32 * half][16 bytes]
       const int blk = row / 32, r = row % 32;
@@ -2009,7 +2336,15 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 }
 
 // the fused table lives in the LDS of the LDS kernels
-bool tile_has_lds_epilogue(int t) { return kTiles[t].reg == 0 || kTiles[t].reg == 3; }
+bool tile_has_lds_epilogue(int t) { return kTiles[t].reg == 0 || kTiles[t].reg == 3 || kTiles[t].reg == 5; }
+
+// the pointwise kernels: 1x1 window, no padding, no dilation (any stride), the input channels
+// within the K the variant holds (and more than half of it, or the smallest variant)
+bool pw_shape_ok(const tpuhip_conv_desc &d, const TileCfg &c) {
+  const int icp = round_up(d.ic, 16);
+  return d.g == 1 && d.kh == 1 && d.kw == 1 && d.pt == 0 && d.pl == 0 && d.pb == 0 && d.pr == 0 && !d.ins_h &&
+         !d.ins_w && !d.relu_first && icp <= c.bk && (c.bk == 64 || icp > c.bk / 2) && d.ic > 4;
+}
 
 // rows of one image a patch tile holds; 0: the layer does not fit the patch kernel
 int patch_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
@@ -2029,6 +2364,7 @@ int patch_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
 bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
   if (c.reg == 4 && patch_rows(d, c) == 0) return false;
+  if (c.reg == 5 && !pw_shape_ok(d, c)) return false;
   if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
@@ -2044,6 +2380,8 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.qmult = w->qplanes;
   a.qshift = w->qplanes + w->nparam;
   a.qhpot = w->qplanes + 2 * w->nparam;
+  a.qclo = w->qc64;
+  a.qchi = w->qc64 + w->nparam;
   a.y = (int8_t *)y;
   a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.x_cs = d.x_cs;
   a.oh = d.oh; a.ow = d.ow; a.y_cs = d.y_cs;
@@ -2088,7 +2426,7 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
       a.pstep_oh = w->c16 == 4 ? 2 : w->c16 == 8 ? 3 : w->c16 == 16 ? 4 : 5;     // log2(C / 16)
       a.pstep_ow = w->c16 == 4 ? 2 : w->c16 == 8 ? 1 : 0;                        // swizzle shift
     }
-    if (t.reg == 3) {
+    if (t.reg == 3 || t.reg == 5) {
       // every XCD owns a run of whole pixel tiles; a workgroup keeps its channel tile
       const int n_pix_tiles = a.n_tiles / a.n_oc_tiles;
       a.tiles_per_xcd = (n_pix_tiles + 7) / 8 * a.n_oc_tiles;
@@ -2105,6 +2443,10 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
 
 void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvArgs &a) {
   dim3 grid((unsigned)(a.wgs_per_xcd * 8));
+  if (kTiles[w->tile].reg == 5) {
+    launch_pw(ctx, w->tile, grid, a);
+    return;
+  }
   const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
   if (w->smallc) {
     if (w->fast)
@@ -2168,6 +2510,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     if (!tile_is_candidate(w->d, t)) continue;
     if (post.lut && !tile_has_lds_epilogue(t)) continue;
     if (w->split_oc && kTiles[t].reg == 4) continue;   // the patch kernel writes one result
+    if (kTiles[t].reg == 5 && (!w->fast || w->split_oc % kTiles[t].bm)) continue;
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
@@ -2325,7 +2668,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   // epilogue parameters, indexed by the true output channel.  `fast` holds when,
   // for every channel, 1 <= rshift and |acc + bias| + 1 + 2^(rshift-1) cannot reach
   // 2^31: |acc| <= 128 * sum|w|, and |x| <= |v| + 1 after the doubling high multiply.
-  const size_t nparam = (size_t)round_up(d.oc, 128) + 16;   // covers every tile's padding
+  const size_t nparam = (size_t)round_up(d.oc, 256) + 16;   // covers every tile's padding
   std::vector<int32_t> b32(nparam, 0);
   std::vector<QParam> qp(nparam);
   bool fast = true;
@@ -2368,6 +2711,16 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
     cw->nparam = (int)nparam;
     rc = tpuhip_malloc(ctx, planes.size() * sizeof(int32_t), (void **)&cw->qplanes);
     if (!rc) rc = tpuhip_upload(ctx, cw->qplanes, planes.data(), planes.size() * sizeof(int32_t));
+    // (acc + bias) * mult + 2^30 == acc * mult + c: the addend of the requantisation's 64-bit
+    // multiply-add, as a plane of low and a plane of high words
+    std::vector<int32_t> c64(2 * nparam);
+    for (size_t i = 0; i < nparam; ++i) {
+      const int64_t c = (int64_t)b32[i] * (int64_t)qp[i].mult + (1ll << 30);
+      c64[i] = (int32_t)(uint32_t)(c & 0xffffffffll);
+      c64[nparam + i] = (int32_t)(c >> 32);
+    }
+    if (!rc) rc = tpuhip_malloc(ctx, c64.size() * sizeof(int32_t), (void **)&cw->qc64);
+    if (!rc) rc = tpuhip_upload(ctx, cw->qc64, c64.data(), c64.size() * sizeof(int32_t));
   }
   if (rc) {
     tpuhip_conv2d_weights_destroy(ctx, cw);
@@ -2384,12 +2737,19 @@ int tpuhip_conv2d_weights_destroy(tpuhip_ctx *ctx, tpuhip_conv_weights *w) {
   int rc2 = tpuhip_free(ctx, w->bias);
   int rc3 = tpuhip_free(ctx, w->qp);
   int rc4 = tpuhip_free(ctx, w->qplanes);
+  int rc5 = tpuhip_free(ctx, w->qc64);
   delete w;
-  return rc ? rc : rc2 ? rc2 : rc3 ? rc3 : rc4;
+  return rc ? rc : rc2 ? rc2 : rc3 ? rc3 : rc4 ? rc4 : rc5;
 }
 
 const char *tpuhip_conv2d_tile_name(int tile) {
   return tile >= 0 && tile < kNumTiles ? kTiles[tile].name : nullptr;
+}
+
+int tpuhip_conv2d_can_fuse_table(const tpuhip_conv_weights *w) {
+  if (!w) return 0;
+  if (w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT || w->algo == ALGO_STEM) return 1;
+  return w->algo == ALGO_MFMA && (!w->tuned || tile_has_lds_epilogue(w->tile)) ? 1 : 0;
 }
 
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
@@ -2428,6 +2788,11 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
   TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 4) || (!w->split_oc && patch_rows(w->d, kTiles[w->tile]) > 0),
                  "conv: tile variant %s needs a single 3x3 / stride 1 / pad 1 conv with 64, 128, 256 or 512 input "
                  "channels on a map narrow enough for its row patch", kTiles[w->tile].name);
+  TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 5) ||
+                     (pw_shape_ok(w->d, kTiles[w->tile]) && w->fast && w->split_oc % kTiles[w->tile].bm == 0),
+                 "conv: tile variant %s needs an unpadded 1x1 conv with 5 to %d input channels, right shifts of at "
+                 "least 1 and sums that cannot overflow the rounding, and a pair split at a tile boundary",
+                 kTiles[w->tile].name, kTiles[w->tile].bk);
   TPUHIP_REQUIRE((w->split_oc != 0) == (post.y2 != nullptr),
                  "conv: weights packed as a pair run through tpuhip_conv2d_pair_i8 (and only they do)");
   ConvArgs a;

@@ -52,6 +52,29 @@ void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
   updateKernelList(module, target_op);
   fuseKernels();
   pairConvs();
+  spreadDirtiness();
+}
+
+// The dirty flag of the reference (MlirModuleInterpreter.cpp:85-116, 383-405) belongs to one
+// kernel; here several kernels can share one launch.  After a partial reload a rebuilt (dirty)
+// add, table op or second conv of a pair may have been folded into a retained (clean) conv
+// whose launch is the only thing that writes its fresh result tensor -- so within a launch
+// group one dirty member makes every member dirty.
+void ModuleInterpreter::spreadDirtiness() {
+  for (bool changed = true; changed;) {   // groups chain through a shared conv: to a fixed point
+    changed = false;
+    for (auto &group : launch_groups_) {
+      bool any = false, all = true;
+      for (auto *k : group) {
+        any = any || k->dirty;
+        all = all && k->dirty;
+      }
+      if (any && !all) {
+        for (auto *k : group) k->dirty = true;
+        changed = true;
+      }
+    }
+  }
 }
 
 // Work that rides in a dense conv's epilogue instead of running as a kernel of its own
@@ -65,6 +88,7 @@ void ModuleInterpreter::fuseKernels() {
   std::map<TensorData *, int> position;                               // tensor -> producing position
   std::vector<Conv2DOpKernel *> fused_convs;
   int pos = 0;
+  launch_groups_.clear();
   for (auto &k : kernel_list_) {
     if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) c->clear_fusion();
     if (auto *e = dynamic_cast<EltwiseAddOpKernel *>(k.get())) e->fused_into_producer = false;
@@ -88,6 +112,7 @@ void ModuleInterpreter::fuseKernels() {
       const int conv_pos = it->second.first;
       conv->fuse_lut(l->table, l->result());
       l->fused_into_producer = true;
+      launch_groups_.push_back({conv, l});
       producer.erase(it);
       producer[l->result().get()] = {conv_pos, conv};   // an add may follow the table
       fused_convs.push_back(conv);
@@ -119,6 +144,7 @@ void ModuleInterpreter::fuseKernels() {
     conv->fuse_add(e->inputs()[1 - conv_idx], e->result(), e->multipliers()[1 - conv_idx],
                    e->multipliers()[conv_idx], e->rshift_value(), e->relu());
     e->fused_into_producer = true;
+    launch_groups_.push_back({conv, e});   // (conv, table) and (conv, add) chain through the conv
     producer.erase(e->inputs()[conv_idx].get());   // one add per conv
     if (std::find(fused_convs.begin(), fused_convs.end(), conv) == fused_convs.end())
       fused_convs.push_back(conv);
@@ -162,6 +188,7 @@ void ModuleInterpreter::pairConvs() {
         if (convs[i]->can_pair_with(*convs[j])) {
           try {
             convs[i]->pair_with(*convs[j]);
+            launch_groups_.push_back({convs[i], convs[j]});
           } catch (const std::exception &) {
             // shapes the packed form does not cover stay two launches
           }

@@ -157,18 +157,20 @@ void TensorFile::load() {
   uint64_t cd_off = rd32(&buf[eocd + 16]);
   if ((entries == 0xffff || cd_off == 0xffffffffu) && eocd >= 20 && rd32(&buf[eocd - 20]) == kEnd64LocSig) {
     const uint64_t e64 = rd64(&buf[eocd - 20 + 8]);
-    if (e64 + 56 > buf.size() || rd32(&buf[e64]) != kEnd64Sig) fail(filename + ": bad zip64 end record");
+    // offsets come from the file: compare against what is left, so that a value near 2^64 cannot wrap
+    if (buf.size() < 56 || e64 > buf.size() - 56 || rd32(&buf[e64]) != kEnd64Sig) fail(filename + ": bad zip64 end record");
     entries = rd64(&buf[e64 + 32]);
     cd_off = rd64(&buf[e64 + 48]);
   }
+  if (cd_off > buf.size()) fail(filename + ": bad central directory");
   size_t p = (size_t)cd_off;
   for (uint64_t e = 0; e < entries; ++e) {
-    if (p + 46 > buf.size() || rd32(&buf[p]) != kCentralSig) fail(filename + ": bad central directory");
+    if (buf.size() - p < 46 || rd32(&buf[p]) != kCentralSig) fail(filename + ": bad central directory");
     const uint16_t method = rd16(&buf[p + 10]);
     uint64_t csize = rd32(&buf[p + 20]), usize = rd32(&buf[p + 24]);
     const uint16_t nlen = rd16(&buf[p + 28]), xlen = rd16(&buf[p + 30]), clen = rd16(&buf[p + 32]);
     uint64_t lho = rd32(&buf[p + 42]);
-    if (p + 46 + nlen + xlen + clen > buf.size()) fail(filename + ": truncated central directory");
+    if (buf.size() - p - 46 < (size_t)nlen + xlen + clen) fail(filename + ": truncated central directory");
     std::string member((const char *)&buf[p + 46], nlen);
     // zip64 extra field: the values that are 0xffffffff above, in this order
     size_t x = p + 46 + nlen;
@@ -184,14 +186,15 @@ void TensorFile::load() {
       x += 4 + (size_t)len;
     }
     p += 46 + (size_t)nlen + xlen + clen;
-    if (lho + 30 > buf.size() || rd32(&buf[lho]) != kLocalSig) fail(filename + ": bad local header of " + member);
+    if (buf.size() < 30 || lho > buf.size() - 30 || rd32(&buf[lho]) != kLocalSig) fail(filename + ": bad local header of " + member);
     const size_t data = (size_t)lho + 30 + rd16(&buf[lho + 26]) + rd16(&buf[lho + 28]);
-    if (data + csize > buf.size()) fail(filename + ": member " + member + " runs past the end of the file");
+    if (data > buf.size() || csize > buf.size() - data) fail(filename + ": member " + member + " runs past the end of the file");
     std::string name = member;
     if (name.size() > 4 && name.compare(name.size() - 4, 4, ".npy") == 0) name.resize(name.size() - 4);
     if (method == 0) {
       map[name] = parse_npy(&buf[data], (size_t)csize, member);
     } else if (method == 8) {
+      if (csize > 0xffffffffu || usize > 0xffffffffu) fail("compressed member " + member + " is too large");
       std::vector<uint8_t> raw((size_t)usize);
       z_stream zs{};
       if (inflateInit2(&zs, -MAX_WBITS) != Z_OK) fail("zlib init failed");
@@ -199,7 +202,6 @@ void TensorFile::load() {
       zs.avail_in = (uInt)csize;
       zs.next_out = raw.data();
       zs.avail_out = (uInt)usize;
-      if (csize > 0xffffffffu || usize > 0xffffffffu) { inflateEnd(&zs); fail("compressed member " + member + " is too large"); }
       const int rc = inflate(&zs, Z_FINISH);
       inflateEnd(&zs);
       if (rc != Z_STREAM_END) fail(filename + ": cannot inflate " + member);
