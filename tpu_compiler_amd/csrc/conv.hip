@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 using namespace tpuhip;
@@ -50,7 +51,7 @@ struct tpuhip_conv_weights {
   int32_t *bias = nullptr;
   QParam *qp = nullptr;
   int32_t *qplanes = nullptr;   // mult | rshift | hpot planes of nparam entries each
-  int32_t *qc64 = nullptr;      // low | high words of bias * mult + 2^30 (the addend of the 64-bit multiply-add)
+  int32_t *qc64 = nullptr;      // (low, high) pairs of bias * mult + 2^30, then the same + 2^(rshift-1) * 2^31
   int nparam = 0;
   int ocp = 0;           // padded output channels (rows of w / entries of bias, qp)
   int kp = 0;            // padded K in bytes (row stride of w) for the MFMA path
@@ -64,7 +65,10 @@ struct ConvArgs {
   const int32_t *bias;
   const QParam *qp;
   const int32_t *qmult, *qshift, *qhpot;   // the same per-channel data as planes (MFMA epilogue)
-  const int32_t *qclo, *qchi;              // bias * mult + 2^30 per channel, low and high words
+  // per channel, as (low, high) word pairs: qc64 = bias * mult + 2^30, the addend of the
+  // requantisation's 64-bit multiply-add; qc64r = qc64 + 2^(rshift-1) * 2^31, which also carries
+  // the rounding term of the right shift (layers with a fused ReLU)
+  const int32_t *qc64, *qc64r;
   int8_t *y;
   int n, ih, iw, x_cs;
   int oh, ow, y_cs;
@@ -1143,27 +1147,46 @@ conv_patch_kernel(ConvArgs a) {
 // whatever follows it in memory (finite integers times zero; past the end of the tensor the
 // buffer descriptor supplies zeros).
 // ---------------------------------------------------------------------------
-template <int TN>
-__device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, const int32_t *pclo,
-                                                 const int32_t *pchi, const int32_t *pmult,
-                                                 const int32_t *pshift, const int32_t *phpot,
-                                                 uint32_t (&outw)[TN][4]) {
+// Requantisation of accumulators that started at zero, for layers whose overflow-free form the
+// host has proved: the bias rides in the addend of the 64-bit multiply-add,
+//   (acc + b) * m + 2^30 == acc * m + c,   c = b * m + 2^30   (pc64: (low, high) pairs per channel).
+// RELU (the layer clamps at 0 after saturation): the rounding right shift needs no sign term, as
+// for x < 0 both (x + h) >> r and (x + h - 1) >> r are <= 0 and the clamp makes them 0; then
+//   ((p >> 31) + h) >> r == (p + h * 2^31) >> (31 + r) == hi32(p + h * 2^31) >> (r - 1),   r >= 1,
+// one multiply-add with c + h * 2^31 as the addend and one shift of the high word (pshift then
+// holds r - 1 and phpot is not read).
+// K slices by which the LDS reads of MFMA operands run ahead of their MFMAs: an LDS read takes
+// some 130 clocks, a 32x32x32 MFMA 32 to 34
+constexpr int frag_prefetch(int mfmas_per_slice) { return mfmas_per_slice >= 8 ? 1 : mfmas_per_slice >= 4 ? 2 : 3; }
+
+template <int TN, bool RELU>
+__device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, const int32_t *pc64,
+                                                 const int32_t *pmult, const int32_t *pshift,
+                                                 const int32_t *phpot, uint32_t (&outw)[TN][4]) {
 #pragma unroll
   for (int qd = 0; qd < 4; ++qd) {
-    const v4i cl = *reinterpret_cast<const v4i *>(pclo + qd * 4);
-    const v4i ch = *reinterpret_cast<const v4i *>(pchi + qd * 4);
+    const v4i c01 = *reinterpret_cast<const v4i *>(pc64 + qd * 8);
+    const v4i c23 = *reinterpret_cast<const v4i *>(pc64 + qd * 8 + 4);
     const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
     const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
-    const v4i h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
+    v4i h4 = {0, 0, 0, 0};
+    if (!RELU) h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
+    const int64_t c[4] = {(int64_t)(((uint64_t)(uint32_t)c01[1] << 32) | (uint32_t)c01[0]),
+                          (int64_t)(((uint64_t)(uint32_t)c01[3] << 32) | (uint32_t)c01[2]),
+                          (int64_t)(((uint64_t)(uint32_t)c23[1] << 32) | (uint32_t)c23[0]),
+                          (int64_t)(((uint64_t)(uint32_t)c23[3] << 32) | (uint32_t)c23[2])};
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       int32_t y[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int64_t c = (int64_t)(((uint64_t)(uint32_t)ch[e] << 32) | (uint32_t)cl[e]);
-        const int64_t p = (int64_t)acc[j][qd * 4 + e] * (int64_t)m4[e] + c;
-        const int32_t x = (int32_t)(p >> 31);
-        y[e] = (x + h4[e] + (x >> 31)) >> r4[e];
+        const int64_t p = (int64_t)acc[j][qd * 4 + e] * (int64_t)m4[e] + c[e];
+        if (RELU) {
+          y[e] = (int32_t)(p >> 32) >> r4[e];
+        } else {
+          const int32_t x = (int32_t)(p >> 31);
+          y[e] = (x + h4[e] + (x >> 31)) >> r4[e];
+        }
       }
       outw[j][qd] = pack_sat4(y[0], y[1], y[2], y[3], lo);
     }
@@ -1172,18 +1195,19 @@ __device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, 
 }
 
 template <int BM, int BN, int WM, int WN, int KP, int SD, int OCC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+__global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_pw_kernel(ConvArgs a) {
-  constexpr int NT = 256;
+  constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
+  static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
   static_assert(KP == 64 || KP == 128 || KP == 256, "padded K");
   constexpr int KC = KP / 64;              // 64-byte K chunks
   constexpr int CPRK = KP / 16;            // 16-byte chunks of a pixel row
   constexpr int RPP = NT / CPRK;           // pixel rows per pass of the loader
-  constexpr int NXC = BN / RPP;            // activation chunks per thread per tile
-  constexpr int NWC = BM * KP / 16 / NT;   // filter chunks per thread
-  static_assert(BN % RPP == 0 && NXC >= 1 && NWC >= 1, "loader shape");
+  constexpr int NXC = (BN + RPP - 1) / RPP;   // activation chunks per thread per tile
+  constexpr int WCH = BM * KP / 16;        // filter chunks of the slice
+  constexpr int NWC = (WCH + NT - 1) / NT; // ... per thread
+  constexpr bool XTAIL = BN % RPP != 0;    // the last pass covers fewer rows than threads
   constexpr int SROW = stage_row_bytes<BM>();
   extern __shared__ __attribute__((aligned(16))) v4i pw_smem[];
   v4i *const wA = pw_smem;                                       // [KC][BM][4 chunks], swizzled
@@ -1224,7 +1248,7 @@ conv_pw_kernel(ConvArgs a) {
 #pragma unroll
     for (int u = 0; u < NXC; ++u) {
       const int row = lrow + RPP * u;
-      const bool pv = exists && lpix0 + row < a.npix;
+      const bool pv = exists && lpix0 + row < a.npix && (!XTAIL || row < BN);
       const uint32_t t1 = (uint32_t)(low + row);
       const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
       const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
@@ -1249,7 +1273,7 @@ conv_pw_kernel(ConvArgs a) {
 #pragma unroll
     for (int u = 0; u < NXC; ++u) {
       const int row = lrow + RPP * u;
-      base[row * 4 + ((c & 3) ^ ((row >> 2) & 3))] = breg[u];
+      if (!XTAIL || row < BN) base[row * 4 + ((c & 3) ^ ((row >> 2) & 3))] = breg[u];
     }
   };
   // does the tile j steps ahead of the current one exist?
@@ -1263,17 +1287,21 @@ conv_pw_kernel(ConvArgs a) {
     const v4i *wsrc = reinterpret_cast<const v4i *>(a.w) + (size_t)(oc0 / BM) * (BM * KP / 16);
     v4i wreg[NWC];
 #pragma unroll
-    for (int u = 0; u < NWC; ++u) wreg[u] = wsrc[tid + u * NT];
+    for (int u = 0; u < NWC; ++u)
+      if (WCH % NT == 0 || tid + u * NT < WCH) wreg[u] = wsrc[tid + u * NT];
     if (tid < BM) {
-      qlds[tid] = a.qclo[oc0 + tid];
-      qlds[BM + tid] = a.qchi[oc0 + tid];
+      // a workgroup whose result is clamped at 0 takes the constants of the short form
+      const int32_t *c64 = out.lo == 0 ? a.qc64r : a.qc64;
+      qlds[2 * tid] = c64[2 * (oc0 + tid)];
+      qlds[2 * tid + 1] = c64[2 * (oc0 + tid) + 1];
       qlds[2 * BM + tid] = a.qmult[oc0 + tid];
-      qlds[3 * BM + tid] = a.qshift[oc0 + tid];
+      qlds[3 * BM + tid] = a.qshift[oc0 + tid] - (out.lo == 0 ? 1 : 0);
       qlds[4 * BM + tid] = a.qhpot[oc0 + tid];
     }
     if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
 #pragma unroll
-    for (int u = 0; u < NWC; ++u) wA[tid + u * NT] = wreg[u];
+    for (int u = 0; u < NWC; ++u)
+      if (WCH % NT == 0 || tid + u * NT < WCH) wA[tid + u * NT] = wreg[u];
   }
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
   store_B(0);
@@ -1309,21 +1337,31 @@ conv_pw_kernel(ConvArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
     const v4i *xb = xB + cur * (KC * BN * 4);
+    // the operands of 32-byte K slice ks are requested PD slices before their MFMAs: with one
+    // or two waves on a SIMD nothing else hides the LDS latency (two MFMAs take 64 clocks, an
+    // LDS read twice that)
+    constexpr int PD0 = OCC >= 4 ? 1 : frag_prefetch(TM * TN);
+    constexpr int NS = KC * 2, PD = PD0 < NS ? PD0 : NS;
+    v4i fa[PD + 1][TM], fb[PD + 1][TN];
+    auto read_slice = [&](int ks, int slot) {
 #pragma unroll
-    for (int kc = 0; kc < KC; ++kc)
+      for (int i = 0; i < TM; ++i) fa[slot][i] = wA[(ks >> 1) * (BM * 4) + ia[i][ks & 1]];
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        v4i fa[TM], fb[TN];
+      for (int j = 0; j < TN; ++j) fb[slot][j] = xb[(ks >> 1) * (BN * 4) + ib[j][ks & 1]];
+    };
 #pragma unroll
-        for (int i = 0; i < TM; ++i) fa[i] = wA[kc * (BM * 4) + ia[i][kk]];
+    for (int ks = 0; ks < PD; ++ks) read_slice(ks, ks);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) fb[j] = xb[kc * (BN * 4) + ib[j][kk]];
+    for (int ks = 0; ks < NS; ++ks) {
+      if (ks + PD < NS) read_slice(ks + PD, (ks + PD) % (PD + 1));
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      }
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks % (PD + 1)][i], fb[ks % (PD + 1)][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
     // the next tile's pixels go to the other LDS tile (free since the barrier of the last
     // epilogue), the one after that is requested
@@ -1339,8 +1377,12 @@ conv_pw_kernel(ConvArgs a) {
     for (int i = 0; i < TM; ++i) {
       uint32_t outw[TN][4];
       const int lc = lch0 + i * 16;
-      requant_rows_c64<TN>(acc[i], out.lo, qlds + lc, qlds + BM + lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
-                           qlds + 4 * BM + lc, outw);
+      if (out.lo == 0)
+        requant_rows_c64<TN, true>(acc[i], 0, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
+                                   qlds + 4 * BM + lc, outw);
+      else
+        requant_rows_c64<TN, false>(acc[i], out.lo, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc,
+                                    qlds + 4 * BM + lc, outw);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         *reinterpret_cast<v4i *>(stage + ((wn * TN + j) * 32 + frow) * SROW + lc) =
@@ -1356,6 +1398,230 @@ conv_pw_kernel(ConvArgs a) {
     if (SD == 2) sd ^= 1;
     else __syncthreads();   // one staging area: everyone has read it before it is written again
   }
+}
+
+// ---------------------------------------------------------------------------
+// 3x3 / stride 1 / pad 1 convolutions, second form of the row-patch kernel: the same tiling
+// as conv_patch_kernel (a workgroup computes BM channels of TH whole rows of one image from a
+// patch of TH + 2 input rows held in LDS, the filter streams through a double-buffered LDS
+// tile), rebuilt around what the counters showed the first form spends its time on -- vector
+// ALU instructions that are not arithmetic of the layer:
+//   * LDS rows are PADDED by 16 bytes (patch position: C + 16 bytes, filter row: BK + 16)
+//     instead of XOR-swizzled: 16 consecutive rows still start in 16 different 16-byte bank
+//     groups (C and BK are multiples of 64), and an operand address becomes lane base +
+//     wave-uniform offset -- one add per fragment and K step, immediates within a step --
+//     where the swizzle cost five operations per fragment;
+//   * the patch is fetched row by row: a lane's global offset is row base + 16 * index;
+//   * K steps of BK = 128 or 256 bytes whatever the channel count (a step of a 64-channel
+//     layer spans four taps), so a 3x3 x 64 layer meets three barriers, not nine;
+//   * accumulators start at zero and the bias rides in the requantisation's 64-bit addend;
+//     layers with a ReLU take the two-instruction form of requant_rows_c64.
+// Layers whose overflow-free requantisation the host cannot prove stay with the first form.
+//   a.stem_pw = W + 2, a.magic_pw = floor(2^20 / (W + 2)) + 1, a.pstep_pix = TH,
+//   a.pstep_n = tiles per image, a.pstep_oh = log2(C), C a power of two from 64 to 1024
+// LDS (dynamic): parameters | two filter tiles | patch; the staged output tile takes the
+// filter tiles' place.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int WM, int WN, int BK, int OCC>
+__global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
+conv_patch2_kernel(ConvArgs a) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int RD = 4;                       // filter tiles in flight in registers (even)
+  constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
+  static_assert(BK == 128 || BK == 256, "K bytes per step");
+  constexpr int AROW = BK + 16;               // bytes of a filter tile row in LDS
+  constexpr int ABYTES = BM * AROW;
+  constexpr int CPA = BK / 16;                // 16-byte chunks of a filter tile row
+  constexpr int NW = BM * CPA / NT;           // filter chunks per thread per step
+  constexpr int KK = BK / 32;
+  constexpr int NPL = 18 * 256 / NT;          // patch chunks per thread at most (72 KiB of input)
+  static_assert(BN * stage_row_bytes<BM>() <= 2 * ABYTES, "the staged tile must fit the filter tiles");
+  extern __shared__ __attribute__((aligned(16))) v4i p2_smem[];
+  int32_t *const qlds = reinterpret_cast<int32_t *>(p2_smem);                 // 5 * BM dwords
+  uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);         // 64 dwords
+  int8_t *const abuf = reinterpret_cast<int8_t *>(lutw + 64);                 // 2 * ABYTES
+  int8_t *const patch = abuf + 2 * ABYTES;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  if (logical >= a.n_tiles) return;
+  const int pt = logical / a.n_oc_tiles;
+  const int oc0 = (logical - pt * a.n_oc_tiles) * BM;
+  const int img = pt / a.pstep_n;
+  const int r0 = (pt - img * a.pstep_n) * a.pstep_pix;
+  const int rows = min(a.pstep_pix, a.oh - r0);
+  const int pix_base = (img * a.oh + r0) * a.ow;
+  const int pix_limit = pix_base + rows * a.ow;
+  const int pw = a.stem_pw;
+  const int lgc = a.pstep_oh;                 // log2(C)
+  const int C = 1 << lgc;
+  const int prow = C + 16;                    // bytes of a patch position in LDS
+  const bool relu = a.lo == 0;
+
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+
+  // ---- the patch: row r of it is pw positions of C bytes = pw * C / 16 chunks, of which chunk
+  // p lies at byte (p - C / 16) * 16 of input row r0 - 1 + r (the first and last position are
+  // the zero border)
+  const int rowchunks = pw << (lgc - 4);
+  const int n_chunks = (a.pstep_pix + 2) * rowchunks;
+  v4i preg[NPL];
+#pragma unroll
+  for (int u = 0; u < NPL; ++u) {
+    const int q = tid + u * NT;
+    const int pr = (int)__umulhi((uint32_t)q, a.magic_c16);      // q / rowchunks
+    const int p = q - pr * rowchunks;
+    const int row = r0 - 1 + pr;
+    const bool ok = q < n_chunks && (unsigned)row < (unsigned)a.ih && p >= (C >> 4) && p < ((a.iw + 1) << (lgc - 4));
+    preg[u] = buffer_load16(xrsrc, ok ? (uint32_t)(((img * a.ih + row) * a.iw - 1) * C + p * 16) : kOobOffset);
+  }
+
+  // ---- the filter: K step s of this output-channel tile is BM * BK contiguous bytes
+  static_assert(NW >= 1, "filter tile smaller than a pass of the workgroup");
+  const uint32_t wbase = (uint32_t)(oc0 / BM) * (uint32_t)(a.kp * BM) + (uint32_t)tid * 16u;
+  const int nsteps = a.kp / BK;
+  v4i wr[RD][NW];
+  auto load_A = [&](int slot, int step) {
+#pragma unroll
+    for (int u = 0; u < NW; ++u)
+      wr[slot][u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(wrsrc, wbase + (uint32_t)(u * NT * 16), step * (BM * BK), 0);
+  };
+  auto store_A = [&](int slot, int buf) {
+#pragma unroll
+    for (int u = 0; u < NW; ++u) {
+      const int q = tid + u * NT;
+      *reinterpret_cast<v4i *>(abuf + buf * ABYTES + (q / CPA) * AROW + (q % CPA) * 16) = wr[slot][u];
+    }
+  };
+#pragma unroll
+  for (int d = 0; d < RD; ++d)
+    if (d < nsteps) load_A(d, d);
+
+  if (tid < BM) {
+    const int32_t *c64 = relu ? a.qc64r : a.qc64;
+    qlds[2 * tid] = c64[2 * (oc0 + tid)];
+    qlds[2 * tid + 1] = c64[2 * (oc0 + tid) + 1];
+    qlds[2 * BM + tid] = a.qmult[oc0 + tid];
+    qlds[3 * BM + tid] = a.qshift[oc0 + tid] - (relu ? 1 : 0);
+    qlds[4 * BM + tid] = a.qhpot[oc0 + tid];
+  }
+  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  const int lch0 = wm * TM * 32 + fk * 16 * TM;
+  // lane bases of the fragment reads
+  int abase[TM], bbase[TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) abase[i] = ((wm * TM + i) * 32 + frow) * AROW + fk * 16;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int p = (wn * TN + j) * 32 + frow;
+    const uint32_t pr = a.ow == 1 ? (uint32_t)p : __umulhi((uint32_t)p, a.magic_ow);
+    const int pc = p - (int)pr * a.ow;
+    bbase[j] = (p < rows * a.ow ? (int)pr * pw + pc : 0) * prow + fk * 16;   // idle slots read position 0
+  }
+
+  // park the patch and the first filter tile
+#pragma unroll
+  for (int u = 0; u < NPL; ++u) {
+    const int q = tid + u * NT;
+    const int pr = (int)__umulhi((uint32_t)q, a.magic_c16);
+    const int p = q - pr * rowchunks;
+    if (q < n_chunks)
+      *reinterpret_cast<v4i *>(patch + (pr * pw + (p >> (lgc - 4))) * prow + (p & ((C >> 4) - 1)) * 16) = preg[u];
+  }
+  store_A(0, 0);
+  __syncthreads();
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS a
+  // step ago -- and receives the tile RD steps ahead; the next step's tile goes from its slot
+  // to the other LDS tile.  Within the step the operands of a 32-byte K slice are requested PD
+  // slices before their MFMAs (see frag_prefetch).
+  constexpr int PD = OCC >= 4 ? 1 : frag_prefetch(TM * TN);
+  auto step = [&](int s, auto slotc) {
+    constexpr int slot = decltype(slotc)::value, buf = slot & 1;
+    if (s + RD < nsteps) load_A(slot, s + RD);
+    const int8_t *ab = abuf + buf * ABYTES;
+    v4i fa[PD + 1][TM], fb[PD + 1][TN];
+    auto read_slice = [&](int kk, int fs) {
+      // the slice lies in one filter tap (C is a multiple of 64); slices past the ninth tap
+      // meet zero weights and read the last tap
+      const int koff = s * BK + kk * 32;
+      const int tap = min(koff >> lgc, 8);
+      const int tkh = (tap * 11) >> 5;
+      const int boff = (tkh * pw + (tap - 3 * tkh)) * prow + (koff & (C - 1));
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(ab + abase[i] + kk * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
+    };
+    // K is padded to whole steps with zero weights: the slices of the last step that lie in
+    // the padding are not multiplied (kreal: slices of this step that hold weights)
+    const int kreal = min(KK, (a.k16 * 16 - s * BK + 31) >> 5);
+#pragma unroll
+    for (int kk = 0; kk < PD; ++kk) read_slice(kk, kk);
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      if (kk + PD < KK) read_slice(kk + PD, (kk + PD) % (PD + 1));
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk < kreal) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[kk % (PD + 1)][i], fb[kk % (PD + 1)][j], acc[i][j], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (s + 1 < nsteps) store_A((slot + 1) % RD, buf ^ 1);
+    __syncthreads();
+  };
+  for (int s = 0; s < nsteps; s += RD) {
+    step(s, std::integral_constant<int, 0>{});
+    if (s + 1 < nsteps) step(s + 1, std::integral_constant<int, 1>{});
+    if (s + 2 < nsteps) step(s + 2, std::integral_constant<int, 2>{});
+    if (s + 3 < nsteps) step(s + 3, std::integral_constant<int, 3>{});
+  }
+
+  // the requantised tile goes through LDS (the filter tiles' space: every wave is past the
+  // last barrier of the K loop) and leaves in memory order
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+  int8_t *const stage = abuf;
+  v4i sv[flush_chunks<BM, BN, NT>()];
+  flush_prefetch<BM, BN, NT>(a, tid, pix_base, pix_limit, oc0, out, sv);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    uint32_t outw[TN][4];
+    const int lc = lch0 + i * 16;
+    if (relu)
+      requant_rows_c64<TN, true>(acc[i], 0, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
+    else
+      requant_rows_c64<TN, false>(acc[i], a.lo, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc,
+                                  outw);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      *reinterpret_cast<v4i *>(stage + ((wn * TN + j) * 32 + frow) * stage_row_bytes<BM>() + lc) =
+          v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+  }
+  __syncthreads();
+  flush_tile<BM, BN, NT>(a, stage, tid, pix_base, pix_limit, oc0, out, lut, sv);
 }
 
 // ---------------------------------------------------------------------------
@@ -2011,7 +2277,8 @@ struct TileCfg {
   const char *name;
   int reg;   // 0: LDS kernel, one tile per workgroup; 1: the LDS-free kernel, bm x bn is the
              // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups;
-             // 4: patch kernel (bn = pixel slots of a tile of whole rows); 5: pointwise kernel
+             // 4: patch kernel (bn = pixel slots of a tile of whole rows); 5: pointwise kernel;
+             // 6: patch kernel, second form
   int bk;    // K bytes per step (pointwise kernel: the padded K it holds)
 };
 
@@ -2057,7 +2324,25 @@ struct TileCfg {
   W(27, "mfma_pw_128x64_k128", 128, 64, 2, 2, 128, 2, 3)    \
   W(28, "mfma_pw_128x64_k256", 128, 64, 2, 2, 256, 1, 2)    \
   W(29, "mfma_pw_256x64_k64", 256, 64, 4, 1, 64, 2, 2)      \
-  W(30, "mfma_pw_256x64_k128", 256, 64, 4, 1, 128, 1, 2)
+  W(30, "mfma_pw_256x64_k128", 256, 64, 4, 1, 128, 1, 2)    \
+  W(36, "mfma_pw_256x64_k64_w8", 256, 64, 4, 2, 64, 2, 4)   \
+  W(37, "mfma_pw_256x64_k128_w8", 256, 64, 4, 2, 128, 1, 4) \
+  W(38, "mfma_pw_128x64_k256_w8", 128, 64, 4, 2, 256, 1, 4) \
+  W(39, "mfma_pw_64x128_k64_w8", 64, 128, 2, 4, 64, 2, 4)   \
+  W(40, "mfma_pw_128x64_k64_w8", 128, 64, 4, 2, 64, 2, 4)
+
+// row-patch kernels, second form (3x3 / stride 1 / pad 1, 64 to 1024 input channels, a power of two):
+// V(index, name, BM, BN, WM, WN, BK, waves per SIMD)
+#define TPUHIP_PATCH2_TILES(V)                          \
+  V(31, "mfma_patch2_64x256", 64, 256, 1, 4, 256, 2)    \
+  V(32, "mfma_patch2_64x128", 64, 128, 2, 2, 256, 2)    \
+  V(33, "mfma_patch2_128x128", 128, 128, 2, 2, 128, 2)  \
+  V(34, "mfma_patch2_64x64", 64, 64, 2, 2, 256, 2)      \
+  V(35, "mfma_patch2_128x256", 128, 256, 2, 2, 128, 1)  \
+  V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4) \
+  V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4) \
+  V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4) \
+  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2)
 
 struct TileTable {
   TileCfg t[64];
@@ -2083,6 +2368,11 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_PW_TILES(W)
 #undef W
+#define V(i, name, BM, BN, WM, WN, BK, O) \
+  t[i] = TileCfg{BM, BN, WM, WN, name, 6, BK}; \
+  n = n > i ? n : i + 1;
+    TPUHIP_PATCH2_TILES(V)
+#undef V
   }
 };
 const TileTable kTileTable;
@@ -2142,9 +2432,9 @@ void launch_pw(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
     constexpr unsigned lds = pw_lds_bytes(BM, BN, KP, SD);                                              \
     if (!pw_prepare(kernel, lds)) break;                                                                \
     if (ctx->prof_start)                                                                                \
-      hipExtLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
+      hipExtLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
     else                                                                                                \
-      hipLaunchKernelGGL(kernel, grid, dim3(256), lds, ctx->stream, a);                                 \
+      hipLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, a);                        \
   } break;
     TPUHIP_PW_TILES(W)
 #undef W
@@ -2159,7 +2449,7 @@ int pw_occupancy(int tile) {
 #define W(i, name, BM, BN, WM, WN, KP, SD, O)                                                           \
   case i:                                                                                               \
     if (pw_prepare(conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>, pw_lds_bytes(BM, BN, KP, SD)))             \
-      e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>, 256, \
+      e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, conv_pw_kernel<BM, BN, WM, WN, KP, SD, O>, WM * WN * 64, \
                                                        pw_lds_bytes(BM, BN, KP, SD));                   \
     break;
     TPUHIP_PW_TILES(W)
@@ -2167,6 +2457,46 @@ int pw_occupancy(int tile) {
   }
   if (e != hipSuccess) (void)hipGetLastError();
   return e == hipSuccess && n > 0 ? n : 1;
+}
+
+// ---- row-patch kernels, second form
+constexpr int kPatch2MaxChunks = 18 * 256;     // 16-byte input chunks a workgroup's patch may hold
+constexpr int kLdsBytes = 160 * 1024;
+
+inline unsigned patch2_lds_bytes(const TileCfg &c, int th, int ow, int ic) {
+  return (unsigned)(5 * c.bm * 4 + 256 + 2 * c.bm * (c.bk + 16) + (th + 2) * (ow + 2) * (ic + 16));
+}
+
+// rows of one image a tile holds; 0: the layer does not fit this kernel
+int patch2_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
+  const bool shape_ok = d.g == 1 && d.kh == 3 && d.kw == 3 && d.sh == 1 && d.sw == 1 && d.dh == 1 && d.dw == 1 &&
+                        d.pt == 1 && d.pb == 1 && d.pl == 1 && d.pr == 1 && !d.ins_h && !d.ins_w && !d.relu_first &&
+                        d.oh == d.ih && d.ow == d.iw && d.x_cs == d.ic && d.ic >= 64 && d.ic <= 1024 &&
+                        (d.ic & (d.ic - 1)) == 0;
+  if (!shape_ok || d.ow > c.bn) return 0;
+  int th = std::min(c.bn / d.ow, d.oh);
+  while (th >= 1 && ((th + 2) * (d.ow + 2) * (d.ic / 16) > kPatch2MaxChunks ||
+                     patch2_lds_bytes(c, th, d.ow, d.ic) > (unsigned)kLdsBytes))
+    --th;
+  if (th < 1) return 0;
+  const int tiles = (d.oh + th - 1) / th;      // evened out over the image
+  return (d.oh + tiles - 1) / tiles;
+}
+
+void launch_patch2(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsigned lds) {
+  switch (tile) {
+#define V(i, name, BM, BN, WM, WN, BK, O)                                                               \
+  case i: {                                                                                             \
+    auto kernel = conv_patch2_kernel<BM, BN, WM, WN, BK, O>;                                            \
+    if (!pw_prepare(kernel, (unsigned)kLdsBytes)) break;                                                \
+    if (ctx->prof_start)                                                                                \
+      hipExtLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
+    else                                                                                                \
+      hipLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, a);                        \
+  } break;
+    TPUHIP_PATCH2_TILES(V)
+#undef V
+  }
 }
 
 template <bool FAST, int MODE>
@@ -2304,6 +2634,12 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
         rowbuf[(size_t)k * kstride + c] = src[(size_t)c * d.kh * d.kw + k];
     if (t.reg == 0 || t.reg == 3 || t.reg == 4) {
       memcpy(packed.data() + (size_t)row * cw->kp, rowbuf.data(), rowbuf.size());
+    } else if (t.reg == 6) {
+      // [output-channel tile][K step][row][BK bytes]: every step's tile is contiguous
+      const int r = row - tile0;
+      int8_t *img = packed.data() + (size_t)(tile0 / t.bm) * t.bm * cw->kp;
+      for (int st = 0; st < cw->kp / t.bk; ++st)
+        memcpy(img + ((size_t)st * t.bm + r) * t.bk, rowbuf.data() + (size_t)st * t.bk, t.bk);
     } else if (t.reg == 5) {
       // the LDS image of every output-channel tile: [64-byte K chunk][row][4 x 16 bytes], the
       // 16-byte position XORed with (row >> 2) & 3
@@ -2336,7 +2672,9 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 }
 
 // the fused table lives in the LDS of the LDS kernels
-bool tile_has_lds_epilogue(int t) { return kTiles[t].reg == 0 || kTiles[t].reg == 3 || kTiles[t].reg == 5; }
+bool tile_has_lds_epilogue(int t) {
+  return kTiles[t].reg == 0 || kTiles[t].reg == 3 || kTiles[t].reg == 5 || kTiles[t].reg == 6;
+}
 
 // the pointwise kernels: 1x1 window, no padding, no dilation (any stride), the input channels
 // within the K the variant holds (and more than half of it, or the smallest variant)
@@ -2365,6 +2703,7 @@ bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   const TileCfg &c = kTiles[t];
   if (c.reg == 4 && patch_rows(d, c) == 0) return false;
   if (c.reg == 5 && !pw_shape_ok(d, c)) return false;
+  if (c.reg == 6 && patch2_rows(d, c) == 0) return false;
   if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
@@ -2380,8 +2719,8 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.qmult = w->qplanes;
   a.qshift = w->qplanes + w->nparam;
   a.qhpot = w->qplanes + 2 * w->nparam;
-  a.qclo = w->qc64;
-  a.qchi = w->qc64 + w->nparam;
+  a.qc64 = w->qc64;
+  a.qc64r = w->qc64 + 2 * w->nparam;
   a.y = (int8_t *)y;
   a.n = d.n; a.ih = d.ih; a.iw = d.iw; a.x_cs = d.x_cs;
   a.oh = d.oh; a.ow = d.ow; a.y_cs = d.y_cs;
@@ -2412,8 +2751,8 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
     const int n_wgs = t.reg == 1 ? (a.n_tiles + 3) / 4 : a.n_tiles;
     a.tiles_per_xcd = (n_wgs + 7) / 8;
     a.wgs_per_xcd = a.tiles_per_xcd;
-    if (t.reg == 4) {
-      const int th = patch_rows(d, t);
+    if (t.reg == 4 || t.reg == 6) {
+      const int th = t.reg == 4 ? patch_rows(d, t) : patch2_rows(d, t);
       const int tiles_per_img = (d.oh + th - 1) / th;
       const int n_pix_tiles = d.n * tiles_per_img;
       a.n_tiles = n_pix_tiles * a.n_oc_tiles;
@@ -2425,6 +2764,14 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
       a.pstep_n = tiles_per_img;
       a.pstep_oh = w->c16 == 4 ? 2 : w->c16 == 8 ? 3 : w->c16 == 16 ? 4 : 5;     // log2(C / 16)
       a.pstep_ow = w->c16 == 4 ? 2 : w->c16 == 8 ? 1 : 0;                        // swizzle shift
+      if (t.reg == 6) {
+        int lgc = 6;
+        while ((1 << lgc) < d.ic) ++lgc;
+        a.pstep_oh = lgc;                                                        // log2(C)
+        const uint32_t rowchunks = (uint32_t)a.stem_pw * (uint32_t)(d.ic / 16);
+        a.magic_c16 = (uint32_t)(((1ull << 32) + rowchunks - 1) / rowchunks);    // q / rowchunks == umulhi(q, magic), q < 2^16
+        a.pstep_ow = (int)patch2_lds_bytes(t, th, d.ow, d.ic);                   // dynamic LDS of the launch
+      }
     }
     if (t.reg == 3 || t.reg == 5) {
       // every XCD owns a run of whole pixel tiles; a workgroup keeps its channel tile
@@ -2445,6 +2792,10 @@ void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvA
   dim3 grid((unsigned)(a.wgs_per_xcd * 8));
   if (kTiles[w->tile].reg == 5) {
     launch_pw(ctx, w->tile, grid, a);
+    return;
+  }
+  if (kTiles[w->tile].reg == 6) {
+    launch_patch2(ctx, w->tile, grid, a, (unsigned)a.pstep_ow);
     return;
   }
   const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
@@ -2511,6 +2862,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     if (post.lut && !tile_has_lds_epilogue(t)) continue;
     if (w->split_oc && kTiles[t].reg == 4) continue;   // the patch kernel writes one result
     if (kTiles[t].reg == 5 && (!w->fast || w->split_oc % kTiles[t].bm)) continue;
+    if (kTiles[t].reg == 6 && (!w->fast || w->split_oc)) continue;
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
@@ -2713,11 +3065,14 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
     if (!rc) rc = tpuhip_upload(ctx, cw->qplanes, planes.data(), planes.size() * sizeof(int32_t));
     // (acc + bias) * mult + 2^30 == acc * mult + c: the addend of the requantisation's 64-bit
     // multiply-add, as a plane of low and a plane of high words
-    std::vector<int32_t> c64(2 * nparam);
+    std::vector<int32_t> c64(4 * nparam);
     for (size_t i = 0; i < nparam; ++i) {
       const int64_t c = (int64_t)b32[i] * (int64_t)qp[i].mult + (1ll << 30);
-      c64[i] = (int32_t)(uint32_t)(c & 0xffffffffll);
-      c64[nparam + i] = (int32_t)(c >> 32);
+      const int64_t cr = c + ((int64_t)qp[i].hpot << 31);
+      c64[2 * i] = (int32_t)(uint32_t)(c & 0xffffffffll);
+      c64[2 * i + 1] = (int32_t)(c >> 32);
+      c64[2 * nparam + 2 * i] = (int32_t)(uint32_t)(cr & 0xffffffffll);
+      c64[2 * nparam + 2 * i + 1] = (int32_t)(cr >> 32);
     }
     if (!rc) rc = tpuhip_malloc(ctx, c64.size() * sizeof(int32_t), (void **)&cw->qc64);
     if (!rc) rc = tpuhip_upload(ctx, cw->qc64, c64.data(), c64.size() * sizeof(int32_t));
@@ -2793,6 +3148,11 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
                  "conv: tile variant %s needs an unpadded 1x1 conv with 5 to %d input channels, right shifts of at "
                  "least 1 and sums that cannot overflow the rounding, and a pair split at a tile boundary",
                  kTiles[w->tile].name, kTiles[w->tile].bk);
+  TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 6) ||
+                     (!w->split_oc && w->fast && patch2_rows(w->d, kTiles[w->tile]) > 0),
+                 "conv: tile variant %s needs a single 3x3 / stride 1 / pad 1 conv with 64, 128, 256, 512 or 1024 input "
+                 "channels on a map narrow enough for its row patch, right shifts of at least 1 and sums that cannot "
+                 "overflow the rounding", kTiles[w->tile].name);
   TPUHIP_REQUIRE((w->split_oc != 0) == (post.y2 != nullptr),
                  "conv: weights packed as a pair run through tpuhip_conv2d_pair_i8 (and only they do)");
   ConvArgs a;
