@@ -20,34 +20,102 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # conv tile variant per layer as an earlier run of this benchmark chose them by timing: used
 # by default so that runs, and the committed profile of this command, execute the same kernels
-RECORDED_TILES = {"cfg3": os.path.join("profiles", "resnet50_b32_tiles.json")}
+RECORDED_TILES = {"cfg3": os.path.join("tpu_compiler_amd", "tiles", "cfg3_b32.json")}
 
 
-def conv_bytes(op, graph):
-    """algorithmic bytes of a conv / fc: int8 input + output + filter, 12 B of int32
-    parameters per output channel"""
+def conv_bytes(op, graph, fused_add=None, stored=True):
+    """algorithmic bytes of a conv / fc launch: int8 input + output + filter, 12 B of int32
+    parameters per output channel; with an eltwise add folded into the epilogue also the add's
+    other operand and its sum; without the conv result itself where that is not written"""
     import numpy as np
     x = graph.by_name[op.inputs[0]].shape
     oc = op.shape[1]
-    return int(np.prod(x)) + int(np.prod(op.shape)) + int(op.weights["filter"].size) + 12 * oc
+    n = int(np.prod(x)) + int(op.weights["filter"].size) + 12 * oc
+    if stored:
+        n += int(np.prod(op.shape))
+    if fused_add is not None:
+        n += 2 * int(np.prod(fused_add.shape))
+    return n
 
 
-def cpu_baseline(graph_fn, images, seconds=12.0):
-    """The oracle (CPU restatement of the reference's arithmetic) on a bounded sample of
-    the same workload, on this host's cores."""
+def host_cpu():
+    """model name, physical cores and logical CPUs of this host (from /proc/cpuinfo)"""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "model name":
+                model = v
+            elif k == "physical id":
+                phys = v
+            elif k == "core id":
+                core = v
+            elif not k and phys is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    return {"model": model, "physical_cores": len(cores) or None, "logical_cpus": os.cpu_count()}
+
+
+def _set_threads(n):
+    """OpenMP threads of the oracle library and of PyTorch's CPU ops"""
+    import ctypes
+    import torch
+    torch.set_num_threads(n)
+    try:
+        ctypes.CDLL("libgomp.so.1").omp_set_num_threads(n)
+    except OSError:
+        pass
+
+
+def _timed(fn, seconds, max_passes=20):
+    fn()                                     # page in
+    passes, t0 = 0, time.perf_counter()
+    while passes < max_passes and (passes == 0 or time.perf_counter() - t0 < seconds):
+        fn()
+        passes += 1
+    return passes, time.perf_counter() - t0
+
+
+def cpu_baseline(graph_fn, images, seconds=12.0, legs=("dataflow_4thr", "dataflow_all", "oracle_all"),
+                 keep_results=None):
+    """CPU restatements of the reference on a bounded sample of the same workload, on this host:
+    dataflow_*: the reference's data flow -- float-stored NCHW tensors, fp32 conv / inner product /
+    pooling through oneDNN (PyTorch CPU ops), float and integer epilogues, the graph run as an N=1
+    graph once per image (MlirModuleInterpreter.cpp:383-405) -- at the 4 threads the reference's
+    regression pins (regression/run_regression.sh:14) and at all CPUs; oracle_all: the integer-exact
+    C/OpenMP oracle.  The top-level value is the data-flow leg at all CPUs."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_dataflow
     import oracle_graph
     g = graph_fn(batch=images)
-    oracle_graph.run(g, keep=g.outputs)      # page in
-    passes, t0 = 0, time.perf_counter()
-    while passes < 20 and (passes == 0 or time.perf_counter() - t0 < seconds):
-        oracle_graph.run(g, keep=g.outputs)
-        passes += 1
-    dt = time.perf_counter() - t0
-    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": round(passes * images / dt, 2), "unit": "images/s", "cores": cores, "kind": "port",
-            "sample": "%s, %d passes of a batch of %d images (%.1f s) through the integer-exact "
-                      "C/OpenMP oracle" % (g.name, passes, images, dt)}
+    all_cpus = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    per_leg = max(0.1, seconds / max(1, len(legs)))
+    out_legs = {}
+    for leg in legs:
+        threads = 4 if leg.endswith("_4thr") else all_cpus
+        _set_threads(threads)
+        if leg.startswith("dataflow"):
+            n_img = max(1, min(images, 4))
+            passes, dt = _timed(lambda: oracle_dataflow.run(g, keep=g.outputs, images=n_img), per_leg)
+            done = passes * n_img
+            what = "%d N=1 passes (%.1f s) of the fp32 data-flow restatement" % (done, dt)
+        else:
+            passes, dt = _timed(lambda: oracle_graph.run(g, keep=g.outputs), per_leg)
+            done = passes * images
+            what = "%d passes of a batch of %d images (%.1f s) through the integer-exact C/OpenMP oracle" % (
+                passes, images, dt)
+        out_legs[leg] = {"value": round(done / dt, 2), "unit": "images/s", "cores": threads, "what": what}
+    _set_threads(all_cpus)
+    if keep_results is not None:
+        keep_results.update(oracle_graph.run(g, guards=keep_results.setdefault("__guards__", {})))
+    head = out_legs.get("dataflow_all") or next(iter(out_legs.values()))
+    return {"value": head["value"], "unit": "images/s", "cores": head["cores"], "kind": "port",
+            "sample": "%s, %d images: %s" % (g.name, images, head["what"]),
+            "host": host_cpu(), "legs": out_legs}
 
 
 def main():
@@ -149,6 +217,19 @@ def main():
     rows = m.time_kernels(iters=max(5, min(args.steps, 20)))
     by_algo = {}
     algo_of = {name: algo for name, algo, _ in rows}
+    ms_of = {name: ms for name, algo, ms in rows}
+    # an eltwise add that launched nothing rides in the epilogue of the later of its conv inputs
+    order = {op.name: i for i, op in enumerate(g.ops)}
+    readers = {}
+    for op in g.ops:
+        for i in op.inputs:
+            readers[i] = readers.get(i, 0) + 1
+    fused_add = {}
+    for op in g.ops:
+        if op.type == "tpu.eltwise_add" and ms_of.get(op.name, 1) == 0:
+            convs = [i for i in op.inputs if g.by_name[i].type == "tpu.conv_2d"]
+            if convs:
+                fused_add[max(convs, key=lambda n: order[n])] = op
     for name, algo, ms in rows:
         op = g.by_name[name]
         if op.type in ("tpu.conv_2d", "tpu.fully_connected"):
@@ -158,7 +239,9 @@ def main():
             d = by_algo.setdefault(key, {"ms": 0.0, "ops": 0.0, "bytes": 0.0, "launches": 0})
             d["ms"] += ms
             d["ops"] += 2.0 * op.macs
-            d["bytes"] += conv_bytes(op, g) - (int(np.prod(g.by_name[op.inputs[0]].shape)) if rides else 0)
+            add = fused_add.get(name)
+            stored = args.keep_all or add is None or readers.get(name, 0) > 1 or name in g.outputs
+            d["bytes"] += conv_bytes(op, g, add, stored) - (int(np.prod(g.by_name[op.inputs[0]].shape)) if rides else 0)
             d["launches"] += 0 if rides else 1
     mfma = {k: v for k, v in by_algo.items() if k.startswith("mfma")}
     conv_ms = sum(v["ms"] for v in mfma.values())
@@ -242,9 +325,45 @@ def main():
         out["host_io"] = {"ms_per_step": round(ms_io, 4), "images_per_s": round(batch / (ms_io / 1e3), 1),
                           "host_bytes_in": int(x_host.nbytes), "host_bytes_out": int(sum(o.nbytes for o in outs)),
                           "what": "set_tensor(fp32, caller's pageable buffer) + invoke + get_tensor(fp32) per step"}
+    # the reference's get_all_tensor mode beside the headline: every tensor of the graph written
+    mk = None
+    if not args.keep_all:
+        mk = module(device=0)
+        mk.set_option("keep_all_tensors", 1)
+        mk.load(g)
+        mk.set_tensor(g.input_op().name, g.input_op().data.astype(np.float32))
+        for _ in range(max(args.warmup, 1)):
+            mk.invoke()
+        mk.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            mk.invoke()
+        mk.sync()
+        ms_keep = (time.perf_counter() - t0) * 1e3 / args.steps
+        out["keep_all"] = {"ms_per_step": round(ms_keep, 4), "images_per_s": round(batch / (ms_keep / 1e3), 1),
+                           "what": "every tensor of the graph written, as the reference's get_all_tensor mode needs"}
+    out["parity_checked"] = False
     if not args.no_cpu_baseline:
-        sample = {"cfg1": 64, "cfg2": 16, "cfg3": 32, "cfg4": 64, "cfg5": 2}[args.config]
-        out["cpu_baseline"] = cpu_baseline(graph_fn, sample)
+        sample = min(batch, {"cfg1": 64, "cfg2": 16, "cfg3": 32, "cfg4": 64, "cfg5": 2}[args.config])
+        want = {}
+        out["cpu_baseline"] = cpu_baseline(graph_fn, sample, keep_results=want)
+        # parity, outside the timed region: the outputs of the timed module, and every tensor of the
+        # keep-all module, against the oracle on the first `sample` images (ops are independent across
+        # the batch, and the generators give image i the same data whatever the batch)
+        guards = want.pop("__guards__")
+        full = graph_fn(batch=sample) if sample != batch else g
+        same_input = np.array_equal(full.input_op().data, g.input_op().data[:sample])
+        outputs_ok = same_input and all(
+            np.array_equal(m.get_tensor_i8(name)[:sample], want[name]) for name in g.outputs)
+        src = mk if mk is not None else m
+        exact = sum(1 for op in g.ops
+                    if np.array_equal(src.get_tensor_i8(op.name)[:sample], want[op.name].reshape((sample,) + tuple(op.shape[1:]))))
+        out["parity_checked"] = bool(outputs_ok)
+        out["parity"] = {"outputs_equal_oracle": bool(outputs_ok), "layers_exact": exact, "layers_total": len(g.ops),
+                         "images_checked": sample,
+                         "fp32_guard_held": bool(max(guards.values()) < (1 << 24)) if guards else None}
+    if mk is not None:
+        mk.close()
     m.close()
     print(json.dumps(out))
 

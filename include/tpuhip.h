@@ -203,6 +203,13 @@ int tpuhip_conv2d_can_fuse_table(const tpuhip_conv_weights *w);
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,
                       const int8_t *filter_nk, const int32_t *bias, int32_t multiplier,
                       int32_t rshift, tpuhip_conv_weights **out);
+/* FullyConnectedOpKernel::invoke (core/fullyconnected.cpp:44-91) for weights packed by
+ * tpuhip_fc_prepack.  Matrices of at most 256 rows run a split-K kernel: K is divided over
+ * workgroups, whose 32x32 int32 partial sums meet in a scratch buffer in device memory that the
+ * library allocates with the context's first such call (and grows when a larger layer comes);
+ * the last workgroup to arrive at a block adds them up and requantises.  Larger matrices take the
+ * conv path.  Same result as tpuhip_conv2d_i8 on the same weights. */
+int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
 
 /* ---- EltwiseAdd ---------------------------------------------------------- */
 

@@ -329,6 +329,45 @@ def test_outputs_only_mode_skips_fused_conv_results_and_keeps_the_rest_exact():
     m.close()
 
 
+def test_benchmark_configuration_full_size_against_the_oracle():
+    """exactly what bench.py times by default: cfg3 at batch 32, the recorded conv tile variants,
+    outputs-only mode -- every tensor that is written, and fc1000, must equal the oracle's"""
+    import json
+    import os
+    import bench
+    g = graphs.cfg3_resnet50()
+    tiles = json.load(open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                                        bench.RECORDED_TILES["cfg3"])))
+    lib = capi.bind()
+    names = []
+    while lib.tpuhip_conv2d_tile_name(len(names)):
+        names.append(lib.tpuhip_conv2d_tile_name(len(names)).decode())
+    for name, algo in tiles.items():
+        g.by_name[name].attrs["algo"] = 16 + names.index(algo)
+    want = oracle_graph.run(g)
+    m = module()
+    m.set_option("keep_all_tensors", 0)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32))
+    m.invoke()
+    kern = dict(m.kernels())
+    for name, algo in tiles.items():
+        assert kern[name] == algo or kern[name].startswith("with "), (name, kern[name], algo)
+    written = skipped = 0
+    for op in g.ops:
+        try:
+            got = m.get_tensor_i8(op.name)
+        except capi.TpuHipError as e:
+            assert "never written" in str(e)
+            skipped += 1
+            continue
+        assert np.array_equal(got, want[op.name].reshape(op.shape)), op.name
+        written += 1
+    assert skipped == 16 and written == len(g.ops) - 16
+    assert np.array_equal(m.get_tensor_i8("fc1000"), want["fc1000"])
+    m.close()
+
+
 def test_module_errors_are_reported():
     g = graphs.cfg1_single_conv()
     m = module()

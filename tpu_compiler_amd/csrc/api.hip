@@ -69,7 +69,10 @@ int tpuhip_ctx_destroy(tpuhip_ctx *ctx) {
   if (ctx->owns_stream && ctx->stream) {
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipStreamDestroy(ctx->stream);
+  } else if (ctx->stream) {
+    (void)hipStreamSynchronize(ctx->stream);
   }
+  if (ctx->workspace) (void)hipFree(ctx->workspace);
   delete ctx;
   return TPUHIP_OK;
 }

@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <string>
 #include <type_traits>
 #include <vector>
 
@@ -2268,6 +2269,74 @@ conv_mfma_splitk_kernel(ConvArgs a) {
 
 
 // ---------------------------------------------------------------------------
+// FullyConnected with few rows (the classifier of a network: 32 x 2048 -> 1000): one 32x32
+// block of outputs per 32 output channels, and a K far too long for one wave per block to be
+// anything but a chain of dependent loads.  So K is split over workgroups of ONE wave: wave
+// (tile, split) multiplies its K range from operands fetched straight in MFMA layout (filter
+// stored fragment by fragment, as for conv_mfma_reg_kernel), leaves its 32x32 int32 partial
+// sum in a scratch buffer in device memory and counts itself in at the tile's arrival
+// counter; the wave that arrives last adds the partial sums and the bias, requantises and
+// stores (ReLU before the requantisation, one multiplier / shift for the tensor:
+// core/fullyconnected.cpp:64-87), and puts the counter back to zero for the next launch.
+// No wave waits for another.  scratch: 1024 counters, then [tile][split][lane][16] int32.
+// ---------------------------------------------------------------------------
+constexpr int kFcMaxTiles = 1024;                              // arrival counters
+constexpr size_t kFcCounterBytes = kFcMaxTiles * sizeof(int32_t);
+constexpr size_t kFcPartialBytes = 64 * 16 * sizeof(int32_t);  // one wave's partial sum
+
+template <bool FAST>
+__global__ __launch_bounds__(64) void fc_splitk_kernel(ConvArgs a, int32_t *scratch, int splits, int steps_per_split) {
+  const int lane = threadIdx.x;
+  const int split = (int)blockIdx.x % splits;
+  const int tile = (int)blockIdx.x / splits;        // pixel block * output-channel blocks + output-channel block
+  const int ob = tile % a.n_oc_tiles, pb = tile / a.n_oc_tiles;
+  const int nsteps = a.kp / 64;
+  const int s0 = split * steps_per_split, s1 = min(nsteps, s0 + steps_per_split);
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+  const int frow = lane & 31, fk = lane >> 5;
+  const int row = pb * 32 + frow;                   // "pixel" = row of the input matrix
+  const uint32_t xoff = row < a.npix ? (uint32_t)(row * a.x_cs + fk * 16) : kOobOffset;
+  const uint32_t woff = (uint32_t)(ob * nsteps) * 2048u + (uint32_t)lane * 16u;
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  for (int s = s0; s < s1; ++s) {
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const v4i af = (v4i)__builtin_amdgcn_raw_buffer_load_b128(wrsrc, woff, s * 2048 + kk * 1024, 0);
+      const v4i bf = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff, s * 64 + kk * 32, 0);
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc, 0, 0, 0);
+    }
+  }
+  int32_t *counters = scratch;
+  v4i *parts = reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(scratch) + kFcCounterBytes);
+  v4i *mine = parts + ((size_t)(tile * splits + split) * 64 + lane) * 4;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) mine[q] = v4i{acc[q * 4 + 0], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+  __threadfence();                                  // the partial sum is visible before the count
+  int arrived = 0;
+  if (lane == 0) arrived = atomicAdd(&counters[tile], 1);
+  arrived = __builtin_amdgcn_readfirstlane(arrived);
+  if (arrived != splits - 1) return;
+  __threadfence();                                  // ... and read only after the last count
+  const int oc = ob * 32 + fk * 16;                 // this lane's 16 channels
+  v16i sum[1];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    v4i t = *reinterpret_cast<const v4i *>(a.bias + oc + q * 4);
+    for (int sp = 0; sp < splits; ++sp) t += parts[((size_t)(tile * splits + sp) * 64 + lane) * 4 + q];
+    sum[0][q * 4 + 0] = t[0]; sum[0][q * 4 + 1] = t[1]; sum[0][q * 4 + 2] = t[2]; sum[0][q * 4 + 3] = t[3];
+  }
+  if (lane == 0) counters[tile] = 0;                // ready for the next launch
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+  if (oc < a.ocw)
+    epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, row, 32, nullptr, out);
+}
+
+// ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
 namespace {
@@ -3326,6 +3395,62 @@ int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
   return run_conv(ctx, w, x, y_a, p);
 }
 
+// how the split-K kernel divides a packed FullyConnected: tiles, splits, K steps per split
+struct FcPlan {
+  int tiles, splits, steps_per_split;
+  size_t bytes;   // scratch the launch needs
+};
+
+static bool fc_splitk_plan(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, FcPlan *p) {
+  const tpuhip_conv_desc &d = w->d;
+  // a packed FullyConnected (1x1 "image", bias before the ReLU) in the fragment order of the
+  // 32x32 LDS-free tile, which is how tpuhip_fc_prepack packs matrices of few rows
+  if (w->algo != ALGO_MFMA || !d.relu_first || d.ih != 1 || d.iw != 1 || w->split_oc ||
+      std::string(kTiles[w->tile].name) != "mfma_reg_32x32")
+    return false;
+  const int n_pb = (d.n + 31) / 32, n_ob = w->ocp / 32, nsteps = w->kp / 64;
+  p->tiles = n_pb * n_ob;
+  if (p->tiles > kFcMaxTiles) return false;
+  // about one wave per SIMD of the chip, at least two K steps each
+  const int want = std::max(1, ctx->num_cu * 4 / p->tiles);
+  p->splits = std::max(1, std::min(want, nsteps / 2));
+  p->steps_per_split = (nsteps + p->splits - 1) / p->splits;
+  p->splits = (nsteps + p->steps_per_split - 1) / p->steps_per_split;
+  p->bytes = kFcCounterBytes + (size_t)p->tiles * p->splits * kFcPartialBytes;
+  return true;
+}
+
+static int run_fc_splitk(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y, void *scratch_ptr,
+                         const FcPlan &p) {
+  ConvArgs a;
+  fill_args(ctx, w, x, y, &a);
+  a.n_oc_tiles = w->ocp / 32;
+  const dim3 grid((unsigned)(p.tiles * p.splits)), block(64);
+  if (w->fast) launch(ctx, fc_splitk_kernel<true>, grid, block, a, (int32_t *)scratch_ptr, p.splits, p.steps_per_split);
+  else launch(ctx, fc_splitk_kernel<false>, grid, block, a, (int32_t *)scratch_ptr, p.splits, p.steps_per_split);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
+int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
+  TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_fc_i8: NULL argument");
+  FcPlan p;
+  if (!fc_splitk_plan(ctx, w, &p)) return run_conv(ctx, w, x, y, PostOps{});   // many rows: the conv path
+  if (ctx->workspace_bytes < p.bytes) {
+    TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+    TPUHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->workspace) TPUHIP_CHECK_HIP(hipFree(ctx->workspace));
+    ctx->workspace = nullptr;
+    ctx->workspace_bytes = 0;
+    TPUHIP_CHECK_HIP(hipMalloc(&ctx->workspace, p.bytes));
+    ctx->workspace_bytes = p.bytes;
+    // the counters start at zero (and every launch leaves them at zero); this first use of a
+    // context cannot be part of a captured graph anyway, it allocates
+    TPUHIP_CHECK_HIP(hipMemsetAsync(ctx->workspace, 0, kFcCounterBytes, ctx->stream));
+  }
+  return run_fc_splitk(ctx, w, x, y, ctx->workspace, p);
+}
+
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,
                       const int8_t *filter_nk, const int32_t *bias, int32_t multiplier,
                       int32_t rshift, tpuhip_conv_weights **out) {
@@ -3338,6 +3463,12 @@ int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, 
   d.with_bias = bias != nullptr;
   d.x_cs = x_cs; d.y_cs = y_cs;
   d.relu_first = 1;
+  // few rows: packed fragment by fragment for the split-K kernel of tpuhip_fc_i8 (the same
+  // bytes serve the LDS-free 32x32 conv tile, so tpuhip_conv2d_i8 runs them too)
+  if (m <= 256 && (n + 31) / 32 * ((m + 31) / 32) <= kFcMaxTiles) {
+    for (int t = 0; t < kNumTiles; ++t)
+      if (std::string(kTiles[t].name) == "mfma_reg_32x32") d.algo = 16 + t;
+  }
   std::vector<int32_t> mult((size_t)n, multiplier), rs((size_t)n, rshift);
   return tpuhip_conv2d_prepack(ctx, &d, filter_nk, bias, mult.data(), rs.data(), out);
 }

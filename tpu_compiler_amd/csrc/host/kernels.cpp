@@ -597,7 +597,7 @@ const char *FullyConnectedOpKernel::algo_name() const {
 }
 
 void FullyConnectedOpKernel::invoke() {
-  ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+  ck(tpuhip_fc_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
 }
 
 // ---------------------------------------------------------------------------
