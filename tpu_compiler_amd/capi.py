@@ -100,6 +100,7 @@ PROTOTYPES = {
                                                                    C.c_int32, C.c_int32,
                                                                    c_void_pp]),
     "tpuhip_fc_i8": (C.c_int, [C.c_void_p] * 4),
+    "tpuhip_fc_i8_noalloc": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_eltwise_add_i8": (C.c_int, [C.c_void_p, c_void_pp, C.c_int, C.c_void_p, C.c_int,
                                         C.c_int, C.c_void_p, C.c_size_t]),
     "tpuhip_pool_max_i8": (C.c_int, [C.c_void_p, C.POINTER(PoolDesc), C.c_void_p, C.c_void_p]),
@@ -439,8 +440,9 @@ class Context:
             None if b is None else b.ctypes.data, int(mult), int(rshift), C.byref(w)))
         return w.value
 
-    def fc(self, w, x, y):
-        self._ck(self.lib.tpuhip_fc_i8(self.h, w, x.ptr, y.ptr))
+    def fc(self, w, x, y, noalloc=False):
+        f = self.lib.tpuhip_fc_i8_noalloc if noalloc else self.lib.tpuhip_fc_i8
+        self._ck(f(self.h, w, x.ptr, y.ptr))
 
     def conv_weights_destroy(self, w):
         self._ck(self.lib.tpuhip_conv2d_weights_destroy(self.h, w))

@@ -39,6 +39,7 @@ static int ctx_create(int device, void *stream, bool own, tpuhip_ctx **out) {
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return set_error(TPUHIP_ERR_UNSUPPORTED, "tpuhip is built for gfx950 only, device %d is %s",
                      device, prop.gcnArchName);
+  if (int rc = tpuhip_static_scratch_init(device)) return rc;
   tpuhip_ctx *c = new tpuhip_ctx();
   c->device = device;
   c->num_cu = prop.multiProcessorCount;

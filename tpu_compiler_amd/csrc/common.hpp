@@ -27,6 +27,10 @@ struct tpuhip_ctx {
   size_t workspace_bytes = 0;
 };
 
+// conv.hip: looks up this device's copy of the library's static scratch array (the one the
+// allocation-free entry point works in); called once per context with the device current
+extern "C" int tpuhip_static_scratch_init(int device);
+
 namespace tpuhip {
 
 int set_error(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -2336,6 +2336,13 @@ __global__ __launch_bounds__(64) void fc_splitk_kernel(ConvArgs a, int32_t *scra
     epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, row, 32, nullptr, out);
 }
 
+// The scratch of the allocation-free entry point: one array per device the library is loaded
+// on, zero at load (the counters must start at zero; every launch leaves them at zero).
+constexpr size_t kFcStaticPartials = 1024;          // (tile, split) pairs: 4 MiB of partial sums
+constexpr size_t kFcStaticBytes = kFcCounterBytes + kFcStaticPartials * kFcPartialBytes;
+static __device__ __align__(256) unsigned char scratch[kFcStaticBytes];
+static void *g_static_scratch[64];                  // device address of `scratch`, per device
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -3432,6 +3439,15 @@ static int run_fc_splitk(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
   return TPUHIP_OK;
 }
 
+int tpuhip_static_scratch_init(int device) {
+  TPUHIP_REQUIRE(device >= 0 && device < 64, "tpuhip: device index %d out of range", device);
+  if (g_static_scratch[device]) return TPUHIP_OK;
+  void *ptr = nullptr;
+  TPUHIP_CHECK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  g_static_scratch[device] = ptr;
+  return TPUHIP_OK;
+}
+
 int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_fc_i8: NULL argument");
   FcPlan p;
@@ -3449,6 +3465,20 @@ int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, v
     TPUHIP_CHECK_HIP(hipMemsetAsync(ctx->workspace, 0, kFcCounterBytes, ctx->stream));
   }
   return run_fc_splitk(ctx, w, x, y, ctx->workspace, p);
+}
+
+int tpuhip_fc_i8_noalloc(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
+  TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_fc_i8_noalloc: NULL argument");
+  FcPlan p;
+  TPUHIP_REQUIRE(fc_splitk_plan(ctx, w, &p),
+                 "tpuhip_fc_i8_noalloc: not a FullyConnected packed by tpuhip_fc_prepack for the split-K kernel "
+                 "(at most 256 rows, at most %d blocks of 32 x 32 outputs)", kFcMaxTiles);
+  TPUHIP_REQUIRE(p.bytes <= kFcStaticBytes,
+                 "tpuhip_fc_i8_noalloc: the layer needs %zu bytes of scratch, the static buffer holds %zu "
+                 "(%zu partial sums of 32 x 32 outputs)", p.bytes, kFcStaticBytes, kFcStaticPartials);
+  void *ptr = ctx->device >= 0 && ctx->device < 64 ? g_static_scratch[ctx->device] : nullptr;
+  TPUHIP_REQUIRE(ptr, "tpuhip_fc_i8_noalloc: the static scratch of device %d was not set up", ctx->device);
+  return run_fc_splitk(ctx, w, x, y, ptr, p);
 }
 
 int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, int do_relu,
