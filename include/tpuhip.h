@@ -207,12 +207,12 @@ int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, 
  * tpuhip_fc_prepack.  Matrices of at most 256 rows run a split-K kernel: K is divided over
  * workgroups, whose 32x32 int32 partial sums meet in a scratch buffer in device memory that the
  * library allocates with the context's first such call (and grows when a larger layer comes);
- * the last workgroup to arrive at a block adds them up and requantises.  Larger matrices take the
+ * a second launch adds them up and requantises.  Larger matrices take the
  * conv path.  Same result as tpuhip_conv2d_i8 on the same weights. */
 int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
 /* The same split-K FullyConnected for callers that cannot allocate (code under HIP graph capture,
  * serving loops, harnesses that forbid hipMalloc): it has no counterpart in the reference.  The
- * partial sums go to a static array in device memory (4 MiB + 4 KiB, one per GPU the library runs
+ * partial sums go to a static array in device memory (4 MiB, one per GPU the library runs
  * on, held until the process ends) whose address is looked up when a context is created; the call
  * itself allocates and frees nothing.  Layers that need more than 1024 partial sums of 32x32 outputs
  * (rows/32 x channels/32 x K splits), or that tpuhip_fc_prepack did not pack for the split-K kernel,

@@ -37,7 +37,7 @@ def test_fc_noalloc_equals_fc_on_two_calls_in_a_row():
         assert np.array_equal(a, want), "the workspace path differs from the oracle"
         assert np.array_equal(b, a), "the static-scratch path differs from the workspace path"
         assert np.array_equal(ctx.raw(y_static), ctx.raw(y_ws))             # pad channels too
-        # once more on the same buffers: the arrival counters were left at zero
+        # once more on the same buffers
         ctx._ck(ctx.lib.tpuhip_memset(ctx.h, y_static.ptr, 0x55, y_static.nbytes))
         ctx.fc(wh, xt, y_static, noalloc=True)
         assert np.array_equal(ctx.raw(y_static), ctx.raw(y_ws))
@@ -50,7 +50,7 @@ def test_fc_noalloc_equals_fc_on_two_calls_in_a_row():
 def test_fc_noalloc_refuses_what_does_not_fit():
     ctx = capi.Context(0)
     rng = np.random.default_rng(5)
-    # 256 rows x 8192 channels: 8 x 256 = 2048 blocks of 32 x 32 outputs, more than the scratch has counters for
+    # 256 rows x 8192 channels: 8 x 256 = 2048 blocks of 32 x 32 outputs, more than the split-K kernels take
     xt, wh, want = _fc_case(ctx, rng, 256, 128, 8192, False)
     yt = ctx.tensor((256, 8192, 1, 1))
     with pytest.raises(capi.TpuHipError, match="blocks of 32 x 32"):

@@ -21,8 +21,7 @@ struct tpuhip_ctx {
   // when set, every kernel launch carries these events: they bracket the dispatch
   // itself (begin / end of execution), not the gaps around it
   hipEvent_t prof_start = nullptr, prof_stop = nullptr;
-  // device memory kernels use beyond their operands (split-K partial sums and arrival
-  // counters): allocated on first need, grown when a larger layer comes, freed with the context
+  // device memory kernels use beyond their operands (split-K partial sums): allocated on first need, grown when a larger layer comes, freed with the context
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
 };

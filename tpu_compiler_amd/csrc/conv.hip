@@ -2273,19 +2273,17 @@ conv_mfma_splitk_kernel(ConvArgs a) {
 // block of outputs per 32 output channels, and a K far too long for one wave per block to be
 // anything but a chain of dependent loads.  So K is split over workgroups of ONE wave: wave
 // (tile, split) multiplies its K range from operands fetched straight in MFMA layout (filter
-// stored fragment by fragment, as for conv_mfma_reg_kernel), leaves its 32x32 int32 partial
-// sum in a scratch buffer in device memory and counts itself in at the tile's arrival
-// counter; the wave that arrives last adds the partial sums and the bias, requantises and
-// stores (ReLU before the requantisation, one multiplier / shift for the tensor:
-// core/fullyconnected.cpp:64-87), and puts the counter back to zero for the next launch.
-// No wave waits for another.  scratch: 1024 counters, then [tile][split][lane][16] int32.
+// stored fragment by fragment, as for conv_mfma_reg_kernel) and leaves its 32x32 int32
+// partial sum in a scratch buffer in device memory, [tile][split][lane][16]; a second launch
+// -- the kernel boundary is what makes the partial sums of all XCDs visible, no fence or
+// atomic is involved and no wave waits for another -- adds them and the bias, requantises
+// and stores (ReLU before the requantisation, one multiplier / shift for the tensor:
+// core/fullyconnected.cpp:64-87).
 // ---------------------------------------------------------------------------
-constexpr int kFcMaxTiles = 1024;                              // arrival counters
-constexpr size_t kFcCounterBytes = kFcMaxTiles * sizeof(int32_t);
+constexpr int kFcMaxTiles = 1024;                              // blocks of 32 x 32 outputs
 constexpr size_t kFcPartialBytes = 64 * 16 * sizeof(int32_t);  // one wave's partial sum
 
-template <bool FAST>
-__global__ __launch_bounds__(64) void fc_splitk_kernel(ConvArgs a, int32_t *scratch, int splits, int steps_per_split) {
+__global__ __launch_bounds__(64) void fc_partial_kernel(ConvArgs a, v4i *parts, int splits, int steps_per_split) {
   const int lane = threadIdx.x;
   const int split = (int)blockIdx.x % splits;
   const int tile = (int)blockIdx.x / splits;        // pixel block * output-channel blocks + output-channel block
@@ -2311,35 +2309,52 @@ __global__ __launch_bounds__(64) void fc_splitk_kernel(ConvArgs a, int32_t *scra
       acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc, 0, 0, 0);
     }
   }
-  int32_t *counters = scratch;
-  v4i *parts = reinterpret_cast<v4i *>(reinterpret_cast<int8_t *>(scratch) + kFcCounterBytes);
   v4i *mine = parts + ((size_t)(tile * splits + split) * 64 + lane) * 4;
 #pragma unroll
   for (int q = 0; q < 4; ++q) mine[q] = v4i{acc[q * 4 + 0], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
-  __threadfence();                                  // the partial sum is visible before the count
-  int arrived = 0;
-  if (lane == 0) arrived = atomicAdd(&counters[tile], 1);
-  arrived = __builtin_amdgcn_readfirstlane(arrived);
-  if (arrived != splits - 1) return;
-  __threadfence();                                  // ... and read only after the last count
+}
+
+// one workgroup per 32x32 block of outputs: wave q adds up dwords 4q .. 4q+3 of every lane's 16
+// partial sums (eight loads in flight per lane), wave 0 collects the four quarters from LDS and
+// runs the epilogue
+template <bool FAST>
+__global__ __launch_bounds__(256) void fc_reduce_kernel(ConvArgs a, const v4i *parts, int splits) {
+  __shared__ v4i quarter[4][64];
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int tile = (int)blockIdx.x;
+  const int ob = tile % a.n_oc_tiles, pb = tile / a.n_oc_tiles;
+  const int frow = lane & 31, fk = lane >> 5;
   const int oc = ob * 32 + fk * 16;                 // this lane's 16 channels
+  const v4i *src = parts + ((size_t)tile * splits * 64 + lane) * 4 + q;
+  v4i t = *reinterpret_cast<const v4i *>(a.bias + oc + q * 4);
+  int sp = 0;
+  for (; sp + 8 <= splits; sp += 8) {
+    v4i v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(sp + u) * 256];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t += v[u];
+  }
+  for (; sp < splits; ++sp) t += src[(size_t)sp * 256];
+  quarter[q][lane] = t;
+  __syncthreads();
+  if (q != 0) return;
   v16i sum[1];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    v4i t = *reinterpret_cast<const v4i *>(a.bias + oc + q * 4);
-    for (int sp = 0; sp < splits; ++sp) t += parts[((size_t)(tile * splits + sp) * 64 + lane) * 4 + q];
-    sum[0][q * 4 + 0] = t[0]; sum[0][q * 4 + 1] = t[1]; sum[0][q * 4 + 2] = t[2]; sum[0][q * 4 + 3] = t[3];
+  for (int k = 0; k < 4; ++k) {
+    const v4i r = quarter[k][lane];
+    sum[0][k * 4 + 0] = r[0]; sum[0][k * 4 + 1] = r[1]; sum[0][k * 4 + 2] = r[2]; sum[0][k * 4 + 3] = r[3];
   }
-  if (lane == 0) counters[tile] = 0;                // ready for the next launch
   const OutRoute out{a.y, a.y_cs, a.lo, 0};
   if (oc < a.ocw)
-    epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, row, 32, nullptr, out);
+    epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pb * 32 + frow, 32, nullptr, out);
 }
 
 // The scratch of the allocation-free entry point: one array per device the library is loaded
-// on, zero at load (the counters must start at zero; every launch leaves them at zero).
+// on.  Nothing in it has to start at zero: every partial sum the second launch reads was
+// written by the first.
 constexpr size_t kFcStaticPartials = 1024;          // (tile, split) pairs: 4 MiB of partial sums
-constexpr size_t kFcStaticBytes = kFcCounterBytes + kFcStaticPartials * kFcPartialBytes;
+constexpr size_t kFcStaticBytes = kFcStaticPartials * kFcPartialBytes;
 static __device__ __align__(256) unsigned char scratch[kFcStaticBytes];
 static void *g_static_scratch[64];                  // device address of `scratch`, per device
 
@@ -3418,12 +3433,12 @@ static bool fc_splitk_plan(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, 
   const int n_pb = (d.n + 31) / 32, n_ob = w->ocp / 32, nsteps = w->kp / 64;
   p->tiles = n_pb * n_ob;
   if (p->tiles > kFcMaxTiles) return false;
-  // about one wave per SIMD of the chip, at least two K steps each
-  const int want = std::max(1, ctx->num_cu * 4 / p->tiles);
+  // about two waves per CU of the chip, at least two K steps each
+  const int want = std::max(1, ctx->num_cu * 2 / p->tiles);
   p->splits = std::max(1, std::min(want, nsteps / 2));
   p->steps_per_split = (nsteps + p->splits - 1) / p->splits;
   p->splits = (nsteps + p->steps_per_split - 1) / p->steps_per_split;
-  p->bytes = kFcCounterBytes + (size_t)p->tiles * p->splits * kFcPartialBytes;
+  p->bytes = (size_t)p->tiles * p->splits * kFcPartialBytes;
   return true;
 }
 
@@ -3432,9 +3447,21 @@ static int run_fc_splitk(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
   ConvArgs a;
   fill_args(ctx, w, x, y, &a);
   a.n_oc_tiles = w->ocp / 32;
-  const dim3 grid((unsigned)(p.tiles * p.splits)), block(64);
-  if (w->fast) launch(ctx, fc_splitk_kernel<true>, grid, block, a, (int32_t *)scratch_ptr, p.splits, p.steps_per_split);
-  else launch(ctx, fc_splitk_kernel<false>, grid, block, a, (int32_t *)scratch_ptr, p.splits, p.steps_per_split);
+  // with per-kernel profiling events set, the pair brackets both launches: begin of the first,
+  // end of the second
+  const dim3 grid1((unsigned)(p.tiles * p.splits)), grid2((unsigned)p.tiles);
+  v4i *parts = (v4i *)scratch_ptr;
+  if (ctx->prof_start)
+    hipExtLaunchKernelGGL(fc_partial_kernel, grid1, dim3(64), 0, ctx->stream, ctx->prof_start, nullptr, 0, a, parts,
+                          p.splits, p.steps_per_split);
+  else
+    hipLaunchKernelGGL(fc_partial_kernel, grid1, dim3(64), 0, ctx->stream, a, parts, p.splits, p.steps_per_split);
+  auto reduce = w->fast ? fc_reduce_kernel<true> : fc_reduce_kernel<false>;
+  if (ctx->prof_stop)
+    hipExtLaunchKernelGGL(reduce, grid2, dim3(256), 0, ctx->stream, nullptr, ctx->prof_stop, 0, a, (const v4i *)parts,
+                          p.splits);
+  else
+    hipLaunchKernelGGL(reduce, grid2, dim3(256), 0, ctx->stream, a, (const v4i *)parts, p.splits);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
@@ -3460,9 +3487,6 @@ int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, v
     ctx->workspace_bytes = 0;
     TPUHIP_CHECK_HIP(hipMalloc(&ctx->workspace, p.bytes));
     ctx->workspace_bytes = p.bytes;
-    // the counters start at zero (and every launch leaves them at zero); this first use of a
-    // context cannot be part of a captured graph anyway, it allocates
-    TPUHIP_CHECK_HIP(hipMemsetAsync(ctx->workspace, 0, kFcCounterBytes, ctx->stream));
   }
   return run_fc_splitk(ctx, w, x, y, ctx->workspace, p);
 }
