@@ -250,7 +250,11 @@ def main():
     roofline = None
     if dom:
         achieved = dom["ops"] / (dom["ms"] / 1e3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<%s>" % dom_name.replace("mfma_", ""),
+        family = next((k for pre, k in (("mfma_pw_", "conv_pw_kernel"), ("mfma_patch2_", "conv_patch2_kernel"),
+                                        ("mfma_patch_", "conv_patch_kernel"), ("mfma_reg_", "conv_mfma_reg_kernel"),
+                                        ("mfma_splitk_", "conv_mfma_splitk_kernel")) if dom_name.startswith(pre)),
+                      "conv_mfma_kernel")
+        roofline = {"bound": "mfma", "kernel": "%s [tile %s]" % (family, dom_name),
                     "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                     "frac": round(achieved / PEAK_INT8_TOPS, 4), "traffic": None,
                     "launches": dom["launches"],
