@@ -220,6 +220,29 @@ int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, v
  * there (two streams, two threads) race; calls on one stream do not. */
 int tpuhip_fc_i8_noalloc(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
 
+/* The batched and transposed forms of FullyConnectedOpKernel::invoke (core/fullyconnected.cpp:44-91,
+ * shapes by parseFullyConnectedParam, TPUOperationSupport.cpp:568-605): batch = batch_high * batch_low
+ * matmuls o_b[m][n] = x_b[m][k] * w_b[n][k]^T + bias_b[n].  With input_transpose the input's logical
+ * shape is [batch_high, m, batch_low, k], else [batch, m, k]; with output_transpose the result's is
+ * [batch_high, m, batch_low, n], else [batch, m, n].  ReLU, then the per-tensor qdm requantisation with
+ * (rshift[i], multiplier[i]) where i = (flat logical index of the RESULT) / (m*n), which is how the
+ * reference indexes after its output permute.  x and y are channels-last device tensors whose 4-d
+ * views (n, c, h, w; missing dims 1) and channel strides are given: the kernel maps logical indices to
+ * them, so no transposed copy is made.  The last logical dim of x must be k, of y n. */
+typedef struct tpuhip_fc_batched_desc {
+  int batch_high, batch_low, m, k, n;
+  int input_transpose, output_transpose, do_relu;
+  int x_c, x_h, x_w, x_cs; /* 4-d view of the input (its n follows from the size) */
+  int y_c, y_h, y_w, y_cs; /* 4-d view of the result */
+} tpuhip_fc_batched_desc;
+typedef struct tpuhip_fc_batched_weights tpuhip_fc_batched_weights;
+/* filter: [batch][n][k]; bias: [batch][n] or NULL; multiplier, rshift: [batch] */
+int tpuhip_fc_batched_prepack(tpuhip_ctx *ctx, const tpuhip_fc_batched_desc *desc, const int8_t *filter,
+                              const int32_t *bias, const int32_t *multiplier, const int32_t *rshift,
+                              tpuhip_fc_batched_weights **out);
+int tpuhip_fc_batched_destroy(tpuhip_ctx *ctx, tpuhip_fc_batched_weights *w);
+int tpuhip_fc_batched_i8(tpuhip_ctx *ctx, const tpuhip_fc_batched_weights *w, const void *x, void *y);
+
 /* ---- EltwiseAdd ---------------------------------------------------------- */
 
 /* Replaces EltwiseAddOpKernel::i8_invoke (core/eltwise.cpp:52-85):

@@ -249,12 +249,15 @@ public:
   ~FullyConnectedOpKernel() override;
   void invoke() override;
   int m = 0, k = 0, n = 0;
-  // "fc/<conv tile variant it runs as>" (the variant is timed on first use)
+  int batch_high = 1, batch_low = 1, batch = 1;   // parseFullyConnectedParam
+  bool ltrans = false, otrans = false;            // input_transpose, output_transpose
+  // "fc/<conv tile variant it runs as>" (the variant is timed on first use), or "fc/batched"
   const char *algo_name() const;
 
 private:
   mutable std::string algo_text;
-  tpuhip_conv_weights *packed = nullptr;
+  tpuhip_conv_weights *packed = nullptr;              // [m,k] x [n,k]: the MFMA path
+  tpuhip_fc_batched_weights *packed_batched = nullptr;  // every other form
   SyncedData input_data, output_data;
 };
 

@@ -253,6 +253,44 @@ void orc_fc_i8(const int8_t *x, const int8_t *w, const float *bias, const float 
   }
 }
 
+/* fullyconnected.cpp:44-91 with the batch loop and both transposes: x in the input's logical
+ * order ([batch_high][m][batch_low][k] under input_transpose, my_permute(0,2,1,3) at :53-57, else
+ * [batch][m][k]); one inner product per batch b = hb*batch_low + lb with filter block b and bias
+ * block b (:62-68); under output_transpose the [batch_high][batch_low][m][n] sums are permuted to
+ * [batch_high][m][batch_low][n] (:69-72); ReLU (:73-75); then element f of the RESULT AS IT LIES
+ * takes rshift / multiplier number f / (m*n) (:77-88) -- after an output permute that is not the
+ * matmul's own batch index. */
+void orc_fc_batched_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                       const float *multiplier, int8_t *y, int batch_high, int batch_low, int m,
+                       int k, int n, int ltrans, int otrans, int do_relu) {
+  const int batch = batch_high * batch_low;
+  const int64_t isz = (int64_t)m * n;
+  float *sum = (float *)malloc(sizeof(float) * (size_t)(batch * isz));
+#pragma omp parallel for collapse(2)
+  for (int b = 0; b < batch; ++b)
+    for (int i = 0; i < m; ++i) {
+      const int hb = b / batch_low, lb = b % batch_low;
+      const int8_t *xr = ltrans ? x + ((((int64_t)hb * m + i) * batch_low + lb) * k)
+                                : x + ((int64_t)b * m + i) * k;
+      for (int j = 0; j < n; ++j) {
+        const int8_t *wr = w + ((int64_t)b * n + j) * k;
+        int32_t s = 0;
+        for (int t = 0; t < k; ++t) s += (int32_t)xr[t] * (int32_t)wr[t];
+        if (bias) s += (int32_t)bias[(int64_t)b * n + j];
+        const int64_t at = otrans ? ((((int64_t)hb * m + i) * batch_low + lb) * n + j)
+                                  : (((int64_t)b * m + i) * n + j);
+        sum[at] = (float)s;
+      }
+    }
+  for (int64_t f = 0; f < batch * isz; ++f) {
+    float v = sum[f];
+    if (do_relu && !(v > 0)) v = 0;
+    const int i = (int)(f / isz);
+    y[f] = orc_apply_mult_rshift_sat8_f(v, orc_f2u32(rshift[i]), orc_f2u32(multiplier[i]), 1);
+  }
+  free(sum);
+}
+
 int64_t orc_fc_guard(const int8_t *x, const int8_t *w, const float *bias, int batch, int m, int k,
                      int n) {
   int64_t worst = 0;

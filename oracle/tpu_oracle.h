@@ -93,6 +93,9 @@ void orc_deconv2d_i8(const int8_t *x, const int8_t *w, const float *bias, const 
  * bias: batch*n or NULL, y: batch*m*n ---- */
 void orc_fc_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
                const float *multiplier, int8_t *y, int batch, int m, int k, int n, int do_relu);
+void orc_fc_batched_i8(const int8_t *x, const int8_t *w, const float *bias, const float *rshift,
+                       const float *multiplier, int8_t *y, int batch_high, int batch_low, int m,
+                       int k, int n, int ltrans, int otrans, int do_relu);
 int64_t orc_fc_guard(const int8_t *x, const int8_t *w, const float *bias, int batch, int m, int k,
                      int n);
 

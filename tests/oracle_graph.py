@@ -35,6 +35,21 @@ _MOVES = {"tpu.pad": ("pad_const", ["pads*"]), "tpu.crop": ("crop", ["crop_offse
           "tpu.pixelshuffle": ("depth_to_space", ["upscale_factor", "mode_dcr"])}
 
 
+def fc_params(a_s, b_s, o_s, ltrans, otrans):
+    """parseFullyConnectedParam (lib/Dialect/TPU/IR/TPUOperationSupport.cpp:568-605)"""
+    o_dim = len(o_s)
+    k, n = int(b_s[-1]), int(b_s[-2])
+    bl = bh = 1
+    if ltrans:
+        bl, m, bh = int(a_s[o_dim - 2]), int(a_s[o_dim - 3]), int(np.prod(a_s[:o_dim - 3], dtype=np.int64))
+    elif otrans:
+        bl, m, bh = int(o_s[o_dim - 2]), int(o_s[o_dim - 3]), int(np.prod(o_s[:o_dim - 3], dtype=np.int64))
+    else:
+        bl = int(np.prod(b_s[:-2], dtype=np.int64))
+        m = int(a_s[o_dim - 2]) if bl > 1 else int(np.prod(a_s[:o_dim - 1], dtype=np.int64))
+    return bh, bl, m, k, n
+
+
 def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=None):
     """Returns {name: int8 NCHW array}.  batch_slice selects images (ops are
     independent across the batch, which is also how the reference runs a batch:
@@ -67,17 +82,28 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             y = O.deconv2d_i8(ins[0], w, op.weights.get("bias"), op.weights["rshift"],
                               op.weights["multiplier"], d)
         elif t == "tpu.fully_connected":
-            x = ins[0].reshape(ins[0].shape[0], -1)
             w = op.weights["filter"].astype(np.int8)
-            y = O.fc_i8(x, w, op.weights.get("bias"), op.weights["rshift"],
-                        op.weights["multiplier"], 1, x.shape[0], x.shape[1], w.shape[0],
-                        bool(op.attrs.get("do_relu", 0)))[0]
-            if guards is not None:
-                guards[op.name] = O.fc_guard(x, w, op.weights.get("bias"), 1, x.shape[0],
-                                             x.shape[1], w.shape[0])
+            lt, ot = int(op.attrs.get("input_transpose", 0)), int(op.attrs.get("output_transpose", 0))
+            if w.ndim == 2 and len(op.shape) == 2 and not lt and not ot:
+                x = ins[0].reshape(ins[0].shape[0], -1)
+                y = O.fc_i8(x, w, op.weights.get("bias"), op.weights["rshift"],
+                            op.weights["multiplier"], 1, x.shape[0], x.shape[1], w.shape[0],
+                            bool(op.attrs.get("do_relu", 0)))[0]
+                if guards is not None:
+                    guards[op.name] = O.fc_guard(x, w, op.weights.get("bias"), 1, x.shape[0],
+                                                 x.shape[1], w.shape[0])
+            else:
+                bh, bl, m, k, n = fc_params(ins[0].shape, w.shape, op.shape, lt, ot)
+                y = O.fc_batched_i8(ins[0], w, op.weights.get("bias"), op.weights["rshift"],
+                                    op.weights["multiplier"], bh, bl, m, k, n, lt, ot,
+                                    bool(op.attrs.get("do_relu", 0))).reshape(op.shape)
+                if guards is not None:
+                    xb = ins[0].reshape(bh, m, bl, k).transpose(0, 2, 1, 3) if lt else ins[0]
+                    guards[op.name] = O.fc_guard(np.ascontiguousarray(xb), w, op.weights.get("bias"),
+                                                 bh * bl, m, k, n)
         elif t == "tpu.eltwise_add":
             y = O.eltwise_add_i8(ins, op.weights["multiplier"], op.weights["rshift"],
-                                 bool(op.attrs["do_relu"]))
+                                 bool(op.attrs.get("do_relu", 0)))
         elif t in _BINARY:
             def nchw(a):
                 return a.reshape(a.shape + (1,) * (4 - a.ndim))
@@ -151,7 +177,8 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             y = O.concat_i8(ins, int(op.attrs["axis"]), op.weights.get("rshift"),
                             op.weights.get("multiplier"), bool(op.attrs.get("do_relu", 0)))
         elif t == "tpu.reshape":
-            y = ins[0].reshape((ins[0].shape[0],) + tuple(op.shape[1:]))
+            full = ins[0].size == int(np.prod(op.shape))
+            y = ins[0].reshape(tuple(op.shape) if full else (ins[0].shape[0],) + tuple(op.shape[1:]))
         else:
             raise NotImplementedError(t)
         vals[op.name] = y

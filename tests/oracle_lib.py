@@ -71,6 +71,7 @@ def _load():
     lib.orc_bf16.restype = C.c_float
     lib.orc_bf16.argtypes = [C.c_float, C.c_int]
     lib.orc_fc_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p] + [C.c_int] * 5
+    lib.orc_fc_batched_i8.argtypes = [i8p, i8p, f32p, f32p, f32p, i8p] + [C.c_int] * 8
     lib.orc_fc_guard.restype = C.c_int64
     lib.orc_fc_guard.argtypes = [i8p, i8p, f32p] + [C.c_int] * 4
     lib.orc_eltwise_add_i8.argtypes = [C.POINTER(i8p), C.c_int, f32p, f32p, C.c_int, i8p,
@@ -191,6 +192,19 @@ def fc_i8(x, w, bias, rshift, multiplier, batch, m, k, n, do_relu):
     b, r, mu = _f32(bias), _f32(rshift), _f32(multiplier)
     lib.orc_fc_i8(_p(x, C.c_int8), _p(w, C.c_int8), _p(b, C.c_float), _p(r, C.c_float),
                   _p(mu, C.c_float), _p(y, C.c_int8), batch, m, k, n, int(do_relu))
+    return y
+
+
+def fc_batched_i8(x, w, bias, rshift, multiplier, batch_high, batch_low, m, k, n, ltrans, otrans, do_relu):
+    """x in the input's logical order; returns the result flat in ITS logical order"""
+    x, w = _i8(x), _i8(w)
+    batch = batch_high * batch_low
+    assert x.size == batch * m * k and w.size == batch * n * k
+    y = np.empty(batch * m * n, np.int8)
+    b, r, mu = _f32(bias), _f32(rshift), _f32(multiplier)
+    lib.orc_fc_batched_i8(_p(x, C.c_int8), _p(w, C.c_int8), _p(b, C.c_float), _p(r, C.c_float),
+                          _p(mu, C.c_float), _p(y, C.c_int8), batch_high, batch_low, m, k, n,
+                          int(ltrans), int(otrans), int(do_relu))
     return y
 
 

@@ -1015,6 +1015,42 @@ def _random_single_op_graph(it):
     return (g, kind)
 
 
+@pytest.mark.parametrize("x_shape,w_shape,y_shape,lt,ot", [
+    ((4, 3, 28), (4, 5, 28), (4, 3, 5), 0, 0),          # the batched form of TPUOperationSupport.cpp:566
+    ((4, 3, 28), (5, 28), (4, 3, 5), 0, 0),             # :567: one matmul with m = 12
+    ((2, 8, 3, 48), (6, 20, 48), (2, 3, 8, 20), 1, 0),  # input_transpose
+    ((2, 3, 8, 48), (6, 20, 48), (2, 8, 3, 20), 0, 1),  # output_transpose
+    ((2, 8, 3, 48), (2, 3, 20, 48), (2, 8, 3, 20), 1, 1),
+])
+def test_fully_connected_batched_and_transposed_graphs(x_shape, w_shape, y_shape, lt, ot):
+    """FullyConnectedOpKernel with a batch and with either transpose (core/fullyconnected.cpp:52-88),
+    through the module interpreter, against the oracle's restatement"""
+    rng = np.random.default_rng(sum(x_shape) + 10 * lt + 20 * ot)
+    f32 = lambda v: np.asarray(v, np.float32).reshape(-1)
+    g = graphs.Graph("fc_batched", 77)
+    x = rng.integers(-128, 128, x_shape).astype(np.int8)
+    g.add(graphs.Op("tpu.input", "input", [], x.shape)).data = x
+    batch = int(np.prod(w_shape[:-2]))
+    w = np.clip(np.rint(rng.normal(0, 25, w_shape)), -127, 127).astype(np.float32)
+    bias = rng.integers(-2000, 2000, (batch, w_shape[-2])).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, batch) * 128).astype(np.float32)
+    rsh = rng.integers(6, 11, batch).astype(np.float32)
+    g.add(graphs.Op("tpu.fully_connected", "y", ["input"], y_shape,
+                    dict(do_relu=1, input_transpose=lt, output_transpose=ot),
+                    dict(filter=w, bias=bias, rshift=rsh, multiplier=mult), "RSHIFT_AND_M_I32"))
+    g.outputs = ["y"]
+    want = oracle_graph.run(g)["y"]
+    m = module()
+    m.load(g)
+    m.set_tensor("input", x.astype(np.float32))
+    m.invoke()
+    got = m.get_tensor_i8("y")
+    assert dict(m.kernels())["y"] == "fc/batched"
+    assert np.array_equal(got.reshape(y_shape), want.reshape(y_shape))
+    assert len(np.unique(want)) > 8
+    m.close()
+
+
 def test_random_deconv_reduce_and_fc_graphs():
     ran = {}
     for it in range(240):

@@ -799,6 +799,60 @@ def test_fully_connected(ctx, m, k, n, relu):
     ctx.conv_weights_destroy(wh)
 
 
+def _view4(shape):
+    return tuple(shape) + (1,) * (4 - len(shape))
+
+
+@pytest.mark.parametrize("bh,bl,m,k,n,lt,ot,relu", [
+    (1, 4, 3, 28, 5, 0, 0, False),     # [4,3,28] x [4,5,28] -> [4,3,5] (TPUOperationSupport.cpp:566)
+    (1, 6, 17, 64, 33, 0, 0, True),
+    (2, 3, 8, 48, 20, 1, 0, True),     # input [2,8,3,48]
+    (2, 3, 8, 48, 20, 0, 1, False),    # result [2,8,3,20]
+    (3, 2, 5, 40, 7, 1, 1, True),
+    (1, 1, 12, 28, 5, 0, 0, False),    # [4,3,28] x [5,28] -> [4,3,5]: one matmul, rank-3 result
+])
+def test_fully_connected_batched_and_transposed(ctx, bh, bl, m, k, n, lt, ot, relu):
+    """core/fullyconnected.cpp:52-88 through tpuhip_fc_batched_i8: tensors lie channels-last on the
+    device in the 4-d views of their logical shapes, the kernel finds its operands through them"""
+    rng = np.random.default_rng(bh * 1000 + bl * 100 + m + k + n + lt * 7 + ot * 13)
+    batch = bh * bl
+    if bh == bl == 1:
+        x_shape, y_shape = (4, m // 4, k), (4, m // 4, n)
+    else:
+        x_shape = (bh, m, bl, k) if lt else ((bh, bl, m, k) if bh > 1 else (batch, m, k))
+        y_shape = (bh, m, bl, n) if ot else ((bh, bl, m, n) if bh > 1 else (batch, m, n))
+    x = rnd_i8(rng, x_shape)
+    w = rnd_w(rng, (batch, n, k), 20)
+    bias = rng.integers(-3000, 3000, (batch, n)).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, batch) * 128).astype(np.float32)
+    rsh = rng.integers(6, 11, batch).astype(np.float32)
+    want = O.fc_batched_i8(x, w, bias, rsh, mult, bh, bl, m, k, n, lt, ot, relu).reshape(y_shape)
+    xt = ctx.from_nchw(x.reshape(_view4(x_shape)))
+    yt = ctx.tensor(_view4(y_shape))
+    xv, yv = _view4(x_shape), _view4(y_shape)
+    d = capi.FcBatchedDesc(bh, bl, m, k, n, lt, ot, int(relu), xv[1], xv[2], xv[3], xt.cs,
+                           yv[1], yv[2], yv[3], yt.cs)
+    wh = ctx.fc_batched_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    ctx.fc_batched(wh, xt, yt)
+    got = ctx.to_nchw(yt).reshape(y_shape)
+    assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 8
+    ctx.fc_batched_destroy(wh)
+
+
+def test_fully_connected_batched_refuses_bad_descriptors(ctx):
+    ok = np.zeros(2, np.int32)
+    w = np.zeros((2, 4, 8), np.int8)
+    good = dict(batch_high=1, batch_low=2, m=3, k=8, n=4, input_transpose=0, output_transpose=0, do_relu=0,
+                x_c=3, x_h=8, x_w=1, x_cs=16, y_c=3, y_h=4, y_w=1, y_cs=16)
+    for bad, msg in ((dict(k=0), "positive"), (dict(x_h=7), "divide"), (dict(x_h=4, x_w=2), "last dim"),
+                     (dict(y_h=2, y_w=2), "last dim"), (dict(x_cs=2), "channel stride")):
+        with pytest.raises(capi.TpuHipError, match=msg):
+            ctx.fc_batched_prepack(capi.FcBatchedDesc(**dict(good, **bad)), w, None, ok, ok)
+    with pytest.raises(capi.TpuHipError, match="rshift"):
+        ctx.fc_batched_prepack(capi.FcBatchedDesc(**good), w, None, ok, np.array([3, 40], np.int32))
+
+
 @pytest.mark.parametrize("nin,relu,rs", [(2, True, 5), (2, False, 0), (3, False, 7), (1, True, 2),
                                          (8, True, 9)])
 def test_eltwise_add(ctx, nin, relu, rs):

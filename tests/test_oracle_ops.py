@@ -195,6 +195,35 @@ def test_fc_per_batch_requant_bias_before_relu():
     assert O.fc_guard(x, w, bias, batch, m, k, n) < (1 << 24)
 
 
+@pytest.mark.parametrize("ltrans,otrans", [(0, 0), (1, 0), (0, 1), (1, 1)])
+def test_fc_batched_and_transposed_vs_numpy_einsum(ltrans, otrans):
+    """core/fullyconnected.cpp:52-88: the permutes are numpy transposes, the matmuls an int64 einsum;
+    the requant pair of an element is picked by its position in the final layout (block f // (m*n)),
+    which differs from its matmul's batch index once the output is permuted"""
+    rng = np.random.default_rng(31 + 2 * ltrans + otrans)
+    bh, bl, m, k, n = 2, 3, 4, 24, 5
+    batch = bh * bl
+    x_l = rnd_i8(rng, (bh, m, bl, k) if ltrans else (batch, m, k))       # logical input
+    w = rnd_i8(rng, (batch, n, k))
+    bias = rng.integers(-3000, 3000, (batch, n)).astype(np.float32)
+    mult = (rng.integers(1 << 23, 1 << 24, batch) * 128).astype(np.float32)
+    rsh = rng.integers(5, 10, batch).astype(np.float32)
+    xb = x_l.transpose(0, 2, 1, 3).reshape(batch, m, k) if ltrans else x_l
+    sums = np.einsum("bmk,bnk->bmn", xb.astype(np.int64), w.astype(np.int64)) + bias.astype(np.int64)[:, None, :]
+    if otrans:
+        sums = sums.reshape(bh, bl, m, n).transpose(0, 2, 1, 3)
+    flat = sums.reshape(-1)
+    for relu in (0, 1):
+        y = O.fc_batched_i8(x_l, w, bias, rsh, mult, bh, bl, m, k, n, ltrans, otrans, relu)
+        for f, s in enumerate(flat):
+            s = max(int(s), 0) if relu else int(s)
+            i = f // (m * n)
+            assert y[f] == qdm_exact(s, int(mult[i]), int(rsh[i])), (f, relu)
+    if not ltrans and not otrans:
+        assert np.array_equal(O.fc_batched_i8(x_l, w, bias, rsh, mult, bh, bl, m, k, n, 0, 0, 1),
+                              O.fc_i8(x_l, w, bias, rsh, mult, batch, m, k, n, True).reshape(-1))
+
+
 def test_eltwise_add_closed_form():
     rng = np.random.default_rng(29)
     xs = [rnd_i8(rng, (2, 3, 4, 5)) for _ in range(3)]

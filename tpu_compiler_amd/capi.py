@@ -44,6 +44,12 @@ class MoveDesc(C.Structure):
  MOVE_REFLECTION_PAD) = range(12)
 
 
+class FcBatchedDesc(C.Structure):
+    _fields_ = [(k, C.c_int) for k in (
+        "batch_high", "batch_low", "m", "k", "n", "input_transpose", "output_transpose", "do_relu",
+        "x_c", "x_h", "x_w", "x_cs", "y_c", "y_h", "y_w", "y_cs")]
+
+
 class PoolDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "n", "c", "ih", "iw", "oh", "ow", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr",
@@ -101,6 +107,10 @@ PROTOTYPES = {
                                                                    c_void_pp]),
     "tpuhip_fc_i8": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_fc_i8_noalloc": (C.c_int, [C.c_void_p] * 4),
+    "tpuhip_fc_batched_prepack": (C.c_int, [C.c_void_p, C.POINTER(FcBatchedDesc)] + [C.c_void_p] * 4 +
+                                  [c_void_pp]),
+    "tpuhip_fc_batched_destroy": (C.c_int, [C.c_void_p] * 2),
+    "tpuhip_fc_batched_i8": (C.c_int, [C.c_void_p] * 4),
     "tpuhip_eltwise_add_i8": (C.c_int, [C.c_void_p, c_void_pp, C.c_int, C.c_void_p, C.c_int,
                                         C.c_int, C.c_void_p, C.c_size_t]),
     "tpuhip_pool_max_i8": (C.c_int, [C.c_void_p, C.POINTER(PoolDesc), C.c_void_p, C.c_void_p]),
@@ -443,6 +453,23 @@ class Context:
     def fc(self, w, x, y, noalloc=False):
         f = self.lib.tpuhip_fc_i8_noalloc if noalloc else self.lib.tpuhip_fc_i8
         self._ck(f(self.h, w, x.ptr, y.ptr))
+
+    def fc_batched_prepack(self, desc, filt, bias, mult, rshift):
+        filt = np.ascontiguousarray(filt, dtype=np.int8)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        mu = np.ascontiguousarray(mult, dtype=np.int32)
+        rs = np.ascontiguousarray(rshift, dtype=np.int32)
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_fc_batched_prepack(
+            self.h, C.byref(desc), filt.ctypes.data, None if b is None else b.ctypes.data,
+            mu.ctypes.data, rs.ctypes.data, C.byref(w)))
+        return w.value
+
+    def fc_batched(self, w, x, y):
+        self._ck(self.lib.tpuhip_fc_batched_i8(self.h, w, x.ptr, y.ptr))
+
+    def fc_batched_destroy(self, w):
+        self._ck(self.lib.tpuhip_fc_batched_destroy(self.h, w))
 
     def conv_weights_destroy(self, w):
         self._ck(self.lib.tpuhip_conv2d_weights_destroy(self.h, w))

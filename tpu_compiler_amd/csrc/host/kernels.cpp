@@ -549,8 +549,8 @@ FullyConnectedOpKernel::FullyConnectedOpKernel(OpDesc &op, value_map_t &valueMap
     : CPUOpKernel(op, valueMapping, weightMapping) {
   require_int8("FullyConnected");
   if (opdTensors.size() != 7) fail("FullyConnected '" + name + "': expected 7 operands");
-  if (op.attr("input_transpose", 0) != 0 || op.attr("output_transpose", 0) != 0)
-    fail("FullyConnected '" + name + "': transposed variants are not implemented");
+  ltrans = op.attr("input_transpose", 0) != 0;
+  otrans = op.attr("output_transpose", 0) != 0;
   input_data = opdTensors[0].act;
   output_data = resTensor;
   auto filter = opdTensors[1].weight;
@@ -559,45 +559,89 @@ FullyConnectedOpKernel::FullyConnectedOpKernel(OpDesc &op, value_map_t &valueMap
   auto multiplier_data = opdTensors[6].weight;
   if (!input_data || !filter || !rshift_data || !multiplier_data)
     fail("FullyConnected '" + name + "': operand missing");
-  // parseFullyConnectedParam (TPUOperationSupport.cpp:568-605), batch_low == batch_high == 1:
-  // m = product of the leading input dims, n = rows of the filter, k = its columns
-  n = output_data->c * output_data->h * output_data->w;
-  if (op.shape.size() != 2) fail("FullyConnected '" + name + "': result must be [m, n]");
-  m = (int)op.shape[0];
-  n = (int)op.shape[1];
-  if (filter->size() % (size_t)n) fail("FullyConnected '" + name + "': filter size mismatch");
-  k = (int)(filter->size() / (size_t)n);
-  if (input_data->size() != (size_t)m * k) fail("FullyConnected '" + name + "': input size mismatch");
-  if (input_data->h * input_data->w != 1)
-    fail("FullyConnected '" + name + "': input must be [m, k] (reshape first)");
+  // parseFullyConnectedParam (TPUOperationSupport.cpp:568-605): k and n are the last dims of the
+  // input and the result (the filter is [..., n, k]); the batch split comes from the input's shape
+  // under input_transpose, from the result's under output_transpose, else from the filter's
+  // leading dims -- here its element count over n*k, since weights carry no shape
+  const SyncedDataShape &o_s = op.shape;
+  auto it = valueMapping.shapes.find(op.operands[0]);
+  if (it == valueMapping.shapes.end()) fail("FullyConnected '" + name + "': input shape unknown");
+  const SyncedDataShape &a_s = it->second;
+  const size_t o_dim = o_s.size();
+  if (o_dim < 2 || a_s.empty()) fail("FullyConnected '" + name + "': result must have rank 2 or more");
+  n = (int)o_s.back();
+  // a rank-2 result is one [m,k] x [n,k] product whatever the input's rank ([m, c, 1, 1] is common):
+  // m = a_s[0] (:595-597 with o_dim == 2), k = what is left
+  const bool rank2 = o_dim == 2 && !ltrans && !otrans;
+  k = rank2 ? (int)(input_data->size() / (size_t)std::max<int64_t>(1, a_s[0])) : (int)a_s.back();
+  auto prod = [](const SyncedDataShape &s, size_t from, size_t to) {
+    int64_t p = 1;
+    for (size_t i = from; i < to; ++i) p *= s[i];
+    return p;
+  };
+  if (ltrans || otrans) {
+    const SyncedDataShape &s = ltrans ? a_s : o_s;
+    if (s.size() != o_dim || o_dim < 3) fail("FullyConnected '" + name + "': a transposed form needs rank 3 or more");
+    batch_low = (int)s[o_dim - 2];
+    m = (int)s[o_dim - 3];
+    batch_high = (int)prod(s, 0, o_dim - 3);
+  } else {
+    if (filter->size() % ((size_t)n * k)) fail("FullyConnected '" + name + "': filter size mismatch");
+    batch_low = (int)(filter->size() / ((size_t)n * k));
+    batch_high = 1;
+    m = rank2 ? (int)a_s[0] : batch_low > 1 ? (int)a_s[a_s.size() - 2] : (int)prod(a_s, 0, a_s.size() - 1);
+  }
+  batch = batch_low * batch_high;
+  if (filter->size() != (size_t)batch * n * k) fail("FullyConnected '" + name + "': filter size mismatch");
+  if (input_data->size() != (size_t)batch * m * k) fail("FullyConnected '" + name + "': input size mismatch");
+  if (output_data->size() != (size_t)batch * m * n) fail("FullyConnected '" + name + "': result size mismatch");
+  if (rshift_data->size() < (size_t)batch || multiplier_data->size() < (size_t)batch)
+    fail("FullyConnected '" + name + "': one rshift and one multiplier per batch needed");
   std::vector<int8_t> w8(filter->size());
   for (size_t i = 0; i < w8.size(); ++i) w8[i] = weight_to_i8(filter->at(i), name, "filter");
   std::vector<int32_t> b32;
   if (bias) {
-    if (bias->size() < (size_t)n) fail("FullyConnected '" + name + "': bias size mismatch");
-    b32.resize((size_t)n);
-    for (int i = 0; i < n; ++i) b32[i] = f2i32(bias->at(i));
+    if (bias->size() < (size_t)batch * n) fail("FullyConnected '" + name + "': bias size mismatch");
+    b32.resize((size_t)batch * n);
+    for (size_t i = 0; i < b32.size(); ++i) b32[i] = f2i32(bias->at(i));
   }
-  // (uint32_t)rshift_data->at(i), (uint32_t)multiplier_data->at(i) with i the batch index
-  // (:78-87); batch == 1 here
-  const int32_t rs = (int32_t)f2u32(rshift_data->at(0));
-  const int32_t mu = (int32_t)f2u32(multiplier_data->at(0));
-  ck(tpuhip_fc_prepack(ctx, m, k, n, input_data->cs, output_data->cs, (int)op.attr("do_relu", 0),
-                       w8.data(), bias ? b32.data() : nullptr, mu, rs, &packed),
-     ("FullyConnected '" + name + "'").c_str());
+  // (uint32_t)rshift_data->at(i), (uint32_t)multiplier_data->at(i) per block i of the result (:78-87)
+  std::vector<int32_t> rs((size_t)batch), mu((size_t)batch);
+  for (int i = 0; i < batch; ++i) {
+    rs[i] = (int32_t)f2u32(rshift_data->at(i));
+    mu[i] = (int32_t)f2u32(multiplier_data->at(i));
+  }
+  const std::string who = "FullyConnected '" + name + "'";
+  const bool plain = rank2 && batch == 1 && input_data->h * input_data->w == 1 && input_data->n == m;
+  if (plain) {
+    ck(tpuhip_fc_prepack(ctx, m, k, n, input_data->cs, output_data->cs, (int)op.attr("do_relu", 0),
+                         w8.data(), bias ? b32.data() : nullptr, mu[0], rs[0], &packed),
+       who.c_str());
+  } else {
+    tpuhip_fc_batched_desc d{};
+    d.batch_high = batch_high; d.batch_low = batch_low; d.m = m; d.k = k; d.n = n;
+    d.input_transpose = ltrans; d.output_transpose = otrans; d.do_relu = (int)op.attr("do_relu", 0);
+    d.x_c = input_data->c; d.x_h = input_data->h; d.x_w = input_data->w; d.x_cs = input_data->cs;
+    d.y_c = output_data->c; d.y_h = output_data->h; d.y_w = output_data->w; d.y_cs = output_data->cs;
+    ck(tpuhip_fc_batched_prepack(ctx, &d, w8.data(), bias ? b32.data() : nullptr, mu.data(), rs.data(),
+                                 &packed_batched),
+       who.c_str());
+  }
 }
 
 FullyConnectedOpKernel::~FullyConnectedOpKernel() {
   if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
+  if (packed_batched) tpuhip_fc_batched_destroy(ctx, packed_batched);
 }
 
 const char *FullyConnectedOpKernel::algo_name() const {
-  algo_text = std::string("fc/") + tpuhip_conv2d_algo_name(packed);
+  algo_text = packed ? std::string("fc/") + tpuhip_conv2d_algo_name(packed) : std::string("fc/batched");
   return algo_text.c_str();
 }
 
 void FullyConnectedOpKernel::invoke() {
-  ck(tpuhip_fc_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+  if (packed) ck(tpuhip_fc_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
+  else ck(tpuhip_fc_batched_i8(ctx, packed_batched, input_data->data(), output_data->data()), name.c_str());
 }
 
 // ---------------------------------------------------------------------------
@@ -1110,7 +1154,10 @@ ConcatOpKernel::ConcatOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
     inputs_data.push_back(opdTensors[i].act);
   }
   output_data = resTensor;
-  if (op.shape.size() != 4 && axis != 1) fail("Concat '" + name + "': only 4-d tensors off axis 1");
+  // shapes of rank 2..4 lie in the 4-d view with trailing dims of 1, so the axis keeps its number;
+  // a rank-1 shape lies along the channels
+  if (axis < 0 || axis >= (int)op.shape.size()) fail("Concat '" + name + "': axis outside the shape");
+  if (op.shape.size() == 1) axis = 1;
 }
 
 void ConcatOpKernel::invoke() {

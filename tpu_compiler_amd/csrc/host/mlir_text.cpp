@@ -748,6 +748,7 @@ MlirModule moduleFromMlir(const MlirFunc &func) {
 
 std::string describeModule(const MlirModule &m) {
   std::ostringstream os;
+  os.precision(17);   // attributes read back to the value the text holds (scales, thresholds)
   os << "weight_file " << (m.weight_file.empty() ? "-" : m.weight_file) << "\n";
   if (!m.chipname.empty()) os << "chipname " << m.chipname << "\n";
   for (auto &w : m.weights) {

@@ -69,6 +69,14 @@ void ModuleInterpreter::loadModuleFile(const std::string &mlir_path, std::string
       if (!wfile.readTensor(w.name, data.data(), count)) {
         auto *a = wfile.find(w.name);
         if (!a) throw std::runtime_error("failed to find tensor " + w.name + " to read in " + wpath);
+        // beyond the reference's float-stored files: arrays kept with their integer storage type
+        // (int8 filters, int32 biases, ...) are widened to float
+        std::vector<float> wide;
+        std::vector<int64_t> wshape;
+        if (wfile.readTensorAsFloat(w.name, wide, wshape) && wide.size() == count) {
+          updateWeightMap(w.name, wide.data(), count);
+          continue;
+        }
         throw std::runtime_error("size does not match for tensor " + w.name + " in " + wpath + " (float32 x " +
                                  std::to_string(count) + " expected)");
       }
