@@ -300,7 +300,7 @@ def main():
                                   "x".join(str(v) for v in g.input_op().shape[1:])),
                    "global_batch": batch,
                    "tensors_written": "all" if args.keep_all else
-                                      "all but the conv results consumed only by their fused add",
+                                      "all but the conv results consumed only by the add or max pool fused into their launch",
                    "conv_tiles": ("recorded: " + os.path.relpath(args.tiles, ROOT)) if args.tiles else
                                  "timed on first use"},
         "tops": round(tops, 2),

@@ -167,6 +167,12 @@ typedef struct tpuhip_conv_post {
   tpuhip_fused_add add;
   const void *add_src;
   void *add_out;
+  /* a max pool (PoolingOpKernel::invoke, core/pooling.cpp, INT8 max branch) over the conv result, run in
+   * the conv's launch: pool_out receives what tpuhip_pool_max_i8 would compute from y; y may then be
+   * NULL (the conv result itself is not written).  Only where tpuhip_conv2d_can_fuse_pool says so; takes
+   * no table and no add.  NULL: no pool. */
+  const struct tpuhip_pool_desc *pool;
+  void *pool_out;
 } tpuhip_conv_post;
 int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                           const tpuhip_conv_post *post);
@@ -192,6 +198,12 @@ const char *tpuhip_conv2d_tile_name(int tile);
  * table op into its producer (the decision MlirModuleInterpreter.cpp:165-344 never has to make: the
  * reference runs every op as its own kernel). */
 int tpuhip_conv2d_can_fuse_table(const tpuhip_conv_weights *w);
+/* 1 when tpuhip_conv2d_post_i8 can run this max pool in the packed conv's launch: a stem conv (at most 4
+ * input channels, 33..64 output channels, 4..7 filter rows, stride_w <= 2) with ReLU and overflow-free
+ * requantisation, a 3x3 / stride 2 pool with top / left padding of at most 1 over exactly the conv's
+ * result.  The conv + ReLU + pool head of the ImageNet networks then costs one launch and the conv
+ * result stays on chip.  No counterpart in the reference (one kernel per op). */
+int tpuhip_conv2d_can_fuse_pool(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const struct tpuhip_pool_desc *pool);
 
 /* ---- FullyConnected ----------------------------------------------------- */
 
@@ -277,7 +289,7 @@ int tpuhip_binary_i8(tpuhip_ctx *ctx, const tpuhip_binary_desc *d, const void *x
 /* ---- Pooling -------------------------------------------------------------- */
 
 /* Field meaning follows parsePoolParam (TPUOperationSupport.cpp:479-522). */
-typedef struct {
+typedef struct tpuhip_pool_desc {
   int n, c, ih, iw, oh, ow, kh, kw, sh, sw, pt, pb, pl, pr;
   int x_cs, y_cs;
 } tpuhip_pool_desc;

@@ -186,6 +186,11 @@ public:
   bool can_fuse_lut() const;
   void fuse_lut(const int8_t *table, SyncedData dst);
   bool has_fused_lut() const { return lut_dst != nullptr; }
+  // Run a max pool over this conv's result in the conv's launch (the stem + pool head of the
+  // ImageNet networks): invoke() then also writes dst.  Takes no table and no add.
+  bool can_fuse_pool(const tpuhip_pool_desc &pool) const;
+  void fuse_pool(const tpuhip_pool_desc &pool, SyncedData dst);
+  bool has_fused_pool() const { return pool_dst != nullptr; }
   bool has_fused_add() const { return fused.enable != 0; }
   // false: table[result] is not written (only the sum fused behind it)
   void set_store_lut(bool store);
@@ -223,6 +228,8 @@ private:
   tpuhip_fused_add fused{};
   bool store_result = true;
   SyncedData lut_dst;
+  SyncedData pool_dst;
+  tpuhip_pool_desc pool_desc{};
   int8_t lut_table[256];
   bool store_lut = true;
   bool plain = false;                      // an ordinary dense conv (not transposed)
@@ -317,6 +324,13 @@ public:
   static constexpr const char *OpName = "CPUPoolingOp";
   PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
   void invoke() override;
+
+  // set by the module interpreter when the producing conv computes this op's result
+  bool fused_into_producer = false;
+  bool is_max() const { return !is_avg; }
+  const tpuhip_pool_desc &pool_desc() const { return desc; }
+  SyncedData input() const { return input_data; }
+  SyncedData result() const { return output_data; }
 
 private:
   tpuhip_pool_desc desc{};

@@ -126,6 +126,79 @@ def test_conv_stem(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
+# n, ic, ih, iw, oc, kh, kw, conv stride, conv pads, pool pads (t, b, l, r), pool out_hw or None
+STEM_POOL_CASES = [
+    (2, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3, 3, 3), (0, 1, 0, 1), None),     # ResNet-50 conv1 + pool1 (Caffe ceil mode)
+    (3, 3, 64, 80, 64, 7, 7, (2, 2), (3, 3, 3, 3), (1, 1, 1, 1), None),        # the torchvision form: pool padded by 1
+    (1, 3, 57, 61, 48, 5, 5, (2, 2), (2, 2, 2, 2), (0, 0, 0, 0), None),        # odd sizes, 48 channels, 5x5
+    (5, 1, 33, 47, 64, 7, 3, (2, 1), (3, 3, 1, 1), (1, 0, 0, 1), None),        # one channel, stride_w 1, mixed pool pads
+    (2, 4, 30, 36, 40, 4, 8, (1, 2), (1, 2, 3, 4), (0, 1, 1, 0), None),        # four channels, kw = 8, stride_h 1
+    (40, 3, 32, 32, 64, 7, 7, (2, 2), (3, 3, 3, 3), (0, 1, 0, 1), None),       # many images: whole maps per workgroup
+]
+
+
+@pytest.mark.parametrize("case", STEM_POOL_CASES)
+@pytest.mark.parametrize("store_conv", [False, True])
+def test_conv_stem_with_the_max_pool_in_its_launch(ctx, case, store_conv):
+    """conv + ReLU + 3x3 / stride 2 max pool as one launch (tpuhip_conv2d_post_i8 with a pool): the
+    pooled tensor equals the oracle's pool of the oracle's conv; the conv result is written only on request"""
+    n, ic, ih, iw, oc, kh, kw, stride, pads, ppads, pout = case
+    rng = np.random.default_rng(n * 7 + ic * 131 + oc + kh * 7 + kw + ih)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    rsh = np.maximum(rsh, 1)
+    conv_want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, (1, 1), (0, 0), True)
+    pool_want = O.pool_max_i8(conv_want, O.make_pool_desc(conv_want.shape, (3, 3), (2, 2), ppads, pout))
+    d = conv_desc(x.shape, w.shape, stride=stride, pads=pads, do_relu=True)
+    pd = pool_desc(conv_want.shape, (3, 3), (2, 2), ppads, pout)
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    assert ctx.conv_algo_name(wh) == "stem" and ctx.conv_can_fuse_pool(wh, pd)
+    xt = ctx.from_nchw(x)
+    yt = ctx.tensor(conv_want.shape)
+    pt = ctx.tensor(pool_want.shape)
+    for t in (yt, pt):
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, t.ptr, 0x55, t.nbytes))
+    ctx.conv_post(wh, xt, yt if store_conv else None, pool=(pd, pt))
+    got = ctx.to_nchw(pt)
+    assert np.array_equal(got, pool_want), "%d mismatches" % (got != pool_want).sum()
+    if pt.cs != oc:
+        assert not ctx.raw(pt)[..., oc:].any(), "pad channels must be zero"
+    if store_conv:
+        assert np.array_equal(ctx.to_nchw(yt), conv_want)
+    else:
+        assert (ctx.raw(yt) == 0x55).all(), "the conv result was not asked for"
+    assert len(np.unique(pool_want)) > 8
+    ctx.conv_weights_destroy(wh)
+
+
+def test_conv_stem_refuses_pools_it_cannot_take(ctx):
+    rng = np.random.default_rng(5)
+    shape = (1, 3, 32, 32)
+    w = rnd_w(rng, (64, 3, 7, 7))
+    bias, rsh, mult = rnd_params(rng, 64)
+    rsh = np.maximum(rsh, 1)
+    out = (1, 64, 16, 16)
+    ok_pool = pool_desc(out, (3, 3), (2, 2), (0, 1, 0, 1))
+
+    def packed(**kw):
+        d = conv_desc(shape, w.shape, stride=(2, 2), pads=(3, 3, 3, 3), **kw)
+        return ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+
+    wh = packed(do_relu=True)
+    assert ctx.conv_can_fuse_pool(wh, ok_pool)
+    for bad in (pool_desc(out, (2, 2), (2, 2), (0, 0, 0, 0)), pool_desc(out, (3, 3), (1, 1), (1, 1, 1, 1)),
+                pool_desc(out, (3, 3), (2, 2), (2, 2, 2, 2)), pool_desc((1, 64, 16, 18), (3, 3), (2, 2), (0, 1, 0, 1))):
+        assert not ctx.conv_can_fuse_pool(wh, bad)
+    xt, pt = ctx.from_nchw(np.zeros(shape, np.int8)), ctx.tensor((1, 64, 8, 8))
+    with pytest.raises(capi.TpuHipError, match="cannot take the max pool"):
+        ctx.conv_post(wh, xt, None, pool=(pool_desc(out, (2, 2), (2, 2), (0, 0, 0, 0)), pt))
+    ctx.conv_weights_destroy(wh)
+    no_relu = packed(do_relu=False)        # the pool stage relies on bytes in 0..127
+    assert not ctx.conv_can_fuse_pool(no_relu, ok_pool)
+    ctx.conv_weights_destroy(no_relu)
+
+
 def test_conv_stem_general_requant_fused_table_and_limits(ctx):
     """parameters outside the overflow-free form, a table fused behind the requantisation, and the
     shapes the stem path refuses"""

@@ -22,7 +22,8 @@ class FusedAdd(C.Structure):
 
 class ConvPost(C.Structure):
     _fields_ = [("lut", C.c_void_p), ("lut_out", C.c_void_p), ("add", FusedAdd),
-                ("add_src", C.c_void_p), ("add_out", C.c_void_p)]
+                ("add_src", C.c_void_p), ("add_out", C.c_void_p),
+                ("pool", C.c_void_p), ("pool_out", C.c_void_p)]
 
 
 class BinaryDesc(C.Structure):
@@ -102,6 +103,7 @@ PROTOTYPES = {
     "tpuhip_dequant_i8_to_f32": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5 + [C.c_float]),
     "tpuhip_move_i8": (C.c_int, [C.c_void_p, C.POINTER(MoveDesc), C.c_void_p, C.c_void_p]),
     "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
+    "tpuhip_conv2d_can_fuse_pool": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc)]),
     "tpuhip_fc_prepack": (C.c_int, [C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_void_p,
                                                                    C.c_int32, C.c_int32,
                                                                    c_void_pp]),
@@ -483,10 +485,17 @@ class Context:
         self._ck(self.lib.tpuhip_conv2d_add_i8(self.h, w, x.ptr, None if y is None else y.ptr,
                                                add_src.ptr, add_out.ptr, C.byref(f)))
 
-    def conv_post(self, w, x, y=None, table=None, lut_out=None, add=None):
-        """conv, then the optional table, then the optional add = (src, out, m_src, m_conv, rshift, relu)"""
+    def conv_can_fuse_pool(self, w, pool_desc):
+        return bool(self.lib.tpuhip_conv2d_can_fuse_pool(self.h, w, C.byref(pool_desc)))
+
+    def conv_post(self, w, x, y=None, table=None, lut_out=None, add=None, pool=None):
+        """conv, then the optional table, then the optional add = (src, out, m_src, m_conv, rshift, relu);
+        or conv, then the max pool = (PoolDesc, out) in the same launch"""
         p = ConvPost()
         t = None
+        if pool is not None:
+            p.pool = C.addressof(pool[0])
+            p.pool_out = pool[1].ptr
         if table is not None:
             t = np.ascontiguousarray(table, dtype=np.int8)
             assert t.size == 256

@@ -12,6 +12,9 @@
 // (lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp:849-871).
 #include "common.hpp"
 
+#include <map>
+#include <mutex>
+
 #include <algorithm>
 #include <atomic>
 #include <cmath>
@@ -1908,6 +1911,202 @@ conv_stem_kernel(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// The stem with the max pool behind it (conv 7x7 / stride 2 + ReLU, pool 3x3 / stride 2: the
+// head of the ImageNet networks) as one launch.  A workgroup of 8 waves owns `rows` pooled rows
+// of one image over its whole width:
+//   1. the input rows those need -- (2 * rows + 1 conv rows - 1) * sh + kh of them, one dword per
+//      pixel, borders zero -- are fetched once into an LDS patch, every load in flight at once;
+//   2. waves walk the tile's conv pixels (rows flattened) in blocks of 32: the MFMAs of
+//      conv_stem_kernel (filter in registers, B operand = 8 consecutive patch dwords), the
+//      two-instruction ReLU form of the requantisation, and the int8 results go to a conv tile in
+//      LDS ([pixel][64 channels], rows padded to 72 bytes so that the 32 pixels of a block land in
+//      different banks);
+//   3. lanes take 8 channels of one pooled pixel: nine 8-byte LDS reads, the maximum with packed
+//      16-bit unsigned ops on the even and odd bytes (values are 0..127 after the ReLU, so an empty
+//      window position counts as 0), one 8-byte store -- 64 contiguous bytes per pixel.
+// The conv result never travels to HBM and back (25.7 + 25.7 MB at ResNet-50's batch 32) unless
+// the caller wants it (a.store_y: rows are then written from the LDS tile, whole lines).
+// Needs: ReLU, the overflow-free requantisation, 33..64 output channels, 4..7 filter rows.
+// ---------------------------------------------------------------------------
+struct StemPoolArgs {
+  int8_t *py;             // pooled result, channels-last
+  int poh, pow, ppt, ppl, p_cs;
+  int rows;               // pooled rows per tile
+  int tiles_per_image, n_tiles;
+  int crows;              // conv rows a tile holds: 2 * rows + 1
+  int crows_last;         // ... the last tile of an image: down to the conv's last row, which a
+                          // pool without bottom padding may not reach (the rows are still stored)
+  int prows;              // patch rows of the larger of the two: (crows - 1) * sh + kh
+  int pw;                 // patch row in dwords: (ow - 1) * sw + 8, rounded up to 4
+  uint32_t magic_pw;      // ceil(2^32 / pw)
+  uint32_t magic_pow;     // ceil(2^32 / pow)
+};
+constexpr int kStemPoolLoads = 20;     // patch dwords per lane at most (40 KiB of patch)
+constexpr int kStemPoolCRow = 72;      // bytes of a conv-tile pixel row in LDS
+
+__host__ __device__ inline unsigned stem_pool_lds_bytes(int prows, int pw, int cpix) {
+  return (unsigned)(prows * pw * 4 + ((cpix * kStemPoolCRow + 15) & ~15));
+}
+
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t x, uint32_t y) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2us, x),
+                                                                __builtin_bit_cast(v2us, y)));
+}
+
+__global__ __launch_bounds__(512) void conv_stem_pool_kernel(ConvArgs a, StemPoolArgs s) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t sp_smem[];
+  uint32_t *const patch = sp_smem;                                              // [prows][pw]
+  int8_t *const ctile = reinterpret_cast<int8_t *>(patch + s.prows * s.pw);      // [crows * ow][72]
+  const int cpix_max = max(s.crows, s.crows_last) * a.ow;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frow = lane & 31, fk = lane >> 5;
+  // a wave owns one half of the channels (32) and every fourth 32-pixel block.  The
+  // requantisation constants of its lanes' 16 channels stay in registers: a lane requantises 16
+  // values per 7 MFMAs, and fetching the parameters from LDS each time kept the LDS pipe busier
+  // than the matrix pipe
+  const int ih_ = wave & 1;                 // channel half
+  const int lc = ih_ * 32 + fk * 16;        // first of this lane's 16 channels
+  int64_t pc[16];
+  int32_t pm[16], pr[16];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const v4i c01 = *reinterpret_cast<const v4i *>(a.qc64r + 2 * (lc + 4 * q));
+    const v4i c23 = *reinterpret_cast<const v4i *>(a.qc64r + 2 * (lc + 4 * q) + 4);
+    const v4i m4 = *reinterpret_cast<const v4i *>(a.qmult + lc + 4 * q);
+    const v4i r4 = *reinterpret_cast<const v4i *>(a.qshift + lc + 4 * q);
+    pc[4 * q + 0] = (int64_t)(((uint64_t)(uint32_t)c01[1] << 32) | (uint32_t)c01[0]);
+    pc[4 * q + 1] = (int64_t)(((uint64_t)(uint32_t)c01[3] << 32) | (uint32_t)c01[2]);
+    pc[4 * q + 2] = (int64_t)(((uint64_t)(uint32_t)c23[1] << 32) | (uint32_t)c23[0]);
+    pc[4 * q + 3] = (int64_t)(((uint64_t)(uint32_t)c23[3] << 32) | (uint32_t)c23[2]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      pm[4 * q + e] = m4[e];
+      pr[4 * q + e] = r4[e] - 1;
+    }
+  }
+  v4i areg[7];
+  {
+    const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + lane;
+#pragma unroll
+    for (int r = 0; r < 7; ++r) areg[r] = afrag[(ih_ * 7 + r) * 64];
+  }
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+
+  for (int tile = (int)blockIdx.x; tile < s.n_tiles; tile += (int)gridDim.x) {
+    const int n = tile / s.tiles_per_image;
+    const int ti = tile - n * s.tiles_per_image;
+    const int r0 = ti * s.rows;                               // first pooled row
+    const int crows = ti == s.tiles_per_image - 1 ? s.crows_last : s.crows;
+    const int cpix = crows * a.ow;
+    const int nblk = (cpix + 31) >> 5;
+    const int patch_dwords = ((crows - 1) * a.sh + a.kh) * s.pw;
+    const int c0 = r0 * 2 - s.ppt;                            // first conv row held (-1 at a padded top)
+    const int iy0 = c0 * a.sh - a.pt;                         // input row of patch row 0
+    // ---- 1. the patch
+    uint32_t stage[kStemPoolLoads];
+#pragma unroll
+    for (int q = 0; q < kStemPoolLoads; ++q) {
+      const int e = tid + q * 512;
+      const int j = (int)__umulhi((uint32_t)e, s.magic_pw);
+      const int d = e - j * s.pw;
+      const int iy = iy0 + j, ix = d - a.pl;
+      const bool ok = (e < patch_dwords) & ((unsigned)iy < (unsigned)a.ih) & ((unsigned)ix < (unsigned)a.iw);
+      stage[q] = __builtin_amdgcn_raw_buffer_load_b32(
+          xrsrc, ok ? (uint32_t)(((n * a.ih + iy) * a.iw + ix) * a.x_cs) : kOobOffset, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < kStemPoolLoads; ++q) {
+      const int e = tid + q * 512;
+      if (e < patch_dwords) patch[e] = stage[q];
+    }
+    __syncthreads();
+    // ---- 2. conv + ReLU requantisation into the LDS tile
+    for (int b = wave >> 1; b < nblk; b += 4) {
+      const int pl = b * 32 + frow;
+      const int p = min(pl, cpix - 1);
+      const int cr = (int)__umulhi((uint32_t)p, a.magic_ow);
+      const int col = p - cr * a.ow;
+      const uint32_t *prow = patch + (cr * a.sh) * s.pw + col * a.sw + fk * 4;
+      v16i acc;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[e] = 0;
+#pragma unroll
+      for (int r = 0; r < 7; ++r) {
+        const uint32_t *src = prow + r * s.pw;
+        v4i bb;
+        bb[0] = (int)src[0]; bb[1] = (int)src[1]; bb[2] = (int)src[2]; bb[3] = (int)src[3];
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[r], bb, acc, 0, 0, 0);
+      }
+      uint32_t outw[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int32_t y[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          // the ReLU form of requant_rows_c64: floor((acc * m + c) / 2^(31 + rshift)), clamped below
+          const int64_t prod = (int64_t)acc[4 * q + e] * (int64_t)pm[4 * q + e] + pc[4 * q + e];
+          y[e] = (int32_t)(prod >> 32) >> pr[4 * q + e];
+        }
+        outw[q] = pack_sat4(y[0], y[1], y[2], y[3], 0);
+      }
+      if (pl < cpix) {
+        uint2 *dst = reinterpret_cast<uint2 *>(ctile + p * kStemPoolCRow + lc);
+        dst[0] = uint2{outw[0], outw[1]};
+        dst[1] = uint2{outw[2], outw[3]};
+      }
+    }
+    __syncthreads();
+    // ---- 3. the pooled rows (and, when asked for, the conv rows themselves)
+    const int rows_here = min(s.rows, s.poh - r0);
+    const int items = rows_here * s.pow * 8;
+    for (int it = tid; it < items; it += 512) {
+      const int cg = it & 7, pp = it >> 3;
+      const int pr = (int)__umulhi((uint32_t)pp, s.magic_pow);
+      const int pc = pp - pr * s.pow;
+      // a window position outside the map is moved onto the nearest one inside, which the window
+      // holds as well (every window starts inside the map): the maximum does not change.  The
+      // 16-bit maximum of the raw words is right in its high bytes whatever the low bytes hold;
+      // the low bytes take a second maximum over the masked words.
+      int roff[3], coff[3];
+#pragma unroll
+      for (int d = 0; d < 3; ++d) {
+        roff[d] = (min(max(c0 + 2 * pr + d, 0), a.oh - 1) - c0) * a.ow * kStemPoolCRow;
+        coff[d] = min(max(2 * pc - s.ppl + d, 0), a.ow - 1) * kStemPoolCRow + cg * 8;
+      }
+      uint32_t e0 = 0, o0 = 0, e1 = 0, o1 = 0;
+#pragma unroll
+      for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < 3; ++dx) {
+          const uint2 v = *reinterpret_cast<const uint2 *>(ctile + roff[dy] + coff[dx]);
+          e0 = pk_max_u16(e0, v.x & 0x00ff00ffu);
+          o0 = pk_max_u16(o0, v.x);
+          e1 = pk_max_u16(e1, v.y & 0x00ff00ffu);
+          o1 = pk_max_u16(o1, v.y);
+        }
+      if (cg * 8 < s.p_cs)
+        *reinterpret_cast<uint2 *>(s.py + ((int64_t)(n * s.poh + r0 + pr) * s.pow + pc) * s.p_cs + cg * 8) =
+            uint2{e0 | (o0 & 0xff00ff00u), e1 | (o1 & 0xff00ff00u)};
+    }
+    if (a.store_y) {
+      for (int it = tid; it < cpix * 8; it += 512) {
+        const int cg = it & 7, p = it >> 3;
+        const int cr = (int)__umulhi((uint32_t)p, a.magic_ow);
+        const int col = p - cr * a.ow;
+        if ((unsigned)(c0 + cr) < (unsigned)a.oh && cg * 8 < a.y_cs)
+          *reinterpret_cast<uint2 *>(a.y + ((int64_t)(n * a.oh + c0 + cr) * a.ow + col) * a.y_cs + cg * 8) =
+              *reinterpret_cast<const uint2 *>(ctile + p * kStemPoolCRow + cg * 8);
+      }
+    }
+    // the next tile's patch goes into LDS nobody reads any more (the conv tile is read above, the
+    // patch was last read before the barrier in front of this stage); its conv stage starts behind
+    // the barrier that follows the patch stores, which every wave reaches only after this stage
+  }
+}
+
+// ---------------------------------------------------------------------------
 // MFMA kernel without LDS: every wave owns a tile of TM*32 output channels x
 // TN*32 pixels and loads its MFMA operands straight from global memory in the
 // fragment layout (lane l: row l & 31, bytes 16*(l >> 5) .. +15 of a 32-byte K
@@ -2481,13 +2680,23 @@ void launch_reg(tpuhip_ctx *ctx, dim3 grid, const ConvArgs &a) {
 }
 
 // the patch kernel's LDS patch is dynamic: (rows + 2) x (W + 2) x C bytes of this layer
+// Raises a kernel's dynamic LDS limit, once per kernel and size (kernels of one signature share
+// their function-pointer type, so the record is keyed by the kernel's address); on failure the
+// runtime's last error stays set for the caller to report.
+bool raise_lds_limit(const void *kernel, unsigned bytes) {
+  static std::mutex mu;
+  static std::map<const void *, unsigned> raised;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = raised.find(kernel);
+  if (it != raised.end() && it->second >= bytes) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return false;
+  raised[kernel] = bytes;
+  return true;
+}
+
 template <typename F>
 void launch_patch(tpuhip_ctx *ctx, F kernel, dim3 grid, const ConvArgs &a, bool dynamic, unsigned stage_bytes) {
-  static bool raised = false;   // per kernel instantiation; the same value from any thread
-  if (dynamic && !raised) {
-    (void)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kPatchBytesDyn);
-    raised = true;
-  }
+  if (dynamic) (void)raise_lds_limit((const void *)kernel, kPatchBytesDyn);
   // the patch, or the staged output tile that takes its place in the epilogue if that is larger
   const unsigned smem = dynamic ? std::max((unsigned)((a.pstep_pix + 2) * a.stem_pw * (a.c16 * 16)), stage_bytes) : 0u;
   if (ctx->prof_start)
@@ -2502,17 +2711,9 @@ constexpr unsigned pw_lds_bytes(int bm, int bn, int kp, int sd) {
   return (unsigned)(bm * kp + 2 * bn * kp + sd * bn * (bm + 16) + 5 * bm * 4 + 256);
 }
 
-// raises the kernel's dynamic LDS limit once; on failure the runtime's last error stays set
-// for the caller to report
 template <typename F>
 bool pw_prepare(F kernel, unsigned lds) {
-  static bool raised = false;   // per kernel instantiation; the same value from any thread
-  if (!raised) {
-    if (hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return false;
-    raised = true;
-  }
-  return true;
+  return raise_lds_limit((const void *)kernel, lds);
 }
 
 void launch_pw(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a) {
@@ -2916,8 +3117,54 @@ struct PostOps {
   const void *add_src = nullptr;
   void *add_out = nullptr;
   void *y2 = nullptr;            // second result of a packed pair
+  const tpuhip_pool_desc *pool = nullptr;   // a 3x3 / stride 2 max pool behind the stem
+  void *pool_out = nullptr;
   bool has_add() const { return f && f->enable; }
 };
+
+// The stem + max pool launch: whether it applies, and its tiling.  rows = pooled rows per
+// workgroup: as many as LDS holds (patch + conv tile), fewer while the launch would leave
+// compute units without a tile, then evened out over the image.
+bool stem_pool_plan(const tpuhip_conv_weights *w, const tpuhip_pool_desc &p, int num_cu, StemPoolArgs *out,
+                    unsigned *lds_bytes) {
+  const tpuhip_conv_desc &d = w->d;
+  if (w->algo != ALGO_STEM || !w->fast || !d.do_relu || d.relu_first) return false;
+  if (d.oc <= 32 || d.oc > 64 || d.kh < 4 || d.kh > 7 || d.kw > 8 || d.sw > 2 || d.ow < 2) return false;
+  if (p.kh != 3 || p.kw != 3 || p.sh != 2 || p.sw != 2 || p.pt < 0 || p.pt > 1 || p.pl < 0 || p.pl > 1) return false;
+  if (p.n != d.n || p.c != d.oc || p.ih != d.oh || p.iw != d.ow || p.x_cs != d.y_cs) return false;
+  if (p.oh < 1 || p.ow < 1 || p.y_cs < round_up(d.oc, 16) || p.y_cs % 8) return false;
+  // every window holds at least one conv pixel
+  if (2 * (p.oh - 1) - p.pt > d.oh - 1 || 2 * (p.ow - 1) - p.pl > d.ow - 1) return false;
+  const int pw = round_up((d.ow - 1) * d.sw + 8, 4);
+  auto bytes_crows = [&](int crows) { return stem_pool_lds_bytes((crows - 1) * d.sh + d.kh, pw, crows * d.ow); };
+  auto fits_crows = [&](int crows) {
+    return bytes_crows(crows) <= 160u * 1024 && crows * d.ow < 65536 &&
+           ((crows - 1) * d.sh + d.kh) * pw <= kStemPoolLoads * 512;
+  };
+  auto fits = [&](int rows) { return fits_crows(2 * rows + 1); };
+  if (!fits(1)) return false;
+  int rows = 1;
+  while (rows < p.oh && fits(rows + 1)) ++rows;
+  while (rows > 1 && (int64_t)d.n * ((p.oh + rows - 1) / rows) < num_cu) --rows;
+  const int per_image = (p.oh + rows - 1) / rows;
+  rows = (p.oh + per_image - 1) / per_image;
+  StemPoolArgs s{};
+  s.poh = p.oh; s.pow = p.ow; s.ppt = p.pt; s.ppl = p.pl; s.p_cs = p.y_cs;
+  s.rows = rows;
+  s.tiles_per_image = per_image;
+  s.n_tiles = d.n * per_image;
+  s.crows = 2 * rows + 1;
+  s.crows_last = std::max(2 * (p.oh - (per_image - 1) * rows) + 1, d.oh - (2 * (per_image - 1) * rows - p.pt));
+  if (!fits_crows(std::max(s.crows, s.crows_last))) return false;
+  s.prows = (std::max(s.crows, s.crows_last) - 1) * d.sh + d.kh;
+  s.pw = pw;
+  s.magic_pw = (uint32_t)(((1ull << 32) + pw - 1) / (uint64_t)pw);
+  s.magic_pow = p.ow > 1 ? (uint32_t)(((1ull << 32) + p.ow - 1) / (uint64_t)p.ow) : 0;
+  if (p.ow == 1) return false;
+  *out = s;
+  *lds_bytes = bytes_crows(std::max(s.crows, s.crows_last));
+  return true;
+}
 
 void apply_fusion(ConvArgs *a, const void *y, const PostOps &p) {
   if (p.lut) {
@@ -3268,6 +3515,20 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
       if (regw) launch(ctx, (conv_depthwise_mfma_kernel<false, true>), grid, block, a);
       else launch(ctx, (conv_depthwise_mfma_kernel<false, false>), grid, block, a);
     }
+  } else if (w->algo == ALGO_STEM && post.pool) {
+    StemPoolArgs sp;
+    unsigned lds = 0;
+    TPUHIP_REQUIRE(!post.lut && !post.has_add() && post.pool_out && stem_pool_plan(w, *post.pool, ctx->num_cu, &sp, &lds),
+                   "conv: this stem cannot take the max pool into its launch (tpuhip_conv2d_can_fuse_pool)");
+    sp.py = (int8_t *)post.pool_out;
+    a.magic_ow = (uint32_t)(((1ull << 32) + a.ow - 1) / (uint64_t)a.ow);
+    TPUHIP_REQUIRE(pw_prepare(conv_stem_pool_kernel, 160u * 1024), "conv: raising the stem + pool kernel's LDS limit failed");
+    const int per_cu = std::max(1, std::min(4, (int)(160u * 1024 / lds)));
+    const dim3 grid((unsigned)std::min<int64_t>(sp.n_tiles, (int64_t)ctx->num_cu * per_cu)), block(512);
+    if (ctx->prof_start)
+      hipExtLaunchKernelGGL(conv_stem_pool_kernel, grid, block, lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a, sp);
+    else
+      hipLaunchKernelGGL(conv_stem_pool_kernel, grid, block, lds, ctx->stream, a, sp);
   } else if (w->algo == ALGO_STEM) {
     // one workgroup per resident slot (3 per CU), each walking (image, output row, 128-pixel
     // segment) tiles
@@ -3353,8 +3614,21 @@ int tpuhip_conv2d_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
     p.add_src = post->add_src;
     p.add_out = post->add_out;
   }
-  TPUHIP_REQUIRE(y || p.lut_out || p.add_out, "conv2d_post: nothing would be written");
+  if (post->pool) {
+    TPUHIP_REQUIRE(post->pool_out, "conv2d_post: fused pool without a result tensor");
+    TPUHIP_REQUIRE(!post->lut && !post->add.enable, "conv2d_post: the fused pool takes no table and no add");
+    p.pool = post->pool;
+    p.pool_out = post->pool_out;
+  }
+  TPUHIP_REQUIRE(y || p.lut_out || p.add_out || p.pool_out, "conv2d_post: nothing would be written");
   return run_conv(ctx, w, x, y, p);
+}
+
+int tpuhip_conv2d_can_fuse_pool(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const tpuhip_pool_desc *pool) {
+  if (!ctx || !w || !pool) return 0;
+  StemPoolArgs sp;
+  unsigned lds = 0;
+  return stem_pool_plan(w, *pool, ctx->num_cu, &sp, &lds) ? 1 : 0;
 }
 
 int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, const tpuhip_conv_desc *db,

@@ -93,6 +93,7 @@ void ModuleInterpreter::fuseKernels() {
     if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) c->clear_fusion();
     if (auto *e = dynamic_cast<EltwiseAddOpKernel *>(k.get())) e->fused_into_producer = false;
     if (auto *l = dynamic_cast<LutOpKernel *>(k.get())) l->fused_into_producer = false;
+    if (auto *q = dynamic_cast<PoolingOpKernel *>(k.get())) q->fused_into_producer = false;
   }
   const char *env = getenv("TPUHIP_FUSE");
   if (!fuse_eltwise || (env && atoi(env) == 0)) return;
@@ -115,6 +116,20 @@ void ModuleInterpreter::fuseKernels() {
       launch_groups_.push_back({conv, l});
       producer.erase(it);
       producer[l->result().get()] = {conv_pos, conv};   // an add may follow the table
+      fused_convs.push_back(conv);
+      continue;
+    }
+    if (auto *q = dynamic_cast<PoolingOpKernel *>(k.get())) {
+      // a max pool straight behind the stem conv runs in the conv's launch
+      position[q->result().get()] = pos;
+      auto it = producer.find(q->input().get());
+      if (!q->is_max() || it == producer.end()) continue;
+      Conv2DOpKernel *conv = it->second.second;
+      if (conv->result().get() != q->input().get() || !conv->can_fuse_pool(q->pool_desc())) continue;
+      conv->fuse_pool(q->pool_desc(), q->result());
+      q->fused_into_producer = true;
+      launch_groups_.push_back({conv, q});
+      producer.erase(it);
       fused_convs.push_back(conv);
       continue;
     }
@@ -440,8 +455,10 @@ std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_
       auto *el = dynamic_cast<EltwiseAddOpKernel *>(krnl.get());
       auto *lu = dynamic_cast<LutOpKernel *>(krnl.get());
       auto *cv = dynamic_cast<Conv2DOpKernel *>(krnl.get());
+      auto *po = dynamic_cast<PoolingOpKernel *>(krnl.get());
       const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) || (cv && cv->is_paired_second()) ||
-                          (el && el->fused_into_producer) || (lu && lu->fused_into_producer));
+                          (el && el->fused_into_producer) || (lu && lu->fused_into_producer) ||
+                          (po && po->fused_into_producer));
       if (runs) ck(tpuhip_ctx_set_kernel_events(ctx_, e0[i], e1[i]), "timeKernels");
       krnl->invoke();
       launched[i] = runs;

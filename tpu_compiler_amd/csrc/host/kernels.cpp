@@ -455,11 +455,15 @@ void Conv2DOpKernel::invoke() {
        name.c_str());
     return;
   }
-  if (!fused.enable && !lut_dst) {
+  if (!fused.enable && !lut_dst && !pool_dst) {
     ck(tpuhip_conv2d_i8(ctx, packed, input_data->data(), output_data->data()), name.c_str());
     return;
   }
   tpuhip_conv_post post{};
+  if (pool_dst) {
+    post.pool = &pool_desc;
+    post.pool_out = pool_dst->data();
+  }
   if (lut_dst) {
     post.lut = lut_table;
     post.lut_out = store_lut ? lut_dst->data() : nullptr;
@@ -476,6 +480,17 @@ void Conv2DOpKernel::invoke() {
 
 bool Conv2DOpKernel::can_fuse_add() const {
   return !pair_packed && !paired_into && std::string(tpuhip_conv2d_algo_name(packed)).rfind("mfma", 0) == 0;
+}
+
+bool Conv2DOpKernel::can_fuse_pool(const tpuhip_pool_desc &pool) const {
+  return !pair_packed && !paired_into && !lut_dst && !fused.enable &&
+         tpuhip_conv2d_can_fuse_pool(ctx, packed, &pool) != 0;
+}
+
+void Conv2DOpKernel::fuse_pool(const tpuhip_pool_desc &pool, SyncedData dst) {
+  if (!dst) fail("Conv2D '" + name + "': fused pool without a result tensor");
+  pool_desc = pool;
+  pool_dst = dst;
 }
 
 void Conv2DOpKernel::fuse_add(SyncedData src, SyncedData dst, int m_src, int m_conv, int rshift,
@@ -515,7 +530,7 @@ void Conv2DOpKernel::set_store_lut(bool store) {
 }
 
 void Conv2DOpKernel::set_store_result(bool store) {
-  if (!store && !fused.enable && !lut_dst)
+  if (!store && !fused.enable && !lut_dst && !pool_dst)
     fail("Conv2D '" + name + "': only a fused conv may drop its own result");
   store_result = store;
   output_data->materialized = store;
@@ -527,6 +542,7 @@ void Conv2DOpKernel::clear_fusion() {
   output_data->materialized = true;
   if (lut_dst) lut_dst->materialized = true;
   lut_dst.reset();
+  pool_dst.reset();
   store_lut = true;
   fused = tpuhip_fused_add{};
   add_src.reset();
@@ -852,6 +868,7 @@ PoolingOpKernel::PoolingOpKernel(OpDesc &op, value_map_t &valueMapping, weight_m
 }
 
 void PoolingOpKernel::invoke() {
+  if (fused_into_producer) return;   // the producing conv wrote this result already
   if (is_avg)
     ck(tpuhip_pool_avg_i8(ctx, &desc, input_data->data(), output_data->data(), multiplier, rshift),
        name.c_str());
