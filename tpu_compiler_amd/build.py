@@ -69,7 +69,29 @@ def build(verbose=True, jobs=None):
     return LIB
 
 
+MICROBENCH = os.path.join(PKG, "machine_ceilings.bin")
+
+
+def build_microbench(verbose=True):
+    """The stand-alone program that measures the machine's ceilings (launch floor, copy bandwidth,
+    MFMA peak, LDS and L2 bandwidth, vector-ALU issue rates): csrc/microbench/machine_ceilings.hip.
+    Not linked into the library."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    src = os.path.join(CSRC, "microbench", "machine_ceilings.hip")
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", src, "-o", MICROBENCH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, res.stdout))
+    return MICROBENCH
+
+
 if __name__ == "__main__":
+    if "--microbench" in sys.argv[1:]:
+        print("built", build_microbench())
+        sys.exit(0)
     build()
     print("built", LIB)
     sys.exit(0)
