@@ -9,8 +9,8 @@
  *
  * Device tensors are int8, channels-last: element (n, h, w, c) of a tensor
  * with channel stride cs lives at byte ((n*H + h)*W + w)*cs + c.  cs is a
- * multiple of 16 (or exactly 4 for a graph input with <= 4 channels) and the
- * bytes c..cs-1 of every pixel are zero; every kernel keeps that invariant.
+ * multiple of 16 and the bytes c..cs-1 of every pixel are zero; every kernel
+ * keeps that invariant.
  * The reference's NCHW float tensors (include/tpuc/Interpreter/cpukernel.h:15-78)
  * are converted at the edge by the tpuhip_*_nchw_* entry points.
  *
