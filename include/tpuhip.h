@@ -456,6 +456,11 @@ int tpuhip_module_load(tpuhip_module *m, const char *target_op);
 /* setTensor / getTensor (:407-430) */
 int tpuhip_module_set_tensor(tpuhip_module *m, const char *name, const float *data, size_t count,
                              int bidx);
+/* set_tensor for callers that hold int8 NCHW data already (no counterpart in the reference, whose
+ * tensors are float-stored): a quarter of the bytes cross the bus and no host pass checks or converts
+ * them.  Not for fp32 graph inputs (a tpu.input in front of a tpu.quant). */
+int tpuhip_module_set_tensor_i8(tpuhip_module *m, const char *name, const int8_t *data, size_t count,
+                                int bidx);
 int tpuhip_module_get_tensor(tpuhip_module *m, const char *name, float *dst, size_t count,
                              int bidx);
 /* same tensor as int8 NCHW, without the float detour */

@@ -72,6 +72,9 @@ public:
   int32_t batch_idx() const { return cur_; }
   // float-stored NCHW host data -> slot bidx (values must be integers in [-128,127])
   void assign(const float *first, size_t num, int32_t bidx);
+  // int8 NCHW host data -> slot bidx, for callers that hold bytes already: a quarter of the
+  // float form's transfer and no host pass over the elements
+  void assign_i8(const int8_t *first, size_t num, int32_t bidx);
   // slot bidx as float-stored NCHW host data
   std::shared_ptr<std::vector<float>> tensor(int32_t bidx) const;
   // slot bidx as int8 NCHW host data (no float detour)
@@ -573,6 +576,8 @@ public:
   void setTensor(std::string &name, const std::vector<float> &data, int32_t bidx);
   // the same from a plain buffer (what a C caller holds): no intermediate vector
   void setTensor(std::string &name, const float *data, size_t count, int32_t bidx);
+  // the same from int8 NCHW data (no counterpart in the reference, whose tensors are float-stored)
+  void setTensorI8(const std::string &name, const int8_t *data, size_t count, int32_t bidx);
   std::shared_ptr<std::vector<float>> getTensor(std::string &name, int32_t bidx);
   void getTensorI8(const std::string &name, int8_t *dst, size_t num, int32_t bidx);
   std::vector<int64_t> getTensorShape(std::string &name);

@@ -371,6 +371,26 @@ def test_benchmark_configuration_full_size_against_the_oracle():
     m.close()
 
 
+def test_int8_host_entry_sets_the_same_tensor_as_the_float_one():
+    g = graphs.cfg3_resnet50(batch=2, hw=64)
+    x = g.input_op().data
+    m = module()
+    m.load(g)
+    m.set_tensor("input", x.astype(np.float32))
+    m.invoke()
+    want = {k: m.get_tensor_i8(k) for k in ("input", "fc1000")}
+    m.set_tensor("input", np.zeros(x.shape, np.float32))
+    m.set_tensor_i8("input", x)
+    m.invoke()
+    for k, v in want.items():
+        assert np.array_equal(m.get_tensor_i8(k), v), k
+    with pytest.raises(capi.TpuHipError, match="size mismatch"):
+        m.set_tensor_i8("input", x[:1])
+    with pytest.raises(TypeError):
+        m.set_tensor_i8("input", x.astype(np.float32))
+    m.close()
+
+
 def test_module_errors_are_reported():
     g = graphs.cfg1_single_conv()
     m = module()

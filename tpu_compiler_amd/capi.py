@@ -148,6 +148,7 @@ PROTOTYPES.update({
     "tpuhip_module_load": (C.c_int, [C.c_void_p, C.c_char_p]),
     "tpuhip_module_set_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,
                                            C.c_int]),
+    "tpuhip_module_set_tensor_i8": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int]),
     "tpuhip_module_get_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,
                                            C.c_int]),
     "tpuhip_module_get_tensor_i8": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t,

@@ -396,6 +396,12 @@ void ModuleInterpreter::setTensor(std::string &name, const float *data, size_t c
   it->second->assign(data, count, bidx);
 }
 
+void ModuleInterpreter::setTensorI8(const std::string &name, const int8_t *data, size_t count, int32_t bidx) {
+  auto it = activationMapping.find(name);
+  if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");
+  it->second->assign_i8(data, count, bidx);
+}
+
 std::shared_ptr<std::vector<float>> ModuleInterpreter::getTensor(std::string &name, int32_t bidx) {
   auto it = activationMapping.find(name);
   if (it == activationMapping.end()) fail(" Not Find Op name: " + name + " tensor");

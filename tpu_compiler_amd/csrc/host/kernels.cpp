@@ -141,6 +141,19 @@ void TensorData::assign(const float *first, size_t num, int32_t bidx) {
      "TensorData::assign");
 }
 
+void TensorData::assign_i8(const int8_t *first, size_t num, int32_t bidx) {
+  if (num != size_) fail("TensorData::assign_i8: size mismatch");
+  if (bidx < 0 || bidx >= batch) fail("TensorData::assign_i8: slot out of range");
+  if (f32) fail("TensorData::assign_i8: this tensor holds fp32 data");
+  // the staging buffers of assign() serve here too (a quarter of them is used)
+  if (!stage_host_) ck(tpuhip_host_malloc(ctx_, num * sizeof(float), &stage_host_), "TensorData::assign_i8");
+  if (!stage_dev_) ck(tpuhip_malloc(ctx_, num * sizeof(float), &stage_dev_), "TensorData::assign_i8");
+  std::memcpy(stage_host_, first, num);
+  ck(tpuhip_upload(ctx_, stage_dev_, stage_host_, num), "TensorData::assign_i8");
+  ck(tpuhip_nchw_to_nhwc_i8(ctx_, stage_dev_, (char *)base_ + slot_bytes() * (size_t)bidx, n, c, h, w, cs),
+     "TensorData::assign_i8");
+}
+
 std::shared_ptr<std::vector<float>> TensorData::tensor(int32_t bidx) const {
   if (!materialized)
     fail("TensorData::tensor: this tensor is fused into its consumer and never written "

@@ -119,6 +119,14 @@ int tpuhip_module_set_tensor(tpuhip_module *m, const char *name, const float *da
   })
 }
 
+int tpuhip_module_set_tensor_i8(tpuhip_module *m, const char *name, const int8_t *data, size_t count,
+                                int bidx) {
+  GUARD(m, {
+    if (!name || !data) throw std::runtime_error("set_tensor_i8: NULL argument");
+    m->interp->setTensorI8(name, data, count, bidx);
+  })
+}
+
 int tpuhip_module_get_tensor(tpuhip_module *m, const char *name, float *dst, size_t count,
                              int bidx) {
   GUARD(m, {

@@ -13,6 +13,7 @@ using namespace tpuhip;
 
 namespace {
 
+typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int kThreads = 256;
 
 struct MoveArgs {
@@ -335,6 +336,100 @@ extern "C" int tpuhip_reduce_i8(tpuhip_ctx *ctx, int kind, const void *x, void *
   return TPUHIP_OK;
 }
 
+namespace {
+
+// ---------------------------------------------------------------------------
+// Permute without the per-byte index map.  S[k]: byte stride of input dimension k in the input,
+// T[k]: byte stride, in the output, of the output dimension that input dimension k becomes.
+// ---------------------------------------------------------------------------
+struct PermArgs {
+  const int8_t *x;
+  int8_t *y;
+  int dim[4];        // input dimensions (n, c, h, w)
+  int64_t S[4], T[4];
+  int ocs;           // channel stride of the output
+  int j, a, b;       // j: the input dimension that becomes the output's channels; a, b: the other two besides c
+};
+
+// channels stay channels (j == 1): a pixel's channel row moves as 16-byte chunks
+__global__ __launch_bounds__(kThreads) void permute_rows_kernel(PermArgs q, int64_t total) {
+  const int c16 = q.ocs >> 4;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int cg = (int)(i % c16);
+    int64_t pix = i / c16;                       // input pixel (n, h, w) in input order
+    const int w = (int)(pix % q.dim[3]);
+    pix /= q.dim[3];
+    const int h = (int)(pix % q.dim[2]);
+    const int n = (int)(pix / q.dim[2]);
+    const v4i v = *reinterpret_cast<const v4i *>(q.x + n * q.S[0] + h * q.S[2] + w * q.S[3] + cg * 16);
+    *reinterpret_cast<v4i *>(q.y + n * q.T[0] + h * q.T[2] + w * q.T[3] + cg * 16) = v;
+  }
+}
+
+// the channels change places with dimension j: 64 x 64 byte tiles through LDS, dword loads along
+// the input's channels, dword stores along the output's (pad channels of the output written as
+// zero: tile rows past the end of dimension j are zero)
+__global__ __launch_bounds__(kThreads) void permute_tile_kernel(PermArgs q) {
+  __shared__ __attribute__((aligned(4))) int8_t tile[64][68];
+  const int c0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  const int ia = (int)(blockIdx.z / q.dim[q.b]), ib = (int)(blockIdx.z % q.dim[q.b]);
+  const int8_t *src = q.x + ia * q.S[q.a] + ib * q.S[q.b];
+  int8_t *dst = q.y + ia * q.T[q.a] + ib * q.T[q.b];
+  const int tq = threadIdx.x & 15, tr = threadIdx.x >> 4;   // 16 dwords per row, 16 rows per pass
+#pragma unroll
+  for (int r = tr; r < 64; r += 16) {
+    const int jj = j0 + r, cc = c0 + tq * 4;
+    uint32_t v = 0;
+    // the input's pad channels are zero and its channel stride is a multiple of 16, so a dword
+    // that starts inside the row may be read whole
+    if (jj < q.dim[q.j] && cc < q.dim[1]) v = *reinterpret_cast<const uint32_t *>(src + jj * q.S[q.j] + cc);
+    *reinterpret_cast<uint32_t *>(&tile[r][tq * 4]) = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = tr; r < 64; r += 16) {
+    const int cc = c0 + r, jj = j0 + tq * 4;
+    if (cc < q.dim[1] && jj < q.ocs) {
+      const uint32_t v = (uint32_t)(uint8_t)tile[tq * 4][r] | ((uint32_t)(uint8_t)tile[tq * 4 + 1][r] << 8) |
+                         ((uint32_t)(uint8_t)tile[tq * 4 + 2][r] << 16) | ((uint32_t)(uint8_t)tile[tq * 4 + 3][r] << 24);
+      *reinterpret_cast<uint32_t *>(dst + cc * q.T[1] + jj) = v;
+    }
+  }
+}
+
+int run_permute(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
+  PermArgs q{};
+  q.x = (const int8_t *)x;
+  q.y = (int8_t *)y;
+  q.dim[0] = d->in; q.dim[1] = d->ic; q.dim[2] = d->ih; q.dim[3] = d->iw;
+  q.S[0] = (int64_t)d->ih * d->iw * d->x_cs; q.S[1] = 1; q.S[2] = (int64_t)d->iw * d->x_cs; q.S[3] = d->x_cs;
+  const int64_t tout[4] = {(int64_t)d->oh * d->ow * d->y_cs, 1, (int64_t)d->ow * d->y_cs, d->y_cs};
+  for (int k = 0; k < 4; ++k) q.T[d->p[k]] = tout[k];   // output dimension k is input dimension p[k]
+  q.ocs = d->y_cs;
+  q.j = d->p[1];
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  if (q.j == 1) {
+    const int64_t total = (int64_t)d->in * d->ih * d->iw * (d->y_cs / 16);
+    const unsigned blocks = (unsigned)std::max<int64_t>(
+        1, std::min<int64_t>(ceil_div64(total, kThreads), (int64_t)ctx->num_cu * 32));
+    launch(ctx, permute_rows_kernel, dim3(blocks), dim3(kThreads), q, total);
+  } else {
+    int rest[2], nr = 0;
+    for (int k = 0; k < 4; ++k)
+      if (k != 1 && k != q.j) rest[nr++] = k;
+    q.a = rest[0];
+    q.b = rest[1];
+    const int64_t batch = (int64_t)q.dim[q.a] * q.dim[q.b];
+    TPUHIP_REQUIRE(batch <= 65535, "permute: more than 65535 planes (%lld)", (long long)batch);
+    const dim3 grid((unsigned)((d->y_cs + 63) / 64), (unsigned)((d->ic + 63) / 64), (unsigned)batch);
+    launch(ctx, permute_tile_kernel, grid, dim3(kThreads), q);
+  }
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
+}  // namespace
+
 extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   TPUHIP_REQUIRE(ctx && d && x && y, "move: NULL argument");
   TPUHIP_REQUIRE(d->kind >= TPUHIP_MOVE_PAD_CONST && d->kind <= TPUHIP_MOVE_REFLECTION_PAD,
@@ -391,6 +486,9 @@ extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const 
         a.p[k] = p[k];
       }
       TPUHIP_REQUIRE(seen == 15, "permute: order is not a permutation");
+      // tiled kernels; the per-byte map below serves the other kinds (and permutes with more
+      // planes than a launch grid holds)
+      if (p[1] == 1 || (int64_t)is[0] * is[2] * is[3] / is[p[1]] <= 65535) return run_permute(ctx, d, x, y);
       break;
     }
     case TPUHIP_MOVE_REORG:

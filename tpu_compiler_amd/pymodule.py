@@ -196,6 +196,14 @@ class module:
         self._ck(self.lib.tpuhip_module_set_tensor(self.h, name.encode(), arr.ctypes.data,
                                                    arr.size, bidx))
 
+    def set_tensor_i8(self, name, data, bidx=0):
+        """int8 NCHW data straight in (no float detour); not for fp32 graph inputs"""
+        arr = np.ascontiguousarray(data)
+        if arr.dtype != np.int8:
+            raise TypeError("set_tensor_i8 takes int8 data, got %s" % arr.dtype)
+        self._ck(self.lib.tpuhip_module_set_tensor_i8(self.h, name.encode(), arr.ctypes.data,
+                                                      arr.size, bidx))
+
     def get_tensor(self, name, bidx=0):
         shape = self.tensor_shape(name)
         out = np.empty(shape, np.float32)
