@@ -390,6 +390,13 @@ typedef struct tpuhip_move_desc {
   int p[8];
 } tpuhip_move_desc;
 int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y);
+/* PermuteOpKernel::invoke (core/permute.cpp:8-44) on DENSE row-major int8 bytes over the full rank
+ * (at most 6): y[..] with dimension d of the result = dimension order[d] of the input.  The module
+ * interpreter uses it for shapes that are not 4-d, between two layout conversions; the reference
+ * folds such shapes to 4-d first (parsePermuteParam, TPUOperationSupport.cpp:690-737) and fails
+ * where that cannot be done. */
+int tpuhip_permute_flat_i8(tpuhip_ctx *ctx, const void *x_dense, void *y_dense, int rank, const int64_t *in_shape,
+                           const int *order);
 
 /* ---- Reduce over consecutive axes ------------------------------------------
  * Replaces ReduceOpKernel::invoke (core/reduce.cpp:54-117) for INT8 tensors.  kind: 0 mean, 1 sum,

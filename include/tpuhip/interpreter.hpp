@@ -504,7 +504,9 @@ public:
   void invoke() override;
 
 protected:
-  MoveOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping, const char *what);
+  // any_rank: the subclass also takes shapes that are not 4-d (and then runs a path of its own)
+  MoveOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping, const char *what,
+               bool any_rank = false);
   tpuhip_move_desc desc{};
   SyncedData input_data, output_data;
 };
@@ -516,7 +518,24 @@ protected:
   };
 TPUHIP_MOVE_KERNEL(PadOpKernel, "CPUPadOp")                          // core/pad.cpp:114-141
 TPUHIP_MOVE_KERNEL(CropOpKernel, "CPUCropOp")                        // core/crop.cpp:34-92
-TPUHIP_MOVE_KERNEL(PermuteOpKernel, "CPUPermuteOp")                  // core/permute.cpp:35-44
+// core/permute.cpp:35-44.  4-d shapes run the tiled kernels on the channels-last tensors; shapes of
+// rank 2, 3, 5 and 6 (the reference folds those to 4-d where it can, parsePermuteParam,
+// TPUOperationSupport.cpp:690-737) go through their row-major bytes: channels-last -> dense,
+// permute of the dense bytes over the full rank, dense -> channels-last.
+class PermuteOpKernel : public MoveOpKernel {
+public:
+  static constexpr const char *OpName = "CPUPermuteOp";
+  PermuteOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping);
+  ~PermuteOpKernel() override;
+  void invoke() override;
+
+private:
+  bool flat = false;
+  int rank = 4;
+  int64_t in_shape[6] = {1, 1, 1, 1, 1, 1};
+  int order[6] = {0, 1, 2, 3, 4, 5};
+  void *dense_in = nullptr, *dense_out = nullptr;
+};
 TPUHIP_MOVE_KERNEL(ReorgOpKernel, "CPUReorgOp")                      // core/reorg.cpp:8-42
 TPUHIP_MOVE_KERNEL(TileOpKernel, "CPUTileOp")                        // core/tile.cpp:8-42
 TPUHIP_MOVE_KERNEL(ReverseOpKernel, "CPUReverseOp")                  // core/reverse.cpp:7-42

@@ -124,6 +124,11 @@ def run(graph, input_data=None, upto=None, keep=None, batch_slice=None, guards=N
             w = op.weights
             y = O.leaky_relu_i8(ins[0], w["rshift_pos"][0], w["multiplier_pos"][0],
                                 w["rshift_neg"][0], w["multiplier_neg"][0])
+        elif t == "tpu.permute" and ins[0].ndim != 4:
+            # core/permute.cpp:8-44 behind parsePermuteParam's folding to 4-d
+            # (TPUOperationSupport.cpp:690-737): result dimension d is input dimension order[d]
+            order = [int(op.attrs["order%d" % d]) for d in range(ins[0].ndim)]
+            y = np.ascontiguousarray(np.transpose(ins[0], order))
         elif t in _MOVES:
             a = op.attrs
             kind, keys = _MOVES[t]

@@ -391,6 +391,60 @@ def test_int8_host_entry_sets_the_same_tensor_as_the_float_one():
     m.close()
 
 
+@pytest.mark.parametrize("shape,order", [
+    ((2, 3, 4, 5, 7), (0, 2, 1, 3, 4)),        # the channel-shuffle form [N, g, C/g, H, W]
+    ((1, 2, 2, 3, 4, 5), (0, 3, 4, 1, 5, 2)),  # the pixel-shuffle form, 6-d: not foldable to 4-d
+    ((3, 2, 5, 4, 6), (4, 0, 3, 1, 2)),
+    ((4, 5, 6), (2, 0, 1)),
+    ((7, 9), (1, 0)),
+])
+def test_permute_of_shapes_that_are_not_4d(shape, order):
+    """PermuteOpKernel on ranks 2, 3, 5, 6 (the reference folds them to 4-d where it can,
+    parsePermuteParam) between reshapes, against numpy's transpose"""
+    rng = np.random.default_rng(sum(shape))
+    size = int(np.prod(shape))
+    flat4 = (shape[0], size // shape[0], 1, 1)
+    x = rng.integers(-128, 128, flat4).astype(np.int8)
+    out_shape = tuple(shape[o] for o in order)
+    g = graphs.Graph("permute_nd", 3)
+    g.add(graphs.Op("tpu.input", "input", [], flat4)).data = x
+    g.add(graphs.Op("tpu.reshape", "nd", ["input"], shape))
+    g.add(graphs.Op("tpu.permute", "perm", ["nd"], out_shape, {"order%d" % d: o for d, o in enumerate(order)}))
+    g.add(graphs.Op("tpu.reshape", "back", ["perm"], (out_shape[0], size // out_shape[0], 1, 1)))
+    g.outputs = ["back"]
+    want = np.transpose(x.reshape(shape), order)
+    assert np.array_equal(oracle_graph.run(g)["perm"], want)
+    m = module()
+    m.set_option("keep_all_tensors", 1)
+    m.load(g)
+    m.set_tensor("input", x.astype(np.float32))
+    m.invoke()
+    assert np.array_equal(m.get_tensor_i8("perm").reshape(out_shape), want)
+    assert np.array_equal(m.get_tensor_i8("back").reshape(-1), want.reshape(-1))
+    m.close()
+
+
+def test_channel_shuffle_written_as_reshape_permute_reshape_equals_the_shuffle_op():
+    rng = np.random.default_rng(8)
+    n, c, h, w, grp = 2, 24, 6, 5, 3
+    x = rng.integers(-128, 128, (n, c, h, w)).astype(np.int8)
+    g = graphs.Graph("shuffle_nd", 4)
+    g.add(graphs.Op("tpu.input", "input", [], x.shape)).data = x
+    g.add(graphs.Op("tpu.reshape", "r5", ["input"], (n, grp, c // grp, h, w)))
+    g.add(graphs.Op("tpu.permute", "p5", ["r5"], (n, c // grp, grp, h, w),
+                    {"order0": 0, "order1": 2, "order2": 1, "order3": 3, "order4": 4}))
+    g.add(graphs.Op("tpu.reshape", "r4", ["p5"], x.shape))
+    g.add(graphs.Op("tpu.shuffle_channel", "sc", ["input"], x.shape, dict(group=grp)))
+    g.outputs = ["r4", "sc"]
+    m = module()
+    m.load(g)
+    m.set_tensor("input", x.astype(np.float32))
+    m.invoke()
+    a, b = m.get_tensor_i8("r4"), m.get_tensor_i8("sc")
+    assert np.array_equal(a, b) and np.array_equal(a, oracle_graph.run(g)["sc"])
+    m.close()
+
+
 def test_module_errors_are_reported():
     g = graphs.cfg1_single_conv()
     m = module()

@@ -101,6 +101,7 @@ PROTOTYPES = {
                                       C.POINTER(C.c_int8)]),
     "tpuhip_quant_f32_to_i8": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5 + [C.c_float]),
     "tpuhip_dequant_i8_to_f32": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 5 + [C.c_float]),
+    "tpuhip_permute_flat_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "tpuhip_move_i8": (C.c_int, [C.c_void_p, C.POINTER(MoveDesc), C.c_void_p, C.c_void_p]),
     "tpuhip_binary_i8": (C.c_int, [C.c_void_p, C.POINTER(BinaryDesc)] + [C.c_void_p] * 3),
     "tpuhip_conv2d_can_fuse_pool": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(PoolDesc)]),

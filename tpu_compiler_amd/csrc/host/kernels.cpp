@@ -42,10 +42,16 @@ int8_t weight_to_i8(float v, const std::string &op, const char *role) {
 }
 
 void view4(const SyncedDataShape &s, int *n, int *c, int *h, int *w) {
-  if (s.empty() || s.size() > 4) fail("tensor rank " + std::to_string(s.size()) + " not supported");
+  if (s.empty() || s.size() > 6) fail("tensor rank " + std::to_string(s.size()) + " not supported");
   int64_t d[4] = {1, 1, 1, 1};
   if (s.size() == 1) {
     d[1] = s[0];
+  } else if (s.size() > 4) {
+    // ranks 5 and 6 (between the reshapes around a permute): the leading dims fold into n,
+    // which keeps the row-major order of the elements
+    const size_t lead = s.size() - 3;
+    for (size_t i = 0; i < lead; ++i) d[0] *= s[i];
+    for (size_t i = 0; i < 3; ++i) d[1 + i] = s[lead + i];
   } else {
     for (size_t i = 0; i < s.size(); ++i) d[i] = s[i];
   }
@@ -757,13 +763,13 @@ void BinaryOpKernel::invoke() {
 // Pad, Crop, Permute, Reorg, Tile, Reverse, ShuffleChannel, DepthToSpace
 // ---------------------------------------------------------------------------
 MoveOpKernel::MoveOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map_t &weightMapping,
-                           const char *what)
+                           const char *what, bool any_rank)
     : CPUOpKernel(op, valueMapping, weightMapping) {
   require_int8(what);
   input_data = opdTensors.at(0).act;
   output_data = resTensor;
   if (!input_data) fail(std::string(what) + " '" + name + "': input missing");
-  if (op.operands.empty() || valueMapping.shapes[op.operands[0]].size() != 4 || shape.size() != 4)
+  if (!any_rank && (op.operands.empty() || valueMapping.shapes[op.operands[0]].size() != 4 || shape.size() != 4))
     fail(std::string(what) + " '" + name + "': only 4-d shapes are supported");
   tpuhip_move_desc &d = desc;
   d.in = input_data->n; d.ic = input_data->c; d.ih = input_data->h; d.iw = input_data->w;
@@ -793,9 +799,47 @@ CropOpKernel::CropOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOp
   numbered(op, "steps", 4, desc.p + 4, 1, false);   // steps default to 1 (parseCropParam)
 }
 PermuteOpKernel::PermuteOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w)
-    : MoveOpKernel(op, v, w, "Permute") {
-  desc.kind = TPUHIP_MOVE_PERMUTE;
-  numbered(op, "order", 4, desc.p, 0, true);
+    : MoveOpKernel(op, v, w, "Permute", true) {
+  const SyncedDataShape &is = v.shapes[op.operands.at(0)];
+  rank = (int)is.size();
+  if (rank == 4 && shape.size() == 4) {
+    desc.kind = TPUHIP_MOVE_PERMUTE;
+    numbered(op, "order", 4, desc.p, 0, true);
+    return;
+  }
+  if (rank < 1 || rank > 6 || (int)shape.size() != rank)
+    fail("Permute '" + name + "': ranks 1 to 6 are supported, input and result of the same rank");
+  flat = true;
+  int seen = 0;
+  for (int d = 0; d < rank; ++d) {
+    in_shape[d] = is[d];
+    order[d] = (int)op.attr("order" + std::to_string(d));
+    if (order[d] < 0 || order[d] >= rank) fail("Permute '" + name + "': order[" + std::to_string(d) + "] out of range");
+    seen |= 1 << order[d];
+    if (shape[d] != is[order[d]]) fail("Permute '" + name + "': result dimension " + std::to_string(d) + " does not match");
+  }
+  if (seen != (1 << rank) - 1) fail("Permute '" + name + "': order is not a permutation");
+  ck(tpuhip_malloc(ctx, input_data->size(), &dense_in), name.c_str());
+  ck(tpuhip_malloc(ctx, input_data->size(), &dense_out), name.c_str());
+}
+
+PermuteOpKernel::~PermuteOpKernel() {
+  if (dense_in) tpuhip_free(ctx, dense_in);
+  if (dense_out) tpuhip_free(ctx, dense_out);
+}
+
+void PermuteOpKernel::invoke() {
+  if (!flat) {
+    MoveOpKernel::invoke();
+    return;
+  }
+  ck(tpuhip_nhwc_to_nchw_i8(ctx, input_data->data(), dense_in, input_data->n, input_data->c, input_data->h,
+                            input_data->w, input_data->cs),
+     name.c_str());
+  ck(tpuhip_permute_flat_i8(ctx, dense_in, dense_out, rank, in_shape, order), name.c_str());
+  ck(tpuhip_nchw_to_nhwc_i8(ctx, dense_out, output_data->data(), output_data->n, output_data->c, output_data->h,
+                            output_data->w, output_data->cs),
+     name.c_str());
 }
 ReorgOpKernel::ReorgOpKernel(OpDesc &op, value_map_t &v, weight_map_t &w) : MoveOpKernel(op, v, w, "Reorg") {
   desc.kind = TPUHIP_MOVE_REORG;

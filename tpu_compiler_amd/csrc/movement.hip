@@ -397,6 +397,27 @@ __global__ __launch_bounds__(kThreads) void permute_tile_kernel(PermArgs q) {
   }
 }
 
+// permute of dense row-major bytes over the full rank (at most 6): a lane owns an output element
+struct FlatPermArgs {
+  const int8_t *x;
+  int8_t *y;
+  int rank;
+  int oshape[6];
+  int64_t istr[6];   // input stride of the input dimension that output dimension d is
+  int64_t total;
+};
+__global__ __launch_bounds__(kThreads) void permute_flat_kernel(FlatPermArgs q) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < q.total; i += (int64_t)gridDim.x * blockDim.x) {
+    int64_t r = i, off = 0;
+    for (int d = q.rank - 1; d >= 0; --d) {
+      const int64_t c = r % q.oshape[d];
+      r /= q.oshape[d];
+      off += c * q.istr[d];
+    }
+    q.y[i] = q.x[off];
+  }
+}
+
 int run_permute(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void *y) {
   PermArgs q{};
   q.x = (const int8_t *)x;
@@ -562,6 +583,38 @@ extern "C" int tpuhip_move_i8(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const 
   const unsigned blocks = (unsigned)std::max<int64_t>(
       1, std::min<int64_t>(ceil_div64(a.total, kThreads), (int64_t)ctx->num_cu * 32));
   launch(ctx, move_kernel, dim3(blocks), dim3(kThreads), a);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
+extern "C" int tpuhip_permute_flat_i8(tpuhip_ctx *ctx, const void *x, void *y, int rank, const int64_t *in_shape,
+                                      const int *order) {
+  TPUHIP_REQUIRE(ctx && x && y && in_shape && order, "permute_flat: NULL argument");
+  TPUHIP_REQUIRE(rank >= 1 && rank <= 6, "permute_flat: rank %d outside [1,6]", rank);
+  FlatPermArgs q{};
+  q.x = (const int8_t *)x;
+  q.y = (int8_t *)y;
+  q.rank = rank;
+  int64_t istride[6], total = 1;
+  int seen = 0;
+  for (int d = rank - 1; d >= 0; --d) {
+    TPUHIP_REQUIRE(in_shape[d] >= 1 && in_shape[d] < (1ll << 31), "permute_flat: bad dimension %d", d);
+    istride[d] = total;
+    total *= in_shape[d];
+  }
+  TPUHIP_REQUIRE(total < (1ll << 31), "permute_flat: tensor too large");
+  for (int d = 0; d < rank; ++d) {
+    TPUHIP_REQUIRE(order[d] >= 0 && order[d] < rank, "permute_flat: order[%d] = %d", d, order[d]);
+    seen |= 1 << order[d];
+    q.oshape[d] = (int)in_shape[order[d]];
+    q.istr[d] = istride[order[d]];
+  }
+  TPUHIP_REQUIRE(seen == (1 << rank) - 1, "permute_flat: order is not a permutation");
+  q.total = total;
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  const unsigned blocks = (unsigned)std::max<int64_t>(
+      1, std::min<int64_t>(ceil_div64(total, kThreads), (int64_t)ctx->num_cu * 32));
+  launch(ctx, permute_flat_kernel, dim3(blocks), dim3(kThreads), q);
   TPUHIP_CHECK_HIP(hipGetLastError());
   return TPUHIP_OK;
 }
