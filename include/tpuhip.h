@@ -216,13 +216,15 @@ int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, 
                       const int8_t *filter_nk, const int32_t *bias, int32_t multiplier,
                       int32_t rshift, tpuhip_conv_weights **out);
 /* FullyConnectedOpKernel::invoke (core/fullyconnected.cpp:44-91) for weights packed by
- * tpuhip_fc_prepack.  Matrices of at most 256 rows run a split-K kernel: K is divided over
- * workgroups, whose 32x32 int32 partial sums meet in a scratch buffer in device memory that the
- * library allocates with the context's first such call (and grows when a larger layer comes);
- * a second launch adds them up and requantises.  Larger matrices take the
- * conv path.  Same result as tpuhip_conv2d_i8 on the same weights. */
+ * tpuhip_fc_prepack.  Matrices of at most 256 rows split K.  With K of 1024 or more, one launch:
+ * sixteen waves per 32x32 block of outputs take a sixteenth of K each and add their partial sums
+ * in LDS.  With a shorter K, K is divided over workgroups, whose 32x32 int32 partial sums meet
+ * in a scratch buffer in device memory that the library allocates with the context's first
+ * such call (and grows when a larger layer comes); a second launch adds them up and
+ * requantises.  Larger matrices take the conv path.  Same result as tpuhip_conv2d_i8 on the
+ * same weights. */
 int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
-/* The same split-K FullyConnected for callers that cannot allocate (code under HIP graph capture,
+/* The two-launch split-K FullyConnected, at any K, for callers that cannot allocate (code under HIP graph capture,
  * serving loops, harnesses that forbid hipMalloc): it has no counterpart in the reference.  The
  * partial sums go to a static array in device memory (4 MiB, one per GPU the library runs
  * on, held until the process ends) whose address is looked up when a context is created; the call

@@ -853,13 +853,24 @@ def test_conv_rejects_bad_arguments(ctx):
 
 
 @pytest.mark.parametrize("m,k,n,relu", [(32, 2048, 1000, False), (5, 100, 37, True),
-                                        (64, 1280, 1000, True)])
+                                        (64, 1280, 1000, True),
+                                        # the one-launch kernel (K of 1024 and more): exactly one K step
+                                        # per wave, waves left without work, an odd number of steps per
+                                        # wave, ragged rows and channels
+                                        (1, 1024, 10, False), (33, 1090, 65, True), (7, 3100, 40, False),
+                                        (256, 1500, 96, True), (40, 4160, 33, False),
+                                        # the two-launch kernels just below that K
+                                        (17, 1000, 70, True),
+                                        # more input channels than the conv kernels index (the first
+                                        # classifier layers of VGG / AlexNet): few rows, and more rows
+                                        # than the K-splitting kernels otherwise take
+                                        (4, 9216, 50, True), (2, 25088, 64, False), (300, 4112, 40, True)])
 def test_fully_connected(ctx, m, k, n, relu):
     rng = np.random.default_rng(m + k + n)
     x = rnd_i8(rng, (m, k))
-    w = rnd_w(rng, (n, k), 20)
+    w = rnd_w(rng, (n, k), 20 if k <= 4160 else 4)     # sums the reference's fp32 holds exactly
     bias = rng.integers(-3000, 3000, n).astype(np.float32)
-    mult, rsh = np.float32((1 << 30) + 128 * 12345), np.float32(9)
+    mult, rsh = np.float32((1 << 30) + 128 * 12345), np.float32(9 if k <= 4160 else 10)
     want = O.fc_i8(x, w, bias, [rsh], [mult], 1, m, k, n, relu)[0]
     xt = ctx.from_nchw(x.reshape(m, k, 1, 1))
     yt = ctx.tensor((m, n, 1, 1))
@@ -868,6 +879,10 @@ def test_fully_connected(ctx, m, k, n, relu):
     ctx.conv(wh, xt, yt)
     got = ctx.to_nchw(yt).reshape(m, n)
     assert np.array_equal(got, want)
+    # the FullyConnected entry point: the K-splitting kernels for matrices of few rows
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.fc(wh, xt, yt)
+    assert np.array_equal(ctx.to_nchw(yt).reshape(m, n), want)
     assert O.fc_guard(x, w, bias, 1, m, k, n) < (1 << 24)
     ctx.conv_weights_destroy(wh)
 

@@ -1,7 +1,8 @@
 """The allocation-free FullyConnected entry point (tpuhip_fc_i8_noalloc) through the C ABI: its
-output must equal that of tpuhip_fc_i8 -- the same split-K kernels with a scratch buffer the
-library allocates -- byte for byte, on two calls in a row, the second on a smaller input (the
-static scratch keeps the first call's partial sums)."""
+output must equal that of tpuhip_fc_i8 -- one launch with the partial sums in LDS for the
+first, long-K layer; for the second the same split-K kernels with a scratch buffer the library
+allocates -- byte for byte, on two calls in a row, the second on a smaller input (the static
+scratch keeps the first call's partial sums)."""
 import numpy as np
 import pytest
 

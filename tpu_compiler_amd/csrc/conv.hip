@@ -50,6 +50,9 @@ struct tpuhip_conv_weights {
   // a pair of convs over one input packed as one: first channel, channel stride and ReLU of
   // the second result (split_oc == 0: an ordinary conv)
   int split_oc = 0, y2_cs = 0, relu2 = 0;
+  // a FullyConnected whose K is beyond what the conv kernels index (more than 4096 input
+  // channels): only the K-splitting FullyConnected kernels, which walk K linearly, run it
+  bool fc_only = false;
   std::vector<int8_t> host_filter;  // OIHW copy, kept while the layer can still be repacked
   int8_t *w = nullptr;   // packed filter
   int32_t *bias = nullptr;
@@ -2636,6 +2639,83 @@ __global__ __launch_bounds__(256) void fc_reduce_kernel(ConvArgs a, const v4i *p
     epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pb * 32 + frow, 32, nullptr, out);
 }
 
+// The same product in ONE launch, for K of at least kFcOneWaves x 64: a workgroup of sixteen waves
+// per 32x32 block of outputs, wave w multiplying K steps [w * spw, (w + 1) * spw) with the
+// loads of two steps in flight at a time.  The sixteen partial sums meet in LDS (64 KiB,
+// [wave][quarter][lane] of four dwords): every thread adds one quarter of four waves in place,
+// wave 0 adds the four groups and the bias and runs the epilogue.  No scratch in device
+// memory and no second launch, which on a classifier of 32 rows is most of the time.
+constexpr int kFcOneWaves = 16;
+
+template <bool FAST>
+__global__ __launch_bounds__(64 * kFcOneWaves) void fc_one_kernel(ConvArgs a, int steps_per_wave) {
+  __shared__ v4i part[kFcOneWaves * 4 * 64];
+  touch_kernargs();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = (int)blockIdx.x;
+  const int ob = tile % a.n_oc_tiles, pb = tile / a.n_oc_tiles;
+  const int nsteps = a.kp / 64;
+  const int s0 = min(nsteps, wave * steps_per_wave), s1 = min(nsteps, s0 + steps_per_wave);
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+  const int frow = lane & 31, fk = lane >> 5;
+  const int row = pb * 32 + frow;
+  const uint32_t xoff = row < a.npix ? (uint32_t)(row * a.x_cs + fk * 16) : kOobOffset;
+  const uint32_t woff = (uint32_t)(ob * nsteps) * 2048u + (uint32_t)lane * 16u;
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  int s = s0;
+  for (; s + 2 <= s1; s += 2) {
+    v4i af[4], bf[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      af[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(wrsrc, woff, s * 2048 + u * 1024, 0);
+      bf[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff, s * 64 + u * 32, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u], bf[u], acc, 0, 0, 0);
+  }
+  if (s < s1) {
+    v4i af[2], bf[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      af[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(wrsrc, woff, s * 2048 + u * 1024, 0);
+      bf[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff, s * 64 + u * 32, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u], bf[u], acc, 0, 0, 0);
+  }
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    part[(wave * 4 + q) * 64 + lane] = v4i{acc[q * 4 + 0], acc[q * 4 + 1], acc[q * 4 + 2], acc[q * 4 + 3]};
+  __syncthreads();
+  {
+    // thread (group g of four waves, quarter q, lane): the sum lands where only it has read
+    const int g = wave >> 2, q = wave & 3;
+    v4i t = part[((g * 4 + 0) * 4 + q) * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) t += part[((g * 4 + w) * 4 + q) * 64 + lane];
+    part[((g * 4) * 4 + q) * 64 + lane] = t;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  const int oc = ob * 32 + fk * 16;                 // this lane's 16 channels
+  v16i sum[1];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    v4i t = *reinterpret_cast<const v4i *>(a.bias + oc + q * 4);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) t += part[((g * 4) * 4 + q) * 64 + lane];
+    sum[0][q * 4 + 0] = t[0]; sum[0][q * 4 + 1] = t[1]; sum[0][q * 4 + 2] = t[2]; sum[0][q * 4 + 3] = t[3];
+  }
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+  if (oc < a.ocw)
+    epilogue_rows<1, FAST>(sum, a, oc, a.qmult + oc, a.qshift + oc, a.qhpot + oc, pb * 32 + frow, 32, nullptr, out);
+}
+
 // The scratch of the allocation-free entry point: one array per device the library is loaded
 // on.  Nothing in it has to start at zero: every partial sum the second launch reads was
 // written by the first.
@@ -3209,6 +3289,7 @@ struct PostOps {
   const tpuhip_pool_desc *pool = nullptr;   // a 3x3 / stride 2 max pool behind the stem
   void *pool_out = nullptr;
   bool has_add() const { return f && f->enable; }
+  bool any() const { return lut || has_add() || y2 || pool; }
 };
 
 // The stem + max pool launch: whether it applies, and its tiling.  rows = pooled rows per
@@ -3369,7 +3450,12 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
                        (int64_t)round_up(d.oc, 128) * (d.kh * d.kw * round_up(d.ic, 16) + 256) <
                            (1ll << 31);
   if (d.algo == ALGO_AUTO && algo == ALGO_MFMA && !mfma_ok) algo = ALGO_DIRECT;
-  TPUHIP_REQUIRE(algo != ALGO_MFMA || mfma_ok,
+  // a matrix product packed fragment by fragment (tpuhip_fc_prepack): the FullyConnected kernels
+  // take any K whose packed filter stays within a buffer descriptor's 2 GiB
+  const bool fc_form = dense && forced_tile >= 0 && std::string(kTiles[forced_tile].name) == "mfma_reg_32x32" &&
+                       d.relu_first && d.ih == 1 && d.iw == 1 && d.kh == 1 && d.kw == 1 &&
+                       (int64_t)round_up(d.oc, 32) * round_up(d.ic, 64) < (1ll << 31);
+  TPUHIP_REQUIRE(algo != ALGO_MFMA || mfma_ok || fc_form,
                  "conv: MFMA path needs g == 1, no inserted zeros, ic <= 4096 and K < 65000");
   TPUHIP_REQUIRE((algo != ALGO_DEPTHWISE && algo != ALGO_DEPTHWISE_DOT) || depthwise,
                  "conv: depthwise path needs g == ic == oc and no inserted zeros");
@@ -3377,6 +3463,7 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   auto *cw = new tpuhip_conv_weights();
   cw->d = d;
   cw->algo = algo;
+  cw->fc_only = algo == ALGO_MFMA && !mfma_ok;
   std::vector<int8_t> packed;
   const size_t per_oc = (size_t)icg * d.kh * d.kw;
   if (algo == ALGO_MFMA) {
@@ -3547,8 +3634,14 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
   return "?";
 }
 
+static int run_fc_one(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
+
 static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                     const PostOps &post) {
+  if (w->fc_only) {
+    TPUHIP_REQUIRE(!post.any() && y, "conv: a FullyConnected of more than 4096 input channels takes no fused work");
+    return run_fc_one(ctx, w, x, y);
+  }
   if (w->algo == ALGO_MFMA && !w->tuned) {
     // first use: pick the tile by measurement (not capturable into a HIP graph).  The
     // fused work is timed with it unless the sum would overwrite its own operand.
@@ -3830,6 +3923,24 @@ static int run_fc_splitk(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
   return TPUHIP_OK;
 }
 
+static int run_fc_one(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y) {
+  ConvArgs a;
+  fill_args(ctx, w, x, y, &a);
+  a.n_oc_tiles = w->ocp / 32;
+  const int nsteps = w->kp / 64;
+  const int64_t tiles = (int64_t)((w->d.n + 31) / 32) * a.n_oc_tiles;
+  TPUHIP_REQUIRE(tiles < (1ll << 31), "fc: too many blocks of 32 x 32 outputs");
+  const int steps_per_wave = (nsteps + kFcOneWaves - 1) / kFcOneWaves;
+  auto kernel = w->fast ? fc_one_kernel<true> : fc_one_kernel<false>;
+  const dim3 grid((unsigned)tiles), block(64 * kFcOneWaves);
+  if (ctx->prof_start || ctx->prof_stop)
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a, steps_per_wave);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, 0, ctx->stream, a, steps_per_wave);
+  TPUHIP_CHECK_HIP(hipGetLastError());
+  return TPUHIP_OK;
+}
+
 int tpuhip_static_scratch_init(int device) {
   TPUHIP_REQUIRE(device >= 0 && device < 64, "tpuhip: device index %d out of range", device);
   if (g_static_scratch[device]) return TPUHIP_OK;
@@ -3843,6 +3954,7 @@ int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, v
   TPUHIP_REQUIRE(ctx && w && x && y, "tpuhip_fc_i8: NULL argument");
   FcPlan p;
   if (!fc_splitk_plan(ctx, w, &p)) return run_conv(ctx, w, x, y, PostOps{});   // many rows: the conv path
+  if (w->kp / 64 >= kFcOneWaves) return run_fc_one(ctx, w, x, y);              // long K: one launch
   if (ctx->workspace_bytes < p.bytes) {
     TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
     TPUHIP_CHECK_HIP(hipStreamSynchronize(ctx->stream));
@@ -3883,7 +3995,8 @@ int tpuhip_fc_prepack(tpuhip_ctx *ctx, int m, int k, int n, int x_cs, int y_cs, 
   d.relu_first = 1;
   // few rows: packed fragment by fragment for the split-K kernel of tpuhip_fc_i8 (the same
   // bytes serve the LDS-free 32x32 conv tile, so tpuhip_conv2d_i8 runs them too)
-  if (m <= 256 && (n + 31) / 32 * ((m + 31) / 32) <= kFcMaxTiles) {
+  // (and so is a K beyond the conv kernels' reach, whatever the rows)
+  if ((m <= 256 && (n + 31) / 32 * ((m + 31) / 32) <= kFcMaxTiles) || k > 4096) {
     for (int t = 0; t < kNumTiles; ++t)
       if (std::string(kTiles[t].name) == "mfma_reg_32x32") d.algo = 16 + t;
   }
