@@ -683,6 +683,55 @@ def test_conv_depthwise(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
+# the row-segment form of the depthwise kernel (windows of at most 3 x 3 taps, right shifts of
+# at least 1): n, c, ih, iw, kh, kw, stride, pads, dil, relu, table
+DEPTHWISE_ROWS = [
+    (3, 144, 56, 56, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True, True),     # 30 + 26 outputs per row, 4.5 channel blocks
+    (2, 64, 28, 28, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), False, False),    # one segment per row
+    (5, 96, 14, 14, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True, True),      # two rows per block
+    (9, 48, 7, 7, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True, False),       # three rows per block, odd row count
+    (2, 32, 33, 61, 3, 3, (1, 1), (0, 0, 0, 0), (1, 1), False, True),     # unpadded, ragged width
+    (2, 16, 20, 35, 3, 3, (1, 1), (1, 2, 2, 1), (1, 1), True, False),     # one channel block, uneven padding
+    (2, 96, 112, 112, 3, 3, (2, 2), (0, 1, 0, 1), (1, 1), True, True),    # stride 2: nine loads, no halo
+    (4, 192, 28, 28, 3, 3, (2, 2), (1, 1, 1, 1), (1, 1), False, False),   # stride 2 onto 14 x 14
+    (3, 40, 15, 13, 3, 3, (2, 2), (1, 1, 1, 1), (1, 1), True, False),     # stride 2 onto 8 x 7
+    (2, 24, 19, 30, 1, 3, (1, 1), (0, 0, 1, 1), (1, 1), True, True),      # one row of taps
+    (2, 24, 30, 19, 3, 1, (1, 1), (1, 1, 0, 0), (1, 1), False, False),    # one column of taps
+    (2, 40, 22, 22, 2, 2, (1, 1), (0, 1, 0, 1), (1, 1), True, False),     # 2 x 2
+    (2, 56, 25, 25, 3, 3, (1, 1), (2, 2, 2, 2), (2, 2), True, True),      # dilated both ways
+    (2, 56, 25, 25, 3, 3, (1, 1), (2, 2, 1, 1), (2, 1), False, False),    # dilated rows only: halo form
+    (2, 32, 17, 40, 3, 3, (1, 2), (1, 1, 1, 1), (1, 1), True, False),     # stride along the width only
+    (1, 32, 9, 70000 // 9, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), True, False),   # a very wide map
+]
+
+
+@pytest.mark.parametrize("case", DEPTHWISE_ROWS)
+def test_conv_depthwise_row_segments(ctx, case):
+    n, c, ih, iw, kh, kw, stride, pads, dil, relu, with_table = case
+    rng = np.random.default_rng(c + kh * 7 + kw + iw)
+    x = rnd_i8(rng, (n, c, ih, iw))
+    w = rnd_w(rng, (c, 1, kh, kw), 24)
+    bias, rsh, mult = rnd_params(rng, c, 5, 12, 2048)
+    want = oracle_conv(x, w, bias, rsh, mult, c, stride, pads, dil, (0, 0), relu)
+    got, name = run_conv(ctx, x, w, bias, rsh, mult, algo=capi.ALGO_DEPTHWISE, g=c, stride=stride, pads=pads,
+                         dil=dil, do_relu=relu)
+    assert name == "depthwise" and np.array_equal(got, want)
+    assert len(np.unique(want)) > 8
+    if with_table:
+        table = rnd_i8(rng, 256)
+        table[0] = 9
+        d = conv_desc(x.shape, w.shape, g=c, stride=stride, pads=pads, dil=dil, do_relu=relu, algo=capi.ALGO_DEPTHWISE)
+        wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+        xt, yt, tt = ctx.from_nchw(x), ctx.tensor(want.shape), ctx.tensor(want.shape)
+        ctx.conv_post(wh, xt, yt, table, tt)
+        assert np.array_equal(ctx.to_nchw(yt), want)
+        assert np.array_equal(ctx.to_nchw(tt), O.lut_i8(want, table))
+        assert tt.cs == c or not ctx.raw(tt)[..., c:].any()
+        ctx.conv_weights_destroy(wh)
+        for t in (xt, yt, tt):
+            t.free()
+
+
 @pytest.mark.parametrize("algo", [capi.ALGO_DEPTHWISE, capi.ALGO_DEPTHWISE_DOT])
 def test_conv_depthwise_dilated_general_requant_and_fused_table(ctx, algo):
     rng = np.random.default_rng(77)

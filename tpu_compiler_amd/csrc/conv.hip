@@ -1832,6 +1832,189 @@ conv_depthwise_mfma_kernel(ConvArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// The same diagonal-MFMA depthwise for windows of at most 3 x 3 taps, laid out so that the
+// vector ALU -- which the per-tap address arithmetic and the general epilogue of the kernel
+// above keep busier than anything else on the large MobileNet layers -- is left with little
+// more than the requantisation:
+//   * a wave's 32 pixels are R whole row segments of W lanes (R * W <= 32) of one image
+//     instead of 32 consecutive pixels of the flattened tensor: image, output rows and first
+//     column of a block are wave-uniform (scalar registers), a lane's row and column within
+//     the block never change, and a tap's address is one multiply-add per filter row;
+//   * SHIFT (3 taps wide, stride 1, no dilation along W): a lane loads only the middle tap
+//     of each filter row; the left and right taps are the same registers moved one lane up
+//     or down the wave (DPP), so a block costs 3 loads instead of 9.  The first and last lane
+//     of every row segment are halo: they load the neighbours' pixels, and what they compute
+//     is not stored (W - 2 outputs per segment);
+//   * accumulators start at zero and the bias rides in the 64-bit multiply-add of the
+//     requantisation (requant_rows_c64; needs the layer's overflow-free form).
+// A wave keeps its 32-channel block (nine A fragments in registers) and walks blocks.
+// ---------------------------------------------------------------------------
+struct DwRowsArgs {
+  int rows, width, valid, halo;   // R, W, outputs per row segment (W - 2 * halo), 1 with SHIFT
+  int xblocks, rblocks;           // column blocks per output row, row blocks per image (both below 2^15)
+  int nblocks;                    // n * rblocks * xblocks
+  // the walk, laid out by the host: blocks in flight per XCD, that step split into (image, row
+  // block, column block) parts, and the first block of every XCD's run split the same way
+  int nslots, d_n, d_rb, d_xb;
+  int start_n[8], start_rb[8], start_xb[8];
+  uint32_t magic_x, magic_r, magic_w;   // ceil(2^32 / d) of xblocks, rblocks, width: x / d == umulhi(x, magic), x, d < 2^16
+};
+
+template <bool SHIFT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SHIFT ? 4 : 3, SHIFT ? 4 : 3))) void
+conv_depthwise_rows_kernel(ConvArgs a, DwRowsArgs r) {
+  __shared__ uint32_t lutw[64];
+  __shared__ int32_t qlds[4][160];   // per wave: 32 (low, high) pairs of c64, then mult, shift, hpot of 32 channels
+  touch_kernargs();
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int p = lane & 31, fk = lane >> 5;
+  const int n_cb = (a.ocw + 31) >> 5;
+  // workgroups are dealt to the 8 XCDs round-robin; each XCD takes a contiguous run of blocks
+  const int per_xcd = (r.nblocks + 7) >> 3;
+  const int xcd = (int)(blockIdx.x & 7);
+  const int b_end = min(r.nblocks, (xcd + 1) * per_xcd);
+  const int gw = (int)(blockIdx.x >> 3) * 4 + wave;
+  const int nslots = r.nslots;                              // blocks in flight per XCD (>= 1)
+  // gw < 2^16 waves per XCD, n_cb < 2^16
+  const int slot = n_cb == 1 ? gw : (int)__umulhi((uint32_t)gw, a.magic_c16);   // gw / n_cb (the host set magic_c16 for it)
+  const int cb = gw - slot * n_cb;
+  const bool relu = a.lo == 0;
+  {
+    int32_t *q = qlds[wave];
+    const int32_t *c64 = relu ? a.qc64r : a.qc64;
+    q[lane] = c64[2 * (cb * 32) + lane];
+    q[64 + lane] = lane < 32 ? a.qmult[cb * 32 + lane] : a.qshift[cb * 32 + lane - 32] - (relu ? 1 : 0);
+    if (lane < 32) q[128 + lane] = a.qhpot[cb * 32 + lane];
+  }
+  if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+  __syncthreads();
+  if (slot >= nslots) return;                               // no barrier below
+  int b = xcd * per_xcd + slot;
+  if (b >= b_end) return;
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+  const int oc = cb * 32 + fk * 16;                         // this lane's 16 channels
+  const bool ch_ok = oc < a.ocw;
+  const __amdgpu_buffer_rsrc_t xrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const int taps = a.kh * a.kw;
+  const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + (size_t)cb * taps * 64 + lane;
+  v4i areg[3][3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      areg[i][j] = (i < a.kh && j < a.kw) ? afrag[(i * a.kw + j) * 64] : v4i{0, 0, 0, 0};
+  const int32_t *q = qlds[wave];
+  const int32_t *pc64 = q + fk * 32, *pmult = q + 64 + fk * 16, *pshift = q + 96 + fk * 16, *phpot = q + 128 + fk * 16;
+
+  // what never changes for a lane
+  const int lr = (int)__umulhi((uint32_t)p, r.magic_w), lc = p - lr * r.width;
+  const bool live = (p < r.rows * r.width) & ch_ok;
+  const bool inner = live & (lc >= r.halo) & (lc < r.halo + r.valid);
+  const int lrow_in = lr * a.sh;                            // input row offset of the lane's segment
+  // column of the tap a lane loads first, relative to the block's first output column times sw:
+  // SHIFT: the middle tap; otherwise the leftmost
+  const int lcol_in = (lc - r.halo) * a.sw - a.pl + (SHIFT ? 1 : 0);
+  const int row_bytes = a.iw * a.x_cs, drow_bytes = a.dh * row_bytes;
+
+  // block -> (image, row block, column block), advanced by nslots blocks at a time
+  int xb = r.start_xb[xcd] + slot;                          // slot < nslots <= 2^15
+  // x / d by umulhi(x, ceil(2^32 / d)) is exact while x * d < 2^32; a divisor of 1 has no such constant
+  int rb = r.start_rb[xcd] + (r.xblocks == 1 ? xb : (int)__umulhi((uint32_t)xb, r.magic_x));
+  xb -= (rb - r.start_rb[xcd]) * r.xblocks;
+  int n = r.start_n[xcd] + (r.rblocks == 1 ? rb : (int)__umulhi((uint32_t)rb, r.magic_r));
+  rb -= (n - r.start_n[xcd]) * r.rblocks;
+  const int d_xb = r.d_xb, d_rb = r.d_rb, d_n = r.d_n;
+
+  uint32_t img_base = 0;                                    // scalar part of the addresses of the loads in flight
+  auto request = [&](v4i (&bt)[3][3]) {
+    const int ihb = rb * r.rows * a.sh - a.pt + lrow_in;    // first filter row's input row
+    const int iw0 = xb * r.valid * a.sw + lcol_in;
+    img_base = (uint32_t)n * (uint32_t)(a.ih * row_bytes);
+    if (SHIFT) {
+      const bool col_ok = live & ((unsigned)iw0 < (unsigned)a.iw);
+      // rows and row pitch are below 2^23 (checked on the host); a first row above the image gives a
+      // negative product, from which the rows below it are still reached
+      const uint32_t off0 = (uint32_t)__mul24(ihb, row_bytes) + (uint32_t)(iw0 * a.x_cs + oc);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        const int ih = ihb + i * a.dh;
+        const bool ok = col_ok & ((unsigned)ih < (unsigned)a.ih) & (i < a.kh);
+        bt[i][1] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, ok ? off0 + (uint32_t)(i * drow_bytes) : kOobOffset,
+                                                              img_base, 0);
+      }
+    } else {
+      bool col_ok[3];
+      uint32_t coff[3];
+      const uint32_t off0 = (uint32_t)__mul24(ihb, row_bytes) + (uint32_t)(iw0 * a.x_cs + oc);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int iw = iw0 + j * a.dw;
+        col_ok[j] = live & ((unsigned)iw < (unsigned)a.iw) & (j < a.kw);
+        coff[j] = off0 + (uint32_t)(j * a.dw * a.x_cs);
+      }
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        const int ih = ihb + i * a.dh;
+        const bool row_ok = ((unsigned)ih < (unsigned)a.ih) & (i < a.kh);
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          bt[i][j] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+              xrsrc, (row_ok & col_ok[j]) ? coff[j] + (uint32_t)(i * drow_bytes) : kOobOffset, img_base, 0);
+      }
+    }
+  };
+  auto shift_lanes = [&](const v4i &m, int ctrl) {
+    v4i o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)   // 0x138: wave_shr:1 (from lane l - 1), 0x130: wave_shl:1; the end lane reads 0
+      o[e] = ctrl == 0 ? __builtin_amdgcn_mov_dpp(m[e], 0x138, 0xf, 0xf, true) : __builtin_amdgcn_mov_dpp(m[e], 0x130, 0xf, 0xf, true);
+    return o;
+  };
+
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+  v4i bt[3][3];
+  request(bt);
+  for (;;) {
+    v16i acc[1];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[0][e] = 0;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      if (SHIFT) {
+        // lane l takes the left tap from lane l - 1 and the right tap from lane l + 1
+        bt[i][0] = shift_lanes(bt[i][1], 0);
+        bt[i][2] = shift_lanes(bt[i][1], 1);
+      }
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(areg[i][j], bt[i][j], acc[0], 0, 0, 0);
+    }
+    // this block's output pixel, before the walk moves on
+    const int oh = rb * r.rows + lr, ow = xb * r.valid + lc - r.halo;
+    const bool st_ok = inner & (oh < a.oh) & (ow < a.ow);
+    const int pix = (n * a.oh + oh) * a.ow + ow;
+    b += nslots;
+    xb += d_xb;
+    if (xb >= r.xblocks) { xb -= r.xblocks; ++rb; }
+    rb += d_rb;
+    if (rb >= r.rblocks) { rb -= r.rblocks; ++n; }
+    n += d_n;
+    const bool more = b < b_end;
+    if (more) request(bt);          // into the registers the MFMAs have just consumed
+    uint32_t outw[1][4];
+    if (relu) requant_rows_c64<1, true>(acc, 0, pc64, pmult, pshift, phpot, outw);
+    else requant_rows_c64<1, false>(acc, a.lo, pc64, pmult, pshift, phpot, outw);
+    if (st_ok) {
+      const v4i o = {(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+      finish_chunk(o, o, (int64_t)pix * out.y_cs + oc, oc, a, out.y, lut);
+    }
+    if (!more) break;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // The network stem: at most 4 input channels, so one pixel is one dword and the kw taps of
 // a filter row are kw consecutive dwords of an input row.  A workgroup computes every
 // output channel (at most 64) of 128 consecutive pixels of ONE output row.  The kh input
@@ -3636,6 +3819,50 @@ const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {
 
 static int run_fc_one(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
 
+// Whether the row-segment depthwise kernel takes the layer, and its blocks: R row segments of
+// W lanes per wave, chosen for the fewest blocks per image.
+static bool dw_rows_plan(const tpuhip_conv_weights *w, const ConvArgs &a, DwRowsArgs *out) {
+  const tpuhip_conv_desc &d = w->d;
+  if (w->algo != ALGO_DEPTHWISE || !w->fast || d.relu_first || d.kh > 3 || d.kw > 3 || a.add_dst) return false;
+  // input rows and the row pitch fit the 24-bit multiply of the address arithmetic
+  if (d.ih >= (1 << 22) || (int64_t)d.iw * d.x_cs >= (1ll << 23) || (int64_t)d.ih * d.iw * d.x_cs >= (1ll << 31)) return false;
+  const int halo = (d.kw == 3 && d.sw == 1 && d.dw == 1) ? 1 : 0;
+  int64_t best = -1;
+  for (int rows = 1; rows <= 4; ++rows) {
+    const int width = 32 / rows, valid = width - 2 * halo;
+    if (valid < 1) continue;
+    const int64_t blocks = (int64_t)((d.oh + rows - 1) / rows) * ((d.ow + valid - 1) / valid);
+    if (best < 0 || blocks < best) {
+      best = blocks;
+      out->rows = rows; out->width = width; out->valid = valid; out->halo = halo;
+      out->rblocks = (d.oh + rows - 1) / rows;
+      out->xblocks = (d.ow + valid - 1) / valid;
+    }
+  }
+  if (best < 0 || best * d.n >= (1ll << 30) || out->rblocks >= (1 << 15) || out->xblocks >= (1 << 15)) return false;
+  out->nblocks = (int)(best * d.n);
+  auto magic = [](int dv) { return dv > 1 ? (uint32_t)(((1ull << 32) + dv - 1) / (uint64_t)dv) : 0u; };
+  out->magic_x = magic(out->xblocks);
+  out->magic_r = magic(out->rblocks);
+  out->magic_w = magic(out->width);
+  return true;
+}
+
+// the walk of the row-segment depthwise kernel for a launch of `wgs` workgroups (a multiple of 8)
+static void dw_rows_walk(DwRowsArgs *r, unsigned wgs, int n_cb) {
+  r->nslots = std::max(1, std::min((int)(wgs / 8) * 4 / n_cb, 1 << 15));
+  r->d_xb = r->nslots % r->xblocks;
+  r->d_rb = (r->nslots / r->xblocks) % r->rblocks;
+  r->d_n = r->nslots / (r->xblocks * r->rblocks);
+  const int per_xcd = (r->nblocks + 7) / 8;
+  for (int x = 0; x < 8; ++x) {
+    const int64_t b = (int64_t)x * per_xcd;
+    r->start_xb[x] = (int)(b % r->xblocks);
+    r->start_rb[x] = (int)((b / r->xblocks) % r->rblocks);
+    r->start_n[x] = (int)(b / ((int64_t)r->xblocks * r->rblocks));
+  }
+}
+
 static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y,
                     const PostOps &post) {
   if (w->fc_only) {
@@ -3685,6 +3912,23 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
     // one wave per (32-channel block, 32-pixel block); a resident set of workgroups, each
     // wave walking pixel blocks of its channel block
     const int n_cb = (a.ocw + 31) / 32, n_pb = (a.npix + 31) / 32;
+    DwRowsArgs dr;
+    if (dw_rows_plan(w, a, &dr)) {
+      // the row-segment form: up to 3 x 3 taps, the layer's overflow-free requantisation, no fused add
+      const int64_t waves_r = (int64_t)n_cb * dr.nblocks;
+      const unsigned wgs = 8 * (unsigned)std::max<int64_t>(
+          (n_cb + 3) / 4, std::min<int64_t>(ceil_div64(waves_r, 32), std::max(1, ctx->num_cu * (dr.halo ? 4 : 3) / 8)));
+      const bool shift = dr.halo == 1;
+      dw_rows_walk(&dr, wgs, n_cb);
+      a.magic_c16 = n_cb > 1 ? (uint32_t)(((1ull << 32) + n_cb - 1) / (uint64_t)n_cb) : 0u;   // wave index / n_cb
+      auto kernel = shift ? conv_depthwise_rows_kernel<true> : conv_depthwise_rows_kernel<false>;
+      if (ctx->prof_start)
+        hipExtLaunchKernelGGL(kernel, dim3(wgs), dim3(256), 0, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a, dr);
+      else
+        hipLaunchKernelGGL(kernel, dim3(wgs), dim3(256), 0, ctx->stream, a, dr);
+      TPUHIP_CHECK_HIP(hipGetLastError());
+      return TPUHIP_OK;
+    }
     const int64_t waves = (int64_t)n_cb * n_pb;
     // a multiple of 8 workgroups, every XCD's share holding at least one wave per channel block
     const unsigned blocks = 8 * (unsigned)std::max<int64_t>(
