@@ -86,6 +86,9 @@ struct ConvArgs {
   uint32_t x_bytes, w_bytes;      // sizes behind x and w (buffer descriptors)
   uint32_t magic_ow, magic_oh;    // ceil(2^32 / d): x / d == umulhi(x, magic) for x, d < 2^16
   int n_oc_tiles, n_tiles, tiles_per_xcd;
+  // ceil(2^32 / n_oc_tiles): tile / n_oc_tiles == umulhi(tile, magic) while tile * n_oc_tiles < 2^32;
+  // 0 where there is nothing to divide by (one channel tile) or the product leaves that range
+  uint32_t magic_oc_tiles;
   // persistent kernels: workgroups per XCD (a multiple of n_oc_tiles) and the pixel
   // advance between two tiles of one workgroup, split into (n, oh, ow) parts
   int wgs_per_xcd, pstep_pix, pstep_n, pstep_oh, pstep_ow;
@@ -113,27 +116,6 @@ struct ConvArgs {
   int8_t *lut_dst;
   Table256 lut;
 };
-
-// The kernel arguments (ConvArgs: six 64-byte lines before the table) arrive through the scalar
-// cache, and the compiler fetches fields where it first needs them: a handful of dependent
-// misses, one after the other, before the first address of the layer is known.  One load per
-// line, all in flight together and one wait, leaves every later fetch a hit.
-__device__ __forceinline__ void touch_kernargs() {
-  auto *ka = __builtin_amdgcn_kernarg_segment_ptr();
-  uint32_t t0, t1, t2, t3, t4, t5;
-  asm volatile(
-      "s_load_dword %0, %6, 0x0\n\t"
-      "s_load_dword %1, %6, 0x40\n\t"
-      "s_load_dword %2, %6, 0x80\n\t"
-      "s_load_dword %3, %6, 0xc0\n\t"
-      "s_load_dword %4, %6, 0x100\n\t"
-      "s_load_dword %5, %6, 0x140\n\t"
-      "s_waitcnt lgkmcnt(0)"
-      : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5)
-      : "s"(ka)
-      : "memory");
-}
-static_assert(sizeof(ConvArgs) >= 0x144, "touch_kernargs reads six lines of the argument segment");
 
 __device__ __forceinline__ int32_t epilogue(int32_t acc, int32_t bias, const QParam &p, int lo,
                                             int relu_first) {
@@ -482,6 +464,34 @@ __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32
 }
 constexpr uint32_t kOobOffset = 0x7fffffffu;
 
+// The kernel arguments (ConvArgs: six 64-byte lines before the table) arrive through the scalar
+// cache.  The compiler fetches a field where it first needs it, and what lies between kernel entry
+// and a layer's first load needs some thirty of them: a dozen and more scalar loads, each with its
+// own wait, one after the other (the first to touch a line a miss), before the first address of
+// the layer is known.  Naming them all as inputs of one (empty) asm statement makes them due at
+// one point: the loads go out together, merged where the fields are neighbours, behind a single
+// wait.
+__device__ __forceinline__ void gather_conv_args(const ConvArgs &a) {
+  asm volatile("" ::"s"(a.x), "s"(a.w), "s"(a.bias), "s"(a.qmult), "s"(a.qshift), "s"(a.qhpot), "s"(a.y), "s"(a.x_bytes),
+               "s"(a.w_bytes), "s"(a.tiles_per_xcd), "s"(a.n_tiles), "s"(a.n_oc_tiles), "s"(a.linear), "s"(a.x_cs),
+               "s"(a.npix), "s"(a.kp), "s"(a.c16), "s"(a.k16), "s"(a.has_lut), "s"(a.wgs_per_xcd), "s"(a.ow), "s"(a.oh),
+               "s"(a.ih), "s"(a.iw), "s"(a.sh), "s"(a.sw), "s"(a.pt), "s"(a.pl), "s"(a.magic_c16), "s"(a.magic_kw));
+}
+// tile index -> pixel tile (the channel tile is the remainder): a multiply where the host could
+// give its constant, the generic division otherwise
+__device__ __forceinline__ int pixel_tile_of(const ConvArgs &a, int tile) {
+  if (a.n_oc_tiles == 1) return tile;
+  if (a.magic_oc_tiles) return (int)__umulhi((uint32_t)tile, a.magic_oc_tiles);
+  return tile / a.n_oc_tiles;
+}
+
+// the second list: what the LDS kernels' tile walk and epilogue set-up read as well
+__device__ __forceinline__ void gather_conv_args_more(const ConvArgs &a) {
+  asm volatile("" ::"s"(a.magic_oc_tiles), "s"(a.split_oc), "s"(a.magic_ow), "s"(a.magic_oh), "s"(a.pstep_pix), "s"(a.stem_pw), "s"(a.lo),
+               "s"(a.ocw), "s"(a.qc64), "s"(a.qc64r), "s"(a.y_cs), "s"(a.store_y), "s"(a.add_dst), "s"(a.relu_first),
+               "s"(a.magic_pw), "s"(a.dh), "s"(a.dw), "s"(a.kh), "s"(a.kw));
+}
+
 // ---------------------------------------------------------------------------
 // depthwise kernel (g == ic == oc).  A lane owns 16 channels and walks pixels with a
 // fixed stride, so its filter taps and requant parameters stay in registers.  The
@@ -629,7 +639,8 @@ template <int BM, int BN, int WM, int WN, int BK, int DEPTH, int OCC, bool PERSI
           int MODE>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC > 0 ? OCC : 1))) void
 conv_mfma_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   constexpr bool UNI = MODE == kModeUniform;
   constexpr bool SMALLC = MODE == kModeSmallC;
   constexpr int NT = WM * WN * 64;
@@ -660,7 +671,7 @@ conv_mfma_kernel(ConvArgs a) {
   int ltile = (int)(blockIdx.x >> 3);                                   // tile index inside the XCD's run
   int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + ltile;
   if (logical >= a.n_tiles) return;
-  const int pix_tile = logical / a.n_oc_tiles;
+  const int pix_tile = pixel_tile_of(a, logical);
   const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;   // the same for every tile of a walk
   const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
   int pix0 = pix_tile * BN;
@@ -981,7 +992,8 @@ constexpr int kPatchBytesDyn = 65536;    // dynamic patch (256-byte K steps: the
 template <int BM, int BN, int BK, int DEPTH, int OCC, bool FAST>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_patch_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   constexpr int WM = 2, WN = 2, NT = 256;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   constexpr int CH = BK / 16;
@@ -1005,7 +1017,7 @@ conv_patch_kernel(ConvArgs a) {
   const int wm = wave / WN, wn = wave % WN;
   const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
   if (logical >= a.n_tiles) return;
-  const int pt = logical / a.n_oc_tiles;
+  const int pt = pixel_tile_of(a, logical);
   const int oc0 = (logical - pt * a.n_oc_tiles) * BM;
   const int img = pt / a.pstep_n;
   const int r0 = (pt - img * a.pstep_n) * a.pstep_pix;
@@ -1274,7 +1286,8 @@ __device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, 
 template <int BM, int BN, int WM, int WN, int KP, int SD, int OCC>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_pw_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   constexpr int NT = WM * WN * 64;
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
@@ -1303,7 +1316,7 @@ conv_pw_kernel(ConvArgs a) {
   int ltile = (int)(blockIdx.x >> 3);
   int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + ltile;
   if (logical >= a.n_tiles) return;
-  const int pix_tile = logical / a.n_oc_tiles;
+  const int pix_tile = pixel_tile_of(a, logical);
   const int oc0 = (logical - pix_tile * a.n_oc_tiles) * BM;
   const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
   int pix0 = pix_tile * BN;
@@ -1314,9 +1327,11 @@ conv_pw_kernel(ConvArgs a) {
   // ---- loader: this thread fetches chunk c of pixel rows lrow + RPP * u
   const int c = tid % CPRK, lrow = tid / CPRK;
   int lpix0 = pix0;                       // first pixel of the tile being fetched
-  int low = pix0 % a.ow;
-  int loh, ln;
-  {
+  // (stride 1: the input pixel has the output pixel's index, no coordinates at all -- three
+  // divisions and the per-row arithmetic out of the path to the first load)
+  int low = 0, loh = 0, ln = 0;
+  if (!a.linear) {
+    low = pix0 % a.ow;
     const int t = pix0 / a.ow;
     loh = t % a.oh;
     ln = t / a.oh;
@@ -1327,6 +1342,10 @@ conv_pw_kernel(ConvArgs a) {
     for (int u = 0; u < NXC; ++u) {
       const int row = lrow + RPP * u;
       const bool pv = exists && lpix0 + row < a.npix && (!XTAIL || row < BN);
+      if (a.linear) {
+        breg[u] = buffer_load16(xrsrc, pv ? (uint32_t)((lpix0 + row) * a.x_cs + c * 16) : kOobOffset);
+        continue;
+      }
       const uint32_t t1 = (uint32_t)(low + row);
       const uint32_t q1 = a.ow == 1 ? t1 : __umulhi(t1, a.magic_ow);
       const int ow = (int)(t1 - q1 * (uint32_t)a.ow);
@@ -1340,6 +1359,7 @@ conv_pw_kernel(ConvArgs a) {
   };
   auto advance_load = [&]() {
     lpix0 += a.pstep_pix;
+    if (a.linear) return;
     low += a.pstep_ow;
     if (low >= a.ow) { low -= a.ow; ++loh; }
     loh += a.pstep_oh;
@@ -1370,11 +1390,15 @@ conv_pw_kernel(ConvArgs a) {
     if (tid < BM) {
       // a workgroup whose result is clamped at 0 takes the constants of the short form
       const int32_t *c64 = out.lo == 0 ? a.qc64r : a.qc64;
-      qlds[2 * tid] = c64[2 * (oc0 + tid)];
-      qlds[2 * tid + 1] = c64[2 * (oc0 + tid) + 1];
-      qlds[2 * BM + tid] = a.qmult[oc0 + tid];
-      qlds[3 * BM + tid] = a.qshift[oc0 + tid] - (out.lo == 0 ? 1 : 0);
-      qlds[4 * BM + tid] = a.qhpot[oc0 + tid];
+      // all five in flight before the first is used (one trip to memory, not two)
+      const int32_t c_lo = c64[2 * (oc0 + tid)], c_hi = c64[2 * (oc0 + tid) + 1];
+      const int32_t qm = a.qmult[oc0 + tid], qs = a.qshift[oc0 + tid], qh = a.qhpot[oc0 + tid];
+      __builtin_amdgcn_sched_barrier(0);
+      qlds[2 * tid] = c_lo;
+      qlds[2 * tid + 1] = c_hi;
+      qlds[2 * BM + tid] = qm;
+      qlds[3 * BM + tid] = qs - (out.lo == 0 ? 1 : 0);
+      qlds[4 * BM + tid] = qh;
     }
     if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
 #pragma unroll
@@ -1503,7 +1527,8 @@ conv_pw_kernel(ConvArgs a) {
 template <int BM, int BN, int WM, int WN, int BK, int OCC>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_patch2_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   constexpr int NT = WM * WN * 64;
   constexpr int RD = 4;                       // filter tiles in flight in registers (even)
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -1528,7 +1553,7 @@ conv_patch2_kernel(ConvArgs a) {
   const int wm = wave / WN, wn = wave % WN;
   const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
   if (logical >= a.n_tiles) return;
-  const int pt = logical / a.n_oc_tiles;
+  const int pt = pixel_tile_of(a, logical);
   const int oc0 = (logical - pt * a.n_oc_tiles) * BM;
   const int img = pt / a.pstep_n;
   const int r0 = (pt - img * a.pstep_n) * a.pstep_pix;
@@ -1865,7 +1890,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SHIFT ? 4 :
 conv_depthwise_rows_kernel(ConvArgs a, DwRowsArgs r) {
   __shared__ uint32_t lutw[64];
   __shared__ int32_t qlds[4][160];   // per wave: 32 (low, high) pairs of c64, then mult, shift, hpot of 32 channels
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int p = lane & 31, fk = lane >> 5;
@@ -2212,7 +2238,8 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t x, uint32_t y) {
 }
 
 __global__ __launch_bounds__(512) void conv_stem_pool_kernel(ConvArgs a, StemPoolArgs s) {
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   extern __shared__ __attribute__((aligned(16))) uint32_t sp_smem[];
   uint32_t *const patch = sp_smem;                                              // [prows][pw]
   int8_t *const ctile = reinterpret_cast<int8_t *>(patch + s.prows * s.pw);      // [crows * ow][72]
@@ -2390,13 +2417,13 @@ __global__ __launch_bounds__(512) void conv_stem_pool_kernel(ConvArgs a, StemPoo
 template <int TM, int TN, int DEPTH, int OCC, bool FAST, bool UNI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_mfma_reg_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int logical_wg = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
   const int wt = logical_wg * 4 + wave;        // this wave's tile; oc tiles of a pixel tile adjacent
   if (wt >= a.n_tiles) return;                 // no barriers anywhere below
-  const int pix_tile = wt / a.n_oc_tiles;
+  const int pix_tile = pixel_tile_of(a, wt);
   const int oc_tile = wt - pix_tile * a.n_oc_tiles;
   const int oc0 = oc_tile * (TM * 32);
   const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
@@ -2553,13 +2580,13 @@ conv_mfma_reg_kernel(ConvArgs a) {
 template <int TM, int TN, int DEPTH, int OCC, bool FAST, bool UNI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_mfma_splitk_kernel(ConvArgs a) {
-  touch_kernargs();
+  gather_conv_args(a);
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int logical_wg = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
   const int wt = logical_wg;                   // the four waves share one tile and split K
   if (wt >= a.n_tiles) return;                 // uniform over the workgroup
-  const int pix_tile = wt / a.n_oc_tiles;
+  const int pix_tile = pixel_tile_of(a, wt);
   const int oc_tile = wt - pix_tile * a.n_oc_tiles;
   const int oc0 = oc_tile * (TM * 32);
   const OutRoute out = route_out(a, __builtin_amdgcn_readfirstlane(oc0));
@@ -2833,7 +2860,8 @@ constexpr int kFcOneWaves = 16;
 template <bool FAST>
 __global__ __launch_bounds__(64 * kFcOneWaves) void fc_one_kernel(ConvArgs a, int steps_per_wave) {
   __shared__ v4i part[kFcOneWaves * 4 * 64];
-  touch_kernargs();
+  gather_conv_args(a);
+  gather_conv_args_more(a);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int tile = (int)blockIdx.x;
   const int ob = tile % a.n_oc_tiles, pb = tile / a.n_oc_tiles;
@@ -3391,6 +3419,7 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
     a.magic_oh = d.oh > 1 ? (uint32_t)(((1ull << 32) + d.oh - 1) / (uint64_t)d.oh) : 0;
     a.n_oc_tiles = w->ocp / t.bm;
     a.n_tiles = (int)(ceil_div64(a.npix, t.bn) * a.n_oc_tiles);
+    a.magic_oc_tiles = 0;   // set below, once the tile count is final
     // workgroups per XCD (a workgroup of the LDS-free kernel holds four wave tiles)
     const int n_wgs = t.reg == 1 ? (a.n_tiles + 3) / 4 : a.n_tiles;
     a.tiles_per_xcd = (n_wgs + 7) / 8;
@@ -3429,6 +3458,9 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
       a.pstep_n = a.pstep_pix / d.ow / d.oh;
     }
   }
+  if (w->algo == ALGO_MFMA && a.n_oc_tiles > 1 &&
+      ((int64_t)a.n_tiles + 8 * (int64_t)a.tiles_per_xcd) * a.n_oc_tiles < (1ll << 32))
+    a.magic_oc_tiles = (uint32_t)(((1ull << 32) + a.n_oc_tiles - 1) / (uint64_t)a.n_oc_tiles);
   *out = a;
 }
 
