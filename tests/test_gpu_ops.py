@@ -727,6 +727,12 @@ def test_conv_depthwise_row_segments(ctx, case):
         assert np.array_equal(ctx.to_nchw(yt), want)
         assert np.array_equal(ctx.to_nchw(tt), O.lut_i8(want, table))
         assert tt.cs == c or not ctx.raw(tt)[..., c:].any()
+        # the table's result alone: the conv result is not written
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, tt.ptr, 0x33, tt.nbytes))
+        ctx.conv_post(wh, xt, None, table, tt)
+        assert (ctx.raw(yt) == 0x55).all()
+        assert np.array_equal(ctx.to_nchw(tt), O.lut_i8(want, table))
         ctx.conv_weights_destroy(wh)
         for t in (xt, yt, tt):
             t.free()
