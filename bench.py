@@ -80,6 +80,25 @@ def _timed(fn, seconds, max_passes=20):
     return passes, time.perf_counter() - t0
 
 
+def activation_stats(ops, tensors, guards):
+    """What the parity check ran on: share of zero and of saturated (-128 / 127) bytes over every int8
+    tensor of the graph as the oracle computed it, and the largest fp32-exactness guard of a conv / fc
+    output (sum |a * w| + |bias|, which has to stay below 2^24 for the reference's fp32 sums to be exact)."""
+    import numpy as np
+    total = zeros = saturated = 0
+    for op in ops:
+        a = tensors.get(op.name)
+        if a is None or a.dtype != np.int8:
+            continue
+        total += a.size
+        zeros += int(np.count_nonzero(a == 0))
+        saturated += int(np.count_nonzero((a == 127) | (a == -128)))
+    if not total:
+        return None
+    return {"int8_elements": total, "zero_frac": round(zeros / total, 4), "saturated_frac": round(saturated / total, 4),
+            "fp32_guard_max": int(max(guards.values())) if guards else None}
+
+
 def cpu_baseline(graph_fn, images, seconds=12.0, legs=("dataflow_4thr", "dataflow_all", "oracle_all"),
                  keep_results=None):
     """CPU restatements of the reference on a bounded sample of the same workload, on this host:
@@ -386,6 +405,10 @@ def main():
         out["parity"] = {"outputs_equal_oracle": bool(outputs_ok), "layers_exact": exact, "layers_total": len(g.ops),
                          "images_checked": sample,
                          "fp32_guard_held": bool(max(guards.values()) < (1 << 24)) if guards else None}
+        try:
+            out["parity"]["activations"] = activation_stats(g.ops, want, guards)
+        except Exception as e:      # statistics only: never in the way of the line
+            out["parity"]["activations"] = {"error": str(e)}
     if mk is not None:
         mk.close()
     m.close()
