@@ -20,7 +20,9 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # conv tile variant per layer as an earlier run of this benchmark chose them by timing: used
 # by default so that runs, and the committed profile of this command, execute the same kernels
-RECORDED_TILES = {"cfg3": os.path.join("tpu_compiler_amd", "tiles", "cfg3_b32.json")}
+RECORDED_TILES = {"cfg3": os.path.join("tpu_compiler_amd", "tiles", "cfg3_b32.json"),
+                  "cfg4": os.path.join("tpu_compiler_amd", "tiles", "cfg4_b64.json"),
+                  "cfg5": os.path.join("tpu_compiler_amd", "tiles", "cfg5_b8.json")}
 
 
 def conv_bytes(op, graph, fused_add=None, stored=True):
@@ -155,7 +157,7 @@ def main():
     ap.add_argument("--save-tiles", default="", help="write the conv tile chosen for every layer")
     ap.add_argument("--tiles", default="", help="use the conv tiles recorded in this file instead "
                                                 "of timing the variants (repeatable profiling); "
-                                                "default for cfg3: " + RECORDED_TILES["cfg3"])
+                                                "default for cfg3 / cfg4 / cfg5: the files under tpu_compiler_amd/tiles")
     ap.add_argument("--autotune", action="store_true",
                     help="time the conv tile variants on first use even where a recorded choice exists")
     ap.add_argument("--keep-all", action="store_true",
