@@ -66,3 +66,19 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     assert d["host_io"]["ms_per_step"] > d["ms_per_step"] and d["host_io"]["host_bytes_in"] > 0
     c = d["cpu_baseline"]
     assert c["kind"] in ("port", "reference") and c["value"] > 0 and c["cores"] >= 1 and c["sample"]
+
+
+def test_activation_statistics_of_the_parity_object():
+    sys.path.insert(0, ROOT)
+    import numpy as np
+    import bench
+
+    class Op:
+        def __init__(self, name):
+            self.name = name
+    a = np.array([0, 0, 127, -128, 5, -5, 1, 2], np.int8)
+    b = np.zeros(8, np.float32)                      # an fp32 edge tensor: not counted
+    s = bench.activation_stats([Op("a"), Op("b"), Op("missing")], {"a": a, "b": b}, {"a": 1000, "x": 77})
+    assert s == {"int8_elements": 8, "zero_frac": 0.25, "saturated_frac": 0.25, "fp32_guard_max": 1000}
+    assert bench.activation_stats([Op("b")], {"b": b}, {}) is None
+
