@@ -82,3 +82,21 @@ def test_activation_statistics_of_the_parity_object():
     assert s == {"int8_elements": 8, "zero_frac": 0.25, "saturated_frac": 0.25, "fp32_guard_max": 1000}
     assert bench.activation_stats([Op("b")], {"b": b}, {}) is None
 
+
+
+def test_op_bench_describes_itself_without_a_gpu():
+    r = subprocess.run([sys.executable, "-m", "tpu_compiler_amd.op_bench", "--help"], capture_output=True, text=True,
+                       timeout=120, cwd=ROOT)
+    assert r.returncode == 0 and "--iters" in r.stdout
+
+
+@pytest.mark.gpu
+def test_op_bench_prints_a_row_per_op():
+    r = subprocess.run([sys.executable, "-m", "tpu_compiler_amd.op_bench", "--iters", "3"], capture_output=True,
+                       text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rows = [l for l in r.stdout.splitlines() if " TB/s " in l]
+    assert len(rows) == 14
+    for l in rows:
+        us = float(l.split(" us (host")[0].split()[-1])
+        assert 1.0 < us < 1000.0, l
