@@ -18,6 +18,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense INT8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+LAUNCH_FLOOR_US = 2.4     # an empty kernel behind another on one stream, measured (profiles/machine_ceilings.txt)
 # conv tile variant per layer as an earlier run of this benchmark chose them by timing: used
 # by default so that runs, and the committed profile of this command, execute the same kernels
 RECORDED_TILES = {"cfg3": os.path.join("tpu_compiler_amd", "tiles", "cfg3_b32.json"),
@@ -252,6 +253,10 @@ def main():
             convs = [i for i in op.inputs if g.by_name[i].type == "tpu.conv_2d"]
             if convs:
                 fused_add[max(convs, key=lambda n: order[n])] = op
+    # likewise a max pool that launched nothing runs inside its producing conv's launch
+    fused_pool = {op.inputs[0]: op for op in g.ops
+                  if op.type == "tpu.pool_max_2d" and ms_of.get(op.name, 1) == 0
+                  and g.by_name[op.inputs[0]].type == "tpu.conv_2d"}
     for name, algo, ms in rows:
         op = g.by_name[name]
         if op.type in ("tpu.conv_2d", "tpu.fully_connected"):
@@ -262,8 +267,12 @@ def main():
             d["ms"] += ms
             d["ops"] += 2.0 * op.macs
             add = fused_add.get(name)
-            stored = args.keep_all or add is None or readers.get(name, 0) > 1 or name in g.outputs
+            pool = fused_pool.get(name)
+            stored = (args.keep_all or (add is None and pool is None) or readers.get(name, 0) > 1
+                      or name in g.outputs)
             d["bytes"] += conv_bytes(op, g, add, stored) - (int(np.prod(g.by_name[op.inputs[0]].shape)) if rides else 0)
+            if pool is not None:
+                d["bytes"] += int(np.prod(pool.shape))
             d["launches"] += 0 if rides else 1
     mfma = {k: v for k, v in by_algo.items() if k.startswith("mfma")}
     conv_ms = sum(v["ms"] for v in mfma.values())
@@ -285,6 +294,15 @@ def main():
                         "achieved": round(conv_ops / (conv_ms / 1e3) / 1e12, 2),
                         "frac": round(conv_ops / (conv_ms / 1e3) / 1e12 / PEAK_INT8_TOPS, 4),
                         "ms": round(conv_ms, 4)}}
+        # the same launches against the other roof: below the ridge (peak ops / peak bytes) a kernel that
+        # moved only its algorithmic bytes at the HBM peak would still be slower than its MFMAs
+        intensity = dom["ops"] / dom["bytes"]
+        ridge = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)
+        gbs = dom["bytes"] / (dom["ms"] / 1e3) / 1e9
+        roofline["against_hbm"] = {"ops_per_byte": round(intensity, 1), "ridge_ops_per_byte": round(ridge, 1),
+                                   "lower_roof": "hbm" if intensity < ridge else "mfma",
+                                   "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / PEAK_HBM_GBS, 4)}
     # HBM bytes per launch of that kernel, from the committed rocprofv3 counter passes
     # (FETCH_SIZE + WRITE_SIZE, scaled against a plain copy kernel) of this same workload
     traffic_file = os.path.join(ROOT, "profiles", "resnet50_b32_bench_traffic.json")
@@ -302,6 +320,25 @@ def main():
             continue
         hbm_bytes += sum(int(np.prod(g.by_name[i].shape)) for i in op.inputs) + int(np.prod(op.shape))
         hbm_ms += ms
+    # what one op per launch can reach at best: every launch's algorithmic bytes at the HBM peak (or its
+    # operations at the MFMA peak, whichever takes longer) behind one launch floor each
+    floor_ms, n_launches, graph_bytes = 0.0, 0, 0.0
+    for d in by_algo.values():
+        floor_ms += max(d["bytes"] / (PEAK_HBM_GBS * 1e9), d["ops"] / (PEAK_INT8_TOPS * 1e12)) * 1e3
+        n_launches += d["launches"]
+        graph_bytes += d["bytes"]
+    n_other = sum(1 for name, algo, ms in rows
+                  if ms > 0 and g.by_name[name].type not in ("tpu.conv_2d", "tpu.fully_connected", "tpu.input"))
+    floor_ms += hbm_bytes / (PEAK_HBM_GBS * 1e9) * 1e3
+    n_launches += n_other
+    graph_bytes += hbm_bytes
+    launch_ms = n_launches * LAUNCH_FLOOR_US / 1e3
+    graph_floor = {"launches": n_launches, "algorithmic_bytes": int(graph_bytes),
+                   "data_ms": round(floor_ms, 4), "launch_ms": round(launch_ms, 4),
+                   "floor_ms": round(floor_ms + launch_ms, 4),
+                   "step_over_floor": round(ms_per_step / (floor_ms + launch_ms), 2),
+                   "what": "per launch max(algorithmic bytes at %g GB/s, operations at %g TOP/s) + %.1f us "
+                           "(an empty dependent launch)" % (PEAK_HBM_GBS, PEAK_INT8_TOPS, LAUNCH_FLOOR_US)}
     if args.per_layer:
         for name, algo, ms in rows:
             op = g.by_name[name]
@@ -329,6 +366,7 @@ def main():
         "ops_per_step": total_ops,
         "event_ms_per_step": round(ev_ms.value / args.steps, 4),
         "roofline": roofline,
+        "graph_floor": graph_floor,
         "hbm_bound_ops": None if hbm_ms <= 0 else {
             "achieved": round(hbm_bytes / (hbm_ms / 1e3) / 1e9, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
             "frac": round(hbm_bytes / (hbm_ms / 1e3) / 1e9 / PEAK_HBM_GBS, 4), "ms": round(hbm_ms, 4)},

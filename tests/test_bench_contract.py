@@ -62,6 +62,9 @@ def test_bench_prints_one_json_line_with_the_contract_keys():
     assert np.isclose(d["value"], d["config"]["global_batch"] / (d["ms_per_step"] / 1e3), rtol=1e-2)
     r_ = d["roofline"]
     assert r_["bound"] in ("hbm", "mfma") and np.isclose(r_["frac"], r_["achieved"] / r_["peak"], atol=1e-3)
+    f = d["graph_floor"]
+    assert f["launches"] >= 2 and np.isclose(f["floor_ms"], f["data_ms"] + f["launch_ms"], atol=2e-4)
+    assert f["step_over_floor"] >= 1.0 and r_["against_hbm"]["lower_roof"] in ("hbm", "mfma")
     # the leg with host buffers in and out every step is reported beside the value, and is slower
     assert d["host_io"]["ms_per_step"] > d["ms_per_step"] and d["host_io"]["host_bytes_in"] > 0
     c = d["cpu_baseline"]
