@@ -1095,6 +1095,24 @@ def test_concat_axes(ctx, axis):
     assert np.array_equal(ctx.to_nchw(yt), want)
 
 
+@pytest.mark.parametrize("channels, in_cs, y_cs", [((16, 48), (None, None), None), ((32, 16, 16, 64), (None, 32, None, 80), None),
+                                                   ((128, 256), (None, None), 400), ((16, 16, 16, 16, 16), (None,) * 5, None)])
+def test_concat_whole_channel_groups(ctx, channels, in_cs, y_cs):
+    """channel concat of inputs with whole 16-channel groups (one launch for two to four inputs; the fifth
+    case has too many and takes a launch per input), with padded strides on either side and identity rescaling"""
+    rng = np.random.default_rng(131 + len(channels))
+    xs = [rnd_i8(rng, (2, c, 7, 9)) for c in channels]
+    want = O.concat_i8(xs, 1)
+    ts = [ctx.from_nchw(a, cs) for a, cs in zip(xs, in_cs)]
+    yt = ctx.tensor(want.shape, y_cs)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0, yt.nbytes))
+    ctx.concat(ts, 1, yt, [0] * len(xs), [1] * len(xs), False)
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., want.shape[1]:].any()
+    for t in ts + [yt]:
+        t.free()
+
+
 def test_concat_channels_unaligned_requant_relu(ctx):
     rng = np.random.default_rng(53)
     xs = [rnd_i8(rng, (2, c, 4, 5)) for c in (24, 7, 40)]

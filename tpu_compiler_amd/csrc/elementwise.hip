@@ -165,6 +165,35 @@ __global__ __launch_bounds__(kThreads) void lut_byte_kernel(LutArgs a, Table256 
   }
 }
 
+// channel concat of up to four inputs whose channel counts are multiples of 16, bytes unchanged:
+// one launch, a lane moves one 16-byte group of one output pixel
+struct ConcatArgs {
+  const int8_t *x[4];
+  int8_t *y;
+  int64_t pixels;
+  int cs[4];       // channel stride of each input
+  int start[5];    // first 16-byte group of each input within an output pixel; start[n] = groups per pixel
+  int n, y_cs;
+};
+
+__global__ __launch_bounds__(kThreads) void concat_channels_kernel(ConcatArgs a) {
+  const int g16 = a.start[a.n];
+  const int64_t total = a.pixels * g16;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t pix = i / g16;
+    const int g = (int)(i - pix * g16);
+    // which input the group comes from: selects, so that no array is indexed by a lane's value
+    const int8_t *src = a.x[0];
+    int cs = a.cs[0], first = 0;
+    if (a.n > 1 && g >= a.start[1]) { src = a.x[1]; cs = a.cs[1]; first = a.start[1]; }
+    if (a.n > 2 && g >= a.start[2]) { src = a.x[2]; cs = a.cs[2]; first = a.start[2]; }
+    if (a.n > 3 && g >= a.start[3]) { src = a.x[3]; cs = a.cs[3]; first = a.start[3]; }
+    const v4i v = *reinterpret_cast<const v4i *>(src + pix * cs + (g - first) * 16);
+    *reinterpret_cast<v4i *>(a.y + pix * a.y_cs + g * 16) = v;
+  }
+}
+
 // zero the channels [c0, c1) of every pixel
 __global__ __launch_bounds__(kThreads) void zero_channels_kernel(int8_t *y, int64_t pixels, int cs,
                                                                  int c0, int c1) {
@@ -605,6 +634,32 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
   }
   const int N = out_dims[0], Cc = out_dims[1], H = out_dims[2], W = out_dims[3];
   TPUHIP_REQUIRE(y_cs >= Cc && y_cs % 16 == 0, "concat: bad output channel stride %d", y_cs);
+
+  // Channel concat that changes no byte (no rescaling that is not the identity; a ReLU would change
+  // negative bytes) of two to four inputs with whole 16-channel groups: one launch for all of them.
+  bool plain = axis == 1 && nin >= 2 && nin <= 4 && !do_relu;
+  for (int i = 0; i < nin && plain; ++i) {
+    plain = in_dims[4 * i + 1] % 16 == 0;
+    if (need_quant && !(multiplier[i] == 1 && rshift[i] == 0)) plain = false;
+  }
+  if (plain) {
+    ConcatArgs a{};
+    a.y = (int8_t *)y;
+    a.pixels = (int64_t)N * H * W;
+    a.n = nin;
+    a.y_cs = y_cs;
+    for (int i = 0; i < nin; ++i) {
+      a.x[i] = (const int8_t *)xs[i];
+      a.cs[i] = in_cs[i];
+      a.start[i + 1] = a.start[i] + in_dims[4 * i + 1] / 16;
+    }
+    // the groups of a pixel are exactly its Cc channels, and Cc <= y_cs was checked above
+    TPUHIP_REQUIRE(a.start[nin] * 16 == Cc, "concat: channel groups %d do not add up to %d channels", a.start[nin], Cc);
+    TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+    launch(ctx, concat_channels_kernel, dim3(grid_for(a.pixels * a.start[nin], kThreads * 4)), dim3(kThreads), a);
+    TPUHIP_CHECK_HIP(hipGetLastError());
+    return TPUHIP_OK;
+  }
 
   // Each input goes through a 256-entry table: requant (unless m == 1, r == 0) then ReLU
   // -- both pure functions of the int8 input (core/concat.cpp:66-88).
