@@ -1083,6 +1083,7 @@ def test_concat_axes(ctx, axis):
     rng = np.random.default_rng(47 + axis)
     base = [2, 32, 5, 6]
     shapes = []
+    # three inputs that change no byte: one launch along any axis
     for extent in (3, 1, 4) if axis != 1 else (32, 16, 48):
         s = list(base)
         s[axis] = extent

@@ -165,32 +165,35 @@ __global__ __launch_bounds__(kThreads) void lut_byte_kernel(LutArgs a, Table256 
   }
 }
 
-// channel concat of up to four inputs whose channel counts are multiples of 16, bytes unchanged:
-// one launch, a lane moves one 16-byte group of one output pixel
+// concat of up to four inputs that changes no byte, along any axis: in channels-last memory every
+// axis is "for each outer index, the inputs' chunks one after the other" (outer = pixel for the
+// channel axis, image row for w, image for h, nothing for n), chunks whole 16-byte groups.
+// One launch, a lane moves one 16-byte group.
 struct ConcatArgs {
   const int8_t *x[4];
   int8_t *y;
-  int64_t pixels;
-  int cs[4];       // channel stride of each input
-  int start[5];    // first 16-byte group of each input within an output pixel; start[n] = groups per pixel
-  int n, y_cs;
+  int64_t outer;       // outer indices
+  int64_t stride[4];   // bytes from one outer index to the next in each input
+  int64_t y_stride;    // ... in the output
+  int64_t start[5];    // first 16-byte group of each input's chunk within an output chunk; start[n] = groups per chunk
+  int n;
 };
 
-__global__ __launch_bounds__(kThreads) void concat_channels_kernel(ConcatArgs a) {
-  const int g16 = a.start[a.n];
-  const int64_t total = a.pixels * g16;
+__global__ __launch_bounds__(kThreads) void concat_chunks_kernel(ConcatArgs a) {
+  const int64_t g16 = a.start[a.n];
+  const int64_t total = a.outer * g16;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
-    const int64_t pix = i / g16;
-    const int g = (int)(i - pix * g16);
+    const int64_t o = i / g16;
+    const int64_t g = i - o * g16;
     // which input the group comes from: selects, so that no array is indexed by a lane's value
     const int8_t *src = a.x[0];
-    int cs = a.cs[0], first = 0;
-    if (a.n > 1 && g >= a.start[1]) { src = a.x[1]; cs = a.cs[1]; first = a.start[1]; }
-    if (a.n > 2 && g >= a.start[2]) { src = a.x[2]; cs = a.cs[2]; first = a.start[2]; }
-    if (a.n > 3 && g >= a.start[3]) { src = a.x[3]; cs = a.cs[3]; first = a.start[3]; }
-    const v4i v = *reinterpret_cast<const v4i *>(src + pix * cs + (g - first) * 16);
-    *reinterpret_cast<v4i *>(a.y + pix * a.y_cs + g * 16) = v;
+    int64_t stride = a.stride[0], first = 0;
+    if (a.n > 1 && g >= a.start[1]) { src = a.x[1]; stride = a.stride[1]; first = a.start[1]; }
+    if (a.n > 2 && g >= a.start[2]) { src = a.x[2]; stride = a.stride[2]; first = a.start[2]; }
+    if (a.n > 3 && g >= a.start[3]) { src = a.x[3]; stride = a.stride[3]; first = a.start[3]; }
+    const v4i v = *reinterpret_cast<const v4i *>(src + o * stride + (g - first) * 16);
+    *reinterpret_cast<v4i *>(a.y + o * a.y_stride + g * 16) = v;
   }
 }
 
@@ -635,28 +638,33 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
   const int N = out_dims[0], Cc = out_dims[1], H = out_dims[2], W = out_dims[3];
   TPUHIP_REQUIRE(y_cs >= Cc && y_cs % 16 == 0, "concat: bad output channel stride %d", y_cs);
 
-  // Channel concat that changes no byte (no rescaling that is not the identity; a ReLU would change
-  // negative bytes) of two to four inputs with whole 16-channel groups: one launch for all of them.
-  bool plain = axis == 1 && nin >= 2 && nin <= 4 && !do_relu;
+  // A concat that changes no byte (no rescaling that is not the identity; a ReLU would change negative
+  // bytes) of two to four inputs is one launch for all of them: along the channels when every input
+  // has whole 16-channel groups; along n, h or w when all tensors have the channel stride of their channel count (a chunk
+  // is then a run of whole pixels, pad channels included, which are zero in every input).
+  bool plain = nin >= 2 && nin <= 4 && !do_relu;
   for (int i = 0; i < nin && plain; ++i) {
-    plain = in_dims[4 * i + 1] % 16 == 0;
+    plain = axis == 1 ? in_dims[4 * i + 1] % 16 == 0 : (in_cs[i] == y_cs && y_cs == round_up(Cc, 16));
     if (need_quant && !(multiplier[i] == 1 && rshift[i] == 0)) plain = false;
   }
   if (plain) {
     ConcatArgs a{};
     a.y = (int8_t *)y;
-    a.pixels = (int64_t)N * H * W;
     a.n = nin;
-    a.y_cs = y_cs;
+    // bytes of one step along the axis, and of everything inside one outer index of the output
+    const int64_t unit = axis == 1 ? 1 : axis == 3 ? y_cs : axis == 2 ? (int64_t)W * y_cs : (int64_t)H * W * y_cs;
+    a.outer = axis == 1 ? (int64_t)N * H * W : axis == 3 ? (int64_t)N * H : axis == 2 ? N : 1;
+    a.y_stride = axis == 1 ? y_cs : unit * out_dims[axis];
     for (int i = 0; i < nin; ++i) {
       a.x[i] = (const int8_t *)xs[i];
-      a.cs[i] = in_cs[i];
-      a.start[i + 1] = a.start[i] + in_dims[4 * i + 1] / 16;
+      a.stride[i] = axis == 1 ? in_cs[i] : unit * in_dims[4 * i + axis];
+      a.start[i + 1] = a.start[i] + unit * in_dims[4 * i + axis] / 16;
     }
-    // the groups of a pixel are exactly its Cc channels, and Cc <= y_cs was checked above
-    TPUHIP_REQUIRE(a.start[nin] * 16 == Cc, "concat: channel groups %d do not add up to %d channels", a.start[nin], Cc);
+    // the chunks of an outer index fill the output's: Cc channels of a pixel, or all of its rows / pixels
+    TPUHIP_REQUIRE(a.start[nin] * 16 == unit * out_dims[axis] && a.start[nin] * 16 <= a.y_stride,
+                   "concat: chunks of %lld groups do not fill axis %d", (long long)a.start[nin], axis);
     TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
-    launch(ctx, concat_channels_kernel, dim3(grid_for(a.pixels * a.start[nin], kThreads * 4)), dim3(kThreads), a);
+    launch(ctx, concat_chunks_kernel, dim3(grid_for(a.outer * a.start[nin], kThreads * 4)), dim3(kThreads), a);
     TPUHIP_CHECK_HIP(hipGetLastError());
     return TPUHIP_OK;
   }
