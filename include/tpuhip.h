@@ -188,6 +188,27 @@ int tpuhip_conv2d_prepack_pair(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc_a, 
                                const int32_t *multiplier_b, const int32_t *rshift_b,
                                tpuhip_conv_weights **out);
 int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y_a, void *y_b);
+/* Two Conv2DOpKernel::invoke calls (core/conv.cpp:80-104), with an EltwiseAddOpKernel::i8_invoke
+ * (core/eltwise.cpp:52-85) between them, as one launch: conv A and conv B are unpadded 1x1 / stride 1
+ * convs, B reads what A produced -- or, with an add, the sum of A's result and add_src.  In a residual
+ * network: the 1x1 expansion + add that closes a bottleneck block and the 1x1 reduction that opens the
+ * next; the sum is written once and not read back.  Shapes covered: A 33..64 -> 256 channels with
+ * B 256 -> 64, A 65..128 -> 512 with B 512 -> 128, dense channel strides, right shifts of at least 1
+ * and sums that cannot overflow the rounding (tpuhip_conv2d_can_chain answers for the shapes; prepack
+ * returns TPUHIP_ERR_UNSUPPORTED otherwise).  y_a (A's own result) and add_out may be NULL: not
+ * written.  Results are those of the separate calls.  No counterpart in the reference (one kernel per
+ * op). */
+typedef struct tpuhip_conv_chain tpuhip_conv_chain;
+int tpuhip_conv2d_can_chain(const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b);
+int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b,
+                                const int8_t *filter_a, const int32_t *bias_a, const int32_t *multiplier_a,
+                                const int32_t *rshift_a, const int8_t *filter_b, const int32_t *bias_b,
+                                const int32_t *multiplier_b, const int32_t *rshift_b, tpuhip_conv_chain **out);
+int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *chain);
+/* f == NULL or f->enable == 0: no add, B reads A's result (add_src / add_out ignored) */
+int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y_a,
+                           const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b);
+const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *chain);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */

@@ -178,6 +178,13 @@ PROTOTYPES.update({
                                              C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                              C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "tpuhip_conv2d_pair_i8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "tpuhip_conv2d_can_chain": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]),
+    "tpuhip_conv2d_chain_prepack": (C.c_int, [C.c_void_p, C.POINTER(ConvDesc), C.POINTER(ConvDesc), C.c_void_p,
+                                              C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                              C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "tpuhip_conv2d_chain_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "tpuhip_conv2d_chain_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd), C.c_void_p]),
+    "tpuhip_conv2d_chain_name": (C.c_char_p, [C.c_void_p]),
     "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
     "tpuhip_module_weight_file": (C.c_char_p, [C.c_void_p]),
     "tpuhip_module_num_ops": (C.c_int, [C.c_void_p]),
@@ -444,6 +451,41 @@ class Context:
 
     def conv_pair(self, w, x, y_a, y_b):
         self._ck(self.lib.tpuhip_conv2d_pair_i8(self.h, w, x.ptr, y_a.ptr, y_b.ptr))
+
+    def conv_can_chain(self, desc_a, desc_b):
+        return bool(self.lib.tpuhip_conv2d_can_chain(C.byref(desc_a), C.byref(desc_b)))
+
+    def conv_chain_prepack(self, desc_a, desc_b, a, b):
+        """a, b: (filter int8, bias int32 or None, multiplier int32, rshift int32) of two pointwise convs,
+        the second reading what the first (or the add behind it) produces -> one handle for conv_chain"""
+        keep, ptrs = [], []
+        for filt, bias, mult, rshift in (a, b):
+            arrs = [np.ascontiguousarray(filt, dtype=np.int8),
+                    None if bias is None else np.ascontiguousarray(bias, dtype=np.int32),
+                    np.ascontiguousarray(mult, dtype=np.int32), np.ascontiguousarray(rshift, dtype=np.int32)]
+            keep += arrs
+            ptrs += [None if x is None else x.ctypes.data for x in arrs]
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_conv2d_chain_prepack(self.h, C.byref(desc_a), C.byref(desc_b), *ptrs,
+                                                      C.byref(w)))
+        return w.value
+
+    def conv_chain(self, ch, x, y_b, y_a=None, add=None):
+        """add = (src, out or None, m_src, m_conv, rshift, relu)"""
+        f = None
+        src = out = None
+        if add is not None:
+            src, out, m_src, m_conv, rshift, relu = add
+            f = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(relu))
+        self._ck(self.lib.tpuhip_conv2d_chain_i8(
+            self.h, ch, x.ptr, None if y_a is None else y_a.ptr, None if src is None else src.ptr,
+            None if out is None else out.ptr, None if f is None else C.byref(f), y_b.ptr))
+
+    def conv_chain_destroy(self, ch):
+        self._ck(self.lib.tpuhip_conv2d_chain_destroy(self.h, ch))
+
+    def conv_chain_name(self, ch):
+        return self.lib.tpuhip_conv2d_chain_name(ch).decode()
 
     def fc_prepack(self, m, k, n, x_cs, y_cs, do_relu, filt, bias, mult, rshift):
         filt = np.ascontiguousarray(filt, dtype=np.int8)

@@ -11,6 +11,7 @@
 // quantizeActivationInt8PerChannelMultiplierAndRShift
 // (lib/Dialect/TPU/Quantization/QuantizationArithmetic.cpp:849-871).
 #include "common.hpp"
+#include "conv_epilogue.hpp"
 
 #include <map>
 #include <mutex>
@@ -26,8 +27,6 @@
 
 using namespace tpuhip;
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum ConvAlgo { ALGO_AUTO = 0, ALGO_DIRECT = 1, ALGO_MFMA = 2, ALGO_DEPTHWISE = 3, ALGO_DEPTHWISE_DOT = 4,
                 ALGO_STEM = 5 };
@@ -188,30 +187,6 @@ __device__ __forceinline__ int32_t sbyte(int32_t word, int i) {
 // consecutive output channels of one pixel: one 16-byte store per block.
 // ---------------------------------------------------------------------------
 
-// tile-local weight row (as the MFMA sees it) -> tile-local output channel
-__host__ __device__ inline int mfma_row_to_oc(int row, int tm) {
-  const int wave_rows = tm * 32;
-  const int wrow = row % wave_rows, wbase = row - wrow;
-  const int i = wrow / 32, ri = wrow % 32;
-  const int fk = (ri >> 2) & 1;
-  const int r = (ri >> 3) * 4 + (ri & 3);
-  return wbase + fk * 16 * tm + i * 16 + r;
-}
-
-typedef short v2s __attribute__((ext_vector_type(2)));
-typedef unsigned short v2us __attribute__((ext_vector_type(2)));
-
-// four int32 -> four saturated int8 in one dword; lo is -128 or 0 (fused ReLU)
-__device__ __forceinline__ uint32_t pack_sat4(int32_t a, int32_t b, int32_t c, int32_t d, int lo) {
-  v2s p0 = __builtin_amdgcn_cvt_pk_i16(a, b);
-  v2s p1 = __builtin_amdgcn_cvt_pk_i16(c, d);
-  const v2s vlo = {(short)lo, (short)lo}, vhi = {127, 127};
-  p0 = __builtin_elementwise_min(__builtin_elementwise_max(p0, vlo), vhi);
-  p1 = __builtin_elementwise_min(__builtin_elementwise_max(p1, vlo), vhi);
-  return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, p1), __builtin_bit_cast(uint32_t, p0),
-                               0x06040200u);
-}
-
 // FAST: every channel has 1 <= rshift <= 31 and |acc + bias| + 1 + 2^(rshift-1) < 2^31
 // (proved on the host from the weights), so RoundingDivideByPOT is
 // (x + 2^(e-1) - (x < 0)) >> e without overflow.
@@ -286,59 +261,9 @@ __device__ __forceinline__ void finish_chunk(v4i o, const v4i &sv, int64_t off, 
     }
     if (a.lut_dst) *reinterpret_cast<v4i *>(a.lut_dst + off) = o;
   }
-  if (a.add_dst && a.add_pk) {
-    // EltwiseAdd (core/eltwise.cpp:52-85, integer form) two outputs per instruction: the bytes
-    // of both operands widen to packed int16 (even and odd bytes apart), src * m_src + y * m_conv
-    // + 2^(r-1) stays inside int16 (the host checked |m| <= 127 and r <= 8), and ReLU / lower
-    // saturation (a floor before the shift), shift and upper saturation are packed ops too
-    const int r = a.add_rshift;
-    const short rnd = (short)(r > 0 ? (1 << (r - 1)) : 0);
-    const short fl = (short)(a.add_relu ? 0 : -(128 << r));
-    const v2s msrc = {(short)a.add_m_src, (short)a.add_m_src}, mconv = {(short)a.add_m_conv, (short)a.add_m_conv};
-    const v2s rnd2 = {rnd, rnd}, fl2 = {fl, fl}, top = {127, 127}, sh = {(short)r, (short)r}, eight = {8, 8};
-    const v2us ueight = {8, 8};
-    v4i z;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int32_t ow = o[q], sw_ = sv[q];   // plain copies: a vector element is no object to bit_cast
-      const v2s o16 = __builtin_bit_cast(v2s, ow), s16 = __builtin_bit_cast(v2s, sw_);
-      // even bytes: up by 8 as unsigned halves (a signed shift may be assumed not to overflow), down arithmetically
-      const v2s olo = __builtin_bit_cast(v2s, __builtin_bit_cast(v2us, ow) << ueight) >> eight, ohi = o16 >> eight;
-      const v2s slo = __builtin_bit_cast(v2s, __builtin_bit_cast(v2us, sw_) << ueight) >> eight, shi = s16 >> eight;
-      v2s tlo = olo * mconv + (slo * msrc + rnd2);
-      v2s thi = ohi * mconv + (shi * msrc + rnd2);
-      tlo = __builtin_elementwise_min(__builtin_elementwise_max(tlo, fl2) >> sh, top);
-      thi = __builtin_elementwise_min(__builtin_elementwise_max(thi, fl2) >> sh, top);
-      z[q] = (int)__builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, thi), __builtin_bit_cast(uint32_t, tlo),
-                                        0x06020400u);
-    }
-    *reinterpret_cast<v4i *>(a.add_dst + off) = z;
-  } else if (a.add_dst) {
-    // EltwiseAdd on the freshly requantised bytes (core/eltwise.cpp:52-85, integer form)
-    // sum = src * m_src + y * m_conv as one 4 x int8 dot product per output (the two
-    // unused byte lanes are zero), with the rounding term as its addend: adding
-    // 2^(r-1) before the ReLU gives the same quotient as after it.
-    int32_t rnd = a.add_rshift > 0 ? (1 << (a.add_rshift - 1)) : 0;
-    int32_t mpair = (a.add_m_src & 0xff) | ((a.add_m_conv & 0xff) << 8);
-    int32_t floor_ = a.add_relu ? 0 : (int32_t)0x80000000;
-    // one scalar and one vector copy of the uniform operands, made once
-    asm volatile("" : "+s"(rnd), "+v"(mpair), "+s"(floor_));
-    v4i z;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      int32_t t[4];
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const uint32_t pair = __builtin_amdgcn_perm((uint32_t)o[q], (uint32_t)sv[q],
-                                                    0x0c0c0000u | ((4u + b) << 8) | (uint32_t)b);
-        int32_t sum;   // the three-operand form: no copy of the addend into the result first
-        asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(sum) : "v"(pair), "v"(mpair), "s"(rnd));
-        t[b] = max(sum, floor_) >> a.add_rshift;
-      }
-      z[q] = (int)pack_sat4(t[0], t[1], t[2], t[3], -128);
-    }
-    *reinterpret_cast<v4i *>(a.add_dst + off) = z;
-  }
+  if (a.add_dst)
+    *reinterpret_cast<v4i *>(a.add_dst + off) =
+        fused_add_chunk(o, sv, a.add_m_src, a.add_m_conv, a.add_rshift, a.add_relu, a.add_pk);
 }
 
 // Epilogue of one wave tile row block, written straight from the MFMA result layout: every
@@ -454,15 +379,6 @@ constexpr int kModeGeneral = 0;   // per-lane tap arithmetic
 constexpr int kModeUniform = 1;   // ic % (BK) == 0: all groups of a step in one tap, scalar arithmetic
 constexpr int kModeSmallC = 2;    // ic <= 4: four taps per 16-byte group
 
-
-// 16-byte load through a buffer descriptor: an offset at or beyond the
-// descriptor's size yields zeros, which is how padding taps, pixels past the end
-// of the tensor and K steps past the end of the filter are fed to the MFMAs
-// without a branch.
-__device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t offset) {
-  return (v4i)__builtin_amdgcn_raw_buffer_load_b128(rsrc, offset, 0, 0);
-}
-constexpr uint32_t kOobOffset = 0x7fffffffu;
 
 // The kernel arguments (ConvArgs: six 64-byte lines before the table) arrive through the scalar
 // cache.  The compiler fetches a field where it first needs it, and what lies between kernel entry
@@ -1247,41 +1163,6 @@ conv_patch_kernel(ConvArgs a) {
 // K slices by which the LDS reads of MFMA operands run ahead of their MFMAs: an LDS read takes
 // some 130 clocks, a 32x32x32 MFMA 32 to 34
 constexpr int frag_prefetch(int mfmas_per_slice) { return mfmas_per_slice >= 8 ? 1 : mfmas_per_slice >= 4 ? 2 : 3; }
-
-template <int TN, bool RELU>
-__device__ __forceinline__ void requant_rows_c64(const v16i (&acc)[TN], int lo, const int32_t *pc64,
-                                                 const int32_t *pmult, const int32_t *pshift,
-                                                 const int32_t *phpot, uint32_t (&outw)[TN][4]) {
-#pragma unroll
-  for (int qd = 0; qd < 4; ++qd) {
-    const v4i c01 = *reinterpret_cast<const v4i *>(pc64 + qd * 8);
-    const v4i c23 = *reinterpret_cast<const v4i *>(pc64 + qd * 8 + 4);
-    const v4i m4 = *reinterpret_cast<const v4i *>(pmult + qd * 4);
-    const v4i r4 = *reinterpret_cast<const v4i *>(pshift + qd * 4);
-    v4i h4 = {0, 0, 0, 0};
-    if (!RELU) h4 = *reinterpret_cast<const v4i *>(phpot + qd * 4);
-    const int64_t c[4] = {(int64_t)(((uint64_t)(uint32_t)c01[1] << 32) | (uint32_t)c01[0]),
-                          (int64_t)(((uint64_t)(uint32_t)c01[3] << 32) | (uint32_t)c01[2]),
-                          (int64_t)(((uint64_t)(uint32_t)c23[1] << 32) | (uint32_t)c23[0]),
-                          (int64_t)(((uint64_t)(uint32_t)c23[3] << 32) | (uint32_t)c23[2])};
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      int32_t y[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int64_t p = (int64_t)acc[j][qd * 4 + e] * (int64_t)m4[e] + c[e];
-        if (RELU) {
-          y[e] = (int32_t)(p >> 32) >> r4[e];
-        } else {
-          const int32_t x = (int32_t)(p >> 31);
-          y[e] = (x + h4[e] + (x >> 31)) >> r4[e];
-        }
-      }
-      outw[j][qd] = pack_sat4(y[0], y[1], y[2], y[3], lo);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-}
 
 template <int BM, int BN, int WM, int WN, int KP, int SD, int OCC>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
