@@ -281,7 +281,7 @@ def main():
     roofline = None
     if dom:
         achieved = dom["ops"] / (dom["ms"] / 1e3) / 1e12
-        family = next((k for pre, k in (("mfma_pw_", "conv_pw_kernel"), ("mfma_patch2_", "conv_patch2_kernel"),
+        family = next((k for pre, k in (("mfma_chain_", "conv_chain_kernel"), ("mfma_pw_", "conv_pw_kernel"), ("mfma_patch2_", "conv_patch2_kernel"),
                                         ("mfma_patch_", "conv_patch_kernel"), ("mfma_reg_", "conv_mfma_reg_kernel"),
                                         ("mfma_splitk_", "conv_mfma_splitk_kernel")) if dom_name.startswith(pre)),
                       "conv_mfma_kernel")

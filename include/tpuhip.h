@@ -209,6 +209,8 @@ int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *chain);
 int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y_a,
                            const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b);
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *chain);
+/* name of chain kernel variant `variant`, NULL past the last one */
+const char *tpuhip_conv2d_chain_variant_name(int variant);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */

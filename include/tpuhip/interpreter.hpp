@@ -218,6 +218,17 @@ public:
   void release_host_weights();
   // dissolves the pair this kernel belongs to (as first or second), leaving no link behind
   void unpair();
+  // A pointwise conv (with the add folded behind it, if any) and the pointwise conv that reads its
+  // final result can run as one launch (tpuhip_conv2d_chain_*): the intermediate tensor is written
+  // once and not read back.  chain_with packs that and makes `next` a no-op; it answers false, and
+  // changes nothing, where the library does not cover the pair.  Results are unchanged.  Only the
+  // module interpreter arranges this, after the add / table fusions and before the pairing.
+  bool can_chain_with(const Conv2DOpKernel &next) const;
+  bool chain_with(Conv2DOpKernel &next);
+  bool is_chain_first() const { return chain_packed != nullptr; }
+  bool is_chain_second() const { return chained_into != nullptr; }
+  // dissolves the chain this kernel belongs to (as first or second)
+  void unchain();
 
 protected:
   // transposed: the attributes describe a DeConv2D; it runs as a stride-1 conv over the
@@ -241,6 +252,9 @@ private:
   tpuhip_conv_weights *pair_packed = nullptr;
   Conv2DOpKernel *pair_second = nullptr;   // runs inside this kernel's launch
   Conv2DOpKernel *paired_into = nullptr;   // this kernel's work is done by that one
+  tpuhip_conv_chain *chain_packed = nullptr;
+  Conv2DOpKernel *chain_second = nullptr;  // runs inside this kernel's launch, on its final result
+  Conv2DOpKernel *chained_into = nullptr;  // this kernel's work is done by that one
   mutable std::string algo_text;           // storage behind algo_name() of a paired kernel
 };
 
@@ -619,6 +633,8 @@ public:
   // convs over the same input with the same geometry run as one launch (on by default;
   // TPUHIP_PAIR=0 disables); applies at the next loadModule
   bool pair_convs = true;
+  // a pointwise conv (+ folded add) followed by the pointwise conv that reads its result: one launch
+  bool chain_convs = true;
   // true (default): every tensor of the graph can be read back after an invoke, like the
   // reference.  false: the result of a conv whose only reader is the add fused into it is
   // never written (reading it back is an error); applies at the next loadModule
@@ -634,6 +650,7 @@ private:
   void updateKernelList(ModuleDesc &module, std::string &target_op);
   bool isKernelDirty(std::shared_ptr<CPUOpKernel> &krnl, OpDesc *op);
   void fuseKernels();
+  void chainConvs();
   void pairConvs();
   void spreadDirtiness();
   // kernels that run as one launch (a conv with the table op / add folded into it, the two

@@ -27,6 +27,11 @@ def test_recorded_tiles_name_layers_and_variants_that_exist():
     names = []
     while lib.tpuhip_conv2d_tile_name(len(names)):
         names.append(lib.tpuhip_conv2d_tile_name(len(names)).decode())
+    # a layer that opens a launch of two chained convs is recorded under that kernel's name
+    n_chain = 0
+    while lib.tpuhip_conv2d_chain_variant_name(n_chain):
+        names.append(lib.tpuhip_conv2d_chain_variant_name(n_chain).decode())
+        n_chain += 1
     for cfg, rel in bench.RECORDED_TILES.items():
         tiles = json.load(open(os.path.join(ROOT, rel)))
         g = graphs.CONFIGS[cfg]()

@@ -185,6 +185,7 @@ PROTOTYPES.update({
     "tpuhip_conv2d_chain_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_conv2d_chain_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd), C.c_void_p]),
     "tpuhip_conv2d_chain_name": (C.c_char_p, [C.c_void_p]),
+    "tpuhip_conv2d_chain_variant_name": (C.c_char_p, [C.c_int]),
     "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
     "tpuhip_module_weight_file": (C.c_char_p, [C.c_void_p]),
     "tpuhip_module_num_ops": (C.c_int, [C.c_void_p]),

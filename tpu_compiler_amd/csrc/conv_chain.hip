@@ -252,7 +252,7 @@ struct ChainVariant {
   X(0, 256, 64, 64, 64, 4, true)     \
   X(1, 512, 128, 128, 64, 2, false)
 const ChainVariant kChainVariants[] = {
-#define X(i, OC1, KP1, OC2, BN, O, L) {OC1, KP1, OC2, BN, O, "chain_" #OC1 "x" #BN "_k" #KP1 "_to" #OC2},
+#define X(i, OC1, KP1, OC2, BN, O, L) {OC1, KP1, OC2, BN, O, "mfma_chain_" #OC1 "x" #BN "_k" #KP1 "_to" #OC2},
     TPUHIP_CHAIN_VARIANTS(X)
 #undef X
 };
@@ -398,6 +398,10 @@ int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *ch) {
 
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *ch) { return ch ? ch->name.c_str() : "null"; }
 
+const char *tpuhip_conv2d_chain_variant_name(int variant) {
+  return variant >= 0 && variant < kNumChainVariants ? kChainVariants[variant].name : nullptr;
+}
+
 int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a,
                            const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b) {
   TPUHIP_REQUIRE(ctx && ch && x && y_b, "tpuhip_conv2d_chain_i8: NULL argument");
@@ -439,7 +443,9 @@ int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const v
     TPUHIP_REQUIRE(raise_chain_lds((const void *)kernel, lds), "conv chain: raising the LDS limit failed"); \
     a.n_tiles = (a.npix + BN - 1) / BN;                                                                    \
     const int per_cu = std::max(1, std::min((int)(160u * 1024 / lds), O / 2));                             \
-    const dim3 grid((unsigned)std::min(a.n_tiles, ctx->num_cu * per_cu)), block(512);                      \
+    int gsz = std::min(a.n_tiles, ctx->num_cu * per_cu);                                                   \
+    if (const char *e = getenv("TPUHIP_CHAIN_GRID")) gsz = std::min(a.n_tiles, atoi(e));                   \
+    const dim3 grid((unsigned)gsz), block(512);                                                            \
     if (ctx->prof_start)                                                                                   \
       hipExtLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
     else                                                                                                   \

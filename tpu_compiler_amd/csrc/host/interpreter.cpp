@@ -51,6 +51,7 @@ void ModuleInterpreter::updateWeightMap(const std::string &name, const float *da
 void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
   updateKernelList(module, target_op);
   fuseKernels();
+  chainConvs();
   pairConvs();
   spreadDirtiness();
 }
@@ -187,6 +188,26 @@ void ModuleInterpreter::fuseKernels() {
   }
 }
 
+// A pointwise conv -- with the add folded into it, if any -- and the pointwise conv that reads its
+// final result become one launch where the library covers the pair (the 1x1 expansion + add that
+// closes a bottleneck block and the 1x1 reduction that opens the next): the second conv's work
+// moves to the position of the first, which is legal because its only activation operand is
+// produced there and nothing reads its result before its own position.  The intermediate tensor
+// is still written (other kernels read it).  Runs after the add / table fusions.
+void ModuleInterpreter::chainConvs() {
+  const char *env = getenv("TPUHIP_CHAIN");
+  if (!chain_convs || (env && atoi(env) == 0)) return;
+  std::vector<Conv2DOpKernel *> convs;
+  for (auto &k : kernel_list_)
+    if (auto *c = dynamic_cast<Conv2DOpKernel *>(k.get())) convs.push_back(c);
+  for (size_t i = 0; i < convs.size(); ++i)
+    for (size_t j = i + 1; j < convs.size(); ++j)
+      if (convs[i]->chain_with(*convs[j])) {
+        launch_groups_.push_back({convs[i], convs[j]});
+        break;
+      }
+}
+
 // Convs that read the same tensor through the same window geometry (the projection shortcut
 // and the first 1x1 of a residual block, for one) become one launch: the second one's work
 // moves to the position of the first, which is legal because its only activation operand
@@ -212,7 +233,8 @@ void ModuleInterpreter::pairConvs() {
   }
   // paired kernels keep their host operands so that a reload can pair them again
   for (auto *c : convs)
-    if (!c->is_paired_first() && !c->is_paired_second()) c->release_host_weights();
+    if (!c->is_paired_first() && !c->is_paired_second() && !c->is_chain_first() && !c->is_chain_second())
+      c->release_host_weights();
 }
 
 // MlirModuleInterpreter.cpp:85-116
@@ -462,7 +484,7 @@ std::vector<std::pair<std::string, float>> ModuleInterpreter::timeKernels(int32_
       auto *lu = dynamic_cast<LutOpKernel *>(krnl.get());
       auto *cv = dynamic_cast<Conv2DOpKernel *>(krnl.get());
       auto *po = dynamic_cast<PoolingOpKernel *>(krnl.get());
-      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) || (cv && cv->is_paired_second()) ||
+      const bool runs = !(dynamic_cast<InputOpKernel *>(krnl.get()) || (cv && (cv->is_paired_second() || cv->is_chain_second())) ||
                           (el && el->fused_into_producer) || (lu && lu->fused_into_producer) ||
                           (po && po->fused_into_producer));
       if (runs) ck(tpuhip_ctx_set_kernel_events(ctx_, e0[i], e1[i]), "timeKernels");

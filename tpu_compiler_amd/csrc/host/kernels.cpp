@@ -412,6 +412,7 @@ Conv2DOpKernel::Conv2DOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
 }
 
 Conv2DOpKernel::~Conv2DOpKernel() {
+  unchain();
   unpair();
   if (packed) tpuhip_conv2d_weights_destroy(ctx, packed);
 }
@@ -435,6 +436,49 @@ void Conv2DOpKernel::unpair() {
   }
 }
 
+// Dissolves the chain this kernel is part of, from either side (a partial reload may destroy one
+// partner and keep the other).
+void Conv2DOpKernel::unchain() {
+  if (chain_packed) {
+    tpuhip_conv2d_chain_destroy(ctx, chain_packed);
+    chain_packed = nullptr;
+  }
+  if (chain_second) {
+    chain_second->chained_into = nullptr;
+    chain_second = nullptr;
+  }
+  if (chained_into) {
+    Conv2DOpKernel *first = chained_into;
+    chained_into = nullptr;
+    first->chain_second = nullptr;
+    first->unchain();
+  }
+}
+
+bool Conv2DOpKernel::can_chain_with(const Conv2DOpKernel &o) const {
+  if (this == &o || !plain || !o.plain || host_w.empty() || o.host_w.empty()) return false;
+  if (pair_packed || paired_into || o.pair_packed || o.paired_into) return false;
+  if (chain_packed || chained_into || o.chain_packed || o.chained_into) return false;
+  if (lut_dst || pool_dst || o.fused.enable || o.lut_dst || o.pool_dst) return false;
+  if (desc.algo != 0 || o.desc.algo != 0) return false;   // a kernel variant asked for by name stays what it is
+  const SyncedData &mid = fused.enable ? add_dst : output_data;
+  if (o.input_data.get() != mid.get()) return false;
+  return tpuhip_conv2d_can_chain(&desc, &o.desc) != 0;
+}
+
+bool Conv2DOpKernel::chain_with(Conv2DOpKernel &next) {
+  if (!can_chain_with(next)) return false;
+  const int rc = tpuhip_conv2d_chain_prepack(
+      ctx, &desc, &next.desc, host_w.data(), desc.with_bias ? host_b.data() : nullptr, host_m.data(), host_r.data(),
+      next.host_w.data(), next.desc.with_bias ? next.host_b.data() : nullptr, next.host_m.data(), next.host_r.data(),
+      &chain_packed);
+  if (rc == TPUHIP_ERR_UNSUPPORTED) return false;   // e.g. a right shift of 0: stays two launches
+  ck(rc, ("Conv2D '" + name + "' -> '" + next.name + "'").c_str());
+  chain_second = &next;
+  next.chained_into = this;
+  return true;
+}
+
 void Conv2DOpKernel::release_host_weights() {
   std::vector<int8_t>().swap(host_w);
   std::vector<int32_t>().swap(host_b);
@@ -445,7 +489,8 @@ void Conv2DOpKernel::release_host_weights() {
 bool Conv2DOpKernel::can_pair_with(const Conv2DOpKernel &o) const {
   if (this == &o || !plain || !o.plain || host_w.empty() || o.host_w.empty()) return false;
   if (pair_packed || paired_into || o.pair_packed || o.paired_into) return false;
-  if (fused.enable || lut_dst || o.fused.enable || o.lut_dst) return false;
+  if (chain_packed || chained_into || o.chain_packed || o.chained_into) return false;
+  if (fused.enable || lut_dst || pool_dst || o.fused.enable || o.lut_dst || o.pool_dst) return false;
   if (input_data.get() != o.input_data.get() || desc.oc % 128 != 0) return false;
   const tpuhip_conv_desc &a = desc, &b = o.desc;
   return a.kh == b.kh && a.kw == b.kw && a.sh == b.sh && a.sw == b.sw && a.pt == b.pt && a.pb == b.pb &&
@@ -467,7 +512,14 @@ void Conv2DOpKernel::pair_with(Conv2DOpKernel &second) {
 }
 
 void Conv2DOpKernel::invoke() {
-  if (paired_into) return;   // computed by the launch of the conv it is paired with
+  if (paired_into || chained_into) return;   // computed by the launch of the conv it is paired / chained with
+  if (chain_packed) {
+    ck(tpuhip_conv2d_chain_i8(ctx, chain_packed, input_data->data(), store_result ? output_data->data() : nullptr,
+                              fused.enable ? add_src->data() : nullptr, fused.enable ? add_dst->data() : nullptr,
+                              fused.enable ? &fused : nullptr, chain_second->output_data->data()),
+       name.c_str());
+    return;
+  }
   if (pair_packed) {
     ck(tpuhip_conv2d_pair_i8(ctx, pair_packed, input_data->data(), output_data->data(),
                              pair_second->output_data->data()),
@@ -556,6 +608,7 @@ void Conv2DOpKernel::set_store_result(bool store) {
 }
 
 void Conv2DOpKernel::clear_fusion() {
+  unchain();
   unpair();
   store_result = true;
   output_data->materialized = true;
@@ -569,10 +622,11 @@ void Conv2DOpKernel::clear_fusion() {
 }
 
 const char *Conv2DOpKernel::algo_name() const {
-  if (paired_into) {
-    algo_text = "with " + paired_into->name;
+  if (paired_into || chained_into) {
+    algo_text = "with " + (paired_into ? paired_into : chained_into)->name;
     return algo_text.c_str();
   }
+  if (chain_packed) return tpuhip_conv2d_chain_name(chain_packed);
   return tpuhip_conv2d_algo_name(pair_packed ? pair_packed : packed);
 }
 

@@ -98,6 +98,8 @@ int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value) {
       m->interp->keep_all_tensors = value != 0;
     else if (k == "pair_convs")
       m->interp->pair_convs = value != 0;
+    else if (k == "chain_convs")
+      m->interp->chain_convs = value != 0;
     else
       throw std::runtime_error("tpuhip_module_set_option: unknown option '" + k + "'");
   })
