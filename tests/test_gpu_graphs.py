@@ -262,6 +262,64 @@ def test_sibling_convs_run_as_one_launch_with_unchanged_results():
         m.close()
 
 
+def test_chained_pointwise_convs_run_as_one_launch_with_unchanged_results():
+    """the 1x1 expansion + add that closes a bottleneck block and the 1x1 reduction that opens the next
+    run as one launch (res2a/b, res3a/b/c of the ResNet-50 shape).  On, off, with every tensor kept and
+    with outputs only, reloaded, partially reloaded and stopped at the second conv of a chain, every
+    tensor written equals the oracle's."""
+    g = graphs.cfg3_resnet50(batch=2, hw=96)
+    want = oracle_graph.run(g)
+    chains = [("res2a_branch2c", "res2b_branch2a"), ("res2b_branch2c", "res2c_branch2a"),
+              ("res3a_branch2c", "res3b_branch2a"), ("res3b_branch2c", "res3c_branch2a"),
+              ("res3c_branch2c", "res3d_branch2a")]
+    x = g.input_op().data.astype(np.float32)
+    for on, keep in ((1, 1), (1, 0), (0, 1)):
+        m = module()
+        m.set_option("chain_convs", on)
+        m.set_option("keep_all_tensors", keep)
+        m.load(g)
+        algo = dict(m.kernels())
+        for first, second in chains:
+            assert algo[first].startswith("mfma_chain_") == bool(on), (on, first, algo[first])
+            assert (algo[second] == "with " + first) == bool(on), (on, second, algo[second])
+        times = {name: ms for name, _, ms in m.time_kernels(iters=2)}
+        if on:
+            assert all(times[second] == 0 and times[first] > 0 for first, second in chains)
+        m.set_tensor("input", x)
+        m.invoke()
+        for op in g.ops:
+            try:
+                got = m.get_tensor_i8(op.name)
+            except capi.TpuHipError as e:
+                assert not keep and "never written" in str(e)
+                continue
+            assert np.array_equal(got, want[op.name].reshape(op.shape)), (on, keep, op.name)
+        if on and keep:
+            # a reload keeps the chains; stopping at the second conv of a chain still produces it
+            m.load(g)
+            assert dict(m.kernels())["res3b_branch2a"] == "with res3a_branch2c"
+            m.set_tensor("input", x)
+            m.invoke_to("res3b_branch2a")
+            assert np.array_equal(m.get_tensor_i8("res3b_branch2a"),
+                                  want["res3b_branch2a"].reshape(g.by_name["res3b_branch2a"].shape))
+        m.close()
+    # partial reloads after fast_invoke_all_batch: only the second conv, the add in the middle, or the
+    # first conv of a chain is rebuilt; the launch that writes the rebuilt kernel's tensor must run
+    g = graphs.cfg3_resnet50(batch=1, hw=64)
+    m = module(max_batch=1)
+    m.load(g)
+    m.set_tensor("input", g.input_op().data.astype(np.float32), 0)
+    m.fast_invoke_all_batch("", 1)
+    for name in ("res2b_branch2a", "res2a", "res3b_branch2c"):
+        g.by_name[name].attrs["do_relu"] = 0 if g.by_name[name].attrs.get("do_relu", 0) else 1
+        m.load(g)
+        m.fast_invoke_all_batch("", 1)
+        want = oracle_graph.run(g)
+        for op in g.ops:
+            assert np.array_equal(m.get_tensor_i8(op.name, 0), want[op.name].reshape(op.shape)), (name, op.name)
+    m.close()
+
+
 @pytest.mark.parametrize("builder,kw", [(graphs.cfg5_yolo_v3, dict(batch=1, hw=96)),
                                         (graphs.cfg4_mobilenet_v2, dict(batch=2, hw=64)),
                                         (graphs.cfg2_mobilenet_block, dict(batch=1))])
