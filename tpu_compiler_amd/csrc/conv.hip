@@ -114,7 +114,15 @@ struct ConvArgs {
   int has_lut;
   int8_t *lut_dst;
   Table256 lut;
+#ifdef TPUHIP_TRACE
+  unsigned long long *trace;   // development builds: 32 shader-clock stamps per workgroup
+#endif
 };
+#ifdef TPUHIP_TRACE
+#define TPUHIP_TS(k) (ts[k] = (unsigned long long)clock64())
+#else
+#define TPUHIP_TS(k) ((void)0)
+#endif
 
 __device__ __forceinline__ int32_t epilogue(int32_t acc, int32_t bias, const QParam &p, int lo,
                                             int relu_first) {
@@ -1405,9 +1413,16 @@ conv_pw_kernel(ConvArgs a) {
 // LDS (dynamic): parameters | two filter tiles | patch; the staged output tile takes the
 // filter tiles' place.
 // ---------------------------------------------------------------------------
+// 2 * (C + 16) + kPatch2RowPad is a multiple of 128 for every C that is a multiple of 64
+constexpr int kPatch2RowPad = 96;
+
 template <int BM, int BN, int WM, int WN, int BK, int OCC>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_patch2_kernel(ConvArgs a) {
+#ifdef TPUHIP_TRACE
+  unsigned long long ts[32] = {};
+#endif
+  TPUHIP_TS(0);
   gather_conv_args(a);
   gather_conv_args_more(a);
   constexpr int NT = WM * WN * 64;
@@ -1445,6 +1460,11 @@ conv_patch2_kernel(ConvArgs a) {
   const int lgc = a.pstep_oh;                 // log2(C)
   const int C = 1 << lgc;
   const int prow = C + 16;                    // bytes of a patch position in LDS
+  // bytes of a patch row: its pw positions and kPatch2RowPad more, which make the pitch congruent to
+  // ow positions modulo the 128 bytes of a bank sweep -- the 32 pixels of a fragment read, which wrap
+  // from one image row into the next on narrow maps, then fall into banks as if they were consecutive
+  // positions, wherever the wraps lie
+  const int rowb = pw * prow + kPatch2RowPad;
   const bool relu = a.lo == 0;
 
   const __amdgpu_buffer_rsrc_t xrsrc =
@@ -1473,10 +1493,24 @@ conv_patch2_kernel(ConvArgs a) {
   const uint32_t wbase = (uint32_t)(oc0 / BM) * (uint32_t)(a.kp * BM) + (uint32_t)tid * 16u;
   const int nsteps = a.kp / BK;
   v4i wr[RD][NW];
+  // (no branch around a load: a step past the end of K reads zeros through the descriptor, so
+  // that every step issues the same loads and the waits before the LDS stores count loads
+  // instead of draining the queue.  The lane offsets are computed once and stay in their own
+  // registers (an offset formed per load tends to land in the registers the load is about to
+  // write, and the write-after-write wait that follows drains the queue just as well); a step
+  // past the end takes an empty descriptor, a scalar select.)
+  const __amdgpu_buffer_rsrc_t wnone = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, 0, 0x00020000);
+  uint32_t woffs[NW];
+#pragma unroll
+  for (int u = 0; u < NW; ++u) {
+    woffs[u] = wbase + (uint32_t)(u * NT * 16);
+    asm volatile("" : "+v"(woffs[u]));
+  }
   auto load_A = [&](int slot, int step) {
+    const bool in_k = step < nsteps;
 #pragma unroll
     for (int u = 0; u < NW; ++u)
-      wr[slot][u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(wrsrc, wbase + (uint32_t)(u * NT * 16), step * (BM * BK), 0);
+      wr[slot][u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(in_k ? wrsrc : wnone, woffs[u], step * (BM * BK), 0);
   };
   auto store_A = [&](int slot, int buf) {
 #pragma unroll
@@ -1486,8 +1520,7 @@ conv_patch2_kernel(ConvArgs a) {
     }
   };
 #pragma unroll
-  for (int d = 0; d < RD; ++d)
-    if (d < nsteps) load_A(d, d);
+  for (int d = 0; d < RD; ++d) load_A(d, d);
 
   if (tid < BM) {
     const int32_t *c64 = relu ? a.qc64r : a.qc64;
@@ -1512,7 +1545,7 @@ conv_patch2_kernel(ConvArgs a) {
     const int p = (wn * TN + j) * 32 + frow;
     const uint32_t pr = a.ow == 1 ? (uint32_t)p : __umulhi((uint32_t)p, a.magic_ow);
     const int pc = p - (int)pr * a.ow;
-    bbase[j] = (p < rows * a.ow ? (int)pr * pw + pc : 0) * prow + fk * 16;   // idle slots read position 0
+    bbase[j] = (p < rows * a.ow ? (int)pr * rowb + pc * prow : 0) + fk * 16;   // idle slots read position 0
   }
 
   // park the patch and the first filter tile
@@ -1522,18 +1555,27 @@ conv_patch2_kernel(ConvArgs a) {
     const int pr = (int)__umulhi((uint32_t)q, a.magic_c16);
     const int p = q - pr * rowchunks;
     if (q < n_chunks)
-      *reinterpret_cast<v4i *>(patch + (pr * pw + (p >> (lgc - 4))) * prow + (p & ((C >> 4) - 1)) * 16) = preg[u];
+      *reinterpret_cast<v4i *>(patch + pr * rowb + (p >> (lgc - 4)) * prow + (p & ((C >> 4) - 1)) * 16) = preg[u];
   }
+  TPUHIP_TS(1);
   store_A(0, 0);
   __syncthreads();
+  TPUHIP_TS(2);
 
-  v16i acc[TM][TN];
+  // A wave whose tile is a single 32x32 block would issue its MFMAs as one dependent chain (every
+  // MFMA waits for the one before); it keeps two sets of accumulators and alternates between them
+  // by K slice -- two independent chains -- and adds them up before the requantisation.
+  constexpr int NACC = TM * TN == 1 ? 2 : 1;
+  v16i accs[NACC][TM][TN];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int c = 0; c < NACC; ++c)
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) accs[c][i][j][e] = 0;
+  v16i (&acc)[TM][TN] = accs[0];
 
   // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS a
   // step ago -- and receives the tile RD steps ahead; the next step's tile goes from its slot
@@ -1542,7 +1584,11 @@ conv_patch2_kernel(ConvArgs a) {
   constexpr int PD = OCC >= 4 ? 1 : frag_prefetch(TM * TN);
   auto step = [&](int s, auto slotc) {
     constexpr int slot = decltype(slotc)::value, buf = slot & 1;
-    if (s + RD < nsteps) load_A(slot, s + RD);
+#ifdef TPUHIP_TRACE
+    const bool tr = s < 4;
+    if (tr) TPUHIP_TS(3 + slot * 6);
+#endif
+    load_A(slot, s + RD);
     const int8_t *ab = abuf + buf * ABYTES;
     v4i fa[PD + 1][TM], fb[PD + 1][TN];
     auto read_slice = [&](int kk, int fs) {
@@ -1551,7 +1597,7 @@ conv_patch2_kernel(ConvArgs a) {
       const int koff = s * BK + kk * 32;
       const int tap = min(koff >> lgc, 8);
       const int tkh = (tap * 11) >> 5;
-      const int boff = (tkh * pw + (tap - 3 * tkh)) * prow + (koff & (C - 1));
+      const int boff = tkh * rowb + (tap - 3 * tkh) * prow + (koff & (C - 1));
 #pragma unroll
       for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(ab + abase[i] + kk * 32);
 #pragma unroll
@@ -1571,12 +1617,24 @@ conv_patch2_kernel(ConvArgs a) {
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[kk % (PD + 1)][i], fb[kk % (PD + 1)][j], acc[i][j], 0, 0, 0);
+            accs[kk % NACC][i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[kk % (PD + 1)][i], fb[kk % (PD + 1)][j],
+                                                                          accs[kk % NACC][i][j], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
+#ifdef TPUHIP_TRACE
+      if (tr && kk == 0) TPUHIP_TS(4 + slot * 6);
+      if (tr && kk == 3) TPUHIP_TS(5 + slot * 6);
+      if (tr && kk == KK - 1) TPUHIP_TS(6 + slot * 6);
+#endif
     }
-    if (s + 1 < nsteps) store_A((slot + 1) % RD, buf ^ 1);
+    store_A((slot + 1) % RD, buf ^ 1);   // (past the last step: zeros, into a tile nobody reads)
+#ifdef TPUHIP_TRACE
+    if (tr) TPUHIP_TS(7 + slot * 6);
+#endif
     __syncthreads();
+#ifdef TPUHIP_TRACE
+    if (tr) TPUHIP_TS(8 + slot * 6);
+#endif
   };
   for (int s = 0; s < nsteps; s += RD) {
     step(s, std::integral_constant<int, 0>{});
@@ -1585,6 +1643,11 @@ conv_patch2_kernel(ConvArgs a) {
     if (s + 3 < nsteps) step(s + 3, std::integral_constant<int, 3>{});
   }
 
+  TPUHIP_TS(27);
+  if (NACC == 2) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) accs[0][0][0][e] += accs[NACC - 1][0][0][e];
+  }
   // the requantised tile goes through LDS (the filter tiles' space: every wave is past the
   // last barrier of the K loop) and leaves in memory order
   const OutRoute out{a.y, a.y_cs, a.lo, 0};
@@ -1605,8 +1668,16 @@ conv_patch2_kernel(ConvArgs a) {
       *reinterpret_cast<v4i *>(stage + ((wn * TN + j) * 32 + frow) * stage_row_bytes<BM>() + lc) =
           v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
   }
+  TPUHIP_TS(28);
   __syncthreads();
+  TPUHIP_TS(29);
   flush_tile<BM, BN, NT>(a, stage, tid, pix_base, pix_limit, oc0, out, lut, sv);
+  TPUHIP_TS(30);
+#ifdef TPUHIP_TRACE
+  if (a.trace && (tid & 63) == 0) {
+    for (int k = 0; k < 32; ++k) a.trace[((size_t)blockIdx.x * 8 + (tid >> 6)) * 32 + k] = ts[k];
+  }
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -2891,7 +2962,9 @@ struct TileCfg {
   V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4) \
   V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4) \
   V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4) \
-  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2)
+  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2) \
+  V(45, "mfma_patch2_32x256_w8", 32, 256, 1, 8, 256, 4) \
+  V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2)
 
 struct TileTable {
   TileCfg t[64];
@@ -3015,7 +3088,7 @@ constexpr int kPatch2MaxChunks = 18 * 256;     // 16-byte input chunks a workgro
 constexpr int kLdsBytes = 160 * 1024;
 
 inline unsigned patch2_lds_bytes(const TileCfg &c, int th, int ow, int ic) {
-  return (unsigned)(5 * c.bm * 4 + 256 + 2 * c.bm * (c.bk + 16) + (th + 2) * (ow + 2) * (ic + 16));
+  return (unsigned)(5 * c.bm * 4 + 256 + 2 * c.bm * (c.bk + 16) + (th + 2) * ((ow + 2) * (ic + 16) + kPatch2RowPad));
 }
 
 // rows of one image a tile holds; 0: the layer does not fit this kernel
@@ -3280,6 +3353,9 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
   a.dh = d.dh; a.dw = d.dw; a.ins_h = d.ins_h; a.ins_w = d.ins_w;
   a.c16 = w->c16; a.k16 = w->k16; a.kp = w->kp;
   a.npix = d.n * d.oh * d.ow;
+#ifdef TPUHIP_TRACE
+  a.trace = getenv("TPUHIP_TRACE_PTR") ? (unsigned long long *)strtoull(getenv("TPUHIP_TRACE_PTR"), nullptr, 16) : nullptr;
+#endif
   a.linear = d.kh == 1 && d.kw == 1 && d.sh == 1 && d.sw == 1 && d.pt == 0 && d.pl == 0 && d.pb == 0 &&
              d.pr == 0 && d.ih == d.oh && d.iw == d.ow && d.ins_h == 0 && d.ins_w == 0;
   a.lo = (d.do_relu && !d.relu_first) ? 0 : -128;
