@@ -253,8 +253,11 @@ int tpuhip_fc_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, v
  * on, held until the process ends) whose address is looked up when a context is created; the call
  * itself allocates and frees nothing.  Layers that need more than 1024 partial sums of 32x32 outputs
  * (rows/32 x channels/32 x K splits), or that tpuhip_fc_prepack did not pack for the split-K kernel,
- * are refused with TPUHIP_ERR_INVALID.  All calls on one GPU share the array: calls that overlap
- * there (two streams, two threads) race; calls on one stream do not. */
+ * are refused with TPUHIP_ERR_INVALID.  All calls on one GPU share the array, so calls that overlap
+ * there would race: calls on one stream do not overlap; a call from another context while the last
+ * user's stream still has work in flight is refused with TPUHIP_ERR_INVALID (a stream query, no
+ * wait); two host threads calling at the same moment on two streams remain the caller's to
+ * serialise. */
 int tpuhip_fc_i8_noalloc(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x, void *y);
 
 /* The batched and transposed forms of FullyConnectedOpKernel::invoke (core/fullyconnected.cpp:44-91,
@@ -265,7 +268,12 @@ int tpuhip_fc_i8_noalloc(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
  * (rshift[i], multiplier[i]) where i = (flat logical index of the RESULT) / (m*n), which is how the
  * reference indexes after its output permute.  x and y are channels-last device tensors whose 4-d
  * views (n, c, h, w; missing dims 1) and channel strides are given: the kernel maps logical indices to
- * them, so no transposed copy is made.  The last logical dim of x must be k, of y n. */
+ * them, so no transposed copy is made.  The last logical dim of x must be k, of y n.  Only the logical
+ * elements of y are written: bytes between its channel count and its channel stride are the caller's to
+ * keep zero (a tensor from tpuhip_malloc + tpuhip_memset, or one every earlier kernel wrote, has them so).
+ * The sums are exact int32 sums; the reference's are fp32 (mkldnn_ip), which agree while
+ * sum |x * w| + |bias| stays below 2^24 per output -- beyond that bound (possible from about 1000 input
+ * channels on) the reference's rounding depends on its summation order and parity is not pinned. */
 typedef struct tpuhip_fc_batched_desc {
   int batch_high, batch_low, m, k, n;
   int input_transpose, output_transpose, do_relu;

@@ -41,6 +41,26 @@ def test_recorded_tiles_name_layers_and_variants_that_exist():
         assert len(tiles) >= {"cfg3": 40, "cfg4": 30, "cfg5": 60}[cfg]      # every MFMA conv of the graph
 
 
+def test_committed_traffic_figures_name_kernel_variants_the_library_still_has():
+    """bench.py takes roofline.traffic from profiles/resnet50_b32_bench_traffic.json by kernel variant name:
+    a variant renamed or removed in the library must not leave a stale entry behind"""
+    from tpu_compiler_amd import capi
+    lib = capi.bind()
+    names = set()
+    i = 0
+    while lib.tpuhip_conv2d_tile_name(i):
+        names.add(lib.tpuhip_conv2d_tile_name(i).decode())
+        i += 1
+    i = 0
+    while lib.tpuhip_conv2d_chain_variant_name(i):
+        names.add(lib.tpuhip_conv2d_chain_variant_name(i).decode())
+        i += 1
+    t = json.load(open(os.path.join(ROOT, "profiles", "resnet50_b32_bench_traffic.json")))
+    assert t["kernels"] and set(t["kernels"]) <= names, sorted(set(t["kernels"]) - names)
+    for k, v in t["kernels"].items():
+        assert v["fetch_KiB"] > 0 and v["write_KiB"] > 0, k
+
+
 def test_cpu_baseline_leg_reports_what_it_ran():
     sys.path.insert(0, ROOT)
     import bench

@@ -1106,7 +1106,7 @@ def test_concat_whole_channel_groups(ctx, channels, in_cs, y_cs):
     want = O.concat_i8(xs, 1)
     ts = [ctx.from_nchw(a, cs) for a, cs in zip(xs, in_cs)]
     yt = ctx.tensor(want.shape, y_cs)
-    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0, yt.nbytes))
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))   # poison: the pad channels must be written
     ctx.concat(ts, 1, yt, [0] * len(xs), [1] * len(xs), False)
     assert np.array_equal(ctx.to_nchw(yt), want)
     assert not ctx.raw(yt)[..., want.shape[1]:].any()
@@ -1238,6 +1238,21 @@ def test_data_movement_ops(ctx, kind, shape, params, out_shape):
     ctx.move(O.MOVE_KINDS.index(kind), xt, yt, params)
     assert np.array_equal(ctx.to_nchw(yt), want)
     assert not ctx.raw(yt)[..., want.shape[1]:].any()
+
+
+@pytest.mark.parametrize("x_cs,y_cs", [(32, 48), (48, 32), (32, 32), (64, 32)])
+def test_permute_that_keeps_the_channels_with_padded_strides(ctx, x_cs, y_cs):
+    """order (0, 1, 3, 2): a pixel's channel row moves as 16-byte groups; with a wider stride on either
+    side no group may come from the neighbouring pixel, and the output's pad groups must be zero"""
+    rng = np.random.default_rng(x_cs * 3 + y_cs)
+    shape = (2, 20, 5, 7)
+    x = rnd_i8(rng, shape)
+    want = O.move_i8("permute", x, [0, 1, 3, 2], None)
+    xt, yt = ctx.from_nchw(x, cs=x_cs), ctx.tensor(want.shape, cs=y_cs)
+    ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+    ctx.move(O.MOVE_KINDS.index("permute"), xt, yt, [0, 1, 3, 2])
+    assert np.array_equal(ctx.to_nchw(yt), want)
+    assert not ctx.raw(yt)[..., shape[1]:].any()
 
 
 def test_data_movement_rejects_bad_arguments(ctx):

@@ -48,6 +48,62 @@ def test_fc_noalloc_equals_fc_on_two_calls_in_a_row():
     ctx.close()
 
 
+def _free_device_bytes():
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_fc_noalloc_leaves_the_free_device_memory_unchanged():
+    """after a first call (which loads the code object) further calls take no device memory: the
+    runtime's free-memory figure is the same before and after"""
+    ctx = capi.Context(0)
+    rng = np.random.default_rng(78)
+    xt, wh, want = _fc_case(ctx, rng, 32, 512, 200, True)
+    yt = ctx.tensor((32, 200, 1, 1))
+    ctx.fc(wh, xt, yt, noalloc=True)
+    ctx.sync()
+    before = _free_device_bytes()
+    for _ in range(3):
+        ctx.fc(wh, xt, yt, noalloc=True)
+    ctx.sync()
+    assert _free_device_bytes() == before
+    assert np.array_equal(ctx.to_nchw(yt).reshape(32, 200), want)
+    ctx.conv_weights_destroy(wh)
+    ctx.close()
+
+
+def test_fc_noalloc_refuses_a_call_that_would_overlap_another_context():
+    """two contexts (two streams) share the GPU's static scratch: while the first one's stream still has
+    work in flight the second one's call is refused; once the first has drained it goes through"""
+    a, b = capi.Context(0), capi.Context(0)
+    rng = np.random.default_rng(79)
+    xa, wa, want_a = _fc_case(a, rng, 32, 512, 200, True)
+    xb, wb, want_b = _fc_case(b, rng, 8, 256, 64, False)
+    ya, yb = a.tensor((32, 200, 1, 1)), b.tensor((8, 64, 1, 1))
+    n = 256 << 20
+    src, dst = a.malloc(n), a.malloc(n)
+    a._ck(a.lib.tpuhip_memset(a.h, src, 1, n))
+    a.sync()
+    for _ in range(100):                 # some milliseconds of queued work on a's stream
+        a._ck(a.lib.tpuhip_relu_i8(a.h, src, dst, n))
+    a.fc(wa, xa, ya, noalloc=True)
+    with pytest.raises(capi.TpuHipError, match="still in flight"):
+        b.fc(wb, xb, yb, noalloc=True)
+    a.sync()
+    b.fc(wb, xb, yb, noalloc=True)
+    assert np.array_equal(a.to_nchw(ya).reshape(32, 200), want_a)
+    assert np.array_equal(b.to_nchw(yb).reshape(8, 64), want_b)
+    a.free(src)
+    a.free(dst)
+    a.conv_weights_destroy(wa)
+    b.conv_weights_destroy(wb)
+    a.close()
+    b.close()
+
+
 def test_fc_noalloc_refuses_what_does_not_fit():
     ctx = capi.Context(0)
     rng = np.random.default_rng(5)

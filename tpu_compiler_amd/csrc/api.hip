@@ -74,6 +74,7 @@ int tpuhip_ctx_destroy(tpuhip_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
   }
   if (ctx->workspace) (void)hipFree(ctx->workspace);
+  tpuhip_static_scratch_forget(ctx);
   delete ctx;
   return TPUHIP_OK;
 }

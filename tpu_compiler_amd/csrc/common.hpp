@@ -29,6 +29,8 @@ struct tpuhip_ctx {
 // conv.hip: looks up this device's copy of the library's static scratch array (the one the
 // allocation-free entry point works in); called once per context with the device current
 extern "C" int tpuhip_static_scratch_init(int device);
+// conv.hip: a context being destroyed stops being the static scratch's last user
+extern "C" void tpuhip_static_scratch_forget(const tpuhip_ctx *ctx);
 
 namespace tpuhip {
 

@@ -2886,6 +2886,11 @@ constexpr size_t kFcStaticPartials = 1024;          // (tile, split) pairs: 4 Mi
 constexpr size_t kFcStaticBytes = kFcStaticPartials * kFcPartialBytes;
 static __device__ __align__(256) unsigned char scratch[kFcStaticBytes];
 static void *g_static_scratch[64];                  // device address of `scratch`, per device
+// who used a device's static scratch last: a call from another stream while that one's work is
+// still in flight would race on the array and is refused
+static std::mutex g_static_mu;
+static const tpuhip_ctx *g_static_user[64];
+static hipStream_t g_static_stream[64];
 
 // ---------------------------------------------------------------------------
 // host side
@@ -4174,6 +4179,16 @@ static int run_fc_one(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void 
   return TPUHIP_OK;
 }
 
+// a context that goes away is forgotten as the static scratch's last user (its stream handle dies with it)
+void tpuhip_static_scratch_forget(const tpuhip_ctx *ctx) {
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  for (int d = 0; d < 64; ++d)
+    if (g_static_user[d] == ctx) {
+      g_static_user[d] = nullptr;
+      g_static_stream[d] = nullptr;
+    }
+}
+
 int tpuhip_static_scratch_init(int device) {
   TPUHIP_REQUIRE(device >= 0 && device < 64, "tpuhip: device index %d out of range", device);
   if (g_static_scratch[device]) return TPUHIP_OK;
@@ -4211,6 +4226,22 @@ int tpuhip_fc_i8_noalloc(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const vo
                  "(%zu partial sums of 32 x 32 outputs)", p.bytes, kFcStaticBytes, kFcStaticPartials);
   void *ptr = ctx->device >= 0 && ctx->device < 64 ? g_static_scratch[ctx->device] : nullptr;
   TPUHIP_REQUIRE(ptr, "tpuhip_fc_i8_noalloc: the static scratch of device %d was not set up", ctx->device);
+  {
+    std::lock_guard<std::mutex> lock(g_static_mu);
+    const tpuhip_ctx *last = g_static_user[ctx->device];
+    if (last && last != ctx && g_static_stream[ctx->device] != ctx->stream) {
+      // (a query, no wait: the call stays free of anything that blocks or allocates)
+      const hipError_t q = hipStreamQuery(g_static_stream[ctx->device]);
+      if (q == hipErrorNotReady)
+        return set_error(TPUHIP_ERR_INVALID,
+                         "tpuhip_fc_i8_noalloc: another context's call on device %d is still in flight on its "
+                         "stream; calls that overlap on one GPU share the static scratch and would race",
+                         ctx->device);
+      (void)hipGetLastError();
+    }
+    g_static_user[ctx->device] = ctx;
+    g_static_stream[ctx->device] = ctx->stream;
+  }
   return run_fc_splitk(ctx, w, x, y, ptr, p);
 }
 

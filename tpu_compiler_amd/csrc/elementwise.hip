@@ -176,11 +176,12 @@ struct ConcatArgs {
   int64_t stride[4];   // bytes from one outer index to the next in each input
   int64_t y_stride;    // ... in the output
   int64_t start[5];    // first 16-byte group of each input's chunk within an output chunk; start[n] = groups per chunk
+  int64_t groups;      // groups written per outer index (>= start[n]; the rest are zero)
   int n;
 };
 
 __global__ __launch_bounds__(kThreads) void concat_chunks_kernel(ConcatArgs a) {
-  const int64_t g16 = a.start[a.n];
+  const int64_t g16 = a.groups;   // groups written per outer index: those of the inputs, then zero pad groups
   const int64_t total = a.outer * g16;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
@@ -192,7 +193,8 @@ __global__ __launch_bounds__(kThreads) void concat_chunks_kernel(ConcatArgs a) {
     if (a.n > 1 && g >= a.start[1]) { src = a.x[1]; stride = a.stride[1]; first = a.start[1]; }
     if (a.n > 2 && g >= a.start[2]) { src = a.x[2]; stride = a.stride[2]; first = a.start[2]; }
     if (a.n > 3 && g >= a.start[3]) { src = a.x[3]; stride = a.stride[3]; first = a.start[3]; }
-    const v4i v = *reinterpret_cast<const v4i *>(src + o * stride + (g - first) * 16);
+    v4i v = {0, 0, 0, 0};
+    if (g < a.start[a.n]) v = *reinterpret_cast<const v4i *>(src + o * stride + (g - first) * 16);
     *reinterpret_cast<v4i *>(a.y + o * a.y_stride + g * 16) = v;
   }
 }
@@ -664,7 +666,9 @@ int tpuhip_concat_i8(tpuhip_ctx *ctx, const void *const *xs, int nin, const int 
     TPUHIP_REQUIRE(a.start[nin] * 16 == unit * out_dims[axis] && a.start[nin] * 16 <= a.y_stride,
                    "concat: chunks of %lld groups do not fill axis %d", (long long)a.start[nin], axis);
     TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
-    launch(ctx, concat_chunks_kernel, dim3(grid_for(a.outer * a.start[nin], kThreads * 4)), dim3(kThreads), a);
+    // along the channels the output's stride may be wider than its channels: the pad groups are written as zero
+    a.groups = axis == 1 ? y_cs / 16 : a.start[nin];
+    launch(ctx, concat_chunks_kernel, dim3(grid_for(a.outer * a.groups, kThreads * 4)), dim3(kThreads), a);
     TPUHIP_CHECK_HIP(hipGetLastError());
     return TPUHIP_OK;
   }

@@ -1148,6 +1148,9 @@ ReduceOpKernel::ReduceOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
   for (int i = 1; i < count; ++i)
     if ((int)op.attr("axes" + std::to_string(i)) != first_axis + i) fail("Reduce '" + name + "': axes must be consecutive");
   if (first_axis < 0 || last_axis > 3) fail("Reduce '" + name + "': axes outside a 4-D tensor");
+  for (const auto &opd : op.operands)
+    if (valueMapping.shapes.count(opd) && valueMapping.shapes[opd].size() > 4)
+      fail("Reduce '" + name + "': tensor rank " + std::to_string(valueMapping.shapes[opd].size()) + " not supported");
   // quant_rshift = opdTensors[3], quant_multiplier = opdTensors[4]; absent: 0 and 1 (reduce.cpp:14-20)
   if (opdTensors.size() > 3 && opdTensors[3].weight) rshift = (int)f2u32(opdTensors[3].weight->at(0));
   if (opdTensors.size() > 4 && opdTensors[4].weight) multiplier = f2u32(opdTensors[4].weight->at(0));
@@ -1285,6 +1288,8 @@ ConcatOpKernel::ConcatOpKernel(OpDesc &op, value_map_t &valueMapping, weight_map
   // shapes of rank 2..4 lie in the 4-d view with trailing dims of 1, so the axis keeps its number;
   // a rank-1 shape lies along the channels
   if (axis < 0 || axis >= (int)op.shape.size()) fail("Concat '" + name + "': axis outside the shape");
+  // (shapes of rank 5 and 6 fold their leading dimensions, which would renumber the axis)
+  if (op.shape.size() > 4) fail("Concat '" + name + "': tensor rank " + std::to_string(op.shape.size()) + " not supported");
   if (op.shape.size() == 1) axis = 1;
 }
 

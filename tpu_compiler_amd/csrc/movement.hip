@@ -348,10 +348,13 @@ struct PermArgs {
   int dim[4];        // input dimensions (n, c, h, w)
   int64_t S[4], T[4];
   int ocs;           // channel stride of the output
+  int ics;           // channel stride of the input
   int j, a, b;       // j: the input dimension that becomes the output's channels; a, b: the other two besides c
 };
 
-// channels stay channels (j == 1): a pixel's channel row moves as 16-byte chunks
+// channels stay channels (j == 1): a pixel's channel row moves as 16-byte chunks.  The two channel
+// strides may differ (a padded stride on either side): groups of the output row beyond the input's
+// stride are written as zero, never read from the next pixel.
 __global__ __launch_bounds__(kThreads) void permute_rows_kernel(PermArgs q, int64_t total) {
   const int c16 = q.ocs >> 4;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
@@ -361,7 +364,8 @@ __global__ __launch_bounds__(kThreads) void permute_rows_kernel(PermArgs q, int6
     pix /= q.dim[3];
     const int h = (int)(pix % q.dim[2]);
     const int n = (int)(pix / q.dim[2]);
-    const v4i v = *reinterpret_cast<const v4i *>(q.x + n * q.S[0] + h * q.S[2] + w * q.S[3] + cg * 16);
+    v4i v = {0, 0, 0, 0};
+    if (cg * 16 < q.ics) v = *reinterpret_cast<const v4i *>(q.x + n * q.S[0] + h * q.S[2] + w * q.S[3] + cg * 16);
     *reinterpret_cast<v4i *>(q.y + n * q.T[0] + h * q.T[2] + w * q.T[3] + cg * 16) = v;
   }
 }
@@ -427,6 +431,7 @@ int run_permute(tpuhip_ctx *ctx, const tpuhip_move_desc *d, const void *x, void 
   const int64_t tout[4] = {(int64_t)d->oh * d->ow * d->y_cs, 1, (int64_t)d->ow * d->y_cs, d->y_cs};
   for (int k = 0; k < 4; ++k) q.T[d->p[k]] = tout[k];   // output dimension k is input dimension p[k]
   q.ocs = d->y_cs;
+  q.ics = d->x_cs;
   q.j = d->p[1];
   TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
   if (q.j == 1) {
