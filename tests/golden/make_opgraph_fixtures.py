@@ -33,7 +33,13 @@ OUT = os.path.join(HERE, "opgraphs")
 # 23 MB of weights; crop, whose second op asks for channels 32..41 of a 16-channel tensor (the
 # reference only compiles that graph; an interpreter would read past the input, this library refuses)
 GRAPHS = ["conv", "conv_1_oc", "deconv", "fc", "eltwise_add", "avg_pool", "max_pool", "relu", "concat",
-          "broadcast_mul", "permute", "reorg", "reverse", "tile"]
+          "broadcast_mul", "permute", "reorg", "reverse", "tile",
+          "broadcast", "conv_large_w", "swap_channel", "permute_large", "lrn", "fc_large"]
+# A quantized tensor of more than this many bytes is not stored: the weight file holds a descriptor
+# "<name>__seeded" = [seed, 100 * sigma, shape...] instead, and materialize() draws the tensor --
+# rint(normal(0, sigma)) clipped to +-127, the statistics of the quantized tensor it stands for --
+# for the HIP path and the oracle alike (fc_large: a 23501 x 512 filter, 12 MB).
+SEEDED_ABOVE = 1 << 20
 _STORAGE = {"INT8": np.int8, "UINT8": np.uint8, "INT16": np.int16, "INT32": np.int32, "UINT32": np.uint32}
 
 
@@ -41,7 +47,18 @@ def prepare(name, tmp, rng):
     """the fp32 graph as the reference holds it, seeded weights under the file name it asks for,
     a calibration table with one seeded threshold per op"""
     path = tmp / (name + ".mlir")
-    path.write_text(open(os.path.join(REF_TESTS, name + ".mlir")).read())
+    text = open(os.path.join(REF_TESTS, name + ".mlir")).read()
+    lrn_thr = np.random.default_rng(77).uniform(0.8, 4.0)   # (a stream of its own: the other graphs' draws stay as they were)
+    if name == "lrn":
+        # the reference splits an LRN into three ops for calibration and folds their thresholds back
+        # into the op as threshold_parts (Quantization.cpp:296-313); the test graph holds the unsplit
+        # op, so the three are stated here from the op's own constants and its input's threshold T:
+        # max of alpha / size * x^2, of its window sum, and of (k + sum)^-beta
+        alpha, size = 9.99999974e-5, 5
+        parts = (alpha / size * lrn_thr ** 2, alpha * lrn_thr ** 2, 1.0)
+        text = text.replace("sum_rshift = 0 : i32}", "sum_rshift = 0 : i32, threshold_parts = [%.9g : f32, %.9g : f32, %.9g : f32]}" % parts)
+        assert "threshold_parts" in text
+    path.write_text(text)
     weights, wfile, ops = {}, None, []
     for line in capi.mlir_describe(str(path)).splitlines():
         w = line.split(" ")
@@ -54,7 +71,8 @@ def prepare(name, tmp, rng):
     if weights:
         np.savez(tmp / wfile, **weights)
     table = tmp / (name + "_table")
-    table.write_text("".join("%s %.5f\n" % (op, rng.uniform(0.8, 4.0)) for op in ops))
+    table.write_text("".join("%s %.5f\n" % (op, lrn_thr if (name == "lrn" and op == "relu") else rng.uniform(0.8, 4.0))
+                             for op in ops))
     return path, table
 
 
@@ -79,10 +97,42 @@ def write_one(name, tmp):
             for k in z.files:
                 t = _STORAGE.get(storage.get(k, "NONE"))
                 a = z[k]
-                typed[k] = a.astype(t) if t is not None and np.array_equal(a.astype(t).astype(np.float32), a) else a
+                a = a.astype(t) if t is not None and np.array_equal(a.astype(t).astype(np.float32), a) else a
+                if a.nbytes > SEEDED_ABOVE:
+                    assert a.dtype == np.int8, (k, a.dtype)
+                    sigma = float(np.std(a.astype(np.float32)))
+                    typed[k + "__seeded"] = np.array([1000 + sum(map(ord, k)), round(100 * sigma)] + list(a.shape), np.int64)
+                else:
+                    typed[k] = a
         np.savez_compressed(os.path.join(OUT, name + "_int8_weights.npz"), **typed)
         wbytes = os.path.getsize(os.path.join(OUT, name + "_int8_weights.npz"))
     print(name, len(text), "bytes of text,", wbytes, "bytes of weights")
+
+
+def materialize(name, dst_dir):
+    """path of the stored quantized graph `name` with a complete weight file beside it: the stored
+    files themselves, or -- where a tensor is held as a seeded descriptor -- copies under dst_dir
+    with that tensor drawn"""
+    src = os.path.join(OUT, name + "_int8.mlir")
+    wsrc = os.path.join(OUT, name + "_int8_weights.npz")
+    if not os.path.exists(wsrc):
+        return src
+    with np.load(wsrc) as z:
+        if not any(k.endswith("__seeded") for k in z.files):
+            return src
+        full = {}
+        for k in z.files:
+            if k.endswith("__seeded"):
+                seed, sigma100, *shape = [int(v) for v in z[k]]
+                rng = np.random.default_rng(seed)
+                full[k[:-len("__seeded")]] = np.clip(np.rint(rng.normal(0, sigma100 / 100.0, shape)), -127, 127).astype(np.int8)
+            else:
+                full[k] = z[k]
+    os.makedirs(dst_dir, exist_ok=True)
+    dst = os.path.join(str(dst_dir), name + "_int8.mlir")
+    open(dst, "w").write(open(src).read())
+    np.savez(os.path.join(str(dst_dir), name + "_int8_weights.npz"), **full)
+    return dst
 
 
 def main():

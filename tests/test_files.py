@@ -8,6 +8,7 @@ import pytest
 from tpu_compiler_amd import capi, graphs, mlir_text
 
 REF_TESTS = "/root/reference/lib/Dialect/TPU/Backend/test"
+HERE = os.path.dirname(os.path.abspath(__file__))
 
 
 def test_npz_written_by_numpy_reads_back(tmp_path):
@@ -166,6 +167,36 @@ def test_reader_accepts_the_references_own_op_test_graphs():
     assert d[-1] == "return conv"
     d = capi.mlir_describe(os.path.join(REF_TESTS, "eltwise_add.mlir"))
     assert "op tpu.eltwise_add " in d
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_TESTS), reason="the reference checkout is not on this machine")
+def test_reader_output_equals_descriptions_typed_in_by_hand():
+    """the reader against an independent statement of what five of the reference's op-test graphs say
+    (tests/golden/reference_graph_facts.json, typed from the files' text): weight file, weights with
+    their shapes, every op in order with type / name / quant mode / param type / shape / operand wiring
+    (none operands included), every attribute value the file writes, the returned values in order"""
+    import json
+    facts = json.load(open(os.path.join(HERE, "golden", "reference_graph_facts.json")))
+    for name, want in facts.items():
+        if name.startswith("_"):
+            continue
+        d = capi.mlir_describe(os.path.join(REF_TESTS, name + ".mlir")).splitlines()
+        assert d[0] == "weight_file " + want["weight_file"], name
+        weights = [l.split(" ") for l in d if l.startswith("weight ")]
+        assert [(w[1], w[2], w[3]) for w in weights] == \
+            [(n, "NONE", "[" + ",".join(map(str, shp)) + "]") for n, shp in want["weights"]], name
+        ops = [l for l in d if l.startswith("op ")]
+        assert len(ops) == len(want["ops"]), name
+        for line, op in zip(ops, want["ops"]):
+            head, attrs = line.split(" {")
+            f = head.split()
+            assert f[1:5] == [op["type"], op["name"], op["quant"], op["param_type"]], line
+            assert f[5] == "[" + ",".join(map(str, op["shape"])) + "]", line
+            assert f[6:] == op["operands"], line
+            got = dict(kv.split("=") for kv in attrs.rstrip("}").split(",") if kv)
+            for k, v in op["attrs"].items():
+                assert k in got and float(got[k]) == float(v), (name, op["name"], k, got.get(k))
+        assert [l.split()[1] for l in d if l.startswith("return ")] == want["returns"], name
 
 
 def test_emitted_text_reads_back_as_the_same_graph(tmp_path):

@@ -36,8 +36,8 @@ def _inputs(g, seed):
 
 
 @pytest.mark.parametrize("name", NAMES)
-def test_stored_op_graphs_are_int8_graphs_the_oracle_covers(name):
-    g = mlir_graph.load(os.path.join(OPGRAPHS, name + "_int8.mlir"))
+def test_stored_op_graphs_are_int8_graphs_the_oracle_covers(name, tmp_path):
+    g = mlir_graph.load(_fx.materialize(name, tmp_path))
     body = [op for op in g.ops if op.type not in ("tpu.input", "tpu.quant", "tpu.reshape")]
     assert body and all(op.quant in ("INT8", "UINT8") for op in body), [(o.name, o.quant) for o in body]
     assert g.outputs and all(g.by_name[o].type == "tpu.quant" for o in g.outputs)
@@ -60,8 +60,8 @@ def test_oracle_runs_the_small_stored_op_graphs(name):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", NAMES)
-def test_hip_path_runs_the_reference_op_graphs_like_the_oracle(name):
-    path = os.path.join(OPGRAPHS, name + "_int8.mlir")
+def test_hip_path_runs_the_reference_op_graphs_like_the_oracle(name, tmp_path):
+    path = _fx.materialize(name, tmp_path)
     g = mlir_graph.load(path)
     xs = _inputs(g, 11 + len(name))
     for k, v in xs.items():
