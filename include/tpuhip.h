@@ -65,6 +65,10 @@ int tpuhip_free(tpuhip_ctx *ctx, void *dptr);
 int tpuhip_host_malloc(tpuhip_ctx *ctx, size_t bytes, void **hptr);
 int tpuhip_host_free(tpuhip_ctx *ctx, void *hptr);
 int tpuhip_memset(tpuhip_ctx *ctx, void *dptr, int value, size_t bytes);
+/* Free and total device memory as the HIP runtime this library is linked with reports them (a process
+ * may hold a second copy of the runtime, e.g. the one a Python package bundles, which sees other
+ * figures or no device).  No counterpart in the reference. */
+int tpuhip_mem_info(tpuhip_ctx *ctx, size_t *free_bytes, size_t *total_bytes);
 int tpuhip_upload(tpuhip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 int tpuhip_download(tpuhip_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
 int tpuhip_sync(tpuhip_ctx *ctx);

@@ -48,14 +48,6 @@ def test_fc_noalloc_equals_fc_on_two_calls_in_a_row():
     ctx.close()
 
 
-def _free_device_bytes():
-    import ctypes
-    hip = ctypes.CDLL("libamdhip64.so")
-    free, total = ctypes.c_size_t(), ctypes.c_size_t()
-    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
-    return free.value
-
-
 def test_fc_noalloc_leaves_the_free_device_memory_unchanged():
     """after a first call (which loads the code object) further calls take no device memory: the
     runtime's free-memory figure is the same before and after"""
@@ -65,11 +57,11 @@ def test_fc_noalloc_leaves_the_free_device_memory_unchanged():
     yt = ctx.tensor((32, 200, 1, 1))
     ctx.fc(wh, xt, yt, noalloc=True)
     ctx.sync()
-    before = _free_device_bytes()
+    before = ctx.mem_info()[0]
     for _ in range(3):
         ctx.fc(wh, xt, yt, noalloc=True)
     ctx.sync()
-    assert _free_device_bytes() == before
+    assert ctx.mem_info()[0] == before
     assert np.array_equal(ctx.to_nchw(yt).reshape(32, 200), want)
     ctx.conv_weights_destroy(wh)
     ctx.close()

@@ -73,6 +73,7 @@ PROTOTYPES = {
     "tpuhip_host_malloc": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
     "tpuhip_host_free": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_memset": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_size_t]),
+    "tpuhip_mem_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tpuhip_upload": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "tpuhip_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "tpuhip_sync": (C.c_int, [C.c_void_p]),
@@ -366,6 +367,12 @@ class Context:
 
     def sync(self):
         self._ck(self.lib.tpuhip_sync(self.h))
+
+    def mem_info(self):
+        """(free, total) device bytes as the library's HIP runtime sees them"""
+        free, total = C.c_size_t(), C.c_size_t()
+        self._ck(self.lib.tpuhip_mem_info(self.h, C.byref(free), C.byref(total)))
+        return free.value, total.value
 
     # -- events ------------------------------------------------------------
     def event(self):

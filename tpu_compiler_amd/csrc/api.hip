@@ -141,6 +141,13 @@ int tpuhip_memset(tpuhip_ctx *ctx, void *dptr, int value, size_t bytes) {
   return TPUHIP_OK;
 }
 
+int tpuhip_mem_info(tpuhip_ctx *ctx, size_t *free_bytes, size_t *total_bytes) {
+  TPUHIP_REQUIRE(ctx && free_bytes && total_bytes, "tpuhip_mem_info: NULL argument");
+  TPUHIP_CHECK_HIP(hipSetDevice(ctx->device));
+  TPUHIP_CHECK_HIP(hipMemGetInfo(free_bytes, total_bytes));
+  return TPUHIP_OK;
+}
+
 int tpuhip_upload(tpuhip_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
   TPUHIP_REQUIRE(ctx && (bytes == 0 || (dst_dev && src_host)), "tpuhip_upload: NULL argument");
   if (bytes == 0) return TPUHIP_OK;

@@ -380,7 +380,6 @@ __device__ __forceinline__ void epilogue_rows(const v16i (&acc)[TN], const ConvA
   epilogue_rows_lim<TN, FAST>(acc, a, oc, pmult, pshift, phpot, pix_first, pix_stride, lut, out, a.npix);
 }
 
-typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 // how a K group maps to filter taps (see load_tile)
 constexpr int kModeGeneral = 0;   // per-lane tap arithmetic

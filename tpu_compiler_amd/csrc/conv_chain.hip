@@ -46,11 +46,20 @@ struct ChainArgs {
   const int8_t *add_src;   // the add's other operand, or null: B reads A's result
   int8_t *add_dst;         // the sum, or null
   int8_t *y_b;
-  int npix, x_cs, n_tiles;
+  int npix, x_cs;
+  int n_tiles, n_full;     // tiles in all; the first n_full hold BN pixels, the rest 32
   uint32_t x_bytes;
   int lo1, lo2;            // 0: the conv clamps at 0 (ReLU) and its planes hold the short form
   int add_m_src, add_m_conv, add_rshift, add_relu, add_pk;
+#ifdef TPUHIP_TRACE
+  unsigned long long *trace;   // development builds: 32 shader-clock stamps per wave
+#endif
 };
+#ifdef TPUHIP_TRACE
+#define CHAIN_TS(k) (ts[k] = (unsigned long long)clock64())
+#else
+#define CHAIN_TS(k) ((void)0)
+#endif
 
 // W2LDS: conv B's filter fragments sit in LDS instead of registers (registers are what limits
 // the workgroups per CU of the narrow variant)
@@ -61,6 +70,11 @@ constexpr unsigned chain_lds_bytes() {
 
 template <int OC1, int KP1, int OC2, int BN, int OCC, bool W2LDS>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void conv_chain_kernel(ChainArgs a) {
+#ifdef TPUHIP_TRACE
+  unsigned long long ts[32] = {};
+  int nt = 0;
+#endif
+  CHAIN_TS(0);
   constexpr int NT = 512, NW = 8;
   constexpr int TM1 = OC1 / NW / 32;      // 32-channel blocks of conv A per wave
   constexpr int TN = BN / 32;             // 32-pixel blocks of a tile
@@ -75,6 +89,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   constexpr int NU = BN * CPR / NT;       // staged chunks per thread
   static_assert(TM1 >= 1 && TM1 * NW * 32 == OC1 && TN >= 1 && TN * 32 == BN, "bad tile");
   static_assert(NB2 >= 1 && NB2 <= NW && XCH <= NT && NU * NT == BN * CPR && KC1 * 64 == KP1, "bad tile");
+  static_assert(TN <= 2 && NU % TN == 0 && NT % CPR == 0 && (NU / TN) * (NT / CPR) == 32, "chunk walk: the first NU / TN chunks are the first 32 rows");
   extern __shared__ __attribute__((aligned(16))) v4i chain_smem[];
   v4i *const xB = chain_smem;                                                  // [2][KC1][BN][4 chunks], swizzled
   int8_t *const stage0 = reinterpret_cast<int8_t *>(xB + 2 * KC1 * BN * 4);    // [2][BN][SROW]
@@ -90,13 +105,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
   if (tile >= a.n_tiles) return;
   const int tstep = gridDim.x;
 
+  // Tiles of the launch: n_full tiles of BN pixels, then (TN == 2) tiles of 32 pixels for what is left,
+  // so that the last round of the workgroups' walk costs half a round where it is not full.
+  // Every tensor is addressed through a buffer descriptor with 32-bit offsets: a pixel past the
+  // end reads zeros and its stores are dropped, no branch and no 64-bit arithmetic per access.
   const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
+  const uint32_t big_bytes = (uint32_t)a.npix * (uint32_t)OC1;
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a.add_src, 0, a.add_src ? big_bytes : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t zrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a.add_dst, 0, a.add_dst ? big_bytes : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t yarsrc = __builtin_amdgcn_make_buffer_rsrc((void *)a.y_a, 0, a.y_a ? big_bytes : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ybrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.y_b, 0, (uint32_t)a.npix * (uint32_t)OC2, 0x00020000);
+  auto tile_pix0 = [&](int t) { return t < a.n_full ? t * BN : a.n_full * BN + (t - a.n_full) * 32; };
+  auto tile_blocks = [&](int t) { return t < a.n_full ? TN : 1; };
+
   const int lc = tid % CPRK, lrow = tid / CPRK;
   const bool loader = XCH == NT || tid < XCH;
   v4i breg;
   auto load_B = [&](int t) {
-    const bool ok = loader && t < a.n_tiles && t * BN + lrow < a.npix;
-    breg = buffer_load16(xrsrc, ok ? (uint32_t)((t * BN + lrow) * a.x_cs + lc * 16) : kOobOffset);
+    const bool ok = loader && t < a.n_tiles && lrow < 32 * tile_blocks(t);
+    breg = buffer_load16(xrsrc, ok ? (uint32_t)((tile_pix0(t) + lrow) * a.x_cs + lc * 16) : kOobOffset);
   };
   auto store_B = [&](int slot) {
     if (loader) xB[slot * (KC1 * BN * 4) + (lc >> 2) * (BN * 4) + lrow * 4 + ((lc & 3) ^ ((lrow >> 2) & 3))] = breg;
@@ -112,31 +140,62 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       fa1[i][ks] = reinterpret_cast<const v4i *>(a.w1)[((wave * TM1 + i) * KS1 + ks) * 64 + lane];
   const int ob = wave / TN, pb = wave % TN;   // conv B: this wave's block of the tile
   v4i fa2[W2LDS ? 1 : KS2];
-  if (W2LDS) {
-    for (int i = tid; i < OC1 * OC2 / 16; i += NT) w2l[i] = reinterpret_cast<const v4i *>(a.w2)[i];
-  } else if (wave < NB2) {
+  if (!W2LDS && wave < NB2) {
 #pragma unroll
     for (int ks = 0; ks < KS2; ++ks) fa2[ks] = reinterpret_cast<const v4i *>(a.w2)[(ob * KS2 + ks) * 64 + lane];
   }
-  for (int i = tid; i < 5 * OC1; i += NT) q1[i] = a.q1[i];
-  for (int i = tid; i < 5 * OC2; i += NT) q2[i] = a.q2[i];
+  // What goes to LDS once -- the parameter planes, conv B's filter (W2LDS) -- is requested in one
+  // go and parked afterwards: one trip to memory for all of it, not one per piece.
+  constexpr int NQ1 = (5 * OC1 / 4 + NT - 1) / NT, NQ2 = (5 * OC2 / 4 + NT - 1) / NT;
+  constexpr int NW2 = W2LDS ? (OC1 * OC2 / 16 + NT - 1) / NT : 0;
+  v4i rq1[NQ1], rq2[NQ2], rw2[NW2 > 0 ? NW2 : 1];
+#pragma unroll
+  for (int u = 0; u < NQ1; ++u)
+    if (tid + u * NT < 5 * OC1 / 4) rq1[u] = reinterpret_cast<const v4i *>(a.q1)[tid + u * NT];
+#pragma unroll
+  for (int u = 0; u < NQ2; ++u)
+    if (tid + u * NT < 5 * OC2 / 4) rq2[u] = reinterpret_cast<const v4i *>(a.q2)[tid + u * NT];
+#pragma unroll
+  for (int u = 0; u < NW2; ++u)
+    if (tid + u * NT < OC1 * OC2 / 16) rw2[u] = reinterpret_cast<const v4i *>(a.w2)[tid + u * NT];
+  __builtin_amdgcn_sched_barrier(0);
+  auto park_constants = [&]() {
+#pragma unroll
+    for (int u = 0; u < NQ1; ++u)
+      if (tid + u * NT < 5 * OC1 / 4) reinterpret_cast<v4i *>(q1)[tid + u * NT] = rq1[u];
+#pragma unroll
+    for (int u = 0; u < NQ2; ++u)
+      if (tid + u * NT < 5 * OC2 / 4) reinterpret_cast<v4i *>(q2)[tid + u * NT] = rq2[u];
+#pragma unroll
+    for (int u = 0; u < NW2; ++u)
+      if (tid + u * NT < OC1 * OC2 / 16) w2l[tid + u * NT] = rw2[u];
+  };
+  park_constants();
   store_B(0);
   load_B(tile + tstep);
   __syncthreads();
+  CHAIN_TS(1);
 
+  // this thread's chunks of a staged tile: chunk u is (row frow_u, 16-byte column fcc) -- rows in
+  // steps of NT / CPR, so that the first NU / TN chunks cover the first 32 rows
+  const int frow0 = tid / CPR, fcc = tid % CPR;
+  const uint32_t foff0 = (uint32_t)(frow0 * OC1 + fcc * 16);
   int cur = 0;
   for (;;) {
-    const int pix0 = tile * BN;
+    const int pix0 = tile_pix0(tile);
+    const int tn = tile_blocks(tile);          // 32-pixel blocks of this tile (uniform)
+    const uint32_t tile_off = (uint32_t)pix0 * (uint32_t)OC1;
+#ifdef TPUHIP_TRACE
+    const bool tr = nt < 4;
+    if (tr) CHAIN_TS(2 + nt * 6);
+#endif
     // the add's other operand for this thread's chunks of the tile: asked for now, used after GEMM 1
     v4i sv[NU];
     if (a.add_src) {
 #pragma unroll
-      for (int u = 0; u < NU; ++u) {
-        const int q = tid + u * NT;
-        const int row = q / CPR, cc = q % CPR;
-        if (pix0 + row < a.npix)
-          sv[u] = *reinterpret_cast<const v4i *>(a.add_src + (int64_t)(pix0 + row) * OC1 + cc * 16);
-      }
+      for (int u = 0; u < NU; ++u)
+        if (u < NU / TN || tn == TN)
+          sv[u] = buffer_load16(srsrc, tile_off + foff0 + (uint32_t)(u * (NT / CPR) * OC1));
     }
     // ---- GEMM 1: this wave's channels x the tile's pixels
     v16i acc[TM1][TN];
@@ -159,8 +218,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
       for (int i = 0; i < TM1; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i][ks], fb[j], acc[i][j], 0, 0, 0);
+          if (j < tn) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i][ks], fb[j], acc[i][j], 0, 0, 0);
     }
+#ifdef TPUHIP_TRACE
+    if (tr) CHAIN_TS(3 + nt * 6);
+#endif
     // the next tile's pixels go to the other LDS tile, the one after that is requested
     const int next = tile + tstep;
     store_B(cur ^ 1);
@@ -169,41 +231,56 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     // ---- requantisation of conv A into the staged tile
     int8_t *const stage = stage0 + cur * (BN * SROW);
 #pragma unroll
-    for (int i = 0; i < TM1; ++i) {
-      uint32_t outw[TN][4];
-      const int cb = wave * (32 * TM1) + fk * (16 * TM1) + i * 16;   // the lane's 16 channels of block i
-      if (a.lo1 == 0)
-        requant_rows_c64<TN, true>(acc[i], 0, q1 + 2 * cb, q1 + 2 * OC1 + cb, q1 + 3 * OC1 + cb, q1 + 4 * OC1 + cb, outw);
-      else
-        requant_rows_c64<TN, false>(acc[i], -128, q1 + 2 * cb, q1 + 2 * OC1 + cb, q1 + 3 * OC1 + cb, q1 + 4 * OC1 + cb, outw);
+    for (int j = 0; j < TN; ++j) {
+      if (j < tn) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        *reinterpret_cast<v4i *>(stage + (j * 32 + frow) * SROW + cb) =
-            v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
+        for (int i = 0; i < TM1; ++i) {
+          uint32_t outw[1][4];
+          const int cb = wave * (32 * TM1) + fk * (16 * TM1) + i * 16;   // the lane's 16 channels of block i
+          const v16i (&blk)[1] = reinterpret_cast<const v16i (&)[1]>(acc[i][j]);
+          if (a.lo1 == 0)
+            requant_rows_c64<1, true>(blk, 0, q1 + 2 * cb, q1 + 2 * OC1 + cb, q1 + 3 * OC1 + cb, q1 + 4 * OC1 + cb, outw);
+          else
+            requant_rows_c64<1, false>(blk, -128, q1 + 2 * cb, q1 + 2 * OC1 + cb, q1 + 3 * OC1 + cb, q1 + 4 * OC1 + cb, outw);
+          *reinterpret_cast<v4i *>(stage + (j * 32 + frow) * SROW + cb) =
+              v4i{(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+        }
+      }
     }
+#ifdef TPUHIP_TRACE
+    if (tr) CHAIN_TS(4 + nt * 6);
+#endif
     __syncthreads();
+#ifdef TPUHIP_TRACE
+    if (tr) CHAIN_TS(5 + nt * 6);
+#endif
 
     // ---- flush in memory order: A's result, the add, the sum back into the staged tile
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-      const int q = tid + u * NT;
-      const int row = q / CPR, cc = q % CPR;
-      if (pix0 + row < a.npix) {
-        const int64_t off = (int64_t)(pix0 + row) * OC1 + cc * 16;
-        v4i *const sp = reinterpret_cast<v4i *>(stage + row * SROW + cc * 16);
+      if (u < NU / TN || tn == TN) {
+        const int row = frow0 + u * (NT / CPR);
+        const uint32_t off = tile_off + foff0 + (uint32_t)(u * (NT / CPR) * OC1);
+        v4i *const sp = reinterpret_cast<v4i *>(stage + row * SROW + fcc * 16);
         const v4i o = *sp;
-        if (a.y_a) *reinterpret_cast<v4i *>(a.y_a + off) = o;
+        if (a.y_a) __builtin_amdgcn_raw_buffer_store_b128((v4u)o, yarsrc, off, 0, 0);
         if (a.add_src) {
           const v4i z = fused_add_chunk(o, sv[u], a.add_m_src, a.add_m_conv, a.add_rshift, a.add_relu, a.add_pk);
-          if (a.add_dst) *reinterpret_cast<v4i *>(a.add_dst + off) = z;
+          if (a.add_dst) __builtin_amdgcn_raw_buffer_store_b128((v4u)z, zrsrc, off, 0, 0);
           *sp = z;
         }
       }
     }
+#ifdef TPUHIP_TRACE
+    if (tr) CHAIN_TS(6 + nt * 6);
+#endif
     __syncthreads();
+#ifdef TPUHIP_TRACE
+    if (tr) CHAIN_TS(7 + nt * 6);
+#endif
 
     // ---- GEMM 2: conv B on the staged tile
-    if (wave < NB2) {
+    if (wave < NB2 && pb < tn) {
       v16i acc2[1];
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc2[0][e] = 0;
@@ -218,15 +295,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
         requant_rows_c64<1, true>(acc2, 0, q2 + 2 * cb, q2 + 2 * OC2 + cb, q2 + 3 * OC2 + cb, q2 + 4 * OC2 + cb, outw);
       else
         requant_rows_c64<1, false>(acc2, -128, q2 + 2 * cb, q2 + 2 * OC2 + cb, q2 + 3 * OC2 + cb, q2 + 4 * OC2 + cb, outw);
-      const int pix = pix0 + pb * 32 + frow;
-      if (pix < a.npix)
-        *reinterpret_cast<v4i *>(a.y_b + (int64_t)pix * OC2 + cb) =
-            v4i{(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+      const v4u o2 = {outw[0][0], outw[0][1], outw[0][2], outw[0][3]};
+      __builtin_amdgcn_raw_buffer_store_b128(o2, ybrsrc, (uint32_t)((pix0 + pb * 32 + frow) * OC2 + cb), 0, 0);
     }
+#ifdef TPUHIP_TRACE
+    ++nt;
+#endif
     if (next >= a.n_tiles) break;
     tile = next;
     cur ^= 1;
   }
+  CHAIN_TS(30);
+#ifdef TPUHIP_TRACE
+  ts[31] = (unsigned long long)nt;
+  if (a.trace && lane == 0)
+    for (int k = 0; k < 32; ++k) a.trace[((size_t)blockIdx.x * 8 + wave) * 32 + k] = ts[k];
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -428,6 +512,9 @@ int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const v
   a.x_bytes = (uint32_t)((int64_t)a.npix * da.x_cs);
   a.lo1 = da.do_relu ? 0 : -128;
   a.lo2 = ch->db.do_relu ? 0 : -128;
+#ifdef TPUHIP_TRACE
+  a.trace = getenv("TPUHIP_TRACE_PTR") ? (unsigned long long *)strtoull(getenv("TPUHIP_TRACE_PTR"), nullptr, 16) : nullptr;
+#endif
   if (add) {
     a.add_m_src = f->m_src;
     a.add_m_conv = f->m_conv;
@@ -441,10 +528,15 @@ int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const v
     auto kernel = conv_chain_kernel<OC1, KP1, OC2, BN, O, L>;                                              \
     constexpr unsigned lds = chain_lds_bytes<OC1, KP1, OC2, BN, L>();                                      \
     TPUHIP_REQUIRE(raise_chain_lds((const void *)kernel, lds), "conv chain: raising the LDS limit failed"); \
-    a.n_tiles = (a.npix + BN - 1) / BN;                                                                    \
     const int per_cu = std::max(1, std::min((int)(160u * 1024 / lds), O / 2));                             \
-    int gsz = std::min(a.n_tiles, ctx->num_cu * per_cu);                                                   \
-    if (const char *e = getenv("TPUHIP_CHAIN_GRID")) gsz = std::min(a.n_tiles, atoi(e));                   \
+    const int slots = ctx->num_cu * per_cu;                                                                \
+    /* whole rounds of BN-pixel tiles over the resident workgroups; what is left runs as 32-pixel */       \
+    /* tiles if one round of those covers it (half a round's time instead of a whole one), else as */      \
+    /* BN-pixel tiles with the ragged end in 32-pixel tiles */                                             \
+    a.n_full = a.npix / BN / slots * slots;                                                                \
+    if (BN == 32 || a.npix - a.n_full * BN > slots * 32) a.n_full = a.npix / BN;                           \
+    a.n_tiles = a.n_full + (a.npix - a.n_full * BN + 31) / 32;                                             \
+    const int gsz = std::min(a.n_tiles, slots);                                                            \
     const dim3 grid((unsigned)gsz), block(512);                                                            \
     if (ctx->prof_start)                                                                                   \
       hipExtLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \

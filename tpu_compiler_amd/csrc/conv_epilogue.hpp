@@ -24,6 +24,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 // tile-local weight row (as the MFMA sees it) -> tile-local output channel
 __host__ __device__ inline int mfma_row_to_oc(int row, int tm) {
