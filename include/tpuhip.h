@@ -204,6 +204,16 @@ int tpuhip_conv2d_pair_i8(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const v
  * op). */
 typedef struct tpuhip_conv_chain tpuhip_conv_chain;
 int tpuhip_conv2d_can_chain(const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b);
+/* A second kind of chain: conv A a depthwise conv (g == ic == oc, at most 3 x 3 taps, any stride,
+ * padding and dilation; core/conv.cpp:11-78, the g != 1 branch), conv B the unpadded 1x1 / stride 1 conv
+ * of at most 384 output channels that reads A's result -- the depthwise + projection half of an
+ * inverted-residual block.  A 256-entry table (LutOpKernel: core/activation.cpp:47-53,
+ * core/clip.cpp:29-40) may ride behind A and an EltwiseAdd (core/eltwise.cpp:52-85) behind B; A's
+ * result, the widest tensor of the block, stays on chip unless the caller keeps it.
+ * tpuhip_conv2d_chain_kind: 0 = the two convs do not chain, 1 = two pointwise convs (an add behind A),
+ * 2 = depthwise then pointwise (a table behind A, an add behind B).  tpuhip_conv2d_can_chain answers
+ * kind != 0 and tpuhip_conv2d_chain_prepack packs either kind. */
+int tpuhip_conv2d_chain_kind(const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b);
 int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc_a, const tpuhip_conv_desc *desc_b,
                                 const int8_t *filter_a, const int32_t *bias_a, const int32_t *multiplier_a,
                                 const int32_t *rshift_a, const int8_t *filter_b, const int32_t *bias_b,
@@ -212,6 +222,12 @@ int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *chain);
 /* f == NULL or f->enable == 0: no add, B reads A's result (add_src / add_out ignored) */
 int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y_a,
                            const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b);
+/* The general call: post_a / post_b (either may be NULL) say what rides behind conv A and conv B, with
+ * tpuhip_conv_post's meaning (no pool); y_a, y_b and the outputs inside the posts may be NULL where the
+ * caller does not keep a tensor, as long as something of B's is written.  A chain refuses, with an error,
+ * the fused work its kind does not take. */
+int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y_a,
+                                const tpuhip_conv_post *post_a, void *y_b, const tpuhip_conv_post *post_b);
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *chain);
 /* name of chain kernel variant `variant`, NULL past the last one */
 const char *tpuhip_conv2d_chain_variant_name(int variant);

@@ -185,6 +185,8 @@ PROTOTYPES.update({
                                               C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "tpuhip_conv2d_chain_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_conv2d_chain_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd), C.c_void_p]),
+    "tpuhip_conv2d_chain_kind": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]),
+    "tpuhip_conv2d_chain_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost), C.c_void_p, C.POINTER(ConvPost)]),
     "tpuhip_conv2d_chain_name": (C.c_char_p, [C.c_void_p]),
     "tpuhip_conv2d_chain_variant_name": (C.c_char_p, [C.c_int]),
     "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
@@ -488,6 +490,30 @@ class Context:
         self._ck(self.lib.tpuhip_conv2d_chain_i8(
             self.h, ch, x.ptr, None if y_a is None else y_a.ptr, None if src is None else src.ptr,
             None if out is None else out.ptr, None if f is None else C.byref(f), y_b.ptr))
+
+    def conv_chain_kind(self, desc_a, desc_b):
+        """0: no chain; 1: two pointwise convs; 2: a depthwise conv and the pointwise conv behind it"""
+        return int(self.lib.tpuhip_conv2d_chain_kind(C.byref(desc_a), C.byref(desc_b)))
+
+    def conv_chain_post(self, ch, x, y_b=None, y_a=None, table_a=None, lut_out_a=None, add_a=None, add_b=None):
+        """the general chain call: a table and / or an add = (src, out or None, m_src, m_conv, rshift, relu)
+        behind conv A, an add behind conv B, as far as the chain's kind takes them"""
+        pa, pb = ConvPost(), ConvPost()
+        keep = None
+        if table_a is not None:
+            keep = np.ascontiguousarray(table_a, dtype=np.int8)
+            assert keep.size == 256
+            pa.lut = keep.ctypes.data
+            pa.lut_out = None if lut_out_a is None else lut_out_a.ptr
+        for post, add in ((pa, add_a), (pb, add_b)):
+            if add is not None:
+                src, out, m_src, m_conv, rshift, relu = add
+                post.add = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(relu))
+                post.add_src = src.ptr
+                post.add_out = None if out is None else out.ptr
+        self._ck(self.lib.tpuhip_conv2d_chain_post_i8(
+            self.h, ch, x.ptr, None if y_a is None else y_a.ptr, C.byref(pa),
+            None if y_b is None else y_b.ptr, C.byref(pb)))
 
     def conv_chain_destroy(self, ch):
         self._ck(self.lib.tpuhip_conv2d_chain_destroy(self.h, ch))

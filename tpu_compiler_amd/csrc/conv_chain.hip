@@ -24,15 +24,9 @@
 //     stored 16 bytes per lane.
 // Two barriers per tile; the staged tile is double-buffered so that GEMM 2 of one tile and the
 // requantisation of the next overlap.
-#include "common.hpp"
-#include "conv_epilogue.hpp"
+#include "conv_chain.hpp"
 
-#include <cstdlib>
 #include <cstring>
-#include <map>
-#include <mutex>
-#include <string>
-#include <vector>
 
 using namespace tpuhip;
 
@@ -316,15 +310,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-struct tpuhip_conv_chain {
-  tpuhip_conv_desc da, db;
-  int variant = -1;
-  int kp1 = 0;
-  int8_t *w1 = nullptr, *w2 = nullptr;
-  int32_t *q1 = nullptr, *q2 = nullptr;
-  std::string name;
-};
-
 namespace {
 
 struct ChainVariant {
@@ -342,13 +327,8 @@ const ChainVariant kChainVariants[] = {
 };
 constexpr int kNumChainVariants = (int)(sizeof(kChainVariants) / sizeof(kChainVariants[0]));
 
-bool is_pointwise(const tpuhip_conv_desc &d) {
-  return d.g == 1 && d.kh == 1 && d.kw == 1 && d.sh == 1 && d.sw == 1 && d.dh == 1 && d.dw == 1 && d.pt == 0 &&
-         d.pb == 0 && d.pl == 0 && d.pr == 0 && !d.ins_h && !d.ins_w && !d.relu_first && d.ih == d.oh && d.iw == d.ow;
-}
-
 int chain_variant_for(const tpuhip_conv_desc &a, const tpuhip_conv_desc &b) {
-  if (!is_pointwise(a) || !is_pointwise(b)) return -1;
+  if (!is_pointwise_conv(a) || !is_pointwise_conv(b)) return -1;
   if (a.n != b.n || a.oh != b.ih || a.ow != b.iw || b.ic != a.oc) return -1;
   for (int v = 0; v < kNumChainVariants; ++v) {
     const ChainVariant &c = kChainVariants[v];
@@ -360,75 +340,24 @@ int chain_variant_for(const tpuhip_conv_desc &a, const tpuhip_conv_desc &b) {
   return -1;
 }
 
-// per-channel planes the kernel copies into LDS: (low, high) of the 64-bit addend, multiplier,
-// shift, 2^(r-1); with a ReLU the short form (addend + 2^(r-1) * 2^31, shift r - 1).
-// false: the overflow-free requantisation cannot be proved for some channel
 bool chain_planes(const tpuhip_conv_desc &d, const int8_t *filter, const int32_t *bias, const int32_t *mult,
                   const int32_t *rshift, std::vector<int32_t> *out) {
-  const int oc = d.oc;
-  const size_t per_oc = (size_t)d.ic;
-  out->assign((size_t)5 * oc, 0);
-  const bool relu = d.do_relu != 0;
-  for (int i = 0; i < oc; ++i) {
-    if (rshift[i] < 1 || rshift[i] > 31) return false;
-    const int32_t b = (d.with_bias && bias) ? bias[i] : 0;
-    const int64_t hpot = 1ll << (rshift[i] - 1);
-    int64_t sumw = 0;
-    for (size_t k = 0; k < per_oc; ++k) sumw += std::abs((int)filter[(size_t)i * per_oc + k]);
-    if (128 * sumw + std::llabs((long long)b) + 1 + hpot >= (1ll << 31)) return false;
-    int64_t c = (int64_t)b * (int64_t)mult[i] + (1ll << 30);
-    if (relu) c += hpot << 31;
-    (*out)[2 * i] = (int32_t)(uint32_t)(c & 0xffffffffll);
-    (*out)[2 * i + 1] = (int32_t)(c >> 32);
-    (*out)[2 * oc + i] = mult[i];
-    (*out)[3 * oc + i] = rshift[i] - (relu ? 1 : 0);
-    (*out)[4 * oc + i] = (int32_t)hpot;
-  }
-  return true;
-}
-
-// MFMA A-operand fragments of a [oc][k] filter: [32-channel block][K slice][lane][16 bytes], lane l
-// holding MFMA row l & 31 -- channel mfma_row_to_oc(row, tm) of its group of tm blocks -- and K
-// bytes 32 * slice + 16 * (l >> 5) .. + 15
-std::vector<int8_t> chain_fragments(const int8_t *filter, int oc, int ic, int kp, int tm) {
-  const int nblk = oc / 32, ks_n = kp / 32;
-  std::vector<int8_t> out((size_t)nblk * ks_n * 1024, 0);
-  for (int blk = 0; blk < nblk; ++blk)
-    for (int ks = 0; ks < ks_n; ++ks)
-      for (int l = 0; l < 64; ++l) {
-        const int group0 = blk / tm * tm * 32;
-        const int ch = group0 + mfma_row_to_oc((blk % tm) * 32 + (l & 31), tm);
-        for (int b = 0; b < 16; ++b) {
-          const int k = ks * 32 + (l >> 5) * 16 + b;
-          if (k < ic) out[((size_t)(blk * ks_n + ks) * 64 + l) * 16 + b] = filter[(size_t)ch * ic + k];
-        }
-      }
-  return out;
-}
-
-bool raise_chain_lds(const void *kernel, unsigned bytes) {
-  static std::mutex mu;
-  static std::map<const void *, unsigned> raised;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = raised.find(kernel);
-  if (it != raised.end() && it->second >= bytes) return true;
-  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return false;
-  raised[kernel] = bytes;
-  return true;
-}
-
-template <typename T>
-int upload_vec(tpuhip_ctx *ctx, const std::vector<T> &v, T **dptr) {
-  if (int rc = tpuhip_malloc(ctx, v.size() * sizeof(T), (void **)dptr)) return rc;
-  return tpuhip_upload(ctx, *dptr, v.data(), v.size() * sizeof(T));
+  return requant_planes(d.oc, d.oc, (size_t)d.ic, d.do_relu != 0, filter, (d.with_bias && bias) ? bias : nullptr, mult,
+                        rshift, out);
 }
 
 }  // namespace
 
 extern "C" {
 
+int tpuhip_conv2d_chain_kind(const tpuhip_conv_desc *da, const tpuhip_conv_desc *db) {
+  if (!da || !db) return 0;
+  if (chain_variant_for(*da, *db) >= 0) return 1;
+  return dwpw_covers(*da, *db) ? 2 : 0;
+}
+
 int tpuhip_conv2d_can_chain(const tpuhip_conv_desc *da, const tpuhip_conv_desc *db) {
-  return da && db && chain_variant_for(*da, *db) >= 0 ? 1 : 0;
+  return tpuhip_conv2d_chain_kind(da, db) != 0 ? 1 : 0;
 }
 
 int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, const tpuhip_conv_desc *db,
@@ -438,10 +367,24 @@ int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, con
   TPUHIP_REQUIRE(ctx && da && db && filter_a && filter_b && mult_a && mult_b && rshift_a && rshift_b && out,
                  "tpuhip_conv2d_chain_prepack: NULL argument");
   const int v = chain_variant_for(*da, *db);
+  if (v < 0 && dwpw_covers(*da, *db)) {
+    auto *ch = new tpuhip_conv_chain();
+    ch->da = *da;
+    ch->db = *db;
+    ch->kind = 2;
+    const int rc = dwpw_prepack(ctx, ch, filter_a, bias_a, mult_a, rshift_a, filter_b, bias_b, mult_b, rshift_b);
+    if (rc) {
+      tpuhip_conv2d_chain_destroy(ctx, ch);
+      return rc;
+    }
+    *out = ch;
+    return TPUHIP_OK;
+  }
   if (v < 0)
     return set_error(TPUHIP_ERR_UNSUPPORTED,
                      "conv chain: needs two unpadded 1x1 / stride 1 convs, the first 33..64 -> 256 or 65..128 -> 512 "
-                     "channels, the second 256 -> 64 or 512 -> 128, dense channel strides");
+                     "channels, the second 256 -> 64 or 512 -> 128, dense channel strides -- or a depthwise conv of "
+                     "at most 3 x 3 taps and the unpadded 1x1 / stride 1 conv of at most 384 channels behind it");
   std::vector<int32_t> p1, p2;
   if (!chain_planes(*da, filter_a, bias_a, mult_a, rshift_a, &p1) ||
       !chain_planes(*db, filter_b, bias_b, mult_b, rshift_b, &p2))
@@ -452,11 +395,12 @@ int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, con
   auto *ch = new tpuhip_conv_chain();
   ch->da = *da;
   ch->db = *db;
+  ch->kind = 1;
   ch->variant = v;
   ch->kp1 = c.kp1;
   ch->name = c.name;
-  const std::vector<int8_t> f1 = chain_fragments(filter_a, c.oc1, da->ic, c.kp1, c.oc1 / 8 / 32);
-  const std::vector<int8_t> f2 = chain_fragments(filter_b, c.oc2, db->ic, c.oc1, 1);
+  const std::vector<int8_t> f1 = mfma_a_fragments(filter_a, c.oc1, c.oc1 / 32, da->ic, c.kp1, c.oc1 / 8 / 32);
+  const std::vector<int8_t> f2 = mfma_a_fragments(filter_b, c.oc2, c.oc2 / 32, db->ic, c.oc1, 1);
   int rc = upload_vec(ctx, f1, &ch->w1);
   if (!rc) rc = upload_vec(ctx, f2, &ch->w2);
   if (!rc) rc = upload_vec(ctx, p1, &ch->q1);
@@ -483,13 +427,30 @@ int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *ch) {
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *ch) { return ch ? ch->name.c_str() : "null"; }
 
 const char *tpuhip_conv2d_chain_variant_name(int variant) {
-  return variant >= 0 && variant < kNumChainVariants ? kChainVariants[variant].name : nullptr;
+  if (variant < 0) return nullptr;
+  return variant < kNumChainVariants ? kChainVariants[variant].name : dwpw_variant_name(variant - kNumChainVariants);
+}
+
+int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a,
+                                const tpuhip_conv_post *post_a, void *y_b, const tpuhip_conv_post *post_b) {
+  TPUHIP_REQUIRE(ctx && ch && x, "tpuhip_conv2d_chain_post_i8: NULL argument");
+  TPUHIP_REQUIRE(!(post_a && post_a->pool) && !(post_b && post_b->pool), "conv chain: takes no fused pool");
+  if (ch->kind == 2) return dwpw_run(ctx, ch, x, y_a, post_a, y_b, post_b);
+  TPUHIP_REQUIRE(!(post_a && post_a->lut) && !(post_b && (post_b->lut || post_b->add.enable)),
+                 "conv chain: two pointwise convs take an add behind the first conv and nothing else");
+  return tpuhip_conv2d_chain_i8(ctx, ch, x, y_a, post_a ? post_a->add_src : nullptr, post_a ? post_a->add_out : nullptr,
+                                post_a ? &post_a->add : nullptr, y_b);
 }
 
 int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a,
                            const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b) {
   TPUHIP_REQUIRE(ctx && ch && x && y_b, "tpuhip_conv2d_chain_i8: NULL argument");
   const bool add = f && f->enable;
+  if (ch->kind == 2) {
+    TPUHIP_REQUIRE(!add, "conv chain: a depthwise -> pointwise chain takes its add behind the second conv "
+                         "(tpuhip_conv2d_chain_post_i8)");
+    return dwpw_run(ctx, ch, x, y_a, nullptr, y_b, nullptr);
+  }
   TPUHIP_REQUIRE(!add || add_src, "conv chain: fused add without its other operand");
   if (add) {
     TPUHIP_REQUIRE(f->rshift >= 0 && f->rshift <= 30, "conv chain: add rshift %d outside [0,30]", f->rshift);
@@ -527,7 +488,7 @@ int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const v
   case i: {                                                                                                \
     auto kernel = conv_chain_kernel<OC1, KP1, OC2, BN, O, L>;                                              \
     constexpr unsigned lds = chain_lds_bytes<OC1, KP1, OC2, BN, L>();                                      \
-    TPUHIP_REQUIRE(raise_chain_lds((const void *)kernel, lds), "conv chain: raising the LDS limit failed"); \
+    TPUHIP_REQUIRE(raise_dynamic_lds((const void *)kernel, lds), "conv chain: raising the LDS limit failed"); \
     const int per_cu = std::max(1, std::min((int)(160u * 1024 / lds), O / 2));                             \
     const int slots = ctx->num_cu * per_cu;                                                                \
     /* whole rounds of BN-pixel tiles over the resident workgroups; what is left runs as 32-pixel */       \
