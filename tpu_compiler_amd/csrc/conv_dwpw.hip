@@ -17,12 +17,21 @@
 //     the requantisation they are four dwords, which is exactly the B-operand fragment of the 1x1
 //     conv's MFMA for that 32-channel K slice.  They go to LDS in that form.
 //   * phase 2, pointwise: the workgroup's P pixel blocks x (output channels / 32) result blocks
-//     are dealt to the four waves; a wave walks the K slices, A fragments (the 1x1 filter, packed
-//     in fragment order) from global memory, B fragments from LDS, then requantises, adds the
+//     are dealt to the four waves -- or, where there are fewer than four, a result block's K slices
+//     are split between waves and the parts added up in LDS (integer adds: any order, same sum).  A
+//     wave requests the A fragments (the 1x1 filter, packed in fragment order) of up to eight K
+//     slices at a time from global memory, takes the B fragments from LDS, then requantises, adds the
 //     residual and stores 16 bytes per lane.
-// A workgroup owns P consecutive pixel blocks (P = 4 for narrow 1x1 convs, so that phase 2 has a
-// block for every wave, down to 1 for wide ones); the waves split the (K slice, pixel block) items
-// of phase 1 in K-slice-major order, so a wave reloads its nine diagonal fragments once per P items.
+// A workgroup owns P consecutive pixel blocks (P = 4 for narrow 1x1 convs, down to 1 for wide ones);
+// the waves split the (K slice, pixel block) items of phase 1 in K-slice-major order, so a wave reloads
+// its nine diagonal fragments once per P items.  The first item's input is requested before the data the
+// workgroup shares (the 1x1 conv's requantisation planes, the table) is copied to LDS.
+//
+// Measured on MobileNetV2's blocks at batch 64 the launch is within +-10 % of the two launches it
+// replaces on maps of 14 x 14 to 56 x 56 and slower on 7 x 7 maps and on 1x1 convs of more than 96
+// channels: both forms issue about nine vector instructions per depthwise output (requantisation,
+// neighbour-lane moves, addresses) and that, not the memory traffic saved, bounds them.  Callers
+// choose per layer pair; the graph interpreter does not chain depthwise convs by itself.
 #include "conv_chain.hpp"
 
 #include <algorithm>
@@ -54,6 +63,7 @@ struct DwPwArgs {
   int xblocks, rblocks, nblocks;     // column blocks per output row, row blocks per image, n * rblocks * xblocks
   uint32_t magic_w;                  // ceil(2^32 / width)
   int log2p, n_cb, n_tm, ngroups;    // P = 1 << log2p pixel blocks per workgroup
+  int nk;                            // phase 2: waves that split the K slices of one result block
 };
 
 template <bool SHIFT, int NT>
@@ -66,6 +76,8 @@ conv_dwpw_kernel(DwPwArgs a) {
   int32_t *q2 = reinterpret_cast<int32_t *>(smem + (size_t)P * a.n_cb * 1024);   // the 1x1 conv's planes
   int32_t *qall = q2 + 5 * ocp;                                                // [4 waves][160]
   uint32_t *lutw = reinterpret_cast<uint32_t *>(qall + 4 * 160);
+  int32_t *red = reinterpret_cast<int32_t *>(lutw + 64);                        // [result block][16][64] when nk > 1
+  const int tiles = a.n_tm << a.log2p;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -79,9 +91,6 @@ conv_dwpw_kernel(DwPwArgs a) {
   const int b0 = g << a.log2p;
   const int nb = min(P, a.nblocks - b0);                    // pixel blocks of this group that exist
 
-  for (int i = threadIdx.x; i < 5 * ocp; i += 256) q2[i] = a.qpw[i];
-  if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
-  __syncthreads();
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
 
   // block b0 -> (image, row block, column block); the next ones follow with carries
@@ -169,6 +178,12 @@ conv_dwpw_kernel(DwPwArgs a) {
     };
 
     if (it < it_end) request(it >> a.log2p, it & (P - 1));
+    // what the whole workgroup shares goes to LDS while the first input is on its way
+    for (int i = threadIdx.x; i < 5 * ocp; i += 256) q2[i] = a.qpw[i];
+    if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+    if (a.nk > 1)
+      for (int i = threadIdx.x; i < tiles * 1024; i += 256) red[i] = 0;
+    __syncthreads();
     while (it < it_end) {
       const int cb = it >> a.log2p, p = it & (P - 1);
       if (cb != cur_cb) {
@@ -234,16 +249,20 @@ conv_dwpw_kernel(DwPwArgs a) {
 
   // ---- phase 2: pointwise --------------------------------------------------
   {
-    const int Tt = a.n_tm << a.log2p;
-    // result block t -> (channel block t >> log2p, pixel block t & (P - 1)); a wave takes t = wave + 4 i
-    int tm[NT], pp[NT];
+    // a unit of work: (result block t, part kp of its K slices); result block t -> (channel block t >> log2p,
+    // pixel block t & (P - 1)).  nk > 1: wave w takes block w % tiles, part w / tiles, and the parts meet in
+    // LDS; nk == 1: wave w takes blocks w, w + 4, ...
+    int tl[NT], tm[NT], pp[NT];
     bool on[NT];
+    const int kp = a.nk > 1 ? wave / tiles : 0;
+    const int kper = (a.n_cb + a.nk - 1) / a.nk;
+    const int k0 = kp * kper, k1 = min(a.n_cb, k0 + kper);
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      const int t = wave + 4 * i;
-      tm[i] = t >> a.log2p;
-      pp[i] = t & (P - 1);
-      on[i] = (t < Tt) & (pp[i] < nb);
+      tl[i] = a.nk > 1 ? wave - kp * tiles : wave + 4 * i;
+      tm[i] = tl[i] >> a.log2p;
+      pp[i] = tl[i] & (P - 1);
+      on[i] = (tl[i] < tiles) & (pp[i] < nb) & (kp < a.nk) & (a.nk == 1 || i == 0);
     }
     v16i acc2[NT][1];
 #pragma unroll
@@ -251,25 +270,37 @@ conv_dwpw_kernel(DwPwArgs a) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc2[i][0][e] = 0;
     const v4i *wfrag = reinterpret_cast<const v4i *>(a.wpw) + lane;
-    v4i an[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-      an[i] = v4i{0, 0, 0, 0};
-      if (on[i]) an[i] = wfrag[(size_t)(tm[i] * a.n_cb) * 64];
-    }
-    for (int cb = 0; cb < a.n_cb; ++cb) {
-      v4i ac[NT];
-#pragma unroll
-      for (int i = 0; i < NT; ++i) ac[i] = an[i];
-      if (cb + 1 < a.n_cb) {
-#pragma unroll
-        for (int i = 0; i < NT; ++i)
-          if (on[i]) an[i] = wfrag[(size_t)(tm[i] * a.n_cb + cb + 1) * 64];
-      }
+    constexpr int U = NT == 1 ? 8 : NT == 2 ? 4 : 2;      // K slices whose A fragments are requested together
+    for (int kb = k0; kb < k1; kb += U) {
+      v4i af[NT][U];
 #pragma unroll
       for (int i = 0; i < NT; ++i)
-        if (on[i])
-          acc2[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ac[i], bfr[(pp[i] * a.n_cb + cb) * 64 + lane], acc2[i][0], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          af[i][u] = v4i{0, 0, 0, 0};
+          if (on[i] && kb + u < k1) af[i][u] = wfrag[(size_t)(tm[i] * a.n_cb + kb + u) * 64];
+        }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+          if (on[i] && kb + u < k1)
+            acc2[i][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i][u], bfr[(pp[i] * a.n_cb + kb + u) * 64 + lane],
+                                                                acc2[i][0], 0, 0, 0);
+    }
+    if (a.nk > 1) {
+      // the parts of a result block are summed in LDS (integer adds: any order gives the same sum)
+      if (on[0]) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) atomicAdd(&red[(tl[0] * 16 + e) * 64 + lane], acc2[0][0][e]);
+      }
+      __syncthreads();
+      if (on[0] && kp == 0) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc2[0][0][e] = red[(tl[0] * 16 + e) * 64 + lane];
+      }
+#pragma unroll
+      for (int i = 0; i < NT; ++i) on[i] = on[i] & (kp == 0);
     }
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
@@ -303,7 +334,7 @@ namespace {
 
 struct DwPwPlan {
   int rows, width, valid, halo, xblocks, rblocks, nblocks;
-  int n_cb, n_tm, log2p, nt;
+  int n_cb, n_tm, log2p, nt, nk;
 };
 
 // the row segments of the depthwise phase (fewest blocks per image) and the pixel blocks per workgroup
@@ -342,6 +373,8 @@ bool dwpw_plan(const tpuhip_conv_desc &a, const tpuhip_conv_desc &b, DwPwPlan *o
   while (log2p > 0 && ((out->n_cb << log2p) > 60 || (out->nblocks >> log2p) < 512)) --log2p;
   out->log2p = log2p;
   out->nt = ((out->n_tm << log2p) + 3) / 4;
+  const int tiles = out->n_tm << log2p;
+  out->nk = tiles < 4 ? std::min(4 / tiles, out->n_cb) : 1;
   return out->nt <= 3;
 }
 
@@ -365,7 +398,8 @@ const char *const kDwPwNames[] = {"mfma_dwpw_shift_nt1", "mfma_dwpw_shift_nt2", 
                                   "mfma_dwpw_taps_nt1",  "mfma_dwpw_taps_nt2",  "mfma_dwpw_taps_nt3"};
 
 unsigned dwpw_lds_bytes(const DwPwPlan &p) {
-  return (unsigned)(((size_t)p.n_cb << p.log2p) * 1024 + (size_t)5 * p.n_tm * 32 * 4 + 4 * 160 * 4 + 256);
+  return (unsigned)(((size_t)p.n_cb << p.log2p) * 1024 + (size_t)5 * p.n_tm * 32 * 4 + 4 * 160 * 4 + 256 +
+                    (p.nk > 1 ? ((size_t)p.n_tm << p.log2p) * 4096 : 0));
 }
 
 }  // namespace
@@ -463,7 +497,7 @@ int dwpw_run(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *
   a.rows = p.rows; a.width = p.width; a.valid = p.valid; a.halo = p.halo;
   a.xblocks = p.xblocks; a.rblocks = p.rblocks; a.nblocks = p.nblocks;
   a.magic_w = p.width > 1 ? (uint32_t)(((1ull << 32) + p.width - 1) / (uint64_t)p.width) : 0u;
-  a.log2p = p.log2p; a.n_cb = p.n_cb; a.n_tm = p.n_tm;
+  a.log2p = p.log2p; a.n_cb = p.n_cb; a.n_tm = p.n_tm; a.nk = p.nk;
   a.ngroups = (p.nblocks + (1 << p.log2p) - 1) >> p.log2p;
   const unsigned lds = dwpw_lds_bytes(p);
   const dim3 grid(8u * (unsigned)((a.ngroups + 7) / 8)), block(256);
