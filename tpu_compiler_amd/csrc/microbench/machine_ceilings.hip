@@ -232,43 +232,110 @@ __global__ __launch_bounds__(256) void k_gload_lds(const v4i *__restrict__ src, 
   if (s[0] + s[1] + s[2] + s[3] == 0x12345678) out[0] = 1;
 }
 
-// ---- VALU op rates: 8 independent chains per lane
+// ---- VALU op rates: 8 independent chains per lane, the 8 instructions of a trip written as one
+// block (the compiler puts a wait state between separate asm statements).  x: %0..%7, q (64-bit): %8..%15, m: %16
+#define V8(F) F(0, 8) F(1, 9) F(2, 10) F(3, 11) F(4, 12) F(5, 13) F(6, 14) F(7, 15)
 template <int OP>
 __global__ __launch_bounds__(256) void k_valu(int *out, int iters, int seed) {
   int x[8];
   long long q[8];
-  double d[8];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) { x[u] = threadIdx.x * 7 + u + seed; q[u] = x[u]; d[u] = x[u]; }
+  for (int u = 0; u < 8; ++u) { x[u] = threadIdx.x * 7 + u + seed; q[u] = x[u]; }
   const int m = seed | 0x40000001;
+#define OPERANDS                                                                                              \
+  : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3]), "+v"(x[4]), "+v"(x[5]), "+v"(x[6]), "+v"(x[7]), "+v"(q[0]), \
+    "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(q[4]), "+v"(q[5]), "+v"(q[6]), "+v"(q[7])                          \
+  : "v"(m)                                                                                                    \
+  : "vcc"
   for (int i = 0; i < iters; ++i) {
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      if (OP == 0) asm volatile("v_mad_i64_i32 %0, vcc, %1, %2, %0" : "+v"(q[u]) : "v"(x[u]), "v"(m) : "vcc");
-      if (OP == 1) asm volatile("v_mul_hi_i32 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 2) asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 3) asm volatile("v_add3_u32 %0, %0, %1, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 4) asm volatile("v_cvt_f64_i32 %0, %1" : "=v"(d[u]) : "v"(x[u]));
-      if (OP == 5) asm volatile("v_fma_f64 %0, %0, %0, %0" : "+v"(d[u]));
-      if (OP == 6) asm volatile("v_floor_f64 %0, %0" : "+v"(d[u]));
-      if (OP == 7) asm volatile("v_cvt_i32_f64 %0, %1" : "=v"(x[u]) : "v"(d[u]));
-      if (OP == 8) asm volatile("v_dot4_i32_i8 %0, %0, %1, %0" : "+v"(x[u]) : "v"(m));
-      if (OP == 9) asm volatile("v_perm_b32 %0, %0, %1, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 10) asm volatile("v_pk_mad_i16 %0, %0, %1, %0" : "+v"(x[u]) : "v"(m));
-      if (OP == 11) asm volatile("v_mul_i32_i24 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 12) asm volatile("v_mul_hi_i32_i24 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 13) asm volatile("v_alignbit_b32 %0, %0, %1, 31" : "+v"(x[u]) : "v"(m));
-      if (OP == 14) asm volatile("v_cvt_pk_i16_i32 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 15) asm volatile("v_pk_max_i16 %0, %0, %1" : "+v"(x[u]) : "v"(m));
-      if (OP == 16) asm volatile("v_mul_f64 %0, %0, %0" : "+v"(d[u]));
-      if (OP == 17) asm volatile("v_ashrrev_i32 %0, %1, %0" : "+v"(x[u]) : "v"(m));
-    }
+#define A(N, Q) "v_add_u32 %" #N ", %" #N ", %16\n"
+    if (OP == 0) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_and_b32 %" #N ", %" #N ", %16\n"
+    if (OP == 1) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_lshrrev_b32 %" #N ", 3, %" #N "\n"
+    if (OP == 2) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_ashrrev_i32 %" #N ", %16, %" #N "\n"
+    if (OP == 3) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_mov_b32 %" #N ", %16\n"
+    if (OP == 4) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_fma_f32 %" #N ", %" #N ", %16, %" #N "\n"
+    if (OP == 5) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_lshlrev_b32 %" #N ", 3, %" #N "\n"
+    if (OP == 6) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_max_i32 %" #N ", %" #N ", %16\n"
+    if (OP == 7) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_med3_i32 %" #N ", %" #N ", %16, 64\n"
+    if (OP == 8) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_add3_u32 %" #N ", %" #N ", %16, %16\n"
+    if (OP == 9) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_perm_b32 %" #N ", %" #N ", %16, %16\n"
+    if (OP == 10) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_alignbit_b32 %" #N ", %" #N ", %16, 31\n"
+    if (OP == 11) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_cvt_pk_i16_i32 %" #N ", %" #N ", %16\n"
+    if (OP == 12) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_pk_max_i16 %" #N ", %" #N ", %16\n"
+    if (OP == 13) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_pk_mad_i16 %" #N ", %" #N ", %16, %" #N "\n"
+    if (OP == 14) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_pk_ashrrev_i16 %" #N ", %16, %" #N "\n"
+    if (OP == 15) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_mul_i32_i24 %" #N ", %" #N ", %16\n"
+    if (OP == 16) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_mul_lo_u32 %" #N ", %" #N ", %16\n"
+    if (OP == 17) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_mul_hi_i32 %" #N ", %" #N ", %16\n"
+    if (OP == 18) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_dot4_i32_i8 %" #N ", %" #N ", %16, %" #N "\n"
+    if (OP == 19) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_mad_i64_i32 %" #Q ", vcc, %" #N ", %16, %" #Q "\n"
+    if (OP == 20) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_lshl_or_b32 %" #N ", %" #N ", 8, %16\n"
+    if (OP == 21) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_sat_pk_u8_i16 %" #N ", %" #N "\n"
+    if (OP == 22) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_fma_f64 %" #Q ", %" #Q ", %" #Q ", %" #Q "\n"
+    if (OP == 23) asm volatile(V8(A) OPERANDS);
+#undef A
+#define A(N, Q) "v_cvt_i32_f64 %" #N ", %" #Q "\n"
+    if (OP == 24) asm volatile(V8(A) OPERANDS);
+#undef A
   }
+#undef OPERANDS
   long long s = 0;
 #pragma unroll
-  for (int u = 0; u < 8; ++u) s += x[u] + q[u] + (long long)d[u];
+  for (int u = 0; u < 8; ++u) s += x[u] + q[u];
   out[blockIdx.x * 256 + threadIdx.x] = (int)s;
 }
+constexpr int kValuOps = 25;
+const char *const kValuNames[kValuOps] = {
+    "v_add_u32", "v_and_b32", "v_lshrrev_b32", "v_ashrrev_i32", "v_mov_b32", "v_fma_f32", "v_lshlrev_b32", "v_max_i32",
+    "v_med3_i32", "v_add3_u32", "v_perm_b32", "v_alignbit_b32", "v_cvt_pk_i16_i32", "v_pk_max_i16", "v_pk_mad_i16",
+    "v_pk_ashrrev_i16", "v_mul_i32_i24", "v_mul_lo_u32", "v_mul_hi_i32", "v_dot4_i32_i8", "v_mad_i64_i32",
+    "v_lshl_or_b32", "v_sat_pk_u8_i16", "v_fma_f64", "v_cvt_i32_f64"};
 
 int main(int argc, char **argv) {
   CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
@@ -356,19 +423,22 @@ int main(int argc, char **argv) {
     }
   }
 
-  printf("== VALU: clocks per wave64 instruction per SIMD (2 waves per SIMD, 8 chains)\n");
+  printf("== VALU: clocks per wave64 instruction per SIMD at 1, 2, 4 and 8 waves per SIMD (8 independent chains per wave)\n");
   {
-    const char *names[] = {"v_mad_i64_i32", "v_mul_hi_i32", "v_mul_lo_u32", "v_add3_u32", "v_cvt_f64_i32", "v_fma_f64",
-                           "v_floor_f64", "v_cvt_i32_f64", "v_dot4_i32_i8", "v_perm_b32", "v_pk_mad_i16", "v_mul_i32_i24",
-                           "v_mul_hi_i32_i24", "v_alignbit_b32", "v_cvt_pk_i16_i32", "v_pk_max_i16", "v_mul_f64", "v_ashrrev_i32"};
-    const int iters = 4000, wgs = ncu * 2;
-    float t[18];
-#define V(OP) t[OP] = time_us([&] { hipLaunchKernelGGL(k_valu<OP>, dim3(wgs), dim3(256), 0, 0, out, iters, 3); }, 3, 1);
-    V(0) V(1) V(2) V(3) V(4) V(5) V(6) V(7) V(8) V(9) V(10) V(11) V(12) V(13) V(14) V(15) V(16) V(17)
+    const int iters = 4000;
+    const int wps[4] = {1, 2, 4, 8};
+    static float t[4][kValuOps];
+    for (int wi = 0; wi < 4; ++wi) {
+      const int wgs = ncu * wps[wi];   // 4 waves per workgroup: one per SIMD
+#define V(OP) t[wi][OP] = time_us([&] { hipLaunchKernelGGL(k_valu<OP>, dim3(wgs), dim3(256), 0, 0, out, iters, 3); }, 3, 1);
+      V(0) V(1) V(2) V(3) V(4) V(5) V(6) V(7) V(8) V(9) V(10) V(11) V(12) V(13) V(14) V(15) V(16) V(17) V(18) V(19) V(20)
+      V(21) V(22) V(23) V(24)
 #undef V
-    for (int op = 0; op < 18; ++op) {
-      const double instr_per_simd = (double)wgs * 4 / (ncu * 4) * iters * 8;
-      printf("%-18s %.2f clk\n", names[op], t[op] * 1e-6 * clk / instr_per_simd);
+    }
+    for (int op = 0; op < kValuOps; ++op) {
+      printf("%-18s", kValuNames[op]);
+      for (int wi = 0; wi < 4; ++wi) printf(" %6.2f", t[wi][op] * 1e-6 * clk / ((double)wps[wi] * iters * 8));
+      printf(" clk\n");
     }
   }
   CK(hipDeviceSynchronize());
