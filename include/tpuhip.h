@@ -10,7 +10,9 @@
  * Device tensors are int8, channels-last: element (n, h, w, c) of a tensor
  * with channel stride cs lives at byte ((n*H + h)*W + w)*cs + c.  cs is a
  * multiple of 16 and the bytes c..cs-1 of every pixel are zero; every kernel
- * keeps that invariant.
+ * keeps that invariant.  One exception: a tensor of at most 4 channels that only
+ * stem convs read may lie at cs = 4 (tpuhip_conv2d_set_input_stride; the layout
+ * conversions below take cs = 4 as well).
  * The reference's NCHW float tensors (include/tpuc/Interpreter/cpukernel.h:15-78)
  * are converted at the edge by the tpuhip_*_nchw_* entry points.
  *
@@ -231,6 +233,13 @@ int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain,
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *chain);
 /* name of chain kernel variant `variant`, NULL past the last one */
 const char *tpuhip_conv2d_chain_variant_name(int variant);
+/* The channel stride of the input a packed conv will be run on, changed after packing.  4 (one dword per
+ * pixel) is taken only by a conv on the stem path -- g == 1, at most 4 input channels, at most 64 output
+ * channels, kh <= 7, kw <= 8, stride_w <= 2, which reads a pixel as one dword anyway (TPUHIP_ERR_UNSUPPORTED
+ * otherwise): a 3-channel image then occupies a quarter of the bytes of the 16-byte stride and the stem
+ * fetches a quarter.  The interpreter lays a graph input out that way when stem convs are its only readers.
+ * No counterpart in the reference (its tensors are dense float NCHW, cpukernel.h:15-24). */
+int tpuhip_conv2d_set_input_stride(tpuhip_conv_weights *w, int x_cs);
 /* name of the kernel variant a prepacked conv dispatches to (for profiling) */
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w);
 /* name of MFMA tile variant `tile` (selected with algo = 16 + tile), NULL past the last one */

@@ -79,6 +79,9 @@ public:
   std::shared_ptr<std::vector<float>> tensor(int32_t bidx) const;
   // slot bidx as int8 NCHW host data (no float detour)
   void read_i8(int8_t *dst, size_t num, int32_t bidx) const;
+  // lays the tensor out again with another channel stride (4 for a tensor of at most 4 channels whose
+  // only readers take one dword per pixel, else a multiple of 16); the contents are lost
+  void set_channel_stride(int new_cs);
 
   int32_t batch;
   int n = 1, c = 1, h = 1, w = 1;  // 4-d view of the shape (missing dims are 1)
@@ -229,6 +232,11 @@ public:
   bool is_chain_second() const { return chained_into != nullptr; }
   // dissolves the chain this kernel belongs to (as first or second)
   void unchain();
+  // true: this conv runs on the stem path, which reads a pixel of its (at most 4-channel) input as one
+  // dword, so the input may lie at a channel stride of 4 instead of 16
+  bool reads_dword_pixels() const;
+  // tells the packed conv its input's channel stride; false where it cannot take it
+  bool set_input_stride(int cs);
 
 protected:
   // transposed: the attributes describe a DeConv2D; it runs as a stride-1 conv over the
@@ -635,6 +643,9 @@ public:
   bool pair_convs = true;
   // a pointwise conv (+ folded add) followed by the pointwise conv that reads its result: one launch
   bool chain_convs = true;
+  // a graph input of at most 4 channels that only stem convs read lies one dword per pixel (a quarter
+  // of the bytes of the 16-byte channel stride; on by default; TPUHIP_PACK_INPUT=0 disables)
+  bool pack_inputs = true;
   // true (default): every tensor of the graph can be read back after an invoke, like the
   // reference.  false: the result of a conv whose only reader is the add fused into it is
   // never written (reading it back is an error); applies at the next loadModule
@@ -652,6 +663,7 @@ private:
   void fuseKernels();
   void chainConvs();
   void pairConvs();
+  void packInputs();
   void spreadDirtiness();
   // kernels that run as one launch (a conv with the table op / add folded into it, the two
   // convs of a pair): rebuilt by every loadModule

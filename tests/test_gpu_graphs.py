@@ -320,6 +320,31 @@ def test_chained_pointwise_convs_run_as_one_launch_with_unchanged_results():
     m.close()
 
 
+@pytest.mark.parametrize("builder,kw,first", [(graphs.cfg3_resnet50, dict(batch=2, hw=96), "conv1"),
+                                              (graphs.cfg4_mobilenet_v2, dict(batch=2, hw=64), "conv1"),
+                                              (graphs.cfg5_yolo_v3, dict(batch=1, hw=96), "conv1")])
+def test_three_channel_graph_input_packed_to_one_dword_per_pixel(builder, kw, first):
+    """the image input of the networks, read only by the stem conv, lies at a channel stride of 4 by default
+    and 16 with the option off: every tensor equals the oracle's either way, the input reads back as it
+    was set, and a reload that changes nothing keeps the layout"""
+    g = builder(**kw)
+    want = oracle_graph.run(g)
+    x = g.input_op().data.astype(np.float32)
+    for on in (1, 0):
+        m = module()
+        m.set_option("pack_inputs", on)
+        m.load(g)
+        assert dict(m.kernels())[first] == "stem"
+        for _ in range(2):
+            m.set_tensor("input", x)
+            m.invoke()
+            assert np.array_equal(m.get_tensor_i8("input"), g.input_op().data.reshape(g.input_op().shape))
+            for op in g.ops:
+                assert np.array_equal(m.get_tensor_i8(op.name), want[op.name].reshape(op.shape)), (on, op.name)
+            m.load(g)
+        m.close()
+
+
 @pytest.mark.parametrize("builder,kw", [(graphs.cfg5_yolo_v3, dict(batch=1, hw=96)),
                                         (graphs.cfg4_mobilenet_v2, dict(batch=2, hw=64)),
                                         (graphs.cfg2_mobilenet_block, dict(batch=1))])

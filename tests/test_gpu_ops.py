@@ -126,6 +126,51 @@ def test_conv_stem(ctx, case, algo):
     assert len(np.unique(want)) > 8
 
 
+@pytest.mark.parametrize("case", STEM_CASES)
+def test_conv_stem_on_an_input_of_one_dword_per_pixel(ctx, case):
+    """the same layers with the input at a channel stride of 4 instead of 16 -- at prepack and switched
+    over afterwards; bytes 3 of a 3-channel pixel are zero as the layout conversion writes them"""
+    n, ic, ih, iw, oc, kh, kw, stride, pads, relu = case
+    rng = np.random.default_rng(ic * 131 + oc + kh * 7 + kw + 1)
+    x = rnd_i8(rng, (n, ic, ih, iw))
+    w = rnd_w(rng, (oc, ic, kh, kw))
+    bias, rsh, mult = rnd_params(rng, oc)
+    want = oracle_conv(x, w, bias, rsh, mult, 1, stride, pads, (1, 1), (0, 0), relu)
+    xt = ctx.from_nchw(x, cs=4)
+    assert xt.cs == 4 and xt.nbytes == n * ih * iw * 4
+    assert not ctx.raw(xt)[..., ic:].any()
+    for at_prepack in (True, False):
+        d = conv_desc(x.shape, w.shape, stride=stride, pads=pads, do_relu=relu, x_cs=4 if at_prepack else None)
+        wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+        assert ctx.conv_algo_name(wh) == "stem"
+        if not at_prepack:
+            ctx.conv_set_input_stride(wh, 4)
+        yt = ctx.tensor(want.shape)
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, yt.ptr, 0x55, yt.nbytes))
+        ctx.conv(wh, xt, yt)
+        got = ctx.to_nchw(yt)
+        assert np.array_equal(got, want), "%d mismatches" % (got != want).sum()
+        ctx.conv_weights_destroy(wh)
+        yt.free()
+    assert np.array_equal(ctx.to_nchw(xt), x)       # and back through the layout conversion
+    xt.free()
+
+
+def test_conv_off_the_stem_path_refuses_a_dword_input(ctx):
+    rng = np.random.default_rng(77)
+    w = rnd_w(rng, (128, 3, 3, 3))                   # 128 output channels: the general MFMA path
+    bias, rsh, mult = rnd_params(rng, 128)
+    with pytest.raises(capi.TpuHipError, match="4-byte channel stride"):
+        ctx.conv_prepack(conv_desc((1, 3, 16, 16), w.shape, pads=(1, 1, 1, 1), x_cs=4), w, f2i32(bias), f2i32(mult),
+                         f2i32(rsh))
+    wh = ctx.conv_prepack(conv_desc((1, 3, 16, 16), w.shape, pads=(1, 1, 1, 1)), w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    with pytest.raises(capi.TpuHipError, match="only the stem path"):
+        ctx.conv_set_input_stride(wh, 4)
+    ctx.conv_weights_destroy(wh)
+    with pytest.raises(capi.TpuHipError, match="channel stride"):
+        ctx.tensor((1, 8, 4, 4), cs=4)               # 8 channels do not fit a dword
+
+
 # n, ic, ih, iw, oc, kh, kw, conv stride, conv pads, pool pads (t, b, l, r), pool out_hw or None
 STEM_POOL_CASES = [
     (2, 3, 224, 224, 64, 7, 7, (2, 2), (3, 3, 3, 3), (0, 1, 0, 1), None),     # ResNet-50 conv1 + pool1 (Caffe ceil mode)

@@ -185,6 +185,7 @@ PROTOTYPES.update({
                                               C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "tpuhip_conv2d_chain_destroy": (C.c_int, [C.c_void_p, C.c_void_p]),
     "tpuhip_conv2d_chain_i8": (C.c_int, [C.c_void_p] * 6 + [C.POINTER(FusedAdd), C.c_void_p]),
+    "tpuhip_conv2d_set_input_stride": (C.c_int, [C.c_void_p, C.c_int]),
     "tpuhip_conv2d_chain_kind": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]),
     "tpuhip_conv2d_chain_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost), C.c_void_p, C.POINTER(ConvPost)]),
     "tpuhip_conv2d_chain_name": (C.c_char_p, [C.c_void_p]),
@@ -317,6 +318,9 @@ class DeviceTensor:
         self.shape = tuple(int(v) for v in shape)
         n, c, h, w = self.shape
         self.cs = cs or channel_stride(c)
+        if self.cs < c or (self.cs % 16 and self.cs != 4):
+            raise TpuHipError(2, "a channel stride is 4 or a multiple of 16 and covers the channels (%d for %d)"
+                              % (self.cs, c))
         self.nbytes = n * h * w * self.cs
         self._owner = owner and ptr is None
         self.ptr = ptr if ptr is not None else ctx.malloc(self.nbytes)
@@ -585,6 +589,9 @@ class Context:
             p.add_src, p.add_out = src.ptr, out.ptr
         self._ck(self.lib.tpuhip_conv2d_post_i8(self.h, w, x.ptr, None if y is None else y.ptr,
                                                 C.byref(p)))
+
+    def conv_set_input_stride(self, w, x_cs):
+        self._ck(self.lib.tpuhip_conv2d_set_input_stride(w, int(x_cs)))
 
     def conv_algo_name(self, w):
         return self.lib.tpuhip_conv2d_algo_name(w).decode()

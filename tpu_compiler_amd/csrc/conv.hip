@@ -3215,7 +3215,8 @@ int check_desc(const tpuhip_conv_desc &d) {
                  "conv: bad kernel/stride/dilation");
   TPUHIP_REQUIRE(d.pt >= 0 && d.pb >= 0 && d.pl >= 0 && d.pr >= 0 && d.ins_h >= 0 && d.ins_w >= 0,
                  "conv: negative padding");
-  TPUHIP_REQUIRE(d.x_cs >= d.ic && d.y_cs >= d.oc && d.x_cs % 16 == 0 && d.y_cs % 16 == 0,
+  // an input of at most 4 channels may lie one dword per pixel (the stem path reads it that way)
+  TPUHIP_REQUIRE(d.x_cs >= d.ic && d.y_cs >= d.oc && (d.x_cs % 16 == 0 || d.x_cs == 4) && d.y_cs % 16 == 0,
                  "conv: channel strides must be multiples of 16 covering the channels "
                  "(x_cs %d ic %d, y_cs %d oc %d)", d.x_cs, d.ic, d.y_cs, d.oc);
   const int ihd = (d.ih - 1) * (d.ins_h + 1) + 1, iwd = (d.iw - 1) * (d.ins_w + 1) + 1;
@@ -3619,6 +3620,9 @@ int tpuhip_conv2d_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *desc, const i
   TPUHIP_REQUIRE(algo != ALGO_STEM || stem_ok,
                  "conv: the stem path needs g == 1, ic <= 4, oc <= 64, kh <= 7, kw <= 8, stride_w <= 2, "
                  "no dilation, no inserted zeros");
+  TPUHIP_REQUIRE(d.x_cs % 16 == 0 || algo == ALGO_STEM,
+                 "conv: only the stem path (g == 1, ic <= 4, oc <= 64, kh <= 7, kw <= 8, stride_w <= 2) reads an input "
+                 "with a 4-byte channel stride");
   // the MFMA kernel locates a K group with multiply-shift divisions that are exact
   // for at most 4094 groups of at most 256 16-channel groups each
   const bool mfma_ok = dense && round_up(d.ic, 16) / 16 <= 256 &&
@@ -3796,6 +3800,17 @@ int tpuhip_conv2d_can_fuse_table(const tpuhip_conv_weights *w) {
   if (!w) return 0;
   if (w->algo == ALGO_DEPTHWISE || w->algo == ALGO_DEPTHWISE_DOT || w->algo == ALGO_STEM) return 1;
   return w->algo == ALGO_MFMA && (!w->tuned || tile_has_lds_epilogue(w->tile)) ? 1 : 0;
+}
+
+int tpuhip_conv2d_set_input_stride(tpuhip_conv_weights *w, int x_cs) {
+  TPUHIP_REQUIRE(w, "tpuhip_conv2d_set_input_stride: NULL argument");
+  TPUHIP_REQUIRE(x_cs >= w->d.ic && (x_cs % 16 == 0 || x_cs == 4), "conv: input channel stride %d must be 4 or a multiple of 16 covering %d channels", x_cs, w->d.ic);
+  if (x_cs == 4 && (w->algo != ALGO_STEM || w->split_oc))
+    return set_error(TPUHIP_ERR_UNSUPPORTED, "conv: only the stem path reads an input with a 4-byte channel stride");
+  TPUHIP_REQUIRE((int64_t)w->d.n * (w->d.ih + w->d.pt + w->d.pb + 2) * (w->d.iw + w->d.pl + w->d.pr + 2) * x_cs < (1ll << 31),
+                 "conv: tensor too large");
+  w->d.x_cs = x_cs;
+  return TPUHIP_OK;
 }
 
 const char *tpuhip_conv2d_algo_name(const tpuhip_conv_weights *w) {

@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kThreads) void nhwc_to_nchw_kernel(const int8_t *sr
 int check_layout_args(const void *a, const void *b, int n, int c, int h, int w, int cs) {
   TPUHIP_REQUIRE(a && b, "layout: NULL pointer");
   TPUHIP_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0, "layout: non-positive dimension");
-  TPUHIP_REQUIRE(cs >= c && cs % 16 == 0, "layout: channel stride %d must be a multiple of 16 >= %d",
+  TPUHIP_REQUIRE(cs >= c && (cs % 16 == 0 || cs == 4), "layout: channel stride %d must be 4 or a multiple of 16, >= %d",
                  cs, c);
   TPUHIP_REQUIRE(n <= 65535 && (c + 63) / 64 <= 65535, "layout: too many images / channels");
   return TPUHIP_OK;

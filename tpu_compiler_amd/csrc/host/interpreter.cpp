@@ -53,6 +53,7 @@ void ModuleInterpreter::loadModule(ModuleDesc &module, std::string target_op) {
   fuseKernels();
   chainConvs();
   pairConvs();
+  packInputs();
   spreadDirtiness();
 }
 
@@ -235,6 +236,41 @@ void ModuleInterpreter::pairConvs() {
   for (auto *c : convs)
     if (!c->is_paired_first() && !c->is_paired_second() && !c->is_chain_first() && !c->is_chain_second())
       c->release_host_weights();
+}
+
+// A graph input of at most 4 channels whose only readers are convs on the stem path -- they take a
+// pixel as one dword -- is laid out at a channel stride of 4 instead of 16: a quarter of the bytes
+// to write at set_tensor and to fetch in the stem.  Decided anew at every load (a reload can change
+// the readers), after pairing, which can take a stem conv off the stem path.
+void ModuleInterpreter::packInputs() {
+  const char *env = getenv("TPUHIP_PACK_INPUT");
+  const bool on = pack_inputs && !(env && atoi(env) == 0);
+  for (auto &k : kernel_list_) {
+    if (!dynamic_cast<InputOpKernel *>(k.get())) continue;
+    auto it = activationMapping.find(k->name);
+    if (it == activationMapping.end()) continue;
+    TensorData *t = it->second.get();
+    if (t->f32 || t->is_unsigned || t->c > 4) continue;
+    std::vector<Conv2DOpKernel *> convs;   // convs whose activation input is t
+    bool all = on;
+    for (auto &r : kernel_list_) {
+      if (r.get() == k.get()) continue;
+      bool reads = false;
+      for (auto &opd : r->operands())
+        if (opd.act && opd.act.get() == t) reads = true;
+      if (!reads) continue;
+      auto *c = dynamic_cast<Conv2DOpKernel *>(r.get());
+      if (c && c->input().get() == t) convs.push_back(c);
+      if (!c || c->input().get() != t || !c->reads_dword_pixels()) all = false;
+    }
+    int want = (all && !convs.empty()) ? 4 : tpuhip_channel_stride(t->c);
+    if (want == 4)
+      for (auto *c : convs)
+        if (!c->set_input_stride(4)) want = tpuhip_channel_stride(t->c);
+    if (want != 4)
+      for (auto *c : convs) c->set_input_stride(want);
+    t->set_channel_stride(want);
+  }
 }
 
 // MlirModuleInterpreter.cpp:85-116

@@ -106,6 +106,17 @@ TensorData::~TensorData() {
   if (base_) tpuhip_free(ctx_, base_);
 }
 
+void TensorData::set_channel_stride(int new_cs) {
+  if (f32 || new_cs == cs) return;
+  if (new_cs < c || (new_cs % 16 != 0 && new_cs != 4)) fail("TensorData::set_channel_stride: bad stride");
+  if (base_) ck(tpuhip_free(ctx_, base_), "TensorData::set_channel_stride");
+  base_ = nullptr;
+  cs = new_cs;
+  ck(tpuhip_malloc(ctx_, slot_bytes() * (size_t)batch, &base_), "TensorData::set_channel_stride");
+  ck(tpuhip_memset(ctx_, base_, 0, slot_bytes() * (size_t)batch), "TensorData::set_channel_stride");
+  ptr_ = (char *)base_ + slot_bytes() * (size_t)cur_;
+}
+
 void TensorData::set_batch_idx(int32_t bidx) {
   if (bidx < 0 || bidx >= batch) fail("TensorData::set_batch_idx: slot out of range");
   ptr_ = (char *)base_ + slot_bytes() * (size_t)bidx;
@@ -476,6 +487,17 @@ bool Conv2DOpKernel::chain_with(Conv2DOpKernel &next) {
   ck(rc, ("Conv2D '" + name + "' -> '" + next.name + "'").c_str());
   chain_second = &next;
   next.chained_into = this;
+  return true;
+}
+
+bool Conv2DOpKernel::reads_dword_pixels() const {
+  return packed && !pair_packed && !paired_into && !chain_packed && !chained_into &&
+         std::string(tpuhip_conv2d_algo_name(packed)) == "stem";
+}
+
+bool Conv2DOpKernel::set_input_stride(int cs) {
+  if (!packed || tpuhip_conv2d_set_input_stride(packed, cs) != TPUHIP_OK) return false;
+  desc.x_cs = cs;
   return true;
 }
 

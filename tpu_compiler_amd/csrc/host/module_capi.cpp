@@ -100,6 +100,8 @@ int tpuhip_module_set_option(tpuhip_module *m, const char *key, int value) {
       m->interp->pair_convs = value != 0;
     else if (k == "chain_convs")
       m->interp->chain_convs = value != 0;
+    else if (k == "pack_inputs")
+      m->interp->pack_inputs = value != 0;
     else
       throw std::runtime_error("tpuhip_module_set_option: unknown option '" + k + "'");
   })
