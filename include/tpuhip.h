@@ -230,6 +230,28 @@ int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, cons
  * the fused work its kind does not take. */
 int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y_a,
                                 const tpuhip_conv_post *post_a, void *y_b, const tpuhip_conv_post *post_b);
+/* A chain of three: the 1x1 expansion (at most 160 input channels), the depthwise conv (at most 3 x 3 taps,
+ * any stride, padding and dilation) and the 1x1 projection (at most 384 output channels) of an
+ * inverted-residual block, with the block's EltwiseAdd behind the projection (post->add; no table, no
+ * pool) -- Conv2DOpKernel::invoke three times (core/conv.cpp:11-104) and EltwiseAddOpKernel::i8_invoke
+ * (core/eltwise.cpp:52-85) as one launch.  Neither expanded tensor is written: the call is for graphs in
+ * which nothing else reads them.  tpuhip_conv2d_can_chain3 answers for the shapes; prepack returns
+ * TPUHIP_ERR_UNSUPPORTED for shapes not covered, a right shift of 0 or sums that could overflow the
+ * rounding.  y may be NULL when only the sum is wanted.  The handle is destroyed with
+ * tpuhip_conv2d_chain_destroy.  No counterpart in the reference (one kernel per op). */
+typedef struct {
+  const int8_t *filter;       /* OIHW */
+  const int32_t *bias;        /* may be NULL */
+  const int32_t *multiplier, *rshift;
+} tpuhip_chain_conv;
+int tpuhip_conv2d_can_chain3(const tpuhip_conv_desc *expand, const tpuhip_conv_desc *depthwise,
+                             const tpuhip_conv_desc *project);
+int tpuhip_conv2d_chain3_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *expand, const tpuhip_conv_desc *depthwise,
+                                 const tpuhip_conv_desc *project, const tpuhip_chain_conv *expand_w,
+                                 const tpuhip_chain_conv *depthwise_w, const tpuhip_chain_conv *project_w,
+                                 tpuhip_conv_chain **out);
+int tpuhip_conv2d_chain3_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *chain, const void *x, void *y,
+                            const tpuhip_conv_post *post);
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *chain);
 /* name of chain kernel variant `variant`, NULL past the last one */
 const char *tpuhip_conv2d_chain_variant_name(int variant);

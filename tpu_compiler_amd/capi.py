@@ -26,6 +26,10 @@ class ConvPost(C.Structure):
                 ("pool", C.c_void_p), ("pool_out", C.c_void_p)]
 
 
+class ChainConv(C.Structure):
+    _fields_ = [("filter", C.c_void_p), ("bias", C.c_void_p), ("multiplier", C.c_void_p), ("rshift", C.c_void_p)]
+
+
 class BinaryDesc(C.Structure):
     _fields_ = [(k, C.c_int) for k in (
         "op", "n", "c", "h", "w", "n0", "c0", "h0", "w0", "n1", "c1", "h1", "w1", "m0", "m1")] + \
@@ -188,6 +192,9 @@ PROTOTYPES.update({
     "tpuhip_conv2d_set_input_stride": (C.c_int, [C.c_void_p, C.c_int]),
     "tpuhip_conv2d_chain_kind": (C.c_int, [C.POINTER(ConvDesc), C.POINTER(ConvDesc)]),
     "tpuhip_conv2d_chain_post_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost), C.c_void_p, C.POINTER(ConvPost)]),
+    "tpuhip_conv2d_can_chain3": (C.c_int, [C.POINTER(ConvDesc)] * 3),
+    "tpuhip_conv2d_chain3_prepack": (C.c_int, [C.c_void_p] + [C.POINTER(ConvDesc)] * 3 + [C.POINTER(ChainConv)] * 3 + [c_void_pp]),
+    "tpuhip_conv2d_chain3_i8": (C.c_int, [C.c_void_p] * 4 + [C.POINTER(ConvPost)]),
     "tpuhip_conv2d_chain_name": (C.c_char_p, [C.c_void_p]),
     "tpuhip_conv2d_chain_variant_name": (C.c_char_p, [C.c_int]),
     "tpuhip_module_load_mlir": (C.c_int, [C.c_void_p, C.c_char_p, C.c_char_p]),
@@ -518,6 +525,34 @@ class Context:
         self._ck(self.lib.tpuhip_conv2d_chain_post_i8(
             self.h, ch, x.ptr, None if y_a is None else y_a.ptr, C.byref(pa),
             None if y_b is None else y_b.ptr, C.byref(pb)))
+
+    def conv_can_chain3(self, desc_e, desc_d, desc_p):
+        return bool(self.lib.tpuhip_conv2d_can_chain3(C.byref(desc_e), C.byref(desc_d), C.byref(desc_p)))
+
+    def conv_chain3_prepack(self, desc_e, desc_d, desc_p, e, d, p):
+        """e, d, p: (filter int8, bias int32 or None, multiplier int32, rshift int32) of the 1x1 expansion, the
+        depthwise conv and the 1x1 projection of an inverted-residual block -> one handle for conv_chain3"""
+        keep, packs = [], []
+        for filt, bias, mult, rshift in (e, d, p):
+            arrs = [np.ascontiguousarray(filt, dtype=np.int8),
+                    None if bias is None else np.ascontiguousarray(bias, dtype=np.int32),
+                    np.ascontiguousarray(mult, dtype=np.int32), np.ascontiguousarray(rshift, dtype=np.int32)]
+            keep += arrs
+            packs.append(ChainConv(*[None if x is None else x.ctypes.data for x in arrs]))
+        w = C.c_void_p()
+        self._ck(self.lib.tpuhip_conv2d_chain3_prepack(self.h, C.byref(desc_e), C.byref(desc_d), C.byref(desc_p),
+                                                       C.byref(packs[0]), C.byref(packs[1]), C.byref(packs[2]),
+                                                       C.byref(w)))
+        return w.value
+
+    def conv_chain3(self, ch, x, y=None, add=None):
+        """add = (src, out, m_src, m_conv, rshift, relu) behind the projection"""
+        post = ConvPost()
+        if add is not None:
+            src, out, m_src, m_conv, rshift, relu = add
+            post.add = FusedAdd(1, int(m_src), int(m_conv), int(rshift), int(relu))
+            post.add_src, post.add_out = src.ptr, out.ptr
+        self._ck(self.lib.tpuhip_conv2d_chain3_i8(self.h, ch, x.ptr, None if y is None else y.ptr, C.byref(post)))
 
     def conv_chain_destroy(self, ch):
         self._ck(self.lib.tpuhip_conv2d_chain_destroy(self.h, ch))

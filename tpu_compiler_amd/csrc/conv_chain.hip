@@ -413,27 +413,68 @@ int tpuhip_conv2d_chain_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *da, con
   return TPUHIP_OK;
 }
 
+int tpuhip_conv2d_can_chain3(const tpuhip_conv_desc *de, const tpuhip_conv_desc *dd, const tpuhip_conv_desc *dp) {
+  return de && dd && dp && irb_covers(*de, *dd, *dp) ? 1 : 0;
+}
+
+int tpuhip_conv2d_chain3_prepack(tpuhip_ctx *ctx, const tpuhip_conv_desc *de, const tpuhip_conv_desc *dd,
+                                 const tpuhip_conv_desc *dp, const tpuhip_chain_conv *ce, const tpuhip_chain_conv *cd,
+                                 const tpuhip_chain_conv *cp, tpuhip_conv_chain **out) {
+  TPUHIP_REQUIRE(ctx && de && dd && dp && ce && cd && cp && out, "tpuhip_conv2d_chain3_prepack: NULL argument");
+  TPUHIP_REQUIRE(ce->filter && cd->filter && cp->filter && ce->multiplier && cd->multiplier && cp->multiplier &&
+                     ce->rshift && cd->rshift && cp->rshift,
+                 "tpuhip_conv2d_chain3_prepack: NULL operand");
+  if (!irb_covers(*de, *dd, *dp))
+    return set_error(TPUHIP_ERR_UNSUPPORTED,
+                     "conv chain: needs an unpadded 1x1 / stride 1 conv of at most 160 input channels, a depthwise conv "
+                     "of at most 3 x 3 taps on its result and an unpadded 1x1 / stride 1 conv of at most 384 channels "
+                     "on that one's, dense channel strides, and LDS for a pixel block's window of the expanded tensor");
+  auto *ch = new tpuhip_conv_chain();
+  ch->da = *de;
+  ch->db = *dd;
+  ch->dc = *dp;
+  ch->kind = 3;
+  const int rc = irb_prepack(ctx, ch, ce, cd, cp);
+  if (rc) {
+    tpuhip_conv2d_chain_destroy(ctx, ch);
+    return rc;
+  }
+  *out = ch;
+  return TPUHIP_OK;
+}
+
+int tpuhip_conv2d_chain3_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y,
+                            const tpuhip_conv_post *post) {
+  TPUHIP_REQUIRE(ctx && ch && x, "tpuhip_conv2d_chain3_i8: NULL argument");
+  TPUHIP_REQUIRE(ch->kind == 3, "tpuhip_conv2d_chain3_i8: not a chain of three");
+  return irb_run(ctx, ch, x, y, post);
+}
+
 int tpuhip_conv2d_chain_destroy(tpuhip_ctx *ctx, tpuhip_conv_chain *ch) {
   if (!ch) return TPUHIP_OK;
   TPUHIP_REQUIRE(ctx, "tpuhip_conv2d_chain_destroy: NULL context");
-  int rc = tpuhip_free(ctx, ch->w1);
-  int rc2 = tpuhip_free(ctx, ch->w2);
-  int rc3 = tpuhip_free(ctx, ch->q1);
-  int rc4 = tpuhip_free(ctx, ch->q2);
+  int rc = 0;
+  for (void *p : {(void *)ch->w1, (void *)ch->w2, (void *)ch->w3, (void *)ch->w2d, (void *)ch->q1, (void *)ch->q2, (void *)ch->q3}) {
+    const int r = p ? tpuhip_free(ctx, p) : 0;
+    if (!rc) rc = r;
+  }
   delete ch;
-  return rc ? rc : rc2 ? rc2 : rc3 ? rc3 : rc4;
+  return rc;
 }
 
 const char *tpuhip_conv2d_chain_name(const tpuhip_conv_chain *ch) { return ch ? ch->name.c_str() : "null"; }
 
 const char *tpuhip_conv2d_chain_variant_name(int variant) {
   if (variant < 0) return nullptr;
-  return variant < kNumChainVariants ? kChainVariants[variant].name : dwpw_variant_name(variant - kNumChainVariants);
+  if (variant < kNumChainVariants) return kChainVariants[variant].name;
+  if (const char *n = dwpw_variant_name(variant - kNumChainVariants)) return n;
+  return irb_variant_name(variant - kNumChainVariants - 6);
 }
 
 int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a,
                                 const tpuhip_conv_post *post_a, void *y_b, const tpuhip_conv_post *post_b) {
   TPUHIP_REQUIRE(ctx && ch && x, "tpuhip_conv2d_chain_post_i8: NULL argument");
+  TPUHIP_REQUIRE(ch->kind != 3, "conv chain: a chain of three runs through tpuhip_conv2d_chain3_i8");
   TPUHIP_REQUIRE(!(post_a && post_a->pool) && !(post_b && post_b->pool), "conv chain: takes no fused pool");
   if (ch->kind == 2) return dwpw_run(ctx, ch, x, y_a, post_a, y_b, post_b);
   TPUHIP_REQUIRE(!(post_a && post_a->lut) && !(post_b && (post_b->lut || post_b->add.enable)),
@@ -445,6 +486,7 @@ int tpuhip_conv2d_chain_post_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, co
 int tpuhip_conv2d_chain_i8(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a,
                            const void *add_src, void *add_out, const tpuhip_fused_add *f, void *y_b) {
   TPUHIP_REQUIRE(ctx && ch && x && y_b, "tpuhip_conv2d_chain_i8: NULL argument");
+  TPUHIP_REQUIRE(ch->kind != 3, "conv chain: a chain of three runs through tpuhip_conv2d_chain3_i8");
   const bool add = f && f->enable;
   if (ch->kind == 2) {
     TPUHIP_REQUIRE(!add, "conv chain: a depthwise -> pointwise chain takes its add behind the second conv "

@@ -14,12 +14,13 @@
 #include <vector>
 
 struct tpuhip_conv_chain {
-  tpuhip_conv_desc da, db;
-  int kind = 0;      // 1: pointwise -> pointwise, 2: depthwise -> pointwise
-  int variant = -1;  // kind 1: index into the chain kernel variants
+  tpuhip_conv_desc da, db, dc;   // dc: the third conv of an inverted-residual chain
+  int kind = 0;      // 1: pointwise -> pointwise, 2: depthwise -> pointwise, 3: pointwise -> depthwise -> pointwise
+  int variant = -1;  // index into the kernel variants of the kind
   int kp1 = 0;
-  int8_t *w1 = nullptr, *w2 = nullptr;
-  int32_t *q1 = nullptr, *q2 = nullptr;
+  int8_t *w1 = nullptr, *w2 = nullptr, *w3 = nullptr;
+  uint32_t *w2d = nullptr;       // kind 3: the depthwise filter as one dword per lane and tap
+  int32_t *q1 = nullptr, *q2 = nullptr, *q3 = nullptr;
   std::string name;
 };
 
@@ -103,5 +104,12 @@ int dwpw_prepack(tpuhip_ctx *ctx, tpuhip_conv_chain *ch, const int8_t *filter_a,
                  const int32_t *mult_b, const int32_t *rshift_b);
 int dwpw_run(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y_a, const tpuhip_conv_post *post_a,
              void *y_b, const tpuhip_conv_post *post_b);
+
+// pointwise -> depthwise -> pointwise (conv_irb.hip)
+bool irb_covers(const tpuhip_conv_desc &e, const tpuhip_conv_desc &d, const tpuhip_conv_desc &p);
+const char *irb_variant_name(int i);    // null past the last one
+int irb_prepack(tpuhip_ctx *ctx, tpuhip_conv_chain *ch, const tpuhip_chain_conv *ce, const tpuhip_chain_conv *cd,
+                const tpuhip_chain_conv *cp);
+int irb_run(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y, const tpuhip_conv_post *post);
 
 }  // namespace tpuhip
