@@ -6,7 +6,8 @@ they replace, on the layer pairs of the benchmark networks:
   * pointwise -> pointwise (ResNet-50: the 1x1 expansion + residual add closing a bottleneck block and
     the 1x1 reduction opening the next);
   * depthwise -> pointwise (MobileNetV2: the depthwise conv and the 1x1 projection of an
-    inverted-residual block, with the block's residual add where it has one).
+    inverted-residual block, with the block's residual add where it has one);
+  * pointwise -> depthwise -> pointwise (the whole inverted-residual block).
 
 Random weights and inputs; both forms write the same bytes (checked).  HIP events around 20 launches."""
 import argparse
@@ -121,6 +122,46 @@ def depthwise_pair(ctx, rng, n, c, oc, hw, stride, add):
     return ts, tc, same, names, ctx.conv_chain_name(ch)
 
 
+def inverted_residual(ctx, rng, n, cin, c, oc, hw, stride, add):
+    """1x1 expansion cin -> c + ReLU, 3x3 depthwise + ReLU, 1x1 projection c -> oc, residual add where the
+    block has one"""
+    we, wa, wb = _weights(rng, (c, cin, 1, 1), 24), _weights(rng, (c, 1, 3, 3), 30), _weights(rng, (oc, c, 1, 1), 20)
+    pe, pa, pb = _params(rng, c), _params(rng, c), _params(rng, oc)
+    xs, es = (n, cin, hw, hw), (n, c, hw, hw)
+    de = _desc(xs, c, 1, relu=True)
+    da = _desc(es, c, 3, g=c, stride=stride, pad=1, relu=True)
+    ms, ys = (n, c, da.oh, da.ow), (n, oc, da.oh, da.ow)
+    db = _desc(ms, oc, 1)
+    xt, et, mt, ot = ctx.tensor(xs), ctx.tensor(es), ctx.tensor(ms), ctx.tensor(ys)
+    r1, r2 = ctx.tensor(ys), ctx.tensor(ys)
+    _fill(ctx, rng, xt)
+    _fill(ctx, rng, ot)
+    whe, wha, whb = ctx.conv_prepack(de, we, *pe), ctx.conv_prepack(da, wa, *pa), ctx.conv_prepack(db, wb, *pb)
+    ch = ctx.conv_chain3_prepack(de, da, db, (we, *pe), (wa, *pa), (wb, *pb))
+
+    def separate():
+        ctx.conv(whe, xt, et)
+        ctx.conv(wha, et, mt)
+        if add:
+            ctx.conv_add(whb, mt, None, ot, r1, 64, 64, 7, False)
+        else:
+            ctx.conv(whb, mt, r1)
+
+    def chained():
+        if add:
+            ctx.conv_chain3(ch, xt, None, (ot, r2, 64, 64, 7, False))
+        else:
+            ctx.conv_chain3(ch, xt, r2)
+
+    separate()
+    ts, tc = _time(ctx, separate), _time(ctx, chained)
+    same = np.array_equal(_bytes(ctx, r1), _bytes(ctx, r2))
+    names = "%s + %s + %s" % (ctx.conv_algo_name(whe), ctx.conv_algo_name(wha), ctx.conv_algo_name(whb))
+    for t in (xt, et, mt, ot, r1, r2):
+        t.free()
+    return ts, tc, same, names, ctx.conv_chain_name(ch)
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--batch-resnet", type=int, default=32)
@@ -144,6 +185,24 @@ def main():
         tot[1] += tc
         print("  %3d dw s%d%s -> %3d at %3dx%-3d  %6.2f | %6.2f  %s | %s  %s"
               % (c, s, " (+add)" if add else "       ", oc, hw, hw, ts, tc, names, cname,
+                 "same bytes" if same else "BYTES DIFFER"), flush=True)
+    print("  sum %.1f | %.1f" % tuple(tot))
+    print("1x1 -> depthwise 3x3 -> 1x1, batch %d: us for the three launches | the chain" % args.batch_mobilenet)
+    tot = [0.0, 0.0]
+    for cin, c, oc, hw, s, add in ((16, 96, 24, 112, 2, False), (24, 144, 24, 56, 1, True), (24, 144, 32, 56, 2, False),
+                                   (32, 192, 32, 28, 1, True), (32, 192, 64, 28, 2, False), (64, 384, 64, 14, 1, True),
+                                   (64, 384, 96, 14, 1, False), (96, 576, 96, 14, 1, True), (96, 576, 160, 14, 2, False),
+                                   (160, 960, 160, 7, 1, True), (160, 960, 320, 7, 1, False)):
+        if not ctx.conv_can_chain3(_desc((args.batch_mobilenet, cin, hw, hw), c, 1, relu=True),
+                                   _desc((args.batch_mobilenet, c, hw, hw), c, 3, g=c, stride=s, pad=1, relu=True),
+                                   _desc((args.batch_mobilenet, c, (hw - 1) // s + 1, (hw - 1) // s + 1), oc, 1)):
+            print("  %3d -> %3d dw s%d -> %3d at %3dx%-3d  not covered" % (cin, c, s, oc, hw, hw))
+            continue
+        ts, tc, same, names, cname = inverted_residual(ctx, rng, args.batch_mobilenet, cin, c, oc, hw, s, add)
+        tot[0] += ts
+        tot[1] += tc
+        print("  %3d -> %3d dw s%d%s -> %3d at %3dx%-3d  %6.2f | %6.2f  %s | %s  %s"
+              % (cin, c, s, " (+add)" if add else "       ", oc, hw, hw, ts, tc, names, cname,
                  "same bytes" if same else "BYTES DIFFER"), flush=True)
     print("  sum %.1f | %.1f" % tuple(tot))
     ctx.close()

@@ -56,6 +56,8 @@ struct IrbArgs {
   uint32_t magic_w, magic_pc;        // ceil(2^32 / width), ceil(2^32 / pcols)
   int pcols, prows;                  // the patch of a group
   int lp16;                          // LDS pitch of a patch pixel in 16-byte chunks (odd)
+  int xc16, xp16;                    // 16-byte chunks of an input pixel, and its LDS pitch in chunks (odd)
+  uint32_t magic_xc;                 // ceil(2^32 / xc16)
   int log2p, n_cb, n_tm, ngroups, nk;
 };
 
@@ -72,6 +74,7 @@ conv_irb_kernel(IrbArgs a) {
   int32_t *qall = q2 + 5 * ocp;                                                     // [NW][160]
   int32_t *red = qall + NW * 160;                                                   // [tiles][16][64] when nk > 1
   v4i *patch = reinterpret_cast<v4i *>(red + (a.nk > 1 ? tiles * 1024 : 0));         // [prows * pcols][lp16 chunks]
+  v4i *xin = patch + a.prows * a.pcols * a.lp16;                                    // [prows * pcols][xp16 chunks]
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -111,6 +114,33 @@ conv_irb_kernel(IrbArgs a) {
     const int prows = (nb * a.rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;   // rows this group's windows span
     const int npp = prows * a.pcols;
     const int npb = (npp + 31) >> 5;
+    // the input pixels under the patch, fetched once by the whole workgroup (one trip to memory instead of
+    // one per result block): 16-byte chunks in memory order, zeros outside the image
+    {
+      const int chunks = npp * a.xc16;
+      for (int q0 = 0; q0 < chunks; q0 += 4 * NW * 64) {
+        v4i v[4];
+        int dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (q0 + u * NW * 64 >= chunks) break;              // the same for the whole workgroup
+          const int q = q0 + u * NW * 64 + (int)threadIdx.x;
+          const int pix = a.xc16 == 1 ? q : (int)__umulhi((uint32_t)q, a.magic_xc), cc = q - pix * a.xc16;
+          const int pr = (int)__umulhi((uint32_t)pix, a.magic_pc), pc = pix - pr * a.pcols;
+          const int ih = prow0 + pr, iw = pcol0 + pc;
+          const bool ok = (q < chunks) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
+          v[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(
+              xrsrc, ok ? (uint32_t)(ih * row_bytes + iw * a.x_cs + cc * 16) : kOobOffset, img_base, 0);
+          dst[u] = q < chunks ? pix * a.xp16 + cc : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          if (q0 + u * NW * 64 >= chunks) break;
+          if (dst[u] >= 0) xin[dst[u]] = v[u];
+        }
+      }
+    }
+    __syncthreads();
     for (int cb = wave; cb < a.n_cb; cb += NW) {
       v4i afr[kIrbMaxKsIn];
       const v4i *afrag = reinterpret_cast<const v4i *>(a.wex) + (size_t)cb * a.ks_in * 64 + lane;
@@ -122,21 +152,16 @@ conv_irb_kernel(IrbArgs a) {
         const int pr = (int)__umulhi((uint32_t)pp, a.magic_pc), pc = pp - pr * a.pcols;
         const int ih = prow0 + pr, iw = pcol0 + pc;
         const bool valid = (pp < npp) & ((unsigned)ih < (unsigned)a.ih) & ((unsigned)iw < (unsigned)a.iw);
-        const uint32_t off = (uint32_t)(ih * row_bytes + iw * a.x_cs + fk * 16);
-        v4i bx[kIrbMaxKsIn];
-#pragma unroll
-        for (int ks = 0; ks < kIrbMaxKsIn; ++ks) {
-          if (ks >= a.ks_in) break;                          // the same for the whole wave
-          const bool ok = valid & (ks * 32 + fk * 16 < a.x_cw);
-          bx[ks] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(xrsrc, ok ? off + (uint32_t)(ks * 32) : kOobOffset, img_base, 0);
-        }
+        const v4i *xp = xin + min(pp, npp - 1) * a.xp16 + fk;
         v16i acc[1];
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[0][e] = 0;
 #pragma unroll
         for (int ks = 0; ks < kIrbMaxKsIn; ++ks) {
-          if (ks >= a.ks_in) break;
-          acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[ks], bx[ks], acc[0], 0, 0, 0);
+          if (ks >= a.ks_in) break;                          // the same for the whole wave
+          // a K slice past the input's last 16 channels meets zero filter columns: any pixel's chunk will do
+          const v4i bx = xp[min(ks * 2, a.xc16 - 1 - fk)];
+          acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[ks], bx, acc[0], 0, 0, 0);
         }
         uint32_t outw[1][4];
         if (a.relu_ex) requant_rows_c64<1, true>(acc, 0, pc64, pmult, pshift, phpot, outw);
@@ -337,7 +362,8 @@ bool irb_plan(const tpuhip_conv_desc &e, const tpuhip_conv_desc &d, const tpuhip
     for (int log2p = (best * d.n >= 1024 ? 1 : 0); log2p >= 0; --log2p) {
       const int P = 1 << log2p, tiles = out->n_tm * P;
       const int prows = (P * rows - 1) * d.sh + (d.kh - 1) * d.dh + 1;
-      const int64_t patch = (int64_t)prows * out->pcols * out->lp16 * 16;
+      const int xp16 = ((e.ic + 15) / 16) | 1;
+      const int64_t patch = (int64_t)prows * out->pcols * (out->lp16 + xp16) * 16;   // the expanded patch and the input under it
       for (int nw = 8; nw <= 16; nw *= 2) {
         const int nt = (tiles + nw - 1) / nw;
         if (irb_shape_index(nw, nt) < 0) continue;
@@ -479,6 +505,9 @@ int irb_run(tpuhip_ctx *ctx, const tpuhip_conv_chain *ch, const void *x, void *y
   a.pcols = plan.pcols; a.prows = plan.prows;
   a.magic_pc = magic(plan.pcols);
   a.lp16 = plan.lp16;
+  a.xc16 = a.x_cw / 16;
+  a.xp16 = a.xc16 | 1;
+  a.magic_xc = magic(a.xc16);
   a.log2p = plan.log2p; a.n_cb = plan.n_cb; a.n_tm = plan.n_tm; a.ngroups = plan.ngroups; a.nk = plan.nk;
   const unsigned lds = plan.lds;
   const dim3 grid(8u * (unsigned)((a.ngroups + 7) / 8)), block((unsigned)plan.nw * 64);
