@@ -262,6 +262,32 @@ def test_sibling_convs_run_as_one_launch_with_unchanged_results():
         m.close()
 
 
+def test_a_stem_that_took_its_max_pool_is_left_out_of_pairing():
+    """two 7x7 / stride 2 convs over the image, the first with 128 output channels (a candidate first of a
+    pair), the second a stem with its max pool folded into its launch: pairing must not swallow the stem, or
+    the pooled tensor would never be written.  Also: with two readers, one of them off the stem path, the
+    image keeps its 16-byte channel stride."""
+    from tpu_compiler_amd.graphs import Builder, BASE_SEED
+    b = Builder("sibling_stems", BASE_SEED + 77, 2, (6, 16))
+    x = b.input("input", 3, 64, 64)
+    wide = b.conv("wide", x, 128, 7, stride=2, pad=3, relu=True)
+    stem = b.conv("stem", x, 64, 7, stride=2, pad=3, relu=True)
+    pooled = b.pool_max("pool", stem, 3, 2, (0, 1, 0, 1))
+    g = b.finish([wide, pooled])
+    want = oracle_graph.run(g)
+    for keep in (1, 0):
+        m = module()
+        m.set_option("keep_all_tensors", keep)
+        m.load(g)
+        algo = dict(m.kernels())
+        assert algo["stem"] == "stem" and not algo["wide"].startswith("with")
+        m.set_tensor("input", g.input_op().data.astype(np.float32))
+        m.invoke()
+        for name in ("wide", "pool") + (("stem",) if keep else ()):
+            assert np.array_equal(m.get_tensor_i8(name), want[name].reshape(g.by_name[name].shape)), (keep, name)
+        m.close()
+
+
 def test_chained_pointwise_convs_run_as_one_launch_with_unchanged_results():
     """the 1x1 expansion + add that closes a bottleneck block and the 1x1 reduction that opens the next
     run as one launch (res2a/b, res3a/b/c of the ResNet-50 shape).  On, off, with every tensor kept and

@@ -9,9 +9,9 @@
 // chip.  A workgroup owns P vertically neighbouring pixel blocks (R rows x W pixels each, R * W <= 32)
 // of one image and runs three phases, all on the matrix cores:
 //   * expansion: the input pixels under the blocks' windows (a patch of prows x pcols pixels, halo
-//     included) times the expansion filter: patch pixels are MFMA columns (B fragments straight from
-//     global memory, 16 bytes per lane; pixels outside the image load zeros), 32-channel blocks of
-//     the filter are A fragments, dealt to the waves.  Requantised results go to an LDS patch
+//     included; fetched into LDS once by the whole workgroup, pixels outside the image as zeros) times
+//     the expansion filter: patch pixels are MFMA columns, 32-channel blocks of the filter are A
+//     fragments, dealt to the waves.  Requantised results go to an LDS patch
 //     [pixel][channels], pixel pitch an odd number of 16-byte chunks; pixels outside the image are
 //     stored as ZEROS -- the depthwise conv pads its input, the expansion's result, with zeros.
 //   * depthwise: a tap is a 32x32 diagonal matrix times 32 channels x 32 pixels read from the patch
