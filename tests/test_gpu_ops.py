@@ -22,7 +22,9 @@ PATCH_TILES = [t for t in range(NUM_TILES) if "mfma_patch_" in capi_tile_name(t)
 PATCH2_TILES = [t for t in range(NUM_TILES) if "mfma_patch2_" in capi_tile_name(t)]
 # the pointwise variants take unpadded 1x1 layers with at most the K in their name
 PW_TILES = [t for t in range(NUM_TILES) if "_pw_" in capi_tile_name(t)]
-GENERAL_TILES = [t for t in range(NUM_TILES) if t not in PATCH_TILES + PATCH2_TILES + PW_TILES]
+# their third form: the same layers again; the four waves of a pixel group split K
+PATCH3_TILES = [t for t in range(NUM_TILES) if "mfma_patch3_" in capi_tile_name(t)]
+GENERAL_TILES = [t for t in range(NUM_TILES) if t not in PATCH_TILES + PATCH2_TILES + PATCH3_TILES + PW_TILES]
 
 
 def tile_bn(tile):
@@ -569,6 +571,84 @@ def test_conv_patch2_tile_variants(ctx, case, tile, post):
         t.free()
 
 
+# cases of the third form beyond PATCH_CASES: tiles of several whole images (with a last tile
+# that holds fewer), 1024 input channels, a K that leaves the four K groups unequal shares
+PATCH3_CASES = PATCH_CASES + [
+    (5, 512, 7, 7, 40, True, False),       # two or five images per tile, the last tile ragged
+    (9, 64, 4, 5, 33, False, False),       # up to twelve images per tile
+    (2, 1024, 3, 3, 64, True, False),
+    (7, 64, 6, 6, 96, True, False),        # 18 K slices: shares of 5, 5, 4 and 4
+    (1, 256, 16, 16, 32, False, False),    # exactly 256 pixels
+]
+
+
+@pytest.mark.parametrize("tile,case", [(t, c) for t in PATCH3_TILES for c in PATCH3_CASES if c[3] <= tile_bn(t)])
+@pytest.mark.parametrize("post", ["plain", "add", "table_add"])
+def test_conv_patch3_tile_variants(ctx, case, tile, post):
+    n, c, h, w_, oc, relu, _ = case
+    rng = np.random.default_rng(c + h * 3 + oc + tile)
+    x = rnd_i8(rng, (n, c, h, w_))
+    w = rnd_w(rng, (oc, c, 3, 3), sigma=14)
+    bias, rsh, mult = rnd_params(rng, oc)
+    rsh[1::5] = 1                      # the smallest shift the overflow-free form takes
+    y_ref = oracle_conv(x, w, bias, rsh, mult, 1, (1, 1), (1, 1, 1, 1), (1, 1), (0, 0), relu)
+    d = conv_desc(x.shape, w.shape, pads=(1, 1, 1, 1), do_relu=relu, algo=16 + tile)
+    xt = ctx.from_nchw(x)
+    yt, tt, zt = ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape), ctx.tensor(y_ref.shape)
+    for t in (yt, tt, zt):
+        ctx._ck(ctx.lib.tpuhip_memset(ctx.h, t.ptr, 0x55, t.nbytes))
+    wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))
+    assert "patch3" in ctx.conv_algo_name(wh)
+    other = rnd_i8(rng, y_ref.shape)
+    ot = ctx.from_nchw(other)
+    if post == "plain":
+        ctx.conv(wh, xt, yt)
+    elif post == "add":
+        z_ref = O.eltwise_add_i8([other, y_ref], [61, -47], [6], True)
+        ctx.conv_add(wh, xt, yt, ot, zt, 61, -47, 6, True)
+        assert np.array_equal(ctx.to_nchw(zt), z_ref) and not ctx.raw(zt)[..., oc:].any()
+    else:
+        table = rnd_i8(rng, 256)
+        table[0] = 77
+        t_ref = O.lut_i8(y_ref, table)
+        z_ref = O.eltwise_add_i8([other, t_ref], [37, 51], [5], False)
+        ctx.conv_post(wh, xt, yt, table, tt, (ot, zt, 37, 51, 5, False))
+        assert np.array_equal(ctx.to_nchw(tt), t_ref) and not ctx.raw(tt)[..., oc:].any()
+        assert np.array_equal(ctx.to_nchw(zt), z_ref) and not ctx.raw(zt)[..., oc:].any()
+    got = ctx.to_nchw(yt)
+    assert np.array_equal(got, y_ref), "%s: %d mismatches" % (ctx.conv_algo_name(wh), (got != y_ref).sum())
+    assert not ctx.raw(yt)[..., oc:].any()
+    assert len(np.unique(y_ref)) > 8
+    ctx.conv_weights_destroy(wh)
+    for t in (xt, ot, yt, tt, zt):
+        t.free()
+
+
+@pytest.mark.parametrize("tile", PATCH3_TILES)
+def test_conv_patch3_tiles_refuse_other_layers(ctx, tile):
+    """stride 2, 96 channels, 1x1, a map wider than the tile, an rshift of 0 (the general requant form)"""
+    z = lambda oc, ic, k: (np.zeros((oc, ic, k, k), np.int8), None, np.full(oc, 1 << 30, np.int32), np.ones(oc, np.int32))
+    for shape, wshape, kw, rs0 in [((1, 64, 8, 8), (64, 64, 3, 3), dict(stride=(2, 2), pads=(1, 1, 1, 1)), False),
+                                   ((1, 96, 8, 8), (64, 96, 3, 3), dict(pads=(1, 1, 1, 1)), False),
+                                   ((1, 64, 8, 8), (64, 64, 1, 1), dict(), False),
+                                   ((1, 64, 8, 300), (64, 64, 3, 3), dict(pads=(1, 1, 1, 1)), False),
+                                   ((1, 64, 8, 8), (64, 64, 3, 3), dict(pads=(1, 1, 1, 1)), True)]:
+        d = conv_desc(shape, wshape, algo=16 + tile, **kw)
+        wt, b, m, r = z(wshape[0], wshape[1], wshape[2])
+        if rs0:
+            r = r.copy()
+            r[5] = 0
+        xt, yt = ctx.tensor(shape), ctx.tensor((d.n, d.oc, d.oh, d.ow))
+        with pytest.raises(capi.TpuHipError, match="3x3 / stride 1 / pad 1"):
+            wh = ctx.conv_prepack(d, wt, b, m, r)
+            try:
+                ctx.conv(wh, xt, yt)
+            finally:
+                ctx.conv_weights_destroy(wh)
+        xt.free()
+        yt.free()
+
+
 def _random_conv_case(rng):
     """a dense conv of one of three families: 3x3 / stride 1 / pad 1 on the channel counts the
     row-patch kernels take, 1x1 with stride 1 or 2, or anything goes"""
@@ -614,7 +694,7 @@ def test_conv_random_shapes_every_tile_variant(ctx, seed):
         z_ref = O.eltwise_add_i8([other, want], [61, 47], [6], True)
         xt, ot = ctx.from_nchw(x), ctx.from_nchw(other)
         yt, zt = ctx.tensor(want.shape), ctx.tensor(want.shape)
-        for tile in GENERAL_TILES + PATCH_TILES + PATCH2_TILES + PW_TILES:
+        for tile in GENERAL_TILES + PATCH_TILES + PATCH2_TILES + PATCH3_TILES + PW_TILES:
             d = conv_desc(x.shape, w.shape, stride=stride, pads=pads, dil=dil, do_relu=relu, algo=16 + tile)
             try:
                 wh = ctx.conv_prepack(d, w, f2i32(bias), f2i32(mult), f2i32(rsh))

@@ -91,6 +91,7 @@ struct ConvArgs {
   // persistent kernels: workgroups per XCD (a multiple of n_oc_tiles) and the pixel
   // advance between two tiles of one workgroup, split into (n, oh, ow) parts
   int wgs_per_xcd, pstep_pix, pstep_n, pstep_oh, pstep_ow;
+  int tile_imgs;          // third form of the patch kernel: whole images per tile
   int npix;
   int linear;             // 1x1, stride 1, no padding: input pixel index == output pixel index
   int stem_pw;            // stem kernel: input columns one row tile needs, (128 - 1) * sw + 8
@@ -1415,7 +1416,7 @@ conv_pw_kernel(ConvArgs a) {
 // 2 * (C + 16) + kPatch2RowPad is a multiple of 128 for every C that is a multiple of 64
 constexpr int kPatch2RowPad = 96;
 
-template <int BM, int BN, int WM, int WN, int BK, int OCC>
+template <int BM, int BN, int WM, int WN, int BK, int OCC, int NB>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_patch2_kernel(ConvArgs a) {
 #ifdef TPUHIP_TRACE
@@ -1425,7 +1426,6 @@ conv_patch2_kernel(ConvArgs a) {
   gather_conv_args(a);
   gather_conv_args_more(a);
   constexpr int NT = WM * WN * 64;
-  constexpr int RD = 4;                       // filter tiles in flight in registers (even)
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
   static_assert(BK == 128 || BK == 256, "K bytes per step");
@@ -1433,14 +1433,18 @@ conv_patch2_kernel(ConvArgs a) {
   constexpr int ABYTES = BM * AROW;
   constexpr int CPA = BK / 16;                // 16-byte chunks of a filter tile row
   constexpr int NW = BM * CPA / NT;           // filter chunks per thread per step
+  // filter tiles in flight in registers (even).  With three LDS tiles a tile is parked two steps
+  // before its step, so it stays in registers for RD - 2 steps only
+  constexpr int RD = NB == 3 && NW <= 2 ? 6 : 4;
+  static_assert(NB == 2 || NB == 3, "LDS filter tiles");
   constexpr int KK = BK / 32;
   constexpr int NPL = 18 * 256 / NT;          // patch chunks per thread at most (72 KiB of input)
-  static_assert(BN * stage_row_bytes<BM>() <= 2 * ABYTES, "the staged tile must fit the filter tiles");
+  static_assert(BN * stage_row_bytes<BM>() <= NB * ABYTES, "the staged tile must fit the filter tiles");
   extern __shared__ __attribute__((aligned(16))) v4i p2_smem[];
   int32_t *const qlds = reinterpret_cast<int32_t *>(p2_smem);                 // 5 * BM dwords
   uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);         // 64 dwords
-  int8_t *const abuf = reinterpret_cast<int8_t *>(lutw + 64);                 // 2 * ABYTES
-  int8_t *const patch = abuf + 2 * ABYTES;
+  int8_t *const abuf = reinterpret_cast<int8_t *>(lutw + 64);                 // NB * ABYTES
+  int8_t *const patch = abuf + NB * ABYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1547,7 +1551,7 @@ conv_patch2_kernel(ConvArgs a) {
     bbase[j] = (p < rows * a.ow ? (int)pr * rowb + pc * prow : 0) + fk * 16;   // idle slots read position 0
   }
 
-  // park the patch and the first filter tile
+  // park the patch and the first filter tile (with three LDS tiles, the first two)
 #pragma unroll
   for (int u = 0; u < NPL; ++u) {
     const int q = tid + u * NT;
@@ -1558,6 +1562,7 @@ conv_patch2_kernel(ConvArgs a) {
   }
   TPUHIP_TS(1);
   store_A(0, 0);
+  if (NB == 3) store_A(1, 1);
   __syncthreads();
   TPUHIP_TS(2);
 
@@ -1576,40 +1581,53 @@ conv_patch2_kernel(ConvArgs a) {
         for (int e = 0; e < 16; ++e) accs[c][i][j][e] = 0;
   v16i (&acc)[TM][TN] = accs[0];
 
-  // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS a
-  // step ago -- and receives the tile RD steps ahead; the next step's tile goes from its slot
-  // to the other LDS tile.  Within the step the operands of a 32-byte K slice are requested PD
-  // slices before their MFMAs (see frag_prefetch).
+  // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS
+  // earlier -- and receives the tile RD steps ahead.  Within the step the operands of a 32-byte K
+  // slice are requested PD slices before their MFMAs (see frag_prefetch).
+  // Two LDS tiles: the next step's tile goes from its slot to the other LDS tile at the end of
+  // the step, and the step after the barrier starts by requesting its first operands.
+  // Three LDS tiles: the tile TWO steps ahead is parked at the end of the step, so the next
+  // step's tile has been visible since the previous barrier and the next step's first operands
+  // are requested BEFORE the barrier: the MFMAs resume right behind it instead of an LDS round
+  // trip later.
   constexpr int PD = OCC >= 4 ? 1 : frag_prefetch(TM * TN);
+  v4i fa[PD + 1][TM], fb[PD + 1][TN];
+  // operands of 32-byte slice kk of K step s, whose filter tile lies at LDS offset aoff
+  auto read_slice = [&](int s, int aoff, int kk, int fs) {
+    // the slice lies in one filter tap (C is a multiple of 64); slices past the ninth tap
+    // meet zero weights and read the last tap
+    const int koff = s * BK + kk * 32;
+    const int tap = min(koff >> lgc, 8);
+    const int tkh = (tap * 11) >> 5;
+    const int boff = tkh * rowb + (tap - 3 * tkh) * prow + (koff & (C - 1));
+#pragma unroll
+    for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(abuf + aoff + abase[i] + kk * 32);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
+  };
+  int cur = 0;   // LDS offset of the running step's filter tile (three tiles: rotates at run time)
+  if (NB == 3) {
+#pragma unroll
+    for (int kk = 0; kk < PD; ++kk) read_slice(0, 0, kk, kk % (PD + 1));
+  }
   auto step = [&](int s, auto slotc) {
-    constexpr int slot = decltype(slotc)::value, buf = slot & 1;
+    constexpr int slot = decltype(slotc)::value;
 #ifdef TPUHIP_TRACE
     const bool tr = s < 4;
-    if (tr) TPUHIP_TS(3 + slot * 6);
+    if (tr) TPUHIP_TS(3 + (slot & 3) * 6);
 #endif
     load_A(slot, s + RD);
-    const int8_t *ab = abuf + buf * ABYTES;
-    v4i fa[PD + 1][TM], fb[PD + 1][TN];
-    auto read_slice = [&](int kk, int fs) {
-      // the slice lies in one filter tap (C is a multiple of 64); slices past the ninth tap
-      // meet zero weights and read the last tap
-      const int koff = s * BK + kk * 32;
-      const int tap = min(koff >> lgc, 8);
-      const int tkh = (tap * 11) >> 5;
-      const int boff = tkh * rowb + (tap - 3 * tkh) * prow + (koff & (C - 1));
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(ab + abase[i] + kk * 32);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fb[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
-    };
+    const int aoff = NB == 3 ? cur : (slot & 1) * ABYTES;
     // K is padded to whole steps with zero weights: the slices of the last step that lie in
     // the padding are not multiplied (kreal: slices of this step that hold weights)
     const int kreal = min(KK, (a.k16 * 16 - s * BK + 31) >> 5);
+    if (NB == 2) {
 #pragma unroll
-    for (int kk = 0; kk < PD; ++kk) read_slice(kk, kk);
+      for (int kk = 0; kk < PD; ++kk) read_slice(s, aoff, kk, kk % (PD + 1));
+    }
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      if (kk + PD < KK) read_slice(kk + PD, (kk + PD) % (PD + 1));
+      if (kk + PD < KK) read_slice(s, aoff, kk + PD, (kk + PD) % (PD + 1));
       __builtin_amdgcn_sched_barrier(0);
       if (kk < kreal) {
 #pragma unroll
@@ -1621,18 +1639,32 @@ conv_patch2_kernel(ConvArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
 #ifdef TPUHIP_TRACE
-      if (tr && kk == 0) TPUHIP_TS(4 + slot * 6);
-      if (tr && kk == 3) TPUHIP_TS(5 + slot * 6);
-      if (tr && kk == KK - 1) TPUHIP_TS(6 + slot * 6);
+      if (tr && kk == 0) TPUHIP_TS(4 + (slot & 3) * 6);
+      if (tr && kk == 3) TPUHIP_TS(5 + (slot & 3) * 6);
+      if (tr && kk == KK - 1) TPUHIP_TS(6 + (slot & 3) * 6);
 #endif
     }
-    store_A((slot + 1) % RD, buf ^ 1);   // (past the last step: zeros, into a tile nobody reads)
+    if (NB == 3) {
+      const int nxt = cur == 2 * ABYTES ? 0 : cur + ABYTES;
+      const int nn = nxt == 2 * ABYTES ? 0 : nxt + ABYTES;
+#pragma unroll
+      for (int kk = 0; kk < PD; ++kk) read_slice(s + 1, nxt, kk, kk % (PD + 1));   // (past the last step: unused)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < NW; ++u) {
+        const int q = tid + u * NT;
+        *reinterpret_cast<v4i *>(abuf + nn + (q / CPA) * AROW + (q % CPA) * 16) = wr[(slot + 2) % RD][u];
+      }
+      cur = nxt;
+    } else {
+      store_A((slot + 1) % RD, (slot & 1) ^ 1);   // (past the last step: zeros, into a tile nobody reads)
+    }
 #ifdef TPUHIP_TRACE
-    if (tr) TPUHIP_TS(7 + slot * 6);
+    if (tr) TPUHIP_TS(7 + (slot & 3) * 6);
 #endif
     __syncthreads();
 #ifdef TPUHIP_TRACE
-    if (tr) TPUHIP_TS(8 + slot * 6);
+    if (tr) TPUHIP_TS(8 + (slot & 3) * 6);
 #endif
   };
   for (int s = 0; s < nsteps; s += RD) {
@@ -1640,6 +1672,10 @@ conv_patch2_kernel(ConvArgs a) {
     if (s + 1 < nsteps) step(s + 1, std::integral_constant<int, 1>{});
     if (s + 2 < nsteps) step(s + 2, std::integral_constant<int, 2>{});
     if (s + 3 < nsteps) step(s + 3, std::integral_constant<int, 3>{});
+    if constexpr (RD == 6) {
+      if (s + 4 < nsteps) step(s + 4, std::integral_constant<int, 4>{});
+      if (s + 5 < nsteps) step(s + 5, std::integral_constant<int, 5>{});
+    }
   }
 
   TPUHIP_TS(27);
@@ -1668,6 +1704,325 @@ conv_patch2_kernel(ConvArgs a) {
           v4i{(int)outw[j][0], (int)outw[j][1], (int)outw[j][2], (int)outw[j][3]};
   }
   TPUHIP_TS(28);
+  __syncthreads();
+  TPUHIP_TS(29);
+  flush_tile<BM, BN, NT>(a, stage, tid, pix_base, pix_limit, oc0, out, lut, sv);
+  TPUHIP_TS(30);
+#ifdef TPUHIP_TRACE
+  if (a.trace && (tid & 63) == 0) {
+    for (int k = 0; k < 32; ++k) a.trace[((size_t)blockIdx.x * 8 + (tid >> 6)) * 32 + k] = ts[k];
+  }
+#endif
+}
+
+// ---------------------------------------------------------------------------
+// 3x3 / stride 1 / pad 1 convolutions, third form of the row-patch kernel, for layers whose K is
+// long and whose pixels are few (the late stages of a residual network, 14x14 and 7x7 maps):
+// there the second form spends its time between barriers -- nine and more K steps, each a
+// filter tile parked in LDS, a barrier, and an LDS round trip before the first MFMA -- and on
+// LDS reads, two fragments per MFMA.  Here the K loop has no barrier and no filter in LDS:
+//   * a workgroup of four waves computes 32 output channels of a tile of whole rows of one image
+//     (or of a few whole images, where two and more fit the tile's NBLK x 32 pixel slots) from
+//     the input patch held in LDS, laid out as in the second form;
+//   * the four waves SPLIT K: wave w multiplies 32-byte K slices w, w + 4, w + 8, ... for ALL
+//     pixel blocks of the tile.  Its filter operand of a slice is one MFMA A fragment, which the
+//     packed filter holds as 1 KB contiguous in memory ([channel block][slice][lane][16 bytes]):
+//     one coalesced load per slice straight into registers, U slices ahead, read by this wave
+//     alone.  One A fragment then meets NBLK B fragments from the patch: NBLK MFMAs per
+//     NBLK + 1 operand reads, and independent accumulators back to back;
+//   * the partial sums meet in LDS (the patch's space): every wave parks the blocks it does not
+//     own, a barrier, and the owner of a block (wave j & 3 for block j) adds the three others';
+//   * requantisation and the staged, row-ordered output as in the other LDS kernels (fused
+//     table and add included).
+//   a.stem_pw = W + 2, a.pstep_pix = TH (rows of a tile), a.pstep_n = tiles per image,
+//   a.tile_imgs = whole images per tile (1: a tile is TH rows of one image),
+//   a.pstep_oh = log2(C), a.magic_c16 = ceil(2^32 / chunks of a patch row),
+//   a.magic_pw = floor(2^16 / (TH + 2)) + 1, a.magic_oh = ceil(2^32 / (H * W)), a.pstep_ow = LDS bytes
+// LDS (dynamic): parameters | table | patch, then the partial sums, then the staged tile.
+// ---------------------------------------------------------------------------
+template <int NB2, int PW>
+__global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
+#ifdef TPUHIP_TRACE
+  unsigned long long ts[32] = {};
+#endif
+  TPUHIP_TS(0);
+  gather_conv_args(a);
+  gather_conv_args_more(a);
+  // 4 * PW waves: wave = pixel group * 4 + K group; a pixel group is NB2 blocks of 32 pixel slots
+  constexpr int NT = 256 * PW, NWAVES = 4 * PW, BM = 32, BN = NB2 * PW * 32;
+  constexpr int U = 8;     // A fragments in flight per wave (even)
+  constexpr int NPL = 16;  // patch chunks per thread and pass
+  extern __shared__ __attribute__((aligned(16))) v4i p3_smem[];
+  int32_t *const qlds = reinterpret_cast<int32_t *>(p3_smem);                 // 5 * BM dwords
+  uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);         // 64 dwords
+  int8_t *const patch = reinterpret_cast<int8_t *>(lutw + 64);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kg = wave & 3;          // K group: slices kg, kg + 4, ...
+  const int pg = wave >> 2;         // pixel group: blocks pg * NB2 ...
+  const int logical = (int)(blockIdx.x & 7) * a.tiles_per_xcd + (int)(blockIdx.x >> 3);
+  if (logical >= a.n_tiles) return;
+  const int pt = pixel_tile_of(a, logical);
+  const int ocb = logical - pt * a.n_oc_tiles;
+  const int oc0 = ocb * BM;
+  const int imgs = a.tile_imgs;
+  int img0, r0, rows, nimg;
+  if (imgs > 1) {
+    img0 = pt * imgs; r0 = 0; rows = a.oh; nimg = min(imgs, a.n - img0);
+  } else {
+    img0 = pt / a.pstep_n; r0 = (pt - img0 * a.pstep_n) * a.pstep_pix; rows = min(a.pstep_pix, a.oh - r0); nimg = 1;
+  }
+  const int pix_base = (img0 * a.oh + r0) * a.ow;
+  const int npx = nimg * rows * a.ow;
+  const int pix_limit = pix_base + npx;
+  const int pw = a.stem_pw;
+  const int lgc = a.pstep_oh;                 // log2(C)
+  const int C = 1 << lgc;
+  const int prow = C + 16;                    // bytes of a patch position in LDS
+  const int rowb = pw * prow + kPatch2RowPad; // bytes of a patch row (see conv_patch2_kernel)
+  const int th2 = a.pstep_pix + 2;            // patch rows per image
+  const bool relu = a.lo == 0;
+  // blocks of this wave's pixel group that hold pixels
+  const int nb = min(NB2, ((npx + 31) >> 5) - pg * NB2);
+
+  const __amdgpu_buffer_rsrc_t wrsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t wnone = __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, 0, 0x00020000);
+
+  // the requantisation parameters are requested first and parked last: loads return in order,
+  // and nothing then waits for these alone
+  int32_t qv[5] = {0, 0, 0, 0, 0};
+  if (tid < BM) {
+    const int32_t *c64 = relu ? a.qc64r : a.qc64;
+    qv[0] = c64[2 * (oc0 + tid)];
+    qv[1] = c64[2 * (oc0 + tid) + 1];
+    qv[2] = a.qmult[oc0 + tid];
+    qv[3] = a.qshift[oc0 + tid];
+    qv[4] = a.qhpot[oc0 + tid];
+  }
+
+  // ---- the filter: slice sl of this channel block is the 1 KB fragment (ocb * nsl + sl)
+  const int nsl = a.kp >> 5;
+  const int trips = nb > 0 ? (nsl - kg + 3) >> 2 : 0;   // slices kg, kg + 4, ... below nsl
+  const uint32_t wlane = (uint32_t)lane * 16u;
+  const uint32_t wblock = (uint32_t)ocb * (uint32_t)nsl * 1024u;
+  // (a request past the wave's last slice repeats the last one: same loads every trip, never used)
+  auto load_A = [&](int i) {
+    const int sl = kg + 4 * min(i, trips - 1);
+    return (v4i)__builtin_amdgcn_raw_buffer_load_b128(trips > 0 ? wrsrc : wnone, wlane, wblock + (uint32_t)sl * 1024u, 0);
+  };
+  v4i af[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) af[u] = load_A(u);
+
+  // ---- the patch.  Patch row pr (image pr / th2 of the tile, input row r0 - 1 + pr % th2) is pw
+  // positions of C bytes; positions 1 .. W are the input row (W * C contiguous bytes), the
+  // first and last position and the rows outside the image are the zero border.  A wave takes
+  // rows wave, wave + NWAVES, ...; its lanes take 16-byte chunks lane, lane + 64, ... of the
+  // input row, through a descriptor that covers what is left of the row from the group's first
+  // chunk on (nothing, for a row outside the image: zeros).  Everything that varies per load is
+  // scalar; the lane offset is one register for all loads (an offset formed per load lands in
+  // the registers the load is about to write, and the wait for that write drains the queue of
+  // loads before it).  NPL chunks per lane are in flight at a time.
+  TPUHIP_TS(13);
+  {
+    const int cshift = lgc - 4;
+    const int row_bytes = a.iw << lgc;
+    const int kpr = (row_bytes + 1023) >> 10;
+    const int total_rows = imgs * th2;
+    // the border positions
+    for (int q = tid; q < (total_rows << (cshift + 1)); q += NT) {
+      const int row = q >> (cshift + 1), side = (q >> cshift) & 1, cc = q & ((1 << cshift) - 1);
+      *reinterpret_cast<v4i *>(patch + row * rowb + (side ? (pw - 1) * prow : 0) + cc * 16) = v4i{0, 0, 0, 0};
+    }
+    uint32_t lane16 = (uint32_t)lane * 16u;
+    asm volatile("" : "+v"(lane16));
+    const int lds_lane = lane * 16 + prow;
+    // scalar state of the walk: patch row, chunk group, the row's offset in x (or -1: no such row)
+    auto row_offset = [&](int pr) {
+      const int il = (int)(((uint32_t)pr * a.magic_pw) >> 16);      // pr / th2
+      const int row = r0 - 1 + (pr - il * th2);
+      const int img = img0 + il;
+      const bool rowok = img < a.n && (unsigned)row < (unsigned)a.ih;
+      return rowok ? ((img * a.ih + row) * a.iw) << lgc : -1;
+    };
+    int pr = wave, k = 0;
+    while (pr < total_rows) {
+      const int pr_first = pr, k_first = k;
+      int xoff = row_offset(pr);
+      v4i preg[NPL];
+#pragma unroll
+      for (int u = 0; u < NPL; ++u) {
+        if (pr < total_rows) {
+          const bool ok = xoff >= 0;
+          const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+              (void *)(a.x + (ok ? (uint32_t)xoff + (uint32_t)(k << 10) : 0u)), 0, ok ? row_bytes - (k << 10) : 0, 0x00020000);
+          preg[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(rs, lane16, 0, 0);
+          if (++k == kpr) {
+            k = 0; pr += NWAVES;
+            xoff = row_offset(pr);
+          }
+        }
+      }
+      pr = pr_first; k = k_first;
+#ifdef TPUHIP_TRACE
+      if (pr_first == wave) TPUHIP_TS(14);
+#endif
+#pragma unroll
+      for (int u = 0; u < NPL; ++u) {
+        if (pr < total_rows) {
+          const int p = lane + (k << 6);
+          if (p < (a.iw << cshift))
+            *reinterpret_cast<v4i *>(patch + pr * rowb + (k << 10) + lds_lane + ((p >> cshift) << 4)) = preg[u];
+#ifdef TPUHIP_TRACE
+          if (pr_first == wave && u == 0) TPUHIP_TS(15);
+          if (pr_first == wave && u == 7) TPUHIP_TS(16);
+#endif
+          if (++k == kpr) { k = 0; pr += NWAVES; }
+        }
+      }
+    }
+  }
+
+  if (tid < BM) {
+    qlds[2 * tid] = qv[0];
+    qlds[2 * tid + 1] = qv[1];
+    qlds[2 * BM + tid] = qv[2];
+    qlds[3 * BM + tid] = qv[3] - (relu ? 1 : 0);
+    qlds[4 * BM + tid] = qv[4];
+  }
+  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
+
+  const int frow = lane & 31;
+  const int fk = lane >> 5;
+  // lane bases of the B fragment reads: pixel slot p of the tile -> its patch position
+  int bbase[NB2];
+  const int ohow = a.oh * a.ow;
+#pragma unroll
+  for (int j = 0; j < NB2; ++j) {
+    const int p = (pg * NB2 + j) * 32 + frow;
+    const int il = imgs > 1 ? (int)__umulhi((uint32_t)p, a.magic_oh) : 0;   // p / (H * W)
+    const int rem = p - il * ohow;
+    const uint32_t pr = a.ow == 1 ? (uint32_t)rem : __umulhi((uint32_t)rem, a.magic_ow);
+    const int pc = rem - (int)pr * a.ow;
+    bbase[j] = (p < npx ? (il * th2 + (int)pr) * rowb + pc * prow : 0) + fk * 16;   // idle slots read position 0
+  }
+  TPUHIP_TS(1);
+  __syncthreads();   // the patch and the parameters are in place
+  TPUHIP_TS(2);
+
+  v16i acc[NB2];
+#pragma unroll
+  for (int j = 0; j < NB2; ++j)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+
+  // The wave's slices advance by 128 bytes of K: the channel offset c0 within the tap and the
+  // tap's patch offset are kept as scalars (taps past the ninth -- one read ahead of the last
+  // slice -- stay on the ninth)
+  int c0 = (kg * 32) & (C - 1), tap = (kg * 32) >> lgc;
+  int tw = tap - 3 * ((tap * 11) >> 5);
+  int tapoff = ((tap * 11) >> 5) * rowb + tw * prow;
+  v4i bf[2][NB2];
+  auto read_B = [&](int fs) {
+    const int boff = tapoff + c0;
+#pragma unroll
+    for (int j = 0; j < NB2; ++j) bf[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
+    c0 += 128;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      if (c0 >= C) {
+        c0 -= C;
+        if (tap < 8) {
+          ++tap;
+          if (++tw == 3) { tw = 0; tapoff += rowb - 2 * prow; } else tapoff += prow;
+        }
+      }
+    }
+  };
+  if (trips > 0) read_B(0);
+  // Whole rounds of U trips run without a branch inside: every trip consumes the fragment
+  // requested U trips earlier and requests one, so the wait before a trip counts loads instead
+  // of draining the queue.  The last trips (fewer than U) take what is already in registers.
+  int i0 = 0;
+  for (; i0 + U <= trips; i0 += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#ifdef TPUHIP_TRACE
+      if (i0 == 0) ts[3 + u] = (unsigned long long)clock64();
+#endif
+      read_B((u + 1) & 1);
+      const v4i afr = af[u];
+      af[u] = load_A(i0 + u + U);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int j = 0; j < NB2; ++j)
+        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr, bf[u & 1][j], acc[j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U - 1; ++u) {
+    if (i0 + u >= trips) break;
+    read_B((u + 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < NB2; ++j)
+      acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u], bf[u & 1][j], acc[j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  TPUHIP_TS(27);
+  // ---- the four partial sums of every block meet at the block's owner, K group j & 3
+  const OutRoute out{a.y, a.y_cs, a.lo, 0};
+  v4i sv[flush_chunks<BM, BN, NT>()];
+  flush_prefetch<BM, BN, NT>(a, tid, pix_base, pix_limit, oc0, out, sv);
+  __syncthreads();   // every wave is done with the patch
+  v4i *const red = reinterpret_cast<v4i *>(patch) + pg * (NB2 * 3 * 4 * 64);   // [block][3 guests][4 quads][64 lanes]
+#pragma unroll
+  for (int j = 0; j < NB2; ++j) {
+    if ((j & 3) != kg && j < nb) {
+      const int slot = (kg - (j & 3) - 1) & 3;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        red[((j * 3 + slot) * 4 + q) * 64 + lane] = v4i{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NB2; ++j) {
+    if ((j & 3) == kg && j < nb) {
+#pragma unroll
+      for (int slot = 0; slot < 3; ++slot)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4i v = red[((j * 3 + slot) * 4 + q) * 64 + lane];
+          acc[j][q * 4] += v[0]; acc[j][q * 4 + 1] += v[1]; acc[j][q * 4 + 2] += v[2]; acc[j][q * 4 + 3] += v[3];
+        }
+    }
+  }
+  __syncthreads();   // the partial sums are read: their space takes the staged tile
+  TPUHIP_TS(28);
+
+  // ---- requantisation into the staging area, then out in memory order
+  int8_t *const stage = patch;
+  const int lc = fk * 16;
+#pragma unroll
+  for (int j = 0; j < NB2; ++j) {
+    if ((j & 3) == kg && j < nb) {
+      const v16i one[1] = {acc[j]};
+      uint32_t outw[1][4];
+      if (relu)
+        requant_rows_c64<1, true>(one, 0, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
+      else
+        requant_rows_c64<1, false>(one, a.lo, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
+      *reinterpret_cast<v4i *>(stage + ((pg * NB2 + j) * 32 + frow) * stage_row_bytes<BM>() + lc) =
+          v4i{(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+    }
+  }
   __syncthreads();
   TPUHIP_TS(29);
   flush_tile<BM, BN, NT>(a, stage, tid, pix_base, pix_limit, oc0, out, lut, sv);
@@ -2902,8 +3257,9 @@ struct TileCfg {
   int reg;   // 0: LDS kernel, one tile per workgroup; 1: the LDS-free kernel, bm x bn is the
              // tile of one wave; 2: its split-K form; 3: LDS kernel, persistent workgroups;
              // 4: patch kernel (bn = pixel slots of a tile of whole rows); 5: pointwise kernel;
-             // 6: patch kernel, second form
+             // 6: patch kernel, second form; 7: patch kernel, third form
   int bk;    // K bytes per step (pointwise kernel: the padded K it holds)
+  int nb = 2;   // second form of the patch kernel: filter tiles it keeps in LDS
 };
 
 // The tile variants, in the order of their public index (conv desc algo = 16 + index).
@@ -2958,17 +3314,30 @@ struct TileCfg {
 // row-patch kernels, second form (3x3 / stride 1 / pad 1, 64 to 1024 input channels, a power of two):
 // V(index, name, BM, BN, WM, WN, BK, waves per SIMD)
 #define TPUHIP_PATCH2_TILES(V)                          \
-  V(31, "mfma_patch2_64x256", 64, 256, 1, 4, 256, 2)    \
-  V(32, "mfma_patch2_64x128", 64, 128, 2, 2, 256, 2)    \
-  V(33, "mfma_patch2_128x128", 128, 128, 2, 2, 128, 2)  \
-  V(34, "mfma_patch2_64x64", 64, 64, 2, 2, 256, 2)      \
-  V(35, "mfma_patch2_128x256", 128, 256, 2, 2, 128, 1)  \
-  V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4) \
-  V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4) \
-  V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4) \
-  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2) \
-  V(45, "mfma_patch2_32x256_w8", 32, 256, 1, 8, 256, 4) \
-  V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2)
+  V(31, "mfma_patch2_64x256", 64, 256, 1, 4, 256, 2, 2)    \
+  V(32, "mfma_patch2_64x128", 64, 128, 2, 2, 256, 2, 2)    \
+  V(33, "mfma_patch2_128x128", 128, 128, 2, 2, 128, 2, 2)  \
+  V(34, "mfma_patch2_64x64", 64, 64, 2, 2, 256, 2, 2)      \
+  V(35, "mfma_patch2_128x256", 128, 256, 2, 2, 128, 1, 2)  \
+  V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4, 2) \
+  V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4, 2) \
+  V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4, 2) \
+  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2, 2) \
+  V(45, "mfma_patch2_32x256_w8", 32, 256, 1, 8, 256, 4, 2) \
+  V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2, 2) \
+  V(47, "mfma_patch2_64x128_w8_b3", 64, 128, 2, 4, 256, 4, 3) \
+  V(48, "mfma_patch2_64x256_w8_b3", 64, 256, 2, 4, 256, 4, 3) \
+  V(49, "mfma_patch2_128x256_w8_b3", 128, 256, 4, 2, 128, 2, 3) \
+  V(50, "mfma_patch2_64x128_b3", 64, 128, 2, 2, 256, 2, 3)
+
+// row-patch kernels, third form (3x3 / stride 1 / pad 1, the four waves split K, 32 channels per
+// workgroup): U(index, name, pixel blocks of a tile)
+#define TPUHIP_PATCH3_TILES(U3)               \
+  U3(51, "mfma_patch3_32x128", 4, 1)          \
+  U3(52, "mfma_patch3_32x224", 7, 1)          \
+  U3(53, "mfma_patch3_32x256", 8, 1)          \
+  U3(54, "mfma_patch3_32x128_w8", 2, 2)       \
+  U3(55, "mfma_patch3_32x256_w8", 4, 2)
 
 struct TileTable {
   TileCfg t[64];
@@ -2994,11 +3363,16 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_PW_TILES(W)
 #undef W
-#define V(i, name, BM, BN, WM, WN, BK, O) \
-  t[i] = TileCfg{BM, BN, WM, WN, name, 6, BK}; \
+#define V(i, name, BM, BN, WM, WN, BK, O, NB) \
+  t[i] = TileCfg{BM, BN, WM, WN, name, 6, BK, NB}; \
   n = n > i ? n : i + 1;
     TPUHIP_PATCH2_TILES(V)
 #undef V
+#define U3(i, name, NB2, PW) \
+  t[i] = TileCfg{32, NB2 * PW * 32, 1, PW, name, 7, 64}; \
+  n = n > i ? n : i + 1;
+    TPUHIP_PATCH3_TILES(U3)
+#undef U3
   }
 };
 const TileTable kTileTable;
@@ -3092,7 +3466,7 @@ constexpr int kPatch2MaxChunks = 18 * 256;     // 16-byte input chunks a workgro
 constexpr int kLdsBytes = 160 * 1024;
 
 inline unsigned patch2_lds_bytes(const TileCfg &c, int th, int ow, int ic) {
-  return (unsigned)(5 * c.bm * 4 + 256 + 2 * c.bm * (c.bk + 16) + (th + 2) * ((ow + 2) * (ic + 16) + kPatch2RowPad));
+  return (unsigned)(5 * c.bm * 4 + 256 + c.nb * c.bm * (c.bk + 16) + (th + 2) * ((ow + 2) * (ic + 16) + kPatch2RowPad));
 }
 
 // rows of one image a tile holds; 0: the layer does not fit this kernel
@@ -3113,9 +3487,9 @@ int patch2_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
 
 void launch_patch2(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsigned lds) {
   switch (tile) {
-#define V(i, name, BM, BN, WM, WN, BK, O)                                                               \
+#define V(i, name, BM, BN, WM, WN, BK, O, NB)                                                           \
   case i: {                                                                                             \
-    auto kernel = conv_patch2_kernel<BM, BN, WM, WN, BK, O>;                                            \
+    auto kernel = conv_patch2_kernel<BM, BN, WM, WN, BK, O, NB>;                                          \
     if (!pw_prepare(kernel, (unsigned)kLdsBytes)) break;                                                \
     if (ctx->prof_start)                                                                                \
       hipExtLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
@@ -3124,6 +3498,62 @@ void launch_patch2(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsi
   } break;
     TPUHIP_PATCH2_TILES(V)
 #undef V
+  }
+}
+
+// ---- row-patch kernels, third form
+struct Patch3Plan {
+  int th = 0;      // rows of a tile (0: the layer does not fit this kernel)
+  int imgs = 1;    // whole images per tile
+  unsigned lds = 0;
+};
+
+Patch3Plan patch3_plan(const tpuhip_conv_desc &d, const TileCfg &c) {
+  Patch3Plan pl;
+  const bool shape_ok = d.g == 1 && d.kh == 3 && d.kw == 3 && d.sh == 1 && d.sw == 1 && d.dh == 1 && d.dw == 1 &&
+                        d.pt == 1 && d.pb == 1 && d.pl == 1 && d.pr == 1 && !d.ins_h && !d.ins_w && !d.relu_first &&
+                        d.oh == d.ih && d.ow == d.iw && d.x_cs == d.ic && d.ic >= 64 && d.ic <= 1024 &&
+                        (d.ic & (d.ic - 1)) == 0;
+  if (!shape_ok || d.ow > c.bn) return pl;
+  const int nblk = c.bn / 32;
+  auto lds_bytes = [&](int th, int imgs) {
+    const int64_t patch = (int64_t)imgs * (th + 2) * ((d.ow + 2) * (d.ic + 16) + kPatch2RowPad);
+    const int64_t red = (int64_t)nblk * 3 * 4096, stage = (int64_t)c.bn * 48;
+    return (int64_t)(5 * 32 * 4 + 256) + std::max(patch, std::max(red, stage));
+  };
+  int imgs = std::min(d.n, c.bn / (d.oh * d.ow));
+  while (imgs > 1 && lds_bytes(d.oh, imgs) > kLdsBytes) --imgs;
+  if (imgs > 1) {
+    // whole images: evened out over the batch
+    const int tiles = (d.n + imgs - 1) / imgs;
+    pl.imgs = (d.n + tiles - 1) / tiles;
+    pl.th = d.oh;
+  } else {
+    int th = std::min(c.bn / d.ow, d.oh);
+    while (th >= 1 && lds_bytes(th, 1) > kLdsBytes) --th;
+    if (th < 1) return pl;
+    const int tiles = (d.oh + th - 1) / th;      // evened out over the image
+    pl.th = (d.oh + tiles - 1) / tiles;
+  }
+  // the kernel's small divisions: patch row / (th + 2) and pixel slot / (oh * ow)
+  if (pl.imgs * (pl.th + 2) * (pl.th + 2) >= 65536) return Patch3Plan{};
+  pl.lds = (unsigned)lds_bytes(pl.th, pl.imgs);
+  return pl;
+}
+
+void launch_patch3(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsigned lds) {
+  switch (tile) {
+#define U3(i, name, NB2, PW)                                                                            \
+  case i: {                                                                                             \
+    auto kernel = conv_patch3_kernel<NB2, PW>;                                                          \
+    if (!pw_prepare(kernel, (unsigned)kLdsBytes)) break;                                                \
+    if (ctx->prof_start)                                                                                \
+      hipExtLaunchKernelGGL(kernel, grid, dim3(256 * PW), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
+    else                                                                                                \
+      hipLaunchKernelGGL(kernel, grid, dim3(256 * PW), lds, ctx->stream, a);                            \
+  } break;
+    TPUHIP_PATCH3_TILES(U3)
+#undef U3
   }
 }
 
@@ -3302,7 +3732,7 @@ int pack_mfma_weights(tpuhip_ctx *ctx, tpuhip_conv_weights *cw, int tile) {
 
 // the fused table lives in the LDS of the LDS kernels
 bool tile_has_lds_epilogue(int t) {
-  return kTiles[t].reg == 0 || kTiles[t].reg == 3 || kTiles[t].reg == 5 || kTiles[t].reg == 6;
+  return kTiles[t].reg == 0 || kTiles[t].reg == 3 || kTiles[t].reg == 5 || kTiles[t].reg == 6 || kTiles[t].reg == 7;
 }
 
 // the pointwise kernels: 1x1 window, no padding, no dilation (any stride), the input channels
@@ -3333,6 +3763,7 @@ bool tile_is_candidate(const tpuhip_conv_desc &d, int t) {
   if (c.reg == 4 && patch_rows(d, c) == 0) return false;
   if (c.reg == 5 && !pw_shape_ok(d, c)) return false;
   if (c.reg == 6 && patch2_rows(d, c) == 0) return false;
+  if (c.reg == 7) return patch3_plan(d, c).th > 0;
   if (d.ic <= 4 && (c.reg == 1 || c.reg == 2)) return false;   // prefer the 4-channel K packing of the LDS kernels
   return !(c.bm > 32 && c.bm / 2 >= round_up(d.oc, 32));   // more than half the rows idle
 }
@@ -3408,6 +3839,26 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
         a.pstep_ow = (int)patch2_lds_bytes(t, th, d.ow, d.ic);                   // dynamic LDS of the launch
       }
     }
+    if (t.reg == 7) {
+      const Patch3Plan pl = patch3_plan(d, t);
+      const int tiles_per_img = (d.oh + pl.th - 1) / pl.th;
+      const int n_pix_tiles = pl.imgs > 1 ? (d.n + pl.imgs - 1) / pl.imgs : d.n * tiles_per_img;
+      a.n_tiles = n_pix_tiles * a.n_oc_tiles;
+      a.tiles_per_xcd = (n_pix_tiles + 7) / 8 * a.n_oc_tiles;
+      a.wgs_per_xcd = a.tiles_per_xcd;
+      a.stem_pw = d.ow + 2;
+      a.pstep_pix = pl.th;
+      a.pstep_n = tiles_per_img;
+      a.tile_imgs = pl.imgs;
+      int lgc = 6;
+      while ((1 << lgc) < d.ic) ++lgc;
+      a.pstep_oh = lgc;                                                          // log2(C)
+      const uint32_t rowchunks = (uint32_t)a.stem_pw * (uint32_t)(d.ic / 16);
+      a.magic_c16 = (uint32_t)(((1ull << 32) + rowchunks - 1) / rowchunks);      // q / rowchunks == umulhi(q, magic), q < 2^16
+      a.magic_pw = 65536u / (uint32_t)(pl.th + 2) + 1;                           // patch row / (th + 2)
+      a.magic_oh = (uint32_t)(((1ull << 32) + (uint64_t)(d.oh * d.ow) - 1) / (uint64_t)(d.oh * d.ow));
+      a.pstep_ow = (int)pl.lds;                                                  // dynamic LDS of the launch
+    }
     if (t.reg == 3 || t.reg == 5) {
       // every XCD owns a run of whole pixel tiles; a workgroup keeps its channel tile
       const int n_pix_tiles = a.n_tiles / a.n_oc_tiles;
@@ -3434,6 +3885,10 @@ void launch_conv_mfma(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const ConvA
   }
   if (kTiles[w->tile].reg == 6) {
     launch_patch2(ctx, w->tile, grid, a, (unsigned)a.pstep_ow);
+    return;
+  }
+  if (kTiles[w->tile].reg == 7) {
+    launch_patch3(ctx, w->tile, grid, a, (unsigned)a.pstep_ow);
     return;
   }
   const bool uni = (w->c16 % (tile_bk(kTiles[w->tile]) / 16)) == 0;
@@ -3548,7 +4003,7 @@ int autotune_mfma(tpuhip_ctx *ctx, tpuhip_conv_weights *w, const void *x, void *
     if (post.lut && !tile_has_lds_epilogue(t)) continue;
     if (w->split_oc && kTiles[t].reg == 4) continue;   // the patch kernel writes one result
     if (kTiles[t].reg == 5 && (!w->fast || w->split_oc % kTiles[t].bm)) continue;
-    if (kTiles[t].reg == 6 && (!w->fast || w->split_oc)) continue;
+    if ((kTiles[t].reg == 6 || kTiles[t].reg == 7) && (!w->fast || w->split_oc)) continue;
     rc = pack_mfma_weights(ctx, w, t);
     if (rc) break;
     ConvArgs a;
@@ -3904,6 +4359,11 @@ static int run_conv(tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *x
                  "conv: tile variant %s needs an unpadded 1x1 conv with 5 to %d input channels, right shifts of at "
                  "least 1 and sums that cannot overflow the rounding, and a pair split at a tile boundary",
                  kTiles[w->tile].name, kTiles[w->tile].bk);
+  TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 7) ||
+                     (!w->split_oc && w->fast && patch3_plan(w->d, kTiles[w->tile]).th > 0),
+                 "conv: tile variant %s needs a single 3x3 / stride 1 / pad 1 conv with 64, 128, 256, 512 or 1024 input "
+                 "channels on a map narrow enough for its row patch, right shifts of at least 1 and sums that cannot "
+                 "overflow the rounding", kTiles[w->tile].name);
   TPUHIP_REQUIRE(!(w->algo == ALGO_MFMA && kTiles[w->tile].reg == 6) ||
                      (!w->split_oc && w->fast && patch2_rows(w->d, kTiles[w->tile]) > 0),
                  "conv: tile variant %s needs a single 3x3 / stride 1 / pad 1 conv with 64, 128, 256, 512 or 1024 input "
