@@ -605,10 +605,11 @@ conv_mfma_kernel(ConvArgs a) {
   const __amdgpu_buffer_rsrc_t wrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
 
-  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  // the fused table and the requant parameters of the channel tile: fetched now, parked in LDS
+  // after the first tile loads have been issued (their latencies overlap instead of adding up)
+  uint32_t lutv = 0;
+  if (a.has_lut && tid < 64) lutv = a.lut.w[tid];
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
-  // requant parameters of the channel tile: fetched now, parked in LDS after the first
-  // tile loads have been issued (their latencies overlap instead of adding up)
   static_assert(!PERSIST || BM <= NT, "one parameter row per thread");
   int32_t qv[4] = {0, 0, 0, 0};
   if (PERSIST && tid < BM) {
@@ -805,6 +806,7 @@ conv_mfma_kernel(ConvArgs a) {
 
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) load_tile(d, d);
+  if (a.has_lut && tid < 64) lutw[tid] = lutv;   // (published by the first barrier of the K loop at the latest)
   if (PERSIST) {
     if (tid < BM) {
       qlds[tid] = qv[0];
@@ -1181,6 +1183,7 @@ conv_pw_kernel(ConvArgs a) {
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
   static_assert(KP == 64 || KP == 128 || KP == 256, "padded K");
+  static_assert(BM >= 64, "the threads that fetch the parameters also fetch the 64 table words");
   constexpr int KC = KP / 64;              // 64-byte K chunks
   constexpr int CPRK = KP / 16;            // 16-byte chunks of a pixel row
   constexpr int RPP = NT / CPRK;           // pixel rows per pass of the loader
@@ -1282,14 +1285,16 @@ conv_pw_kernel(ConvArgs a) {
       // all five in flight before the first is used (one trip to memory, not two)
       const int32_t c_lo = c64[2 * (oc0 + tid)], c_hi = c64[2 * (oc0 + tid) + 1];
       const int32_t qm = a.qmult[oc0 + tid], qs = a.qshift[oc0 + tid], qh = a.qhpot[oc0 + tid];
+      uint32_t lutv = 0;
+      if (a.has_lut && tid < 64) lutv = a.lut.w[tid];   // BM >= 64: these threads cover the table
       __builtin_amdgcn_sched_barrier(0);
+      if (a.has_lut && tid < 64) lutw[tid] = lutv;
       qlds[2 * tid] = c_lo;
       qlds[2 * tid + 1] = c_hi;
       qlds[2 * BM + tid] = qm;
       qlds[3 * BM + tid] = qs - (out.lo == 0 ? 1 : 0);
       qlds[4 * BM + tid] = qh;
     }
-    if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
 #pragma unroll
     for (int u = 0; u < NWC; ++u)
       if (WCH % NT == 0 || tid + u * NT < WCH) wA[tid + u * NT] = wreg[u];
