@@ -1421,7 +1421,7 @@ conv_pw_kernel(ConvArgs a) {
 // 2 * (C + 16) + kPatch2RowPad is a multiple of 128 for every C that is a multiple of 64
 constexpr int kPatch2RowPad = 96;
 
-template <int BM, int BN, int WM, int WN, int BK, int OCC, int NB>
+template <int BM, int BN, int WM, int WN, int BK, int OCC>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void
 conv_patch2_kernel(ConvArgs a) {
 #ifdef TPUHIP_TRACE
@@ -1431,6 +1431,7 @@ conv_patch2_kernel(ConvArgs a) {
   gather_conv_args(a);
   gather_conv_args_more(a);
   constexpr int NT = WM * WN * 64;
+  constexpr int RD = 4;                       // filter tiles in flight in registers (even)
   constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
   static_assert((WM * WN == 4 || WM * WN == 8) && TM >= 1 && TN >= 1 && TM * WM * 32 == BM && TN * WN * 32 == BN, "bad tile");
   static_assert(BK == 128 || BK == 256, "K bytes per step");
@@ -1438,18 +1439,14 @@ conv_patch2_kernel(ConvArgs a) {
   constexpr int ABYTES = BM * AROW;
   constexpr int CPA = BK / 16;                // 16-byte chunks of a filter tile row
   constexpr int NW = BM * CPA / NT;           // filter chunks per thread per step
-  // filter tiles in flight in registers (even).  With three LDS tiles a tile is parked two steps
-  // before its step, so it stays in registers for RD - 2 steps only
-  constexpr int RD = NB == 3 && NW <= 2 ? 6 : 4;
-  static_assert(NB == 2 || NB == 3, "LDS filter tiles");
   constexpr int KK = BK / 32;
   constexpr int NPL = 18 * 256 / NT;          // patch chunks per thread at most (72 KiB of input)
-  static_assert(BN * stage_row_bytes<BM>() <= NB * ABYTES, "the staged tile must fit the filter tiles");
+  static_assert(BN * stage_row_bytes<BM>() <= 2 * ABYTES, "the staged tile must fit the filter tiles");
   extern __shared__ __attribute__((aligned(16))) v4i p2_smem[];
   int32_t *const qlds = reinterpret_cast<int32_t *>(p2_smem);                 // 5 * BM dwords
   uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);         // 64 dwords
-  int8_t *const abuf = reinterpret_cast<int8_t *>(lutw + 64);                 // NB * ABYTES
-  int8_t *const patch = abuf + NB * ABYTES;
+  int8_t *const abuf = reinterpret_cast<int8_t *>(lutw + 64);                 // 2 * ABYTES
+  int8_t *const patch = abuf + 2 * ABYTES;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1556,7 +1553,7 @@ conv_patch2_kernel(ConvArgs a) {
     bbase[j] = (p < rows * a.ow ? (int)pr * rowb + pc * prow : 0) + fk * 16;   // idle slots read position 0
   }
 
-  // park the patch and the first filter tile (with three LDS tiles, the first two)
+  // park the patch and the first filter tile
 #pragma unroll
   for (int u = 0; u < NPL; ++u) {
     const int q = tid + u * NT;
@@ -1567,7 +1564,6 @@ conv_patch2_kernel(ConvArgs a) {
   }
   TPUHIP_TS(1);
   store_A(0, 0);
-  if (NB == 3) store_A(1, 1);
   __syncthreads();
   TPUHIP_TS(2);
 
@@ -1586,53 +1582,40 @@ conv_patch2_kernel(ConvArgs a) {
         for (int e = 0; e < 16; ++e) accs[c][i][j][e] = 0;
   v16i (&acc)[TM][TN] = accs[0];
 
-  // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS
-  // earlier -- and receives the tile RD steps ahead.  Within the step the operands of a 32-byte K
-  // slice are requested PD slices before their MFMAs (see frag_prefetch).
-  // Two LDS tiles: the next step's tile goes from its slot to the other LDS tile at the end of
-  // the step, and the step after the barrier starts by requesting its first operands.
-  // Three LDS tiles: the tile TWO steps ahead is parked at the end of the step, so the next
-  // step's tile has been visible since the previous barrier and the next step's first operands
-  // are requested BEFORE the barrier: the MFMAs resume right behind it instead of an LDS round
-  // trip later.
+  // One K step; its register slot (compile-time, step % RD) is free -- its tile went to LDS a
+  // step ago -- and receives the tile RD steps ahead; the next step's tile goes from its slot
+  // to the other LDS tile.  Within the step the operands of a 32-byte K slice are requested PD
+  // slices before their MFMAs (see frag_prefetch).
   constexpr int PD = OCC >= 4 ? 1 : frag_prefetch(TM * TN);
-  v4i fa[PD + 1][TM], fb[PD + 1][TN];
-  // operands of 32-byte slice kk of K step s, whose filter tile lies at LDS offset aoff
-  auto read_slice = [&](int s, int aoff, int kk, int fs) {
-    // the slice lies in one filter tap (C is a multiple of 64); slices past the ninth tap
-    // meet zero weights and read the last tap
-    const int koff = s * BK + kk * 32;
-    const int tap = min(koff >> lgc, 8);
-    const int tkh = (tap * 11) >> 5;
-    const int boff = tkh * rowb + (tap - 3 * tkh) * prow + (koff & (C - 1));
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(abuf + aoff + abase[i] + kk * 32);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
-  };
-  int cur = 0;   // LDS offset of the running step's filter tile (three tiles: rotates at run time)
-  if (NB == 3) {
-#pragma unroll
-    for (int kk = 0; kk < PD; ++kk) read_slice(0, 0, kk, kk % (PD + 1));
-  }
   auto step = [&](int s, auto slotc) {
-    constexpr int slot = decltype(slotc)::value;
+    constexpr int slot = decltype(slotc)::value, buf = slot & 1;
 #ifdef TPUHIP_TRACE
     const bool tr = s < 4;
-    if (tr) TPUHIP_TS(3 + (slot & 3) * 6);
+    if (tr) TPUHIP_TS(3 + slot * 6);
 #endif
     load_A(slot, s + RD);
-    const int aoff = NB == 3 ? cur : (slot & 1) * ABYTES;
+    const int8_t *ab = abuf + buf * ABYTES;
+    v4i fa[PD + 1][TM], fb[PD + 1][TN];
+    auto read_slice = [&](int kk, int fs) {
+      // the slice lies in one filter tap (C is a multiple of 64); slices past the ninth tap
+      // meet zero weights and read the last tap
+      const int koff = s * BK + kk * 32;
+      const int tap = min(koff >> lgc, 8);
+      const int tkh = (tap * 11) >> 5;
+      const int boff = tkh * rowb + (tap - 3 * tkh) * prow + (koff & (C - 1));
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[fs][i] = *reinterpret_cast<const v4i *>(ab + abase[i] + kk * 32);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[fs][j] = *reinterpret_cast<const v4i *>(patch + bbase[j] + boff);
+    };
     // K is padded to whole steps with zero weights: the slices of the last step that lie in
     // the padding are not multiplied (kreal: slices of this step that hold weights)
     const int kreal = min(KK, (a.k16 * 16 - s * BK + 31) >> 5);
-    if (NB == 2) {
 #pragma unroll
-      for (int kk = 0; kk < PD; ++kk) read_slice(s, aoff, kk, kk % (PD + 1));
-    }
+    for (int kk = 0; kk < PD; ++kk) read_slice(kk, kk);
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
-      if (kk + PD < KK) read_slice(s, aoff, kk + PD, (kk + PD) % (PD + 1));
+      if (kk + PD < KK) read_slice(kk + PD, (kk + PD) % (PD + 1));
       __builtin_amdgcn_sched_barrier(0);
       if (kk < kreal) {
 #pragma unroll
@@ -1644,32 +1627,18 @@ conv_patch2_kernel(ConvArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
 #ifdef TPUHIP_TRACE
-      if (tr && kk == 0) TPUHIP_TS(4 + (slot & 3) * 6);
-      if (tr && kk == 3) TPUHIP_TS(5 + (slot & 3) * 6);
-      if (tr && kk == KK - 1) TPUHIP_TS(6 + (slot & 3) * 6);
+      if (tr && kk == 0) TPUHIP_TS(4 + slot * 6);
+      if (tr && kk == 3) TPUHIP_TS(5 + slot * 6);
+      if (tr && kk == KK - 1) TPUHIP_TS(6 + slot * 6);
 #endif
     }
-    if (NB == 3) {
-      const int nxt = cur == 2 * ABYTES ? 0 : cur + ABYTES;
-      const int nn = nxt == 2 * ABYTES ? 0 : nxt + ABYTES;
-#pragma unroll
-      for (int kk = 0; kk < PD; ++kk) read_slice(s + 1, nxt, kk, kk % (PD + 1));   // (past the last step: unused)
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int u = 0; u < NW; ++u) {
-        const int q = tid + u * NT;
-        *reinterpret_cast<v4i *>(abuf + nn + (q / CPA) * AROW + (q % CPA) * 16) = wr[(slot + 2) % RD][u];
-      }
-      cur = nxt;
-    } else {
-      store_A((slot + 1) % RD, (slot & 1) ^ 1);   // (past the last step: zeros, into a tile nobody reads)
-    }
+    store_A((slot + 1) % RD, buf ^ 1);   // (past the last step: zeros, into a tile nobody reads)
 #ifdef TPUHIP_TRACE
-    if (tr) TPUHIP_TS(7 + (slot & 3) * 6);
+    if (tr) TPUHIP_TS(7 + slot * 6);
 #endif
     __syncthreads();
 #ifdef TPUHIP_TRACE
-    if (tr) TPUHIP_TS(8 + (slot & 3) * 6);
+    if (tr) TPUHIP_TS(8 + slot * 6);
 #endif
   };
   for (int s = 0; s < nsteps; s += RD) {
@@ -1677,10 +1646,6 @@ conv_patch2_kernel(ConvArgs a) {
     if (s + 1 < nsteps) step(s + 1, std::integral_constant<int, 1>{});
     if (s + 2 < nsteps) step(s + 2, std::integral_constant<int, 2>{});
     if (s + 3 < nsteps) step(s + 3, std::integral_constant<int, 3>{});
-    if constexpr (RD == 6) {
-      if (s + 4 < nsteps) step(s + 4, std::integral_constant<int, 4>{});
-      if (s + 5 < nsteps) step(s + 5, std::integral_constant<int, 5>{});
-    }
   }
 
   TPUHIP_TS(27);
@@ -3264,7 +3229,6 @@ struct TileCfg {
              // 4: patch kernel (bn = pixel slots of a tile of whole rows); 5: pointwise kernel;
              // 6: patch kernel, second form; 7: patch kernel, third form
   int bk;    // K bytes per step (pointwise kernel: the padded K it holds)
-  int nb = 2;   // second form of the patch kernel: filter tiles it keeps in LDS
 };
 
 // The tile variants, in the order of their public index (conv desc algo = 16 + index).
@@ -3319,30 +3283,29 @@ struct TileCfg {
 // row-patch kernels, second form (3x3 / stride 1 / pad 1, 64 to 1024 input channels, a power of two):
 // V(index, name, BM, BN, WM, WN, BK, waves per SIMD)
 #define TPUHIP_PATCH2_TILES(V)                          \
-  V(31, "mfma_patch2_64x256", 64, 256, 1, 4, 256, 2, 2)    \
-  V(32, "mfma_patch2_64x128", 64, 128, 2, 2, 256, 2, 2)    \
-  V(33, "mfma_patch2_128x128", 128, 128, 2, 2, 128, 2, 2)  \
-  V(34, "mfma_patch2_64x64", 64, 64, 2, 2, 256, 2, 2)      \
-  V(35, "mfma_patch2_128x256", 128, 256, 2, 2, 128, 1, 2)  \
-  V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4, 2) \
-  V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4, 2) \
-  V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4, 2) \
-  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2, 2) \
-  V(45, "mfma_patch2_32x256_w8", 32, 256, 1, 8, 256, 4, 2) \
-  V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2, 2) \
-  V(47, "mfma_patch2_64x128_w8_b3", 64, 128, 2, 4, 256, 4, 3) \
-  V(48, "mfma_patch2_64x256_w8_b3", 64, 256, 2, 4, 256, 4, 3) \
-  V(49, "mfma_patch2_128x256_w8_b3", 128, 256, 4, 2, 128, 2, 3) \
-  V(50, "mfma_patch2_64x128_b3", 64, 128, 2, 2, 256, 2, 3)
+  V(31, "mfma_patch2_64x256", 64, 256, 1, 4, 256, 2)    \
+  V(32, "mfma_patch2_64x128", 64, 128, 2, 2, 256, 2)    \
+  V(33, "mfma_patch2_128x128", 128, 128, 2, 2, 128, 2)  \
+  V(34, "mfma_patch2_64x64", 64, 64, 2, 2, 256, 2)      \
+  V(35, "mfma_patch2_128x256", 128, 256, 2, 2, 128, 1)  \
+  V(41, "mfma_patch2_64x256_w8", 64, 256, 2, 4, 256, 4) \
+  V(42, "mfma_patch2_64x128_w8", 64, 128, 2, 4, 256, 4) \
+  V(43, "mfma_patch2_128x128_w8", 128, 128, 4, 2, 128, 4) \
+  V(44, "mfma_patch2_128x256_w8", 128, 256, 4, 2, 128, 2) \
+  V(45, "mfma_patch2_32x256_w8", 32, 256, 1, 8, 256, 4) \
+  V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2) \
+  V(47, "mfma_patch2_128x256_w8_k256", 128, 256, 4, 2, 256, 2) \
+  V(48, "mfma_patch2_128x256_w8t_k256", 128, 256, 2, 4, 256, 2) \
+  V(49, "mfma_patch2_128x256_w8t", 128, 256, 2, 4, 128, 2)
 
 // row-patch kernels, third form (3x3 / stride 1 / pad 1, the four waves split K, 32 channels per
 // workgroup): U(index, name, pixel blocks of a tile)
 #define TPUHIP_PATCH3_TILES(U3)               \
-  U3(51, "mfma_patch3_32x128", 4, 1)          \
-  U3(52, "mfma_patch3_32x224", 7, 1)          \
-  U3(53, "mfma_patch3_32x256", 8, 1)          \
-  U3(54, "mfma_patch3_32x128_w8", 2, 2)       \
-  U3(55, "mfma_patch3_32x256_w8", 4, 2)
+  U3(50, "mfma_patch3_32x128", 4, 1)          \
+  U3(51, "mfma_patch3_32x224", 7, 1)          \
+  U3(52, "mfma_patch3_32x256", 8, 1)          \
+  U3(53, "mfma_patch3_32x128_w8", 2, 2)       \
+  U3(54, "mfma_patch3_32x256_w8", 4, 2)
 
 struct TileTable {
   TileCfg t[64];
@@ -3368,8 +3331,8 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_PW_TILES(W)
 #undef W
-#define V(i, name, BM, BN, WM, WN, BK, O, NB) \
-  t[i] = TileCfg{BM, BN, WM, WN, name, 6, BK, NB}; \
+#define V(i, name, BM, BN, WM, WN, BK, O) \
+  t[i] = TileCfg{BM, BN, WM, WN, name, 6, BK}; \
   n = n > i ? n : i + 1;
     TPUHIP_PATCH2_TILES(V)
 #undef V
@@ -3471,7 +3434,7 @@ constexpr int kPatch2MaxChunks = 18 * 256;     // 16-byte input chunks a workgro
 constexpr int kLdsBytes = 160 * 1024;
 
 inline unsigned patch2_lds_bytes(const TileCfg &c, int th, int ow, int ic) {
-  return (unsigned)(5 * c.bm * 4 + 256 + c.nb * c.bm * (c.bk + 16) + (th + 2) * ((ow + 2) * (ic + 16) + kPatch2RowPad));
+  return (unsigned)(5 * c.bm * 4 + 256 + 2 * c.bm * (c.bk + 16) + (th + 2) * ((ow + 2) * (ic + 16) + kPatch2RowPad));
 }
 
 // rows of one image a tile holds; 0: the layer does not fit this kernel
@@ -3492,9 +3455,9 @@ int patch2_rows(const tpuhip_conv_desc &d, const TileCfg &c) {
 
 void launch_patch2(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsigned lds) {
   switch (tile) {
-#define V(i, name, BM, BN, WM, WN, BK, O, NB)                                                           \
+#define V(i, name, BM, BN, WM, WN, BK, O)                                                               \
   case i: {                                                                                             \
-    auto kernel = conv_patch2_kernel<BM, BN, WM, WN, BK, O, NB>;                                          \
+    auto kernel = conv_patch2_kernel<BM, BN, WM, WN, BK, O>;                                            \
     if (!pw_prepare(kernel, (unsigned)kLdsBytes)) break;                                                \
     if (ctx->prof_start)                                                                                \
       hipExtLaunchKernelGGL(kernel, grid, dim3(WM * WN * 64), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
