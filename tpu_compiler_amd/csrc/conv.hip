@@ -1706,8 +1706,8 @@ conv_patch2_kernel(ConvArgs a) {
 //     table and add included).
 //   a.stem_pw = W + 2, a.pstep_pix = TH (rows of a tile), a.pstep_n = tiles per image,
 //   a.tile_imgs = whole images per tile (1: a tile is TH rows of one image),
-//   a.pstep_oh = log2(C), a.magic_c16 = ceil(2^32 / chunks of a patch row),
-//   a.magic_pw = floor(2^16 / (TH + 2)) + 1, a.magic_oh = ceil(2^32 / (H * W)), a.pstep_ow = LDS bytes
+//   a.pstep_oh = log2(C), a.magic_c16 = ceil(2^32 / 16-byte chunks of an input row),
+//   a.magic_kw = ceil(2^32 / H), a.magic_oh = ceil(2^32 / (H * W)), a.pstep_ow = LDS bytes
 // LDS (dynamic): parameters | table | patch, then the partial sums, then the staged tile.
 // ---------------------------------------------------------------------------
 template <int NB2, int PW>
@@ -1721,7 +1721,7 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
   // 4 * PW waves: wave = pixel group * 4 + K group; a pixel group is NB2 blocks of 32 pixel slots
   constexpr int NT = 256 * PW, NWAVES = 4 * PW, BM = 32, BN = NB2 * PW * 32;
   constexpr int U = 8;     // A fragments in flight per wave (even)
-  constexpr int NPL = 16;  // patch chunks per thread and pass
+  constexpr int NPL = 16 / PW;  // pieces of the input span per wave and pass
   extern __shared__ __attribute__((aligned(16))) v4i p3_smem[];
   int32_t *const qlds = reinterpret_cast<int32_t *>(p3_smem);                 // 5 * BM dwords
   uint32_t *const lutw = reinterpret_cast<uint32_t *>(qlds + 5 * BM);         // 64 dwords
@@ -1789,71 +1789,64 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
 
   // ---- the patch.  Patch row pr (image pr / th2 of the tile, input row r0 - 1 + pr % th2) is pw
   // positions of C bytes; positions 1 .. W are the input row (W * C contiguous bytes), the
-  // first and last position and the rows outside the image are the zero border.  A wave takes
-  // rows wave, wave + NWAVES, ...; its lanes take 16-byte chunks lane, lane + 64, ... of the
-  // input row, through a descriptor that covers what is left of the row from the group's first
-  // chunk on (nothing, for a row outside the image: zeros).  Everything that varies per load is
-  // scalar; the lane offset is one register for all loads (an offset formed per load lands in
-  // the registers the load is about to write, and the wait for that write drains the queue of
-  // loads before it).  NPL chunks per lane are in flight at a time.
+  // first and last position and the rows outside the image are the zero border.  The input rows
+  // a tile needs are ONE contiguous span of x (consecutive rows of an image, consecutive whole
+  // images), so the span is fetched as a byte stream: wave w takes its 1 KB pieces w, w + NWAVES,
+  // ... through a descriptor that begins at the piece and ends with the span (a piece past the
+  // end: nothing), every lane 16 bytes at one fixed offset -- scalar work and no branch per
+  // load -- and each lane finds the patch position of its chunk (row = chunk / chunks of a row)
+  // when it parks it.  NPL pieces per wave are in flight at a time.  The whole patch is zeroed
+  // first (border positions, rows outside the image, images the last tile lacks).
   TPUHIP_TS(13);
   {
     const int cshift = lgc - 4;
-    const int row_bytes = a.iw << lgc;
-    const int kpr = (row_bytes + 1023) >> 10;
-    const int total_rows = imgs * th2;
-    // the border positions
-    for (int q = tid; q < (total_rows << (cshift + 1)); q += NT) {
-      const int row = q >> (cshift + 1), side = (q >> cshift) & 1, cc = q & ((1 << cshift) - 1);
-      *reinterpret_cast<v4i *>(patch + row * rowb + (side ? (pw - 1) * prow : 0) + cc * 16) = v4i{0, 0, 0, 0};
-    }
+    const int chunks_in = a.iw << cshift;                 // chunks of an input row
+    // first and last input row of the span (single image), or all rows of the tile's images
+    const int row_f = imgs > 1 ? 0 : max(r0 - 1, 0);
+    const int row_l = imgs > 1 ? nimg * a.ih - 1 : min(r0 + rows, a.ih - 1);
+    const int span_chunks = (row_l - row_f + 1) * chunks_in;
+    const int span_bytes = span_chunks << 4;
+    const int8_t *span = a.x + ((size_t)((img0 * a.ih + row_f) * a.iw) << lgc);
+    const int pieces = (span_bytes + 1023) >> 10;
     uint32_t lane16 = (uint32_t)lane * 16u;
     asm volatile("" : "+v"(lane16));
-    const int lds_lane = lane * 16 + prow;
-    // scalar state of the walk: patch row, chunk group, the row's offset in x (or -1: no such row)
-    auto row_offset = [&](int pr) {
-      const int il = (int)(((uint32_t)pr * a.magic_pw) >> 16);      // pr / th2
-      const int row = r0 - 1 + (pr - il * th2);
-      const int img = img0 + il;
-      const bool rowok = img < a.n && (unsigned)row < (unsigned)a.ih;
-      return rowok ? ((img * a.ih + row) * a.iw) << lgc : -1;
-    };
-    int pr = wave, k = 0;
-    while (pr < total_rows) {
-      const int pr_first = pr, k_first = k;
-      int xoff = row_offset(pr);
+    const int total_chunks = imgs * th2 * rowb >> 4;      // (rowb is a multiple of 16)
+    // (every wave makes the first pass, whatever the span: the barrier inside is the workgroup's)
+    int piece0 = wave;
+    do {
       v4i preg[NPL];
 #pragma unroll
       for (int u = 0; u < NPL; ++u) {
-        if (pr < total_rows) {
-          const bool ok = xoff >= 0;
-          const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-              (void *)(a.x + (ok ? (uint32_t)xoff + (uint32_t)(k << 10) : 0u)), 0, ok ? row_bytes - (k << 10) : 0, 0x00020000);
-          preg[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(rs, lane16, 0, 0);
-          if (++k == kpr) {
-            k = 0; pr += NWAVES;
-            xoff = row_offset(pr);
-          }
-        }
+        const int off = (piece0 + u * NWAVES) << 10;
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc((void *)(span + min(off, span_bytes)), 0, max(span_bytes - off, 0), 0x00020000);
+        preg[u] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(rs, lane16, 0, 0);
       }
-      pr = pr_first; k = k_first;
+      if (piece0 == wave) {
+        // (first pass only) the zeros, and the barrier that orders them before the data
+        for (int q = tid; q < total_chunks; q += NT) *reinterpret_cast<v4i *>(patch + q * 16) = v4i{0, 0, 0, 0};
+        __syncthreads();
+      }
 #ifdef TPUHIP_TRACE
-      if (pr_first == wave) TPUHIP_TS(14);
+      if (piece0 == wave) TPUHIP_TS(14);
 #endif
 #pragma unroll
       for (int u = 0; u < NPL; ++u) {
-        if (pr < total_rows) {
-          const int p = lane + (k << 6);
-          if (p < (a.iw << cshift))
-            *reinterpret_cast<v4i *>(patch + pr * rowb + (k << 10) + lds_lane + ((p >> cshift) << 4)) = preg[u];
+        const int c = ((piece0 + u * NWAVES) << 6) + lane;                 // chunk of the span
+        const int g = (int)__umulhi((uint32_t)c, a.magic_c16);            // its row in the span
+        const int p = c - g * chunks_in;
+        // patch row: a single image's span begins at patch row row_f - (r0 - 1); whole images
+        // have a border row before and after each
+        const int pr = imgs > 1 ? g + 1 + 2 * (int)__umulhi((uint32_t)g, a.magic_kw) : g + row_f - (r0 - 1);
+        if (c < span_chunks)
+          *reinterpret_cast<v4i *>(patch + pr * rowb + prow + p * 16 + ((p >> cshift) << 4)) = preg[u];
 #ifdef TPUHIP_TRACE
-          if (pr_first == wave && u == 0) TPUHIP_TS(15);
-          if (pr_first == wave && u == 7) TPUHIP_TS(16);
+        if (piece0 == wave && u == 0) TPUHIP_TS(15);
+        if (piece0 == wave && u == 7) TPUHIP_TS(16);
 #endif
-          if (++k == kpr) { k = 0; pr += NWAVES; }
-        }
       }
-    }
+      piece0 += NWAVES * NPL;
+    } while (piece0 < pieces);
   }
 
   if (tid < BM) {
@@ -3503,8 +3496,6 @@ Patch3Plan patch3_plan(const tpuhip_conv_desc &d, const TileCfg &c) {
     const int tiles = (d.oh + th - 1) / th;      // evened out over the image
     pl.th = (d.oh + tiles - 1) / tiles;
   }
-  // the kernel's small divisions: patch row / (th + 2) and pixel slot / (oh * ow)
-  if (pl.imgs * (pl.th + 2) * (pl.th + 2) >= 65536) return Patch3Plan{};
   pl.lds = (unsigned)lds_bytes(pl.th, pl.imgs);
   return pl;
 }
@@ -3821,9 +3812,9 @@ void fill_args(const tpuhip_ctx *ctx, const tpuhip_conv_weights *w, const void *
       int lgc = 6;
       while ((1 << lgc) < d.ic) ++lgc;
       a.pstep_oh = lgc;                                                          // log2(C)
-      const uint32_t rowchunks = (uint32_t)a.stem_pw * (uint32_t)(d.ic / 16);
+      const uint32_t rowchunks = (uint32_t)d.iw * (uint32_t)(d.ic / 16);
       a.magic_c16 = (uint32_t)(((1ull << 32) + rowchunks - 1) / rowchunks);      // q / rowchunks == umulhi(q, magic), q < 2^16
-      a.magic_pw = 65536u / (uint32_t)(pl.th + 2) + 1;                           // patch row / (th + 2)
+      a.magic_kw = (uint32_t)(((1ull << 32) + (uint64_t)d.oh - 1) / (uint64_t)d.oh);   // span row / H
       a.magic_oh = (uint32_t)(((1ull << 32) + (uint64_t)(d.oh * d.ow) - 1) / (uint64_t)(d.oh * d.ow));
       a.pstep_ow = (int)pl.lds;                                                  // dynamic LDS of the launch
     }
