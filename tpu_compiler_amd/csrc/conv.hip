@@ -2175,14 +2175,31 @@ conv_depthwise_rows_kernel(ConvArgs a, DwRowsArgs r) {
   const int slot = n_cb == 1 ? gw : (int)__umulhi((uint32_t)gw, a.magic_c16);   // gw / n_cb (the host set magic_c16 for it)
   const int cb = gw - slot * n_cb;
   const bool relu = a.lo == 0;
+  // Everything the wave fetches before its first block -- the parameters of its 32 channels, the
+  // fused table, the filter fragments -- is requested in one go and parked afterwards: one trip
+  // to memory, not one per array (a load under its own condition is waited for where it stands).
+  // The parameter arrays are padded past the last channel block, so every lane may read them.
+  const int32_t *c64 = relu ? a.qc64r : a.qc64;
+  const int32_t qv0 = c64[2 * (cb * 32) + lane];
+  const int32_t qv1 = a.qmult[cb * 32 + p], qv2 = a.qshift[cb * 32 + p], qv3 = a.qhpot[cb * 32 + p];
+  uint32_t lutv = 0;
+  if (a.has_lut && threadIdx.x < 64) lutv = a.lut.w[threadIdx.x];
+  const int taps = a.kh * a.kw;
+  const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + (size_t)cb * taps * 64 + lane;
+  v4i areg[3][3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+      areg[i][j] = (i < a.kh && j < a.kw) ? afrag[(i * a.kw + j) * 64] : v4i{0, 0, 0, 0};
+  __builtin_amdgcn_sched_barrier(0);
   {
     int32_t *q = qlds[wave];
-    const int32_t *c64 = relu ? a.qc64r : a.qc64;
-    q[lane] = c64[2 * (cb * 32) + lane];
-    q[64 + lane] = lane < 32 ? a.qmult[cb * 32 + lane] : a.qshift[cb * 32 + lane - 32] - (relu ? 1 : 0);
-    if (lane < 32) q[128 + lane] = a.qhpot[cb * 32 + lane];
+    q[lane] = qv0;
+    q[64 + lane] = fk == 0 ? qv1 : qv2 - (relu ? 1 : 0);
+    if (fk == 0) q[128 + lane] = qv3;
   }
-  if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = a.lut.w[threadIdx.x];
+  if (a.has_lut && threadIdx.x < 64) lutw[threadIdx.x] = lutv;
   __syncthreads();
   if (slot >= nslots) return;                               // no barrier below
   int b = xcd * per_xcd + slot;
@@ -2192,14 +2209,6 @@ conv_depthwise_rows_kernel(ConvArgs a, DwRowsArgs r) {
   const bool ch_ok = oc < a.ocw;
   const __amdgpu_buffer_rsrc_t xrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
-  const int taps = a.kh * a.kw;
-  const v4i *afrag = reinterpret_cast<const v4i *>(a.w) + (size_t)cb * taps * 64 + lane;
-  v4i areg[3][3];
-#pragma unroll
-  for (int i = 0; i < 3; ++i)
-#pragma unroll
-    for (int j = 0; j < 3; ++j)
-      areg[i][j] = (i < a.kh && j < a.kw) ? afrag[(i * a.kw + j) * 64] : v4i{0, 0, 0, 0};
   const int32_t *q = qlds[wave];
   const int32_t *pc64 = q + fk * 32, *pmult = q + 64 + fk * 16, *pshift = q + 96 + fk * 16, *phpot = q + 128 + fk * 16;
 
@@ -2341,12 +2350,17 @@ conv_stem_kernel(ConvArgs a) {
   const int frow = lane & 31, fk = lane >> 5;
   const int ib = SPLIT ? (wave & 1) : 0;                  // first channel block of this wave
   const int pbase = SPLIT ? (wave >> 1) * 64 : wave * 32; // first pixel of this wave in the tile
-  for (int e = tid; e < 4 * TM * 32; e += 256) {
-    const int k = e / (TM * 32), c = e - k * (TM * 32);
-    const int32_t *src = k == 0 ? a.bias : k == 1 ? a.qmult : k == 2 ? a.qshift : a.qhpot;
-    qlds[k][c] = src[c];
+  // parameters, table and filter fragments are requested together and parked afterwards (one
+  // trip to memory; a thread holds one of the 4 * TM * 32 <= 256 parameter words)
+  static_assert(4 * TM * 32 <= 256, "one parameter word per thread");
+  int32_t qv = 0;
+  const int qk = tid / (TM * 32), qc = tid - qk * (TM * 32);
+  if (tid < 4 * TM * 32) {
+    const int32_t *src = qk == 0 ? a.bias : qk == 1 ? a.qmult : qk == 2 ? a.qshift : a.qhpot;
+    qv = src[qc];
   }
-  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  uint32_t lutv = 0;
+  if (a.has_lut && tid < 64) lutv = a.lut.w[tid];
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
   const OutRoute out{a.y, a.y_cs, a.lo, 0};
 
@@ -2358,6 +2372,9 @@ conv_stem_kernel(ConvArgs a) {
 #pragma unroll
       for (int r = 0; r < KH; ++r) areg[i][r] = afrag[((ib + i) * KH + r) * 64];
   }
+  __builtin_amdgcn_sched_barrier(0);
+  if (tid < 4 * TM * 32) qlds[qk][qc] = qv;
+  if (a.has_lut && tid < 64) lutw[tid] = lutv;
   const __amdgpu_buffer_rsrc_t xrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.x, 0, a.x_bytes, 0x00020000);
   const int nseg = (a.ow + 127) >> 7;
