@@ -579,6 +579,8 @@ PATCH3_CASES = PATCH_CASES + [
     (2, 1024, 3, 3, 64, True, False),
     (7, 64, 6, 6, 96, True, False),        # 18 K slices: shares of 5, 5, 4 and 4
     (1, 256, 16, 16, 32, False, False),    # exactly 256 pixels
+    (8, 128, 1, 30, 20, False, False),     # images of one row, several per tile (a division by H = 1)
+    (9, 64, 1, 1, 40, True, False),        # images of one pixel (a division by H * W = 1)
 ]
 
 

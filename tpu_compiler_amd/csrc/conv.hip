@@ -1837,7 +1837,8 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
         const int p = c - g * chunks_in;
         // patch row: a single image's span begins at patch row row_f - (r0 - 1); whole images
         // have a border row before and after each
-        const int pr = imgs > 1 ? g + 1 + 2 * (int)__umulhi((uint32_t)g, a.magic_kw) : g + row_f - (r0 - 1);
+        // (x / d by umulhi(x, ceil(2^32 / d)) has no constant for d == 1)
+        const int pr = imgs > 1 ? g + 1 + 2 * (a.ih == 1 ? g : (int)__umulhi((uint32_t)g, a.magic_kw)) : g + row_f - (r0 - 1);
         if (c < span_chunks)
           *reinterpret_cast<v4i *>(patch + pr * rowb + prow + p * 16 + ((p >> cshift) << 4)) = preg[u];
 #ifdef TPUHIP_TRACE
@@ -1867,7 +1868,7 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
 #pragma unroll
   for (int j = 0; j < NB2; ++j) {
     const int p = (pg * NB2 + j) * 32 + frow;
-    const int il = imgs > 1 ? (int)__umulhi((uint32_t)p, a.magic_oh) : 0;   // p / (H * W)
+    const int il = imgs > 1 ? (ohow == 1 ? p : (int)__umulhi((uint32_t)p, a.magic_oh)) : 0;   // p / (H * W)
     const int rem = p - il * ohow;
     const uint32_t pr = a.ow == 1 ? (uint32_t)rem : __umulhi((uint32_t)rem, a.magic_ow);
     const int pc = rem - (int)pr * a.ow;
