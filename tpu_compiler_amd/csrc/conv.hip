@@ -563,6 +563,11 @@ template <int BM, int BN, int WM, int WN, int BK, int DEPTH, int OCC, bool PERSI
           int MODE>
 __global__ __launch_bounds__(WM *WN * 64) __attribute__((amdgpu_waves_per_eu(OCC > 0 ? OCC : 1))) void
 conv_mfma_kernel(ConvArgs a) {
+#ifdef TPUHIP_TRACE
+  unsigned long long ts[32] = {};
+  bool first_tile = true;
+#endif
+  TPUHIP_TS(0);
   gather_conv_args(a);
   gather_conv_args_more(a);
   constexpr bool UNI = MODE == kModeUniform;
@@ -837,8 +842,14 @@ conv_mfma_kernel(ConvArgs a) {
         }
       }
     }
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(1);
+#endif
     store_tile(0, 0);
     __syncthreads();
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(2);
+#endif
     read_frag(0, 0, 0);
 
     // Whole groups of DEPTH steps: ring slots and LDS buffers are compile-time indices
@@ -859,6 +870,9 @@ conv_mfma_kernel(ConvArgs a) {
     for (int d = 0; d < DEPTH - 1; ++d)
       if (d < rem) step_body(d);
 
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(27);
+#endif
     const int pix_done = pix0;
     bool more = false;
     if (PERSIST) {
@@ -891,8 +905,23 @@ conv_mfma_kernel(ConvArgs a) {
     else
       stage_rows<TM, TN, BM, FAST>(acc, a.relu_first, out.lo, stage, wn * TN * 32 + frow, lch0,
                                    a.qmult + ocw0, a.qshift + ocw0, a.qhpot + ocw0);
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(28);
+#endif
     __syncthreads();
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(29);
+#endif
     flush_tile<BM, BN, NT>(a, stage, tid, pix_done, a.npix, oc0, out, lut, sv);
+#ifdef TPUHIP_TRACE
+    if (first_tile) TPUHIP_TS(30);
+    first_tile = false;
+    if (!PERSIST || !more) {
+      ts[31] = (unsigned long long)clock64();
+      if (a.trace && (tid & 63) == 0)
+        for (int kq = 0; kq < 32; ++kq) a.trace[((size_t)blockIdx.x * 8 + (tid >> 6)) * 32 + kq] = ts[kq];
+    }
+#endif
     if (!PERSIST || !more) break;
     __syncthreads();   // the next tile's first K tile lands where the staged bytes are still read
   }
