@@ -1733,13 +1733,19 @@ conv_patch2_kernel(ConvArgs a) {
 //     own, a barrier, and the owner of a block (wave j & 3 for block j) adds the three others';
 //   * requantisation and the staged, row-ordered output as in the other LDS kernels (fused
 //     table and add included).
+// OB = 2: the workgroup computes 64 channels, every wave two A fragments per slice against the
+// same NBLK B fragments (2 * NBLK MFMAs per NBLK + 2 operand reads).  A workgroup then fetches
+// its patch once for twice the channels: on maps whose patch is large against the filter slice
+// (19x19 x 512 channels: 134 KB per tile) the launch is bound by what the CUs can pull out of
+// L2, patches and filter fragments together, and this form moves about half of it.  The partial
+// sums meet in one round per channel block (the space holds one block's guests).
 //   a.stem_pw = W + 2, a.pstep_pix = TH (rows of a tile), a.pstep_n = tiles per image,
 //   a.tile_imgs = whole images per tile (1: a tile is TH rows of one image),
 //   a.pstep_oh = log2(C), a.magic_c16 = ceil(2^32 / 16-byte chunks of an input row),
 //   a.magic_kw = ceil(2^32 / H), a.magic_oh = ceil(2^32 / (H * W)), a.pstep_ow = LDS bytes
 // LDS (dynamic): parameters | table | patch, then the partial sums, then the staged tile.
 // ---------------------------------------------------------------------------
-template <int NB2, int PW>
+template <int NB2, int PW, int OB>
 __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
 #ifdef TPUHIP_TRACE
   unsigned long long ts[32] = {};
@@ -1748,8 +1754,8 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
   gather_conv_args(a);
   gather_conv_args_more(a);
   // 4 * PW waves: wave = pixel group * 4 + K group; a pixel group is NB2 blocks of 32 pixel slots
-  constexpr int NT = 256 * PW, NWAVES = 4 * PW, BM = 32, BN = NB2 * PW * 32;
-  constexpr int U = 8;     // A fragments in flight per wave (even)
+  constexpr int NT = 256 * PW, NWAVES = 4 * PW, BM = 32 * OB, BN = NB2 * PW * 32;
+  constexpr int U = OB == 1 ? 8 : 4;   // K slices in flight per wave (even), OB A fragments each
   constexpr int NPL = 16 / PW;  // pieces of the input span per wave and pass
   extern __shared__ __attribute__((aligned(16))) v4i p3_smem[];
   int32_t *const qlds = reinterpret_cast<int32_t *>(p3_smem);                 // 5 * BM dwords
@@ -1805,16 +1811,20 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
   // ---- the filter: slice sl of this channel block is the 1 KB fragment (ocb * nsl + sl)
   const int nsl = a.kp >> 5;
   const int trips = nb > 0 ? (nsl - kg + 3) >> 2 : 0;   // slices kg, kg + 4, ... below nsl
-  const uint32_t wlane = (uint32_t)lane * 16u;
-  const uint32_t wblock = (uint32_t)ocb * (uint32_t)nsl * 1024u;
+  uint32_t wlane = (uint32_t)lane * 16u;
+  asm volatile("" : "+v"(wlane));
+  const uint32_t wblock = (uint32_t)(ocb * OB) * (uint32_t)nsl * 1024u;   // block ob of the tile: nsl KB further each
   // (a request past the wave's last slice repeats the last one: same loads every trip, never used)
-  auto load_A = [&](int i) {
+  auto load_A = [&](v4i (&dst)[OB], int i) {
     const int sl = kg + 4 * min(i, trips - 1);
-    return (v4i)__builtin_amdgcn_raw_buffer_load_b128(trips > 0 ? wrsrc : wnone, wlane, wblock + (uint32_t)sl * 1024u, 0);
-  };
-  v4i af[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) af[u] = load_A(u);
+    for (int ob = 0; ob < OB; ++ob)
+      dst[ob] = (v4i)__builtin_amdgcn_raw_buffer_load_b128(trips > 0 ? wrsrc : wnone, wlane,
+                                                           wblock + (uint32_t)(ob * nsl + sl) * 1024u, 0);
+  };
+  v4i af[U][OB];
+#pragma unroll
+  for (int u = 0; u < U; ++u) load_A(af[u], u);
 
   // ---- the patch.  Patch row pr (image pr / th2 of the tile, input row r0 - 1 + pr % th2) is pw
   // positions of C bytes; positions 1 .. W are the input row (W * C contiguous bytes), the
@@ -1907,11 +1917,13 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
   __syncthreads();   // the patch and the parameters are in place
   TPUHIP_TS(2);
 
-  v16i acc[NB2];
+  v16i acc[OB][NB2];
 #pragma unroll
-  for (int j = 0; j < NB2; ++j)
+  for (int ob = 0; ob < OB; ++ob)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[j][e] = 0;
+    for (int j = 0; j < NB2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[ob][j][e] = 0;
 
   // The wave's slices advance by 128 bytes of K: the channel offset c0 within the tap and the
   // tap's patch offset are kept as scalars (taps past the ninth -- one read ahead of the last
@@ -1948,12 +1960,16 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
       if (i0 == 0) ts[3 + u] = (unsigned long long)clock64();
 #endif
       read_B((u + 1) & 1);
-      const v4i afr = af[u];
-      af[u] = load_A(i0 + u + U);
+      v4i afr[OB];
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob) afr[ob] = af[u][ob];
+      load_A(af[u], i0 + u + U);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int j = 0; j < NB2; ++j)
-        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr, bf[u & 1][j], acc[j], 0, 0, 0);
+#pragma unroll
+        for (int ob = 0; ob < OB; ++ob)
+          acc[ob][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(afr[ob], bf[u & 1][j], acc[ob][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -1964,7 +1980,9 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < NB2; ++j)
-      acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u], bf[u & 1][j], acc[j], 0, 0, 0);
+#pragma unroll
+      for (int ob = 0; ob < OB; ++ob)
+        acc[ob][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[u][ob], bf[u & 1][j], acc[ob][j], 0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
   }
 
@@ -1975,45 +1993,54 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
   flush_prefetch<BM, BN, NT>(a, tid, pix_base, pix_limit, oc0, out, sv);
   __syncthreads();   // every wave is done with the patch
   v4i *const red = reinterpret_cast<v4i *>(patch) + pg * (NB2 * 3 * 4 * 64);   // [block][3 guests][4 quads][64 lanes]
+  // (one round per channel block of the wave: the space holds the guests' sums of NB2 blocks)
 #pragma unroll
-  for (int j = 0; j < NB2; ++j) {
-    if ((j & 3) != kg && j < nb) {
-      const int slot = (kg - (j & 3) - 1) & 3;
+  for (int ob = 0; ob < OB; ++ob) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        red[((j * 3 + slot) * 4 + q) * 64 + lane] = v4i{acc[j][q * 4], acc[j][q * 4 + 1], acc[j][q * 4 + 2], acc[j][q * 4 + 3]};
+    for (int j = 0; j < NB2; ++j) {
+      if ((j & 3) != kg && j < nb) {
+        const int slot = (kg - (j & 3) - 1) & 3;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          red[((j * 3 + slot) * 4 + q) * 64 + lane] =
+              v4i{acc[ob][j][q * 4], acc[ob][j][q * 4 + 1], acc[ob][j][q * 4 + 2], acc[ob][j][q * 4 + 3]};
+      }
     }
-  }
-  __syncthreads();
+    __syncthreads();
 #pragma unroll
-  for (int j = 0; j < NB2; ++j) {
-    if ((j & 3) == kg && j < nb) {
+    for (int j = 0; j < NB2; ++j) {
+      if ((j & 3) == kg && j < nb) {
 #pragma unroll
-      for (int slot = 0; slot < 3; ++slot)
+        for (int slot = 0; slot < 3; ++slot)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4i v = red[((j * 3 + slot) * 4 + q) * 64 + lane];
-          acc[j][q * 4] += v[0]; acc[j][q * 4 + 1] += v[1]; acc[j][q * 4 + 2] += v[2]; acc[j][q * 4 + 3] += v[3];
-        }
+          for (int q = 0; q < 4; ++q) {
+            const v4i v = red[((j * 3 + slot) * 4 + q) * 64 + lane];
+            acc[ob][j][q * 4] += v[0]; acc[ob][j][q * 4 + 1] += v[1]; acc[ob][j][q * 4 + 2] += v[2]; acc[ob][j][q * 4 + 3] += v[3];
+          }
+      }
     }
+    __syncthreads();   // the partial sums are read: their space takes the next round's, then the staged tile
   }
-  __syncthreads();   // the partial sums are read: their space takes the staged tile
   TPUHIP_TS(28);
 
-  // ---- requantisation into the staging area, then out in memory order
+  // ---- requantisation into the staging area, then out in memory order (a lane's 16 results of
+  // channel block ob are channels fk * 16 * OB + ob * 16 ... of the tile: see mfma_row_to_oc)
   int8_t *const stage = patch;
-  const int lc = fk * 16;
 #pragma unroll
-  for (int j = 0; j < NB2; ++j) {
-    if ((j & 3) == kg && j < nb) {
-      const v16i one[1] = {acc[j]};
-      uint32_t outw[1][4];
-      if (relu)
-        requant_rows_c64<1, true>(one, 0, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
-      else
-        requant_rows_c64<1, false>(one, a.lo, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
-      *reinterpret_cast<v4i *>(stage + ((pg * NB2 + j) * 32 + frow) * stage_row_bytes<BM>() + lc) =
-          v4i{(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+  for (int ob = 0; ob < OB; ++ob) {
+    const int lc = fk * 16 * OB + ob * 16;
+#pragma unroll
+    for (int j = 0; j < NB2; ++j) {
+      if ((j & 3) == kg && j < nb) {
+        const v16i one[1] = {acc[ob][j]};
+        uint32_t outw[1][4];
+        if (relu)
+          requant_rows_c64<1, true>(one, 0, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
+        else
+          requant_rows_c64<1, false>(one, a.lo, qlds + 2 * lc, qlds + 2 * BM + lc, qlds + 3 * BM + lc, qlds + 4 * BM + lc, outw);
+        *reinterpret_cast<v4i *>(stage + ((pg * NB2 + j) * 32 + frow) * stage_row_bytes<BM>() + lc) =
+            v4i{(int)outw[0][0], (int)outw[0][1], (int)outw[0][2], (int)outw[0][3]};
+      }
     }
   }
   __syncthreads();
@@ -3336,16 +3363,20 @@ struct TileCfg {
   V(46, "mfma_patch2_32x128", 32, 128, 1, 4, 256, 2) \
   V(47, "mfma_patch2_128x256_w8_k256", 128, 256, 4, 2, 256, 2) \
   V(48, "mfma_patch2_128x256_w8t_k256", 128, 256, 2, 4, 256, 2) \
-  V(49, "mfma_patch2_128x256_w8t", 128, 256, 2, 4, 128, 2)
+  V(49, "mfma_patch2_128x256_w8t", 128, 256, 2, 4, 128, 2) \
+  V(55, "mfma_patch2_256x256_w8", 256, 256, 2, 4, 128, 2) \
+  V(56, "mfma_patch2_128x192_w8", 128, 192, 4, 2, 256, 2)
 
 // row-patch kernels, third form (3x3 / stride 1 / pad 1, the four waves split K, 32 channels per
-// workgroup): U(index, name, pixel blocks of a tile)
+// workgroup, or 64: two channel blocks per wave): U3(index, name, pixel blocks of a pixel group, pixel groups, channel blocks)
 #define TPUHIP_PATCH3_TILES(U3)               \
-  U3(50, "mfma_patch3_32x128", 4, 1)          \
-  U3(51, "mfma_patch3_32x224", 7, 1)          \
-  U3(52, "mfma_patch3_32x256", 8, 1)          \
-  U3(53, "mfma_patch3_32x128_w8", 2, 2)       \
-  U3(54, "mfma_patch3_32x256_w8", 4, 2)
+  U3(50, "mfma_patch3_32x128", 4, 1, 1)       \
+  U3(51, "mfma_patch3_32x224", 7, 1, 1)       \
+  U3(52, "mfma_patch3_32x256", 8, 1, 1)       \
+  U3(53, "mfma_patch3_32x128_w8", 2, 2, 1)    \
+  U3(54, "mfma_patch3_32x256_w8", 4, 2, 1)    \
+  U3(57, "mfma_patch3_64x256_w8", 4, 2, 2)    \
+  U3(58, "mfma_patch3_64x192_w8", 3, 2, 2)
 
 struct TileTable {
   TileCfg t[64];
@@ -3376,8 +3407,8 @@ struct TileTable {
   n = n > i ? n : i + 1;
     TPUHIP_PATCH2_TILES(V)
 #undef V
-#define U3(i, name, NB2, PW) \
-  t[i] = TileCfg{32, NB2 * PW * 32, 1, PW, name, 7, 64}; \
+#define U3(i, name, NB2, PW, OB) \
+  t[i] = TileCfg{32 * OB, NB2 * PW * 32, 1, PW, name, 7, 64}; \
   n = n > i ? n : i + 1;
     TPUHIP_PATCH3_TILES(U3)
 #undef U3
@@ -3526,8 +3557,8 @@ Patch3Plan patch3_plan(const tpuhip_conv_desc &d, const TileCfg &c) {
   const int nblk = c.bn / 32;
   auto lds_bytes = [&](int th, int imgs) {
     const int64_t patch = (int64_t)imgs * (th + 2) * ((d.ow + 2) * (d.ic + 16) + kPatch2RowPad);
-    const int64_t red = (int64_t)nblk * 3 * 4096, stage = (int64_t)c.bn * 48;
-    return (int64_t)(5 * 32 * 4 + 256) + std::max(patch, std::max(red, stage));
+    const int64_t red = (int64_t)nblk * 3 * 4096, stage = (int64_t)c.bn * (c.bm + 16);
+    return (int64_t)(5 * c.bm * 4 + 256) + std::max(patch, std::max(red, stage));
   };
   int imgs = std::min(d.n, c.bn / (d.oh * d.ow));
   while (imgs > 1 && lds_bytes(d.oh, imgs) > kLdsBytes) --imgs;
@@ -3549,9 +3580,9 @@ Patch3Plan patch3_plan(const tpuhip_conv_desc &d, const TileCfg &c) {
 
 void launch_patch3(tpuhip_ctx *ctx, int tile, dim3 grid, const ConvArgs &a, unsigned lds) {
   switch (tile) {
-#define U3(i, name, NB2, PW)                                                                            \
+#define U3(i, name, NB2, PW, OB)                                                                        \
   case i: {                                                                                             \
-    auto kernel = conv_patch3_kernel<NB2, PW>;                                                          \
+    auto kernel = conv_patch3_kernel<NB2, PW, OB>;                                                      \
     if (!pw_prepare(kernel, (unsigned)kLdsBytes)) break;                                                \
     if (ctx->prof_start)                                                                                \
       hipExtLaunchKernelGGL(kernel, grid, dim3(256 * PW), lds, ctx->stream, ctx->prof_start, ctx->prof_stop, 0, a); \
