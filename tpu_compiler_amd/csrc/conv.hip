@@ -3345,7 +3345,8 @@ struct TileCfg {
   W(37, "mfma_pw_256x64_k128_w8", 256, 64, 4, 2, 128, 1, 4) \
   W(38, "mfma_pw_128x64_k256_w8", 128, 64, 4, 2, 256, 1, 4) \
   W(39, "mfma_pw_64x128_k64_w8", 64, 128, 2, 4, 64, 2, 4)   \
-  W(40, "mfma_pw_128x64_k64_w8", 128, 64, 4, 2, 64, 2, 4)
+  W(40, "mfma_pw_128x64_k64_w8", 128, 64, 4, 2, 64, 2, 4)   \
+  W(59, "mfma_pw_96x128_k64", 96, 128, 1, 4, 64, 2, 3)
 
 // row-patch kernels, second form (3x3 / stride 1 / pad 1, 64 to 1024 input channels, a power of two):
 // V(index, name, BM, BN, WM, WN, BK, waves per SIMD)
