@@ -1506,6 +1506,20 @@ conv_patch2_kernel(ConvArgs a) {
   const __amdgpu_buffer_rsrc_t wrsrc =
       __builtin_amdgcn_make_buffer_rsrc((void *)a.w, 0, a.w_bytes, 0x00020000);
 
+  // the requantisation parameters and the fused table are requested first and parked last: loads
+  // return in order, and nothing then waits for these alone
+  int32_t qv[5] = {0, 0, 0, 0, 0};
+  uint32_t lutv = 0;
+  if (tid < BM) {
+    const int32_t *c64 = relu ? a.qc64r : a.qc64;
+    qv[0] = c64[2 * (oc0 + tid)];
+    qv[1] = c64[2 * (oc0 + tid) + 1];
+    qv[2] = a.qmult[oc0 + tid];
+    qv[3] = a.qshift[oc0 + tid];
+    qv[4] = a.qhpot[oc0 + tid];
+  }
+  if (a.has_lut && tid < 64) lutv = a.lut.w[tid];
+
   // ---- the patch: row r of it is pw positions of C bytes = pw * C / 16 chunks, of which chunk
   // p lies at byte (p - C / 16) * 16 of input row r0 - 1 + r (the first and last position are
   // the zero border)
@@ -1556,15 +1570,6 @@ conv_patch2_kernel(ConvArgs a) {
 #pragma unroll
   for (int d = 0; d < RD; ++d) load_A(d, d);
 
-  if (tid < BM) {
-    const int32_t *c64 = relu ? a.qc64r : a.qc64;
-    qlds[2 * tid] = c64[2 * (oc0 + tid)];
-    qlds[2 * tid + 1] = c64[2 * (oc0 + tid) + 1];
-    qlds[2 * BM + tid] = a.qmult[oc0 + tid];
-    qlds[3 * BM + tid] = a.qshift[oc0 + tid] - (relu ? 1 : 0);
-    qlds[4 * BM + tid] = a.qhpot[oc0 + tid];
-  }
-  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
 
   const int frow = lane & 31;
@@ -1591,6 +1596,14 @@ conv_patch2_kernel(ConvArgs a) {
     if (q < n_chunks)
       *reinterpret_cast<v4i *>(patch + pr * rowb + (p >> (lgc - 4)) * prow + (p & ((C >> 4) - 1)) * 16) = preg[u];
   }
+  if (tid < BM) {
+    qlds[2 * tid] = qv[0];
+    qlds[2 * tid + 1] = qv[1];
+    qlds[2 * BM + tid] = qv[2];
+    qlds[3 * BM + tid] = qv[3] - (relu ? 1 : 0);
+    qlds[4 * BM + tid] = qv[4];
+  }
+  if (a.has_lut && tid < 64) lutw[tid] = lutv;
   TPUHIP_TS(1);
   store_A(0, 0);
   __syncthreads();
@@ -1807,6 +1820,8 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
     qv[3] = a.qshift[oc0 + tid];
     qv[4] = a.qhpot[oc0 + tid];
   }
+  uint32_t lutv = 0;
+  if (a.has_lut && tid < 64) lutv = a.lut.w[tid];
 
   // ---- the filter: slice sl of this channel block is the 1 KB fragment (ocb * nsl + sl)
   const int nsl = a.kp >> 5;
@@ -1896,7 +1911,7 @@ __global__ __launch_bounds__(256 * PW) void conv_patch3_kernel(ConvArgs a) {
     qlds[3 * BM + tid] = qv[3] - (relu ? 1 : 0);
     qlds[4 * BM + tid] = qv[4];
   }
-  if (a.has_lut && tid < 64) lutw[tid] = a.lut.w[tid];
+  if (a.has_lut && tid < 64) lutw[tid] = lutv;
   const uint8_t *lut = a.has_lut ? reinterpret_cast<const uint8_t *>(lutw) : nullptr;
 
   const int frow = lane & 31;
