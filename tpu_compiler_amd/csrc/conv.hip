@@ -666,7 +666,13 @@ conv_mfma_kernel(ConvArgs a) {
       const int n = n_first + (int)q2;
       ih0[s] = pv ? oh * a.sh - a.pt : -(1 << 28);   // an invalid pixel never passes the bounds test
       iw0[s] = ow * a.sw - a.pl;
-      poff[s] = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[s]) * a.x_cs + (UNI ? kc * 16 : 0);
+      // (the product is pinned before the chunk offset is added: left to itself the compiler forms a
+      // 64-bit multiply-add whose upper addend register is undefined, picks one that a parameter
+      // load above is still due to write, and waits for that load before the first tile load is
+      // issued -- a trip to memory for a value nobody reads)
+      int pixel_bytes = ((n * a.ih + (oh * a.sh - a.pt)) * a.iw + iw0[s]) * a.x_cs;
+      asm volatile("" : "+v"(pixel_bytes));
+      poff[s] = pixel_bytes + (UNI ? kc * 16 : 0);
       // keep the three values in registers instead of recomputing them every K step
       asm volatile("" : "+v"(poff[s]), "+v"(ih0[s]), "+v"(iw0[s]));
     }
@@ -2873,14 +2879,25 @@ conv_mfma_reg_kernel(ConvArgs a) {
     }
   };
 
+  // (the bias is requested, then the first K steps, and only then does it go into the accumulators:
+  // one trip to memory before the first MFMA, not two)
   v16i acc[TM][TN];
   const int ocw0 = oc0 + fk * 16 * TM;
+  v4i bias4[TM][4];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
 #pragma unroll
+    for (int q = 0; q < 4; ++q) bias4[i][q] = bp[q];
+  }
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const v4i b = bp[q];
+      const v4i b = bias4[i][q];
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         acc[i][j][q * 4 + 0] = b[0];
@@ -2890,9 +2907,6 @@ conv_mfma_reg_kernel(ConvArgs a) {
       }
     }
   }
-
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
 
   auto mfma_step = [&](int slot) {
 #pragma unroll
@@ -3039,14 +3053,26 @@ conv_mfma_splitk_kernel(ConvArgs a) {
     }
   };
 
+  // the bias is requested, then the first K steps, and only then does the bias go into the
+  // accumulators: taken the other way round the first operand loads leave after the bias has
+  // come back, two trips to memory in a row
   v16i acc[TM][TN];
   const int ocw0 = oc0 + fk * 16 * TM;
+  v4i bias4[TM][4];
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const v4i *bp = reinterpret_cast<const v4i *>(a.bias + ocw0 + i * 16);
 #pragma unroll
+    for (int q = 0; q < 4; ++q) bias4[i][q] = bp[q];
+  }
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
     for (int q = 0; q < 4; ++q) {
-      v4i b = bp[q];
+      v4i b = bias4[i][q];
       if (wave != 0) b = v4i{0, 0, 0, 0};
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -3057,9 +3083,6 @@ conv_mfma_splitk_kernel(ConvArgs a) {
       }
     }
   }
-
-#pragma unroll
-  for (int d = 0; d < DEPTH; ++d) load_step(d, d);
 
   auto mfma_step = [&](int slot) {
 #pragma unroll
